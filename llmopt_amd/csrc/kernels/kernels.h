@@ -1,0 +1,121 @@
+// Host-visible launch interface of the HIP kernels.  Plain structs and raw
+// device pointers; every launcher is asynchronous on the given stream and
+// assumes the caller has validated shapes and buffer sizes.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace llmopt {
+
+// One packed W4 matrix: weight u8 [n, k/2] row-major, scale f16 [n, k/64].
+struct W4Matrix {
+  const uint8_t *weight;
+  const uint16_t *scale;
+};
+
+// y[r, c] = half(sum_k x[r,k] * q[c,k] * s[c,k/64] (+ addend[r*addend_row_stride + c]))
+// Semantics of llmopt_w4a16_linear_f16_g64{,_m4,_m8}
+// (lib/metal_w4a16_source.ml:8-194): addend is a bias when the stride is 0 and a
+// residual when it is n.
+struct W4LinearArgs {
+  const uint16_t *x;  // f16 [m, k]
+  W4Matrix w;
+  const uint16_t *addend;  // may be null when has_addend == 0
+  uint32_t has_addend;
+  uint32_t addend_row_stride;
+  uint16_t *y;  // f16 [m, n]
+  uint32_t m, n, k;
+};
+
+// Three projections of one activation in one launch
+// (llmopt_w4a16_qkv_linear_f16_g64*, lib/metal_w4a16_source.ml:218-480).
+struct W4QkvArgs {
+  const uint16_t *x;  // f16 [m, k]
+  W4Matrix w[3];
+  uint16_t *y[3];  // f16 [m, n[i]]
+  uint32_t n[3];
+  uint32_t m, k;
+};
+
+// product[r, c] = half(silu(gate[r,c]) * up[r,c]) with gate, up fp32
+// (llmopt_w4a16_dual_swiglu_f16_g64*, lib/metal_w4a16_source.ml:533-577).
+struct W4DualSwigluArgs {
+  const uint16_t *x;  // f16 [m, k]
+  W4Matrix gate, up;  // each [n, k/2]
+  uint16_t *product;  // f16 [m, n]
+  uint32_t m, n, k;
+};
+
+hipError_t launch_w4a16_linear(const W4LinearArgs &args, hipStream_t stream);
+hipError_t launch_w4a16_qkv(const W4QkvArgs &args, hipStream_t stream);
+hipError_t launch_w4a16_dual_swiglu(const W4DualSwigluArgs &args, hipStream_t stream);
+
+// Bit-exact dequantisation q * s to float32 [n, k] (debug / parity check of the
+// unpack arithmetic; python/llmopt_backend/quantization.py:91-121).
+hipError_t launch_w4_dequant_f32(const W4Matrix &w, float *out, uint32_t n, uint32_t k,
+                                 hipStream_t stream);
+
+// ---- grouped-Q8 KV cache -----------------------------------------------------
+
+// AttentionCacheParams / AttentionCachePairParams
+// (lib/metal_cache_source.ml:9-34).  For the single-segment kernels only
+// source[0] / segment_offset[0] are used; the pair kernel packs K and V.
+struct Q8PackArgs {
+  const uint16_t *source[2];  // f16 head-major [heads, source_items, head_dim]
+  const uint32_t *slots;      // [items]
+  uint8_t *pool;
+  uint32_t items;
+  uint32_t segment_offset[2];
+  uint32_t heads, head_dim;
+  uint32_t token_elements, token_stride;
+  uint32_t source_items, source_offset;
+};
+
+struct Q8UnpackArgs {
+  const uint8_t *pool;
+  const uint32_t *slots;
+  uint16_t *destination;  // f16 head-major [heads, items, head_dim]
+  uint32_t items;
+  uint32_t segment_offset;
+  uint32_t heads, head_dim;
+  uint32_t token_elements, token_stride;
+};
+
+hipError_t launch_q8_pack(const Q8PackArgs &args, bool pair, hipStream_t stream);
+hipError_t launch_q8_unpack(const Q8UnpackArgs &args, hipStream_t stream);
+
+// Q8PagedAttentionParams (lib/metal_cache_source.ml:352-369) plus the
+// per-sequence extension: when past_lengths is not null, sequence b attends to
+// past_lengths[b] pool tokens whose slot indices start at
+// slots[slot_offsets[b]]; otherwise all sequences share slots[0..past_length)
+// as in the reference kernels (:391,:429).
+struct Q8AttentionArgs {
+  const uint16_t *query;          // f16 [b, h, q, D]
+  const uint16_t *current_key;    // f16 [b, kvh, q, D]
+  const uint16_t *current_value;  // f16 [b, kvh, q, D]
+  const uint8_t *pool;
+  const uint32_t *slots;
+  const uint8_t *mask;  // may be null
+  uint16_t *output;     // f16 token-major [b, q, h, D]
+  const uint32_t *past_lengths;  // extension, may be null
+  const uint32_t *slot_offsets;  // extension, may be null
+  uint32_t batches, query_heads, kv_heads, past_length, head_dim;
+  uint32_t mask_batches, mask_heads, token_elements, key_offset, value_offset;
+  uint32_t token_stride;
+  float scale;
+  uint32_t query_length, mask_dtype, window;
+  uint32_t max_past_length;  // >= every past length (bounds the split grid)
+  void *workspace;           // split-context partials
+  size_t workspace_bytes;
+};
+
+// Bytes of workspace launch_q8_attention needs for these arguments (0 when the
+// row-serial kernel is used).
+size_t q8_attention_workspace_bytes(const Q8AttentionArgs &args);
+hipError_t launch_q8_attention(const Q8AttentionArgs &args, hipStream_t stream);
+
+// The largest m the streaming GEMV path takes; above it the MFMA GEMM runs.
+constexpr uint32_t kGemvMaxRows = 8;
+
+}  // namespace llmopt

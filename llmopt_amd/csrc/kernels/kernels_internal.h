@@ -1,0 +1,19 @@
+// Launchers shared between kernel translation units (not part of the host
+// interface): the m-based choice between the streaming GEMV and the MFMA GEMM
+// is made in w4a16_linear.hip.
+#pragma once
+
+#include "kernels.h"
+
+namespace llmopt {
+
+int device_compute_units();
+
+hipError_t launch_w4a16_gemv_linear(const W4LinearArgs &args, hipStream_t stream);
+hipError_t launch_w4a16_gemv_qkv(const W4QkvArgs &args, hipStream_t stream);
+hipError_t launch_w4a16_gemv_dual_swiglu(const W4DualSwigluArgs &args, hipStream_t stream);
+
+hipError_t launch_w4a16_gemm_linear(const W4LinearArgs &args, hipStream_t stream);
+hipError_t launch_w4a16_gemm_dual_swiglu(const W4DualSwigluArgs &args, hipStream_t stream);
+
+}  // namespace llmopt

@@ -1,0 +1,107 @@
+// Device helpers shared by the W4A16 kernels (gfx950, wave64).
+//
+// Packed format (python/llmopt_backend/quantization.py:63-121, lib/cpu.ml:131-139):
+// byte b of a weight row holds K = 2b in its low nibble and K = 2b + 1 in its
+// high nibble, both two's-complement int4; one fp16 scale per 64 K values.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace llmopt {
+
+typedef _Float16 h2_t __attribute__((ext_vector_type(2)));
+typedef _Float16 h4_t __attribute__((ext_vector_type(4)));
+typedef _Float16 h8_t __attribute__((ext_vector_type(8)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef float f4_t __attribute__((ext_vector_type(4)));
+typedef float f16x_t __attribute__((ext_vector_type(16)));
+
+__device__ __forceinline__ h2_t as_h2(uint32_t bits) {
+  return __builtin_bit_cast(h2_t, bits);
+}
+
+__device__ __forceinline__ uint32_t as_u32(h2_t value) {
+  return __builtin_bit_cast(uint32_t, value);
+}
+
+__device__ __forceinline__ float half_bits_to_float(uint16_t bits) {
+  return (float)__builtin_bit_cast(_Float16, bits);
+}
+
+__device__ __forceinline__ uint16_t float_to_half_bits(float value) {
+  return __builtin_bit_cast(uint16_t, (_Float16)value);  // round to nearest even
+}
+
+// Exact int4 -> fp16 decode of one dword (8 nibbles = K offsets 0..7).
+//
+// XOR with 0x88888888 turns two's complement into offset binary (q + 8).
+// OR-ing a 4-bit field into the mantissa of 1024.0 (0x6400, ulp 1) or of 64.0
+// (0x5400, ulp 1/16, field at bits 4..7) gives 1024 + (q + 8) or 64 + (q + 8)
+// exactly, so one packed subtract yields q.  The four results hold the pairs
+// (k0,k4) (k1,k5) (k2,k6) (k3,k7): the activation is arranged to match.
+struct W4Pairs {
+  h2_t p04, p15, p26, p37;
+};
+
+__device__ __forceinline__ W4Pairs w4_decode_pairs(uint32_t word) {
+  const uint32_t v = word ^ 0x88888888u;
+  const uint32_t hi = v >> 8;
+  const h2_t bias_lo = {(_Float16)1032.0f, (_Float16)1032.0f};
+  const h2_t bias_hi = {(_Float16)72.0f, (_Float16)72.0f};
+  W4Pairs out;
+  out.p04 = as_h2((v & 0x000F000Fu) | 0x64006400u) - bias_lo;
+  out.p15 = as_h2((v & 0x00F000F0u) | 0x54005400u) - bias_hi;
+  out.p26 = as_h2((hi & 0x000F000Fu) | 0x64006400u) - bias_lo;
+  out.p37 = as_h2((hi & 0x00F000F0u) | 0x54005400u) - bias_hi;
+  return out;
+}
+
+// Rearranges 8 consecutive fp16 activations (x0..x7) into the pair order of
+// w4_decode_pairs: {(x0,x4), (x1,x5), (x2,x6), (x3,x7)}.
+__device__ __forceinline__ uint4 pair_order(uint4 x) {
+  uint4 out;
+  out.x = __builtin_amdgcn_perm(x.z, x.x, 0x05040100u);
+  out.y = __builtin_amdgcn_perm(x.z, x.x, 0x07060302u);
+  out.z = __builtin_amdgcn_perm(x.w, x.y, 0x05040100u);
+  out.w = __builtin_amdgcn_perm(x.w, x.y, 0x07060302u);
+  return out;
+}
+
+// Sum over the 64 lanes of a wave with DPP row operations; every lane of each
+// 16-lane row ends with the row sum, then the four row sums are combined.
+__device__ __forceinline__ float wave_sum(float value) {
+  value += __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, value), 0xB1, 0xF, 0xF, false));
+  value += __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, value), 0x4E, 0xF, 0xF, false));
+  value += __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, value), 0x141, 0xF, 0xF, false));
+  value += __builtin_bit_cast(
+      float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, value), 0x140, 0xF, 0xF, false));
+  const int bits = __builtin_bit_cast(int, value);
+  const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 0));
+  const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 16));
+  const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 32));
+  const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 48));
+  return (r0 + r1) + (r2 + r3);
+}
+
+__device__ __forceinline__ float wave_max(float value) {
+  value = fmaxf(value, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+                           0, __builtin_bit_cast(int, value), 0xB1, 0xF, 0xF, false)));
+  value = fmaxf(value, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+                           0, __builtin_bit_cast(int, value), 0x4E, 0xF, 0xF, false)));
+  value = fmaxf(value, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+                           0, __builtin_bit_cast(int, value), 0x141, 0xF, 0xF, false)));
+  value = fmaxf(value, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+                           0, __builtin_bit_cast(int, value), 0x140, 0xF, 0xF, false)));
+  const int bits = __builtin_bit_cast(int, value);
+  const float r0 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 0));
+  const float r1 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 16));
+  const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 32));
+  const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 48));
+  return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
+}
+
+}  // namespace llmopt

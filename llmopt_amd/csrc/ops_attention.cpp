@@ -1,0 +1,246 @@
+// Entry points of the grouped-Q8 KV cache and paged decode attention family:
+// buffer order and parameter-block layout of lib/metal_cache_source.ml:9-34,
+// 46-243,352-583 (host side lib/metal_cache.ml:230-511,
+// lib/metal_dispatch_attention.ml:104-217, lib/metal_parameters.ml:119-140).
+#include "kernels/kernels.h"
+#include "runtime.h"
+
+namespace llmopt {
+namespace {
+
+int launched(hipError_t status, const char *name) {
+  if (status != hipSuccess)
+    return fail(LLMOPT_ERR_FAILURE, "%s launch failed: %s", name, hipGetErrorString(status));
+  return LLMOPT_OK;
+}
+
+int check_cache_geometry(const char *name, uint32_t heads, uint32_t head_dim, uint32_t group_size,
+                         uint32_t token_elements, uint32_t token_stride) {
+  if (group_size != 64)
+    return fail(LLMOPT_ERR_INVALID, "%s supports the Q8 group size 64 only, got %u", name, group_size);
+  if (heads == 0 || head_dim == 0 || head_dim % 64 != 0)
+    return fail(LLMOPT_ERR_INVALID, "%s requires head_dim to be a positive multiple of 64", name);
+  if (token_elements % 64 != 0 || token_stride < token_elements + 2 * (token_elements / 64))
+    return fail(LLMOPT_ERR_INVALID, "%s received an inconsistent Q8 token layout", name);
+  return LLMOPT_OK;
+}
+
+// AttentionCacheParams, 10 x u32 (lib/metal_cache_source.ml:9-20).
+// buffers: source, slots, pool.
+int cache_pack(llmopt_hip_context *context, const DispatchRecord &record) {
+  if (int status = require_buffer_count(record, 3)) return status;
+  if (int status = require_parameter_bytes(record, 40)) return status;
+  Q8PackArgs args = {};
+  args.items = param_u32(record, 0);
+  args.segment_offset[0] = param_u32(record, 4);
+  args.heads = param_u32(record, 8);
+  args.head_dim = param_u32(record, 12);
+  const uint32_t group_size = param_u32(record, 16);
+  args.token_elements = param_u32(record, 20);
+  args.token_stride = param_u32(record, 28);
+  args.source_items = param_u32(record, 32);
+  args.source_offset = param_u32(record, 36);
+  if (int status = check_cache_geometry(record.name.c_str(), args.heads, args.head_dim, group_size,
+                                        args.token_elements, args.token_stride))
+    return status;
+  if (args.segment_offset[0] % 64 != 0 ||
+      (uint64_t)args.segment_offset[0] + (uint64_t)args.heads * args.head_dim > args.token_elements)
+    return fail(LLMOPT_ERR_INVALID, "%s segment lies outside the token", record.name.c_str());
+  if ((uint64_t)args.source_offset + args.items > args.source_items)
+    return fail(LLMOPT_ERR_INVALID, "%s source window lies outside the source", record.name.c_str());
+  if (int status = require_buffer_size(
+          record.buffers[0], (uint64_t)args.heads * args.source_items * args.head_dim * 2, "cache source"))
+    return status;
+  if (int status = require_buffer_size(record.buffers[1], (uint64_t)args.items * 4, "slots")) return status;
+  if (int status = require_buffer_size(record.buffers[2], args.token_stride, "pool")) return status;
+  args.source[0] = reinterpret_cast<const uint16_t *>(record.buffers[0].device);
+  args.slots = reinterpret_cast<const uint32_t *>(record.buffers[1].device);
+  args.pool = record.buffers[2].device;
+  return launched(launch_q8_pack(args, false, context->stream), record.name.c_str());
+}
+
+// AttentionCachePairParams, 11 x u32 (lib/metal_cache_source.ml:22-34).
+// buffers: key_source, value_source, slots, pool.
+int cache_pack_pair(llmopt_hip_context *context, const DispatchRecord &record) {
+  if (int status = require_buffer_count(record, 4)) return status;
+  if (int status = require_parameter_bytes(record, 44)) return status;
+  Q8PackArgs args = {};
+  args.items = param_u32(record, 0);
+  args.segment_offset[0] = param_u32(record, 4);
+  args.segment_offset[1] = param_u32(record, 8);
+  args.heads = param_u32(record, 12);
+  args.head_dim = param_u32(record, 16);
+  const uint32_t group_size = param_u32(record, 20);
+  args.token_elements = param_u32(record, 24);
+  args.token_stride = param_u32(record, 32);
+  args.source_items = param_u32(record, 36);
+  args.source_offset = param_u32(record, 40);
+  if (int status = check_cache_geometry(record.name.c_str(), args.heads, args.head_dim, group_size,
+                                        args.token_elements, args.token_stride))
+    return status;
+  for (int which = 0; which < 2; ++which)
+    if (args.segment_offset[which] % 64 != 0 ||
+        (uint64_t)args.segment_offset[which] + (uint64_t)args.heads * args.head_dim > args.token_elements)
+      return fail(LLMOPT_ERR_INVALID, "%s segment lies outside the token", record.name.c_str());
+  if ((uint64_t)args.source_offset + args.items > args.source_items)
+    return fail(LLMOPT_ERR_INVALID, "%s source window lies outside the source", record.name.c_str());
+  const uint64_t source_bytes = (uint64_t)args.heads * args.source_items * args.head_dim * 2;
+  if (int status = require_buffer_size(record.buffers[0], source_bytes, "key source")) return status;
+  if (int status = require_buffer_size(record.buffers[1], source_bytes, "value source")) return status;
+  if (int status = require_buffer_size(record.buffers[2], (uint64_t)args.items * 4, "slots")) return status;
+  if (int status = require_buffer_size(record.buffers[3], args.token_stride, "pool")) return status;
+  args.source[0] = reinterpret_cast<const uint16_t *>(record.buffers[0].device);
+  args.source[1] = reinterpret_cast<const uint16_t *>(record.buffers[1].device);
+  args.slots = reinterpret_cast<const uint32_t *>(record.buffers[2].device);
+  args.pool = record.buffers[3].device;
+  return launched(launch_q8_pack(args, true, context->stream), record.name.c_str());
+}
+
+// buffers: pool, slots, destination; AttentionCacheParams.
+int cache_unpack(llmopt_hip_context *context, const DispatchRecord &record) {
+  if (int status = require_buffer_count(record, 3)) return status;
+  if (int status = require_parameter_bytes(record, 40)) return status;
+  Q8UnpackArgs args = {};
+  args.items = param_u32(record, 0);
+  args.segment_offset = param_u32(record, 4);
+  args.heads = param_u32(record, 8);
+  args.head_dim = param_u32(record, 12);
+  const uint32_t group_size = param_u32(record, 16);
+  args.token_elements = param_u32(record, 20);
+  args.token_stride = param_u32(record, 28);
+  if (int status = check_cache_geometry(record.name.c_str(), args.heads, args.head_dim, group_size,
+                                        args.token_elements, args.token_stride))
+    return status;
+  if (args.segment_offset % 64 != 0 ||
+      (uint64_t)args.segment_offset + (uint64_t)args.heads * args.head_dim > args.token_elements)
+    return fail(LLMOPT_ERR_INVALID, "%s segment lies outside the token", record.name.c_str());
+  if (int status = require_buffer_size(record.buffers[0], args.token_stride, "pool")) return status;
+  if (int status = require_buffer_size(record.buffers[1], (uint64_t)args.items * 4, "slots")) return status;
+  if (int status = require_buffer_size(
+          record.buffers[2], (uint64_t)args.heads * args.items * args.head_dim * 2, "cache destination"))
+    return status;
+  args.pool = record.buffers[0].device;
+  args.slots = reinterpret_cast<const uint32_t *>(record.buffers[1].device);
+  args.destination = reinterpret_cast<uint16_t *>(record.buffers[2].device);
+  return launched(launch_q8_unpack(args, context->stream), record.name.c_str());
+}
+
+// Q8PagedAttentionParams, 64 bytes (lib/metal_cache_source.ml:352-369):
+// batches 0, query_heads 4, kv_heads 8, past_length 12, head_dim 16,
+// mask_batches 20, mask_heads 24, token_elements 28, key_offset 32,
+// value_offset 36, group_size 40, token_stride 44, scale(f32) 48,
+// query_length 52, mask_dtype 56, window 60.
+// buffers: query, current_key, current_value, pool, slots, mask (the slots
+// buffer again when there is no mask), output.
+//
+// The batched extension appends u32 max_past_length at byte 64 and two
+// buffers: past_lengths u32[batches], slot_offsets u32[batches].
+int paged_attention(llmopt_hip_context *context, const DispatchRecord &record, bool batched) {
+  if (int status = require_buffer_count(record, batched ? 9 : 7)) return status;
+  if (int status = require_parameter_bytes(record, batched ? 68 : 64)) return status;
+  Q8AttentionArgs args = {};
+  args.batches = param_u32(record, 0);
+  args.query_heads = param_u32(record, 4);
+  args.kv_heads = param_u32(record, 8);
+  args.past_length = param_u32(record, 12);
+  args.head_dim = param_u32(record, 16);
+  args.mask_batches = param_u32(record, 20);
+  args.mask_heads = param_u32(record, 24);
+  args.token_elements = param_u32(record, 28);
+  args.key_offset = param_u32(record, 32);
+  args.value_offset = param_u32(record, 36);
+  const uint32_t group_size = param_u32(record, 40);
+  args.token_stride = param_u32(record, 44);
+  args.scale = param_f32(record, 48);
+  args.query_length = param_u32(record, 52);
+  args.mask_dtype = param_u32(record, 56);
+  args.window = param_u32(record, 60);
+  args.max_past_length = batched ? param_u32(record, 64) : args.past_length;
+  const char *name = record.name.c_str();
+  if (int status = check_cache_geometry(name, args.kv_heads, args.head_dim, group_size,
+                                        args.token_elements, args.token_stride))
+    return status;
+  if (args.batches == 0 || args.query_heads == 0 || args.query_heads % args.kv_heads != 0)
+    return fail(LLMOPT_ERR_INVALID, "%s requires query heads to be a multiple of kv heads", name);
+  if (args.head_dim > 512)
+    return fail(LLMOPT_ERR_INVALID, "%s supports head_dim up to 512, got %u", name, args.head_dim);
+  const uint64_t segment = (uint64_t)args.kv_heads * args.head_dim;
+  if (args.key_offset % 64 != 0 || args.value_offset % 64 != 0 ||
+      args.key_offset + segment > args.token_elements || args.value_offset + segment > args.token_elements)
+    return fail(LLMOPT_ERR_INVALID, "%s K/V segments lie outside the token", name);
+  if (args.mask_dtype > 2) return fail(LLMOPT_ERR_INVALID, "%s mask dtype %u is unsupported", name, args.mask_dtype);
+  const uint32_t q_len = args.query_length == 0 ? 1 : args.query_length;
+  const uint64_t q_bytes = (uint64_t)args.batches * args.query_heads * q_len * args.head_dim * 2;
+  const uint64_t kv_bytes = (uint64_t)args.batches * args.kv_heads * q_len * args.head_dim * 2;
+  if (int status = require_buffer_size(record.buffers[0], q_bytes, "query")) return status;
+  if (int status = require_buffer_size(record.buffers[1], kv_bytes, "current key")) return status;
+  if (int status = require_buffer_size(record.buffers[2], kv_bytes, "current value")) return status;
+  if (args.max_past_length > 0) {
+    if (int status = require_buffer_size(record.buffers[3], args.token_stride, "pool")) return status;
+    if (int status = require_buffer_size(record.buffers[4], (uint64_t)args.max_past_length * 4, "slots"))
+      return status;
+  }
+  const bool masked = args.mask_batches > 0 && args.mask_dtype != 0;
+  if (masked) {
+    const uint64_t mask_elements = (uint64_t)args.mask_batches * args.mask_heads * q_len *
+                                   ((uint64_t)args.max_past_length + q_len);
+    if (int status = require_buffer_size(record.buffers[5], mask_elements * (args.mask_dtype == 2 ? 2 : 1), "mask"))
+      return status;
+    if (batched && args.mask_batches != 0)
+      return fail(LLMOPT_ERR_INVALID, "%s does not take a mask", name);
+  }
+  if (int status = require_buffer_size(record.buffers[6], q_bytes, "output")) return status;
+  args.query = reinterpret_cast<const uint16_t *>(record.buffers[0].device);
+  args.current_key = reinterpret_cast<const uint16_t *>(record.buffers[1].device);
+  args.current_value = reinterpret_cast<const uint16_t *>(record.buffers[2].device);
+  args.pool = record.buffers[3].device;
+  args.slots = reinterpret_cast<const uint32_t *>(record.buffers[4].device);
+  args.mask = masked ? record.buffers[5].device : nullptr;
+  args.output = reinterpret_cast<uint16_t *>(record.buffers[6].device);
+  if (batched) {
+    if (int status = require_buffer_size(record.buffers[7], (uint64_t)args.batches * 4, "past lengths")) return status;
+    if (int status = require_buffer_size(record.buffers[8], (uint64_t)args.batches * 4, "slot offsets")) return status;
+    args.past_lengths = reinterpret_cast<const uint32_t *>(record.buffers[7].device);
+    args.slot_offsets = reinterpret_cast<const uint32_t *>(record.buffers[8].device);
+  }
+  const size_t workspace_bytes = q8_attention_workspace_bytes(args);
+  if (workspace_bytes > 0) {
+    args.workspace = context_workspace(context, workspace_bytes);
+    if (args.workspace == nullptr) return LLMOPT_ERR_FAILURE;
+    args.workspace_bytes = workspace_bytes;
+  }
+  return launched(launch_q8_attention(args, context->stream), name);
+}
+
+int paged_attention_reference(llmopt_hip_context *context, const DispatchRecord &record) {
+  return paged_attention(context, record, false);
+}
+
+int paged_attention_batched(llmopt_hip_context *context, const DispatchRecord &record) {
+  return paged_attention(context, record, true);
+}
+
+}  // namespace
+
+void register_cache_kernels(std::vector<KernelEntryPoint> &table) {
+  static const char *const cache = "cache";
+  table.push_back({"llmopt_cache_pack_attention_q8", cache, cache_pack});
+  table.push_back({"llmopt_cache_pack_attention_q8_simd", cache, cache_pack});
+  table.push_back({"llmopt_cache_pack_attention_q8_pair_simd", cache, cache_pack_pair});
+  table.push_back({"llmopt_cache_unpack_attention_q8", cache, cache_unpack});
+  table.push_back({"llmopt_cache_unpack_attention_q8_vec4", cache, cache_unpack});
+}
+
+void register_attention_kernels(std::vector<KernelEntryPoint> &table) {
+  static const char *const attention = "attention";
+  static const char *const names[] = {
+      "llmopt_attention_q8_paged_simd_generic",   "llmopt_attention_q8_paged_simd_h64",
+      "llmopt_attention_q8_paged_simd_h64_gqa3",  "llmopt_attention_q8_paged_simd_h256",
+      "llmopt_attention_q8_paged_simd_h512",      "llmopt_attention_q8_paged_simd_h64_split8",
+      "llmopt_attention_q8_paged_simd_h64_gqa3_split8"};
+  for (const char *name : names) table.push_back({name, attention, paged_attention_reference});
+  // Extension: per-sequence context lengths and slot tables in one launch.
+  table.push_back({"llmopt_attention_q8_paged_batched", attention, paged_attention_batched});
+}
+
+}  // namespace llmopt

@@ -1,0 +1,173 @@
+// Entry points of the W4A16 linear family: buffer order, parameter-block
+// layout and size checks of the reference's kernels
+// (lib/metal_w4a16_source.ml; host side lib/metal_dispatch_linear.ml:252-455,
+// 938-982), bound to the gfx950 launchers.
+#include "kernels/kernels.h"
+#include "runtime.h"
+
+namespace llmopt {
+namespace {
+
+const uint16_t *as_f16(const BoundBuffer &buffer) {
+  return reinterpret_cast<const uint16_t *>(buffer.device);
+}
+
+int check_w4_shape(const char *name, uint32_t m, uint32_t n, uint32_t k) {
+  if (m == 0 || n == 0 || k == 0)
+    return fail(LLMOPT_ERR_INVALID, "%s requires positive m, n and k", name);
+  if (k % 64 != 0)
+    return fail(LLMOPT_ERR_INVALID, "%s requires k to be a multiple of the group size 64, got %u",
+                name, k);
+  return LLMOPT_OK;
+}
+
+int check_w4_matrix(const BoundBuffer &weight, const BoundBuffer &scale, uint64_t n, uint64_t k,
+                    const char *label) {
+  std::string weight_name = std::string(label) + " packed weight";
+  std::string scale_name = std::string(label) + " scale";
+  if (int status = require_buffer_size(weight, n * (k / 2), weight_name.c_str())) return status;
+  return require_buffer_size(scale, n * (k / 64) * 2, scale_name.c_str());
+}
+
+int launched(hipError_t status, const char *name) {
+  if (status != hipSuccess) return fail(LLMOPT_ERR_FAILURE, "%s launch failed: %s", name, hipGetErrorString(status));
+  return LLMOPT_OK;
+}
+
+// W4A16Params {u32 m, n, k, has_bias, bias_row_stride}  (lib/metal_w4a16_source.ml:7)
+// buffers: input, packed_weight, scale, bias_or_scale, output.
+int w4a16_linear(llmopt_hip_context *context, const DispatchRecord &record) {
+  if (int status = require_buffer_count(record, 5)) return status;
+  if (int status = require_parameter_bytes(record, 20)) return status;
+  const uint32_t m = param_u32(record, 0), n = param_u32(record, 4), k = param_u32(record, 8);
+  const uint32_t has_bias = param_u32(record, 12), stride = param_u32(record, 16);
+  if (int status = check_w4_shape(record.name.c_str(), m, n, k)) return status;
+  if (int status = require_buffer_size(record.buffers[0], (uint64_t)m * k * 2, "input")) return status;
+  if (int status = check_w4_matrix(record.buffers[1], record.buffers[2], n, k, "W4A16")) return status;
+  if (has_bias) {
+    const uint64_t last = (uint64_t)(m - 1) * stride + n;
+    if (int status = require_buffer_size(record.buffers[3], last * 2, "bias")) return status;
+  }
+  if (int status = require_buffer_size(record.buffers[4], (uint64_t)m * n * 2, "output")) return status;
+  W4LinearArgs args = {};
+  args.x = as_f16(record.buffers[0]);
+  args.w = {record.buffers[1].device, as_f16(record.buffers[2])};
+  args.addend = as_f16(record.buffers[3]);
+  args.has_addend = has_bias;
+  args.addend_row_stride = stride;
+  args.y = reinterpret_cast<uint16_t *>(record.buffers[4].device);
+  args.m = m;
+  args.n = n;
+  args.k = k;
+  return launched(launch_w4a16_linear(args, context->stream), record.name.c_str());
+}
+
+// W4A16QKVParams {u32 m, k, n_q, n_k, n_v}  (lib/metal_w4a16_source.ml:211-217)
+// buffers: input, qW, qS, kW, kS, vW, vS, qOut, kOut, vOut.
+int w4a16_qkv_linear(llmopt_hip_context *context, const DispatchRecord &record) {
+  if (int status = require_buffer_count(record, 10)) return status;
+  if (int status = require_parameter_bytes(record, 20)) return status;
+  const uint32_t m = param_u32(record, 0), k = param_u32(record, 4);
+  const uint32_t n[3] = {param_u32(record, 8), param_u32(record, 12), param_u32(record, 16)};
+  W4QkvArgs args = {};
+  static const char *const labels[3] = {"query", "key", "value"};
+  for (int i = 0; i < 3; ++i) {
+    if (int status = check_w4_shape(record.name.c_str(), m, n[i], k)) return status;
+    if (int status = check_w4_matrix(record.buffers[1 + 2 * i], record.buffers[2 + 2 * i], n[i], k, labels[i]))
+      return status;
+    if (int status = require_buffer_size(record.buffers[7 + i], (uint64_t)m * n[i] * 2, "output")) return status;
+    args.w[i] = {record.buffers[1 + 2 * i].device, as_f16(record.buffers[2 + 2 * i])};
+    args.y[i] = reinterpret_cast<uint16_t *>(record.buffers[7 + i].device);
+    args.n[i] = n[i];
+  }
+  if (int status = require_buffer_size(record.buffers[0], (uint64_t)m * k * 2, "input")) return status;
+  args.x = as_f16(record.buffers[0]);
+  args.m = m;
+  args.k = k;
+  return launched(launch_w4a16_qkv(args, context->stream), record.name.c_str());
+}
+
+// W4A16SwiGLUFFNParams {u32 m, n, k; f32 eps}: n = intermediate width, k = hidden width
+// (lib/metal_parameters.ml:45-50).  buffers: normalized, gateW, gateS, upW, upS, product.
+int w4a16_dual_swiglu(llmopt_hip_context *context, const DispatchRecord &record) {
+  if (int status = require_buffer_count(record, 6)) return status;
+  if (int status = require_parameter_bytes(record, 16)) return status;
+  const uint32_t m = param_u32(record, 0), n = param_u32(record, 4), k = param_u32(record, 8);
+  if (int status = check_w4_shape(record.name.c_str(), m, n, k)) return status;
+  if (int status = require_buffer_size(record.buffers[0], (uint64_t)m * k * 2, "normalized")) return status;
+  if (int status = check_w4_matrix(record.buffers[1], record.buffers[2], n, k, "gate")) return status;
+  if (int status = check_w4_matrix(record.buffers[3], record.buffers[4], n, k, "up")) return status;
+  if (int status = require_buffer_size(record.buffers[5], (uint64_t)m * n * 2, "product")) return status;
+  W4DualSwigluArgs args = {};
+  args.x = as_f16(record.buffers[0]);
+  args.gate = {record.buffers[1].device, as_f16(record.buffers[2])};
+  args.up = {record.buffers[3].device, as_f16(record.buffers[4])};
+  args.product = reinterpret_cast<uint16_t *>(record.buffers[5].device);
+  args.m = m;
+  args.n = n;
+  args.k = k;
+  return launched(launch_w4a16_dual_swiglu(args, context->stream), record.name.c_str());
+}
+
+// Same parameter block; the contraction runs over n and the output has k
+// columns: output[m,k] = half(product[m,n] . downW[k,n/2]^T + residual[m,k]).
+// buffers: product, downW, downS, residual, output.
+int w4a16_down_add(llmopt_hip_context *context, const DispatchRecord &record) {
+  if (int status = require_buffer_count(record, 5)) return status;
+  if (int status = require_parameter_bytes(record, 16)) return status;
+  const uint32_t m = param_u32(record, 0), n = param_u32(record, 4), k = param_u32(record, 8);
+  if (int status = check_w4_shape(record.name.c_str(), m, k, n)) return status;
+  if (int status = require_buffer_size(record.buffers[0], (uint64_t)m * n * 2, "product")) return status;
+  if (int status = check_w4_matrix(record.buffers[1], record.buffers[2], k, n, "down")) return status;
+  if (int status = require_buffer_size(record.buffers[3], (uint64_t)m * k * 2, "residual")) return status;
+  if (int status = require_buffer_size(record.buffers[4], (uint64_t)m * k * 2, "output")) return status;
+  W4LinearArgs args = {};
+  args.x = as_f16(record.buffers[0]);
+  args.w = {record.buffers[1].device, as_f16(record.buffers[2])};
+  args.addend = as_f16(record.buffers[3]);
+  args.has_addend = 1;
+  args.addend_row_stride = k;
+  args.y = reinterpret_cast<uint16_t *>(record.buffers[4].device);
+  args.m = m;
+  args.n = k;
+  args.k = n;
+  return launched(launch_w4a16_linear(args, context->stream), record.name.c_str());
+}
+
+// Extension (no reference kernel): float32 [n,k] = q * scale, for checking the
+// unpack arithmetic bit for bit.  Parameters {u32 n, k}; buffers: packed, scale, output.
+int w4_dequant_f32(llmopt_hip_context *context, const DispatchRecord &record) {
+  if (int status = require_buffer_count(record, 3)) return status;
+  if (int status = require_parameter_bytes(record, 8)) return status;
+  const uint32_t n = param_u32(record, 0), k = param_u32(record, 4);
+  if (int status = check_w4_shape(record.name.c_str(), 1, n, k)) return status;
+  if (int status = check_w4_matrix(record.buffers[0], record.buffers[1], n, k, "W4A16")) return status;
+  if (int status = require_buffer_size(record.buffers[2], (uint64_t)n * k * 4, "output")) return status;
+  W4Matrix w = {record.buffers[0].device, as_f16(record.buffers[1])};
+  return launched(launch_w4_dequant_f32(w, reinterpret_cast<float *>(record.buffers[2].device), n, k,
+                                        context->stream),
+                  record.name.c_str());
+}
+
+}  // namespace
+
+void register_linear_kernels(std::vector<KernelEntryPoint> &table) {
+  static const char *const linear = "w4a16-linear-g64";
+  static const char *const qkv = "w4a16-qkv-linear-g64";
+  static const char *const ffn = "w4a16-swiglu-ffn-g64";
+  table.push_back({"llmopt_w4a16_linear_f16_g64", linear, w4a16_linear});
+  table.push_back({"llmopt_w4a16_linear_f16_g64_m4", linear, w4a16_linear});
+  table.push_back({"llmopt_w4a16_linear_f16_g64_m8", linear, w4a16_linear});
+  table.push_back({"llmopt_w4a16_qkv_linear_f16_g64", qkv, w4a16_qkv_linear});
+  table.push_back({"llmopt_w4a16_qkv_linear_f16_g64_m4", qkv, w4a16_qkv_linear});
+  table.push_back({"llmopt_w4a16_qkv_linear_f16_g64_m8", qkv, w4a16_qkv_linear});
+  table.push_back({"llmopt_w4a16_dual_swiglu_f16_g64", ffn, w4a16_dual_swiglu});
+  table.push_back({"llmopt_w4a16_dual_swiglu_f16_g64_m4", ffn, w4a16_dual_swiglu});
+  table.push_back({"llmopt_w4a16_dual_swiglu_f16_g64_m8", ffn, w4a16_dual_swiglu});
+  table.push_back({"llmopt_w4a16_down_add_f16_g64", ffn, w4a16_down_add});
+  table.push_back({"llmopt_w4a16_down_add_f16_g64_m4", ffn, w4a16_down_add});
+  table.push_back({"llmopt_w4a16_down_add_f16_g64_m8", ffn, w4a16_down_add});
+  table.push_back({"llmopt_w4_dequant_f32", linear, w4_dequant_f32});
+}
+
+}  // namespace llmopt

@@ -1,0 +1,187 @@
+"""GPU parity of the W4A16 linear kernels against the CPU oracle, through the C ABI."""
+import numpy as np
+import pytest
+
+import oracle
+from tests.gpu_util import assert_close_to_oracle, linear_grid, u32s, w4_case
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def runtime():
+    from llmopt_amd.native import Runtime
+    rt = Runtime()
+    yield rt
+    rt.close()
+
+
+def run_linear(runtime, x, packed, scale, bias=None, residual=None, name=None):
+    m, k = x.shape
+    n = packed.shape[0]
+    addend = bias if bias is not None else residual
+    stride = n if residual is not None else 0
+    bx = runtime.buffer_of_bytes(x)
+    bw = runtime.buffer_of_bytes(packed)
+    bs = runtime.buffer_of_bytes(scale)
+    ba = runtime.buffer_of_bytes(addend) if addend is not None else bs
+    out = runtime.buffer_of_bytes(np.full((m, n), np.nan, dtype=np.float16))  # NaN sentinel
+    if name is None:
+        name = "llmopt_w4a16_linear_f16_g64" if m == 1 else "llmopt_w4a16_linear_f16_g64_m4"
+    columns = m * n if m == 1 else ((m + 3) // 4) * n
+    runtime.dispatch(name, [bx, bw, bs, ba, out],
+                     u32s(m, n, k, 1 if addend is not None else 0, stride),
+                     grid=(linear_grid(columns), 1, 1), group=(256, 1, 1))
+    return out.numpy(np.float16, (m, n))
+
+
+def test_dequant_is_bit_exact(runtime):
+    rng = np.random.default_rng(0)
+    packed = np.arange(256, dtype=np.uint8).repeat(32).reshape(64, 128)  # every byte value
+    rng.shuffle(packed, axis=1)
+    scale = rng.uniform(0.005, 0.02, size=(64, 4)).astype(np.float16)
+    bw, bs = runtime.buffer_of_bytes(packed), runtime.buffer_of_bytes(scale)
+    out = runtime.create_buffer(64 * 256 * 4)
+    runtime.dispatch("llmopt_w4_dequant_f32", [bw, bs, out], u32s(64, 256))
+    got = out.numpy(np.float32, (64, 256))
+    np.testing.assert_array_equal(got.view(np.uint32), oracle.w4_dequant(packed, scale).view(np.uint32))
+
+
+def test_reference_fixture_golden_bits(runtime, golden):
+    case = golden["w4a16_linear_fixture"]
+    packed = np.arange(96, dtype=np.uint8).reshape(3, 32)
+    packed[0, 0] = 0x78
+    scale = np.array(case["scale"], dtype=np.float16).reshape(3, 1)
+    bias = np.array(case["bias"], dtype=np.float16)
+    x = np.full((2, 64), 1.0, dtype=np.float16)
+    out = run_linear(runtime, x, packed, scale, bias=bias)
+    assert out.view(np.uint16).reshape(-1).tolist() == case["expected_output_bits"]
+
+
+@pytest.mark.parametrize("with_bias", [True, False])
+def test_runtime_smoke_is_exact(runtime, golden, with_bias):
+    case = golden["w4a16_runtime_smoke"]
+    m, n, k = case["m"], case["n"], case["k"]
+    packed = np.empty((n, k // 2), dtype=np.uint8)
+    packed[0::2] = case["even_row_byte"]
+    packed[1::2] = case["odd_row_byte"]
+    scale = np.full((n, 1), case["scale"], dtype=np.float16)
+    bias = np.arange(n, dtype=np.float16) if with_bias else None
+    x = np.ones((m, k), dtype=np.float16)
+    out = run_linear(runtime, x, packed, scale, bias=bias)
+    expected = oracle.w4a16_linear(x, packed, scale, bias).astype(np.float16)
+    np.testing.assert_array_equal(out.view(np.uint16), expected.view(np.uint16))
+
+
+GEMV_SHAPES = [(1, 1536, 576), (1, 4096, 4096), (2, 512, 4096), (3, 260, 1024), (4, 96, 14336),
+               (5, 64, 640), (8, 200, 4096), (8, 33, 14336), (7, 1, 64)]
+
+
+@pytest.mark.parametrize("m,n,k", GEMV_SHAPES)
+def test_gemv_matches_oracle(runtime, m, n, k):
+    rng = np.random.default_rng(1000 * m + n + k)
+    x, packed, scale, bias = w4_case(rng, m, n, k, bias=True)
+    expected = oracle.w4a16_linear(x, packed, scale, None)
+    assert_close_to_oracle(run_linear(runtime, x, packed, scale), expected, f"gemv {m}x{n}x{k}")
+    expected_bias = oracle.add(expected, bias.astype(np.float32).reshape(1, -1))
+    assert_close_to_oracle(run_linear(runtime, x, packed, scale, bias=bias), expected_bias,
+                           f"gemv+bias {m}x{n}x{k}")
+
+
+def test_gemv_residual_epilogue(runtime):
+    rng = np.random.default_rng(5)
+    m, n, k = 4, 576, 1536
+    x, packed, scale, _ = w4_case(rng, m, n, k)
+    residual = rng.standard_normal((m, n)).astype(np.float16)
+    expected = oracle.add(oracle.w4a16_linear(x, packed, scale, None), residual.astype(np.float32))
+    assert_close_to_oracle(run_linear(runtime, x, packed, scale, residual=residual), expected,
+                           "gemv+residual")
+
+
+GEMM_SHAPES = [(9, 64, 64), (16, 128, 128), (100, 29, 192), (128, 256, 512), (130, 300, 1024),
+               (512, 128, 4096)]
+
+
+@pytest.mark.parametrize("m,n,k", GEMM_SHAPES)
+def test_gemm_matches_oracle(runtime, m, n, k):
+    rng = np.random.default_rng(7 * m + n + k)
+    x, packed, scale, bias = w4_case(rng, m, n, k, bias=True)
+    expected = oracle.w4a16_linear(x, packed, scale, bias)
+    assert_close_to_oracle(run_linear(runtime, x, packed, scale, bias=bias), expected,
+                           f"gemm {m}x{n}x{k}")
+
+
+def test_gemm_linearity_at_full_size(runtime):
+    """M=2048, K=4096, N=4096: too large for the serial oracle, so check sampled
+    output columns against it and linearity (2x activation -> 2x output, exact in fp16)."""
+    rng = np.random.default_rng(77)
+    m, n, k = 2048, 4096, 4096
+    x, packed, scale, _ = w4_case(rng, m, n, k)
+    out = run_linear(runtime, x, packed, scale)
+    doubled = run_linear(runtime, (x.astype(np.float32) * 2).astype(np.float16), packed, scale)
+    base, twice = out.astype(np.float32), doubled.astype(np.float32)
+    normal = np.abs(base) >= 2.0 ** -13  # doubling is exact in fp16 except from the subnormal range
+    np.testing.assert_array_equal(twice[normal], 2 * base[normal])
+    assert normal.mean() > 0.99
+    columns = rng.choice(n, size=24, replace=False)
+    rows = rng.choice(m, size=64, replace=False)
+    expected = oracle.w4a16_linear(x[rows], packed[columns], scale[columns], None)
+    assert_close_to_oracle(out[np.ix_(rows, columns)], expected, "gemm sampled")
+
+
+def qkv_params(m, k, nq, nk, nv):
+    return u32s(m, k, nq, nk, nv)
+
+
+@pytest.mark.parametrize("m", [1, 4, 8, 40])
+def test_qkv_linear(runtime, m):
+    rng = np.random.default_rng(31 + m)
+    k, sizes = 576, (576, 192, 192)
+    x = rng.standard_normal((m, k)).astype(np.float16)
+    mats = [w4_case(rng, 1, n, k)[1:3] for n in sizes]
+    buffers = [runtime.buffer_of_bytes(x)]
+    for packed, scale in mats:
+        buffers += [runtime.buffer_of_bytes(packed), runtime.buffer_of_bytes(scale)]
+    outs = [runtime.buffer_of_bytes(np.full((m, n), np.nan, dtype=np.float16)) for n in sizes]
+    name = "llmopt_w4a16_qkv_linear_f16_g64" + ("" if m == 1 else "_m4")
+    runtime.dispatch(name, buffers + outs, qkv_params(m, k, *sizes),
+                     grid=(linear_grid(m * sum(sizes)), 1, 1), group=(256, 1, 1))
+    for (packed, scale), out, n in zip(mats, outs, sizes):
+        assert_close_to_oracle(out.numpy(np.float16, (m, n)),
+                               oracle.w4a16_linear(x, packed, scale, None), f"qkv n={n}")
+
+
+@pytest.mark.parametrize("m", [1, 2, 4, 8, 48])
+def test_swiglu_ffn_chain(runtime, m):
+    """dual-SwiGLU then down+residual, the two W4A16 stages of the reference's
+    FFN macro-op; the intermediate product is rounded to f16 between stages
+    (lib/metal_w4a16_source.ml:574-575)."""
+    import struct
+    rng = np.random.default_rng(91 + m)
+    k, n = 576, 1536
+    x = rng.standard_normal((m, k)).astype(np.float16)
+    _, gate_w, gate_s, _ = w4_case(rng, 1, n, k)
+    _, up_w, up_s, _ = w4_case(rng, 1, n, k)
+    _, down_w, down_s, _ = w4_case(rng, 1, k, n)
+    residual = rng.standard_normal((m, k)).astype(np.float16)
+    params = u32s(m, n, k) + struct.pack("<f", 1e-5)
+    suffix = "" if m == 1 else "_m4"
+    product = runtime.buffer_of_bytes(np.full((m, n), np.nan, dtype=np.float16))
+    runtime.dispatch("llmopt_w4a16_dual_swiglu_f16_g64" + suffix,
+                     [runtime.buffer_of_bytes(x), runtime.buffer_of_bytes(gate_w),
+                      runtime.buffer_of_bytes(gate_s), runtime.buffer_of_bytes(up_w),
+                      runtime.buffer_of_bytes(up_s), product], params,
+                     grid=(linear_grid(m * n), 1, 1), group=(256, 1, 1))
+    gate = oracle.w4a16_linear(x, gate_w, gate_s, None)
+    up = oracle.w4a16_linear(x, up_w, up_s, None)
+    expected_product = oracle.silu_mul(gate, up)
+    got_product = product.numpy(np.float16, (m, n))
+    assert_close_to_oracle(got_product, expected_product, "dual swiglu")
+    output = runtime.buffer_of_bytes(np.full((m, k), np.nan, dtype=np.float16))
+    runtime.dispatch("llmopt_w4a16_down_add_f16_g64" + suffix,
+                     [product, runtime.buffer_of_bytes(down_w), runtime.buffer_of_bytes(down_s),
+                      runtime.buffer_of_bytes(residual), output], params,
+                     grid=(linear_grid(m * k), 1, 1), group=(256, 1, 1))
+    expected = oracle.add(oracle.w4a16_linear(got_product, down_w, down_s, None),
+                          residual.astype(np.float32))
+    assert_close_to_oracle(output.numpy(np.float16, (m, k)), expected, "down+residual")
