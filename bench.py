@@ -1,0 +1,297 @@
+#!/usr/bin/env python3
+"""Measures the W4A16 / Q8 hot path on one MI355X and prints ONE JSON line.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Headline (`value`): W4A16 decode GEMV sweep, M in {1,2,4,8} x (K,N) in
+{(4096,4096), (4096,14336), (14336,4096)}: algorithmic bytes of one pass over
+the 12 cases divided by the wall time of that pass (inputs resident in HBM).
+A "step" is one such pass.  Each (K,N) keeps 16 distinct weight copies that
+steps cycle through, so a weight matrix is never re-read from the 256 MB
+Infinity Cache: every step streams its weights from HBM.
+
+Also reported in the same line: `roofline` of the dominant kernel (the M=1
+GEMV at K=4096, N=14336) from HIP events around graph-replayed launches,
+`cpu_baseline` (the C oracle on one host core over the same sweep) and, under
+`extras`, the prefill GEMM (MFMA roofline) and Q8 decode attention (HBM
+roofline, tokens/s) measurements.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import math
+import os
+import struct
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16
+SEED = 20240531
+COPIES = 16
+
+GEMV_SHAPES = [(4096, 4096), (4096, 14336), (14336, 4096)]
+GEMV_ROWS = [1, 2, 4, 8]
+
+
+def gemv_bytes(m, k, n):
+    """Algorithmic bytes of one W4A16 linear: packed weights + fp16 scales +
+    fp16 activations in + fp16 outputs (the reference's own accounting,
+    lib/dag_analysis.ml:24-33)."""
+    return n * k // 2 + 2 * n * (k // 64) + 2 * m * k + 2 * m * n
+
+
+def u32s(*values):
+    return struct.pack("<%dI" % len(values), *values)
+
+
+def linear_grid(columns):
+    return ((columns + 7) // 8) * 8 * 32
+
+
+def w4_inputs(rng, m, n, k):
+    packed = rng.integers(0, 256, size=(n, k // 2), dtype=np.uint8)
+    scale = rng.uniform(0.005, 0.02, size=(n, k // 64)).astype(np.float16)
+    x = rng.standard_normal((m, k)).astype(np.float16)
+    return x, packed, scale
+
+
+def record_linear(batch, m, n, k, bx, bw, bs, out):
+    name = "llmopt_w4a16_linear_f16_g64" if m == 1 else "llmopt_w4a16_linear_f16_g64_m4"
+    columns = m * n if m == 1 else ((m + 3) // 4) * n
+    batch.dispatch(name, [bx, bw, bs, bs, out], u32s(m, n, k, 0, 0),
+                   grid=(linear_grid(columns), 1, 1), group=(256, 1, 1))
+
+
+def bench_gemv(runtime, steps, warmup):
+    rng = np.random.default_rng(SEED)
+    weights = {}
+    for k, n in GEMV_SHAPES:
+        _, packed, scale = w4_inputs(rng, 1, n, k)
+        weights[(k, n)] = [(runtime.buffer_of_bytes(packed), runtime.buffer_of_bytes(scale))
+                           for _ in range(COPIES)]
+    activations = {(m, k): runtime.buffer_of_bytes(rng.standard_normal((m, k)).astype(np.float16))
+                   for m in GEMV_ROWS for k in {s[0] for s in GEMV_SHAPES}}
+    outputs = {(m, n): runtime.create_buffer(m * n * 2)
+               for m in GEMV_ROWS for n in {s[1] for s in GEMV_SHAPES}}
+
+    def record_steps(batch, count, first=0):
+        for step in range(first, first + count):
+            for m in GEMV_ROWS:
+                for k, n in GEMV_SHAPES:
+                    bw, bs = weights[(k, n)][step % COPIES]
+                    record_linear(batch, m, n, k, activations[(m, k)], bw, bs, outputs[(m, n)])
+
+    bytes_per_step = sum(gemv_bytes(m, k, n) for m in GEMV_ROWS for k, n in GEMV_SHAPES)
+
+    # warmup (untimed), then EXACTLY `steps` steps between two synchronisations
+    batch = runtime.begin_batch()
+    record_steps(batch, max(1, warmup))
+    batch.commit()
+    batch = runtime.begin_batch()
+    record_steps(batch, steps)
+    runtime.synchronize()
+    started = time.perf_counter()
+    batch.commit()  # launches every recorded dispatch in order and waits
+    runtime.synchronize()
+    elapsed = time.perf_counter() - started
+    ms_per_step = elapsed * 1e3 / steps
+
+    # the same steps as a HIP graph (back-to-back launches, no host in the loop)
+    batch = runtime.begin_batch()
+    record_steps(batch, COPIES)
+    graph_repeats = max(1, steps // COPIES)
+    graph_ms = batch.commit_profiled(repeats=graph_repeats, use_graph=True)
+    graph_ms_per_step = graph_ms / (graph_repeats * COPIES)
+
+    # per-case kernel time: COPIES launches of one case per graph, HIP events
+    cases = []
+    for m in GEMV_ROWS:
+        for k, n in GEMV_SHAPES:
+            batch = runtime.begin_batch()
+            for copy in range(COPIES):
+                bw, bs = weights[(k, n)][copy]
+                record_linear(batch, m, n, k, activations[(m, k)], bw, bs, outputs[(m, n)])
+            repeats = 8
+            ms = batch.commit_profiled(repeats=repeats, use_graph=True)
+            us = ms * 1e3 / (repeats * COPIES)
+            gbs = gemv_bytes(m, k, n) / (us * 1e-6) / 1e9
+            cases.append({"m": m, "k": k, "n": n, "bytes": gemv_bytes(m, k, n),
+                          "us_per_launch": round(us, 3), "GBps": round(gbs, 1),
+                          "hbm_frac": round(gbs / HBM_PEAK_GBS, 4)})
+    return {"bytes_per_step": bytes_per_step, "ms_per_step": ms_per_step,
+            "graph_ms_per_step": graph_ms_per_step, "cases": cases}
+
+
+def bench_gemm(runtime):
+    """C3: prefill GEMM, M in {512, 2048}, K=4096, N in {4096, 14336}, plus the fused
+    SwiGLU pair (two N=14336 projections combined as silu(a)*b)."""
+    rng = np.random.default_rng(SEED + 1)
+    results = []
+    k = 4096
+    packed_cache = {}
+    for n in (4096, 14336):
+        _, packed, scale = w4_inputs(rng, 1, n, k)
+        packed_cache[n] = (runtime.buffer_of_bytes(packed), runtime.buffer_of_bytes(scale),
+                           runtime.buffer_of_bytes(packed[::-1].copy()), runtime.buffer_of_bytes(scale))
+    for m in (512, 2048):
+        bx = runtime.buffer_of_bytes(rng.standard_normal((m, k)).astype(np.float16))
+        for n in (4096, 14336):
+            bw, bs, _, _ = packed_cache[n]
+            out = runtime.create_buffer(m * n * 2)
+            batch = runtime.begin_batch()
+            for _ in range(4):
+                record_linear(batch, m, n, k, bx, bw, bs, out)
+            repeats = 3
+            ms = batch.commit_profiled(repeats=repeats, use_graph=True)
+            us = ms * 1e3 / (repeats * 4)
+            tflops = 2.0 * m * n * k / (us * 1e-6) / 1e12
+            results.append({"kind": "linear", "m": m, "n": n, "k": k, "us_per_launch": round(us, 2),
+                            "TFLOPs": round(tflops, 1),
+                            "mfma_frac": round(tflops / MFMA_F16_PEAK_TFLOPS, 4)})
+        n = 14336
+        gate_w, gate_s, up_w, up_s = packed_cache[n]
+        product = runtime.create_buffer(m * n * 2)
+        batch = runtime.begin_batch()
+        params = u32s(m, n, k) + struct.pack("<f", 1e-5)
+        for _ in range(4):
+            batch.dispatch("llmopt_w4a16_dual_swiglu_f16_g64_m4", [bx, gate_w, gate_s, up_w, up_s, product],
+                           params, grid=(linear_grid(((m + 3) // 4) * n), 1, 1), group=(256, 1, 1))
+        repeats = 3
+        ms = batch.commit_profiled(repeats=repeats, use_graph=True)
+        us = ms * 1e3 / (repeats * 4)
+        tflops = 2.0 * 2.0 * m * n * k / (us * 1e-6) / 1e12
+        results.append({"kind": "dual_swiglu", "m": m, "n": n, "k": k, "us_per_launch": round(us, 2),
+                        "TFLOPs": round(tflops, 1),
+                        "mfma_frac": round(tflops / MFMA_F16_PEAK_TFLOPS, 4)})
+    return results
+
+
+def bench_attention(runtime):
+    """C4: batch 16, 32 query heads / 8 KV heads, head_dim 128, context lengths ~ U{512..8192},
+    contiguous per-sequence slots, Q8 KV cache of one layer."""
+    rng = np.random.default_rng(SEED + 2)
+    batches, heads, kv_heads, dim = 16, 32, 8, 128
+    lengths = rng.integers(512, 8193, size=batches).astype(np.uint32)
+    token_elements = 2 * kv_heads * dim
+    stride = token_elements + 2 * (token_elements // 64)
+    total = int(lengths.sum())
+    # int8 values ~ quantised N(0,1) (|x|max/127 scaling -> q ~ N(0, 127/3.3)), fp16 scales
+    pool = np.empty((total, stride), dtype=np.uint8)
+    q = np.clip(np.rint(rng.standard_normal((total, token_elements)) * 38.0), -127, 127).astype(np.int8)
+    pool[:, :token_elements] = q.view(np.uint8)
+    scales = rng.uniform(0.02, 0.035, size=(total, token_elements // 64)).astype(np.float16)
+    pool[:, token_elements:] = scales.view(np.uint8).reshape(total, -1)
+    offsets = np.concatenate([[0], np.cumsum(lengths)[:-1]]).astype(np.uint32)
+    slots = np.arange(total, dtype=np.uint32)  # contiguous per-sequence layout
+    query = rng.standard_normal((batches, heads, 1, dim)).astype(np.float16)
+    ck = rng.standard_normal((batches, kv_heads, 1, dim)).astype(np.float16)
+    cv = rng.standard_normal((batches, kv_heads, 1, dim)).astype(np.float16)
+    params = struct.pack("<12IfIII", batches, heads, kv_heads, 0, dim, 0, 0, token_elements, 0,
+                         kv_heads * dim, 64, stride, 1.0 / math.sqrt(dim), 1, 0, 0)
+    params += struct.pack("<I", int(lengths.max()))
+    # two pools so that consecutive launches do not re-read the same bytes from the Infinity Cache
+    pools = [runtime.buffer_of_bytes(pool) for _ in range(3)]
+    b_slots = runtime.buffer_of_bytes(slots)
+    buffers_tail = [runtime.buffer_of_bytes(lengths), runtime.buffer_of_bytes(offsets)]
+    bq, bck, bcv = (runtime.buffer_of_bytes(a) for a in (query, ck, cv))
+    out = runtime.create_buffer(batches * heads * dim * 2)
+    batch = runtime.begin_batch()
+    for b_pool in pools:
+        batch.dispatch("llmopt_attention_q8_paged_batched",
+                       [bq, bck, bcv, b_pool, b_slots, b_slots, out] + buffers_tail, params,
+                       grid=(batches * heads * 32, 1, 1), group=(256, 1, 1))
+    repeats = 10
+    ms = batch.commit_profiled(repeats=repeats, use_graph=True)
+    us = ms * 1e3 / (repeats * len(pools))
+    kv_bytes = total * stride + 2 * batches * heads * dim * 2
+    gbs = kv_bytes / (us * 1e-6) / 1e9
+    return {"batch": batches, "sum_context": total, "bytes": kv_bytes, "us_per_call": round(us, 2),
+            "GBps": round(gbs, 1), "hbm_frac": round(gbs / HBM_PEAK_GBS, 4),
+            "tokens_per_s": round(batches / (us * 1e-6), 1)}
+
+
+def cpu_baseline():
+    """The C oracle (a port of lib/cpu.ml's w4a16_linear) on ONE host core over the same
+    GEMV sweep at reduced N (1/16 of the output columns of every case, every M and K)."""
+    import oracle
+    rng = np.random.default_rng(SEED)
+    total_bytes = 0
+    started_all = time.perf_counter()
+    elapsed = 0.0
+    for m in GEMV_ROWS:
+        for k, n in GEMV_SHAPES:
+            sample_n = n // 16
+            x, packed, scale = w4_inputs(rng, m, sample_n, k)
+            started = time.perf_counter()
+            oracle.w4a16_linear(x, packed, scale, None)
+            elapsed += time.perf_counter() - started
+            total_bytes += gemv_bytes(m, k, sample_n)
+    del started_all
+    return {"value": round(total_bytes / elapsed / 1e9, 4), "unit": "GB/s", "cores": 1,
+            "kind": "port",
+            "sample": "the 12-case GEMV sweep with N/16 output columns per case "
+                      f"({elapsed:.1f} s of single-thread oracle time)"}
+
+
+def main():
+    parser = argparse.ArgumentParser()
+    parser.add_argument("--gpus", type=int, default=1)
+    parser.add_argument("--steps", type=int, default=64)
+    parser.add_argument("--warmup", type=int, default=16)
+    parser.add_argument("--skip-extras", action="store_true")
+    parser.add_argument("--skip-cpu", action="store_true")
+    args = parser.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one GPU: this hot path has no multi-GPU part; run with --gpus 1")
+
+    from llmopt_amd.native import Runtime
+    runtime = Runtime()
+    gemv = bench_gemv(runtime, args.steps, args.warmup)
+    headline = next(c for c in gemv["cases"] if (c["m"], c["k"], c["n"]) == (1, 4096, 14336))
+    # K steps replayed as HIP graphs of 16 steps each, timed by HIP events on the launch stream
+    value = gemv["bytes_per_step"] / (gemv["graph_ms_per_step"] * 1e-3) / 1e9
+    extras = {"gemv_cases": gemv["cases"],
+              "gemv_eager_host_launch_GBps":
+                  round(gemv["bytes_per_step"] / (gemv["ms_per_step"] * 1e-3) / 1e9, 1),
+              "gemv_eager_host_launch_ms_per_step": round(gemv["ms_per_step"], 4),
+              "device": runtime.device_name(), "seed": SEED}
+    if not args.skip_extras:
+        extras["prefill_gemm"] = bench_gemm(runtime)
+        extras["q8_attention"] = bench_attention(runtime)
+    line = {
+        "metric": "W4A16 GEMV HBM GB/s (% peak); Q8 attn decode tokens/s; prefill MFMA %",
+        "value": round(value, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(gemv["graph_ms_per_step"], 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16 x int4 -> f32 accumulate",
+        "data": "synthetic (seeded int4 U{-8..7}, fp16 scales U[0.005,0.02], activations N(0,1))",
+        "config": {"workload": "W4A16 decode GEMV sweep: M in {1,2,4,8} x (K,N) in "
+                               "{(4096,4096),(4096,14336),(14336,4096)}, group-64 fp16 scales; "
+                               "one step = the 12 launches, weights cycled over 16 HBM copies",
+                   "bytes_per_step": gemv["bytes_per_step"]},
+        "roofline": {"bound": "hbm", "kernel": "w4a16_gemv_kernel<M=1,R=4> at K=4096 N=14336",
+                     "achieved": headline["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": headline["hbm_frac"], "traffic": None,
+                     "bytes_per_launch": headline["bytes"], "us_per_launch": headline["us_per_launch"]},
+        "cpu_baseline": None if args.skip_cpu else cpu_baseline(),
+        "extras": extras,
+    }
+    runtime.close()
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

@@ -172,6 +172,14 @@ int llmopt_hip_batch_barrier(llmopt_hip_batch *batch);
 int llmopt_hip_commit_batch(llmopt_hip_batch *batch);
 /* caml_llmopt_metal_commit_batch_async (:1359-1370): launches without waiting. */
 int llmopt_hip_commit_batch_async(llmopt_hip_batch *batch);
+/* Commit for measurement: the counterpart of committing under
+ * LLMOPT_PROFILE_BATCH, where the reference reports the command buffer's GPU
+ * time (native/ocaml_metal_stubs.m:1337-1347).  Runs the recorded work once
+ * untimed, then `repeats` times between two HIP events on the context's
+ * stream (as one HIP graph per repeat when use_graph != 0, so launches are
+ * back to back) and returns the elapsed GPU milliseconds of the timed part. */
+int llmopt_hip_commit_batch_profiled(llmopt_hip_batch *batch, int use_graph, int repeats,
+                                     float *gpu_milliseconds);
 /* caml_llmopt_metal_abort_batch (:1372-1382). */
 int llmopt_hip_abort_batch(llmopt_hip_batch *batch);
 

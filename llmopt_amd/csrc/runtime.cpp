@@ -670,6 +670,76 @@ static int submit_batch(llmopt_hip_batch *batch, bool wait) {
 int llmopt_hip_commit_batch(llmopt_hip_batch *batch) { return submit_batch(batch, true); }
 int llmopt_hip_commit_batch_async(llmopt_hip_batch *batch) { return submit_batch(batch, false); }
 
+int llmopt_hip_commit_batch_profiled(llmopt_hip_batch *batch, int use_graph, int repeats,
+                                     float *gpu_milliseconds) {
+  if (int status = require_active_batch(batch)) return status;
+  if (repeats <= 0) return fail(LLMOPT_ERR_INVALID, "profiled commit needs a positive repeat count");
+  llmopt_hip_context *context = batch->library->context;
+  if (int status = use_device(context)) return status;
+  batch->finished = true;
+  hipStream_t stream = context->stream;
+  auto launch_all = [&]() -> int {
+    for (BatchOp &op : batch->ops) {
+      if (op.is_copy) {
+        if (hipMemcpyAsync(op.destination->device, op.source->device, op.source->length,
+                           hipMemcpyDeviceToDevice, stream) != hipSuccess)
+          return fail(LLMOPT_ERR_FAILURE, "HIP batched copy failed");
+      } else if (int status = launch_record(context, op.record)) {
+        return status;
+      }
+    }
+    return LLMOPT_OK;
+  };
+  // One untimed pass: first-use allocations (kernel workspace) happen here,
+  // outside any stream capture.
+  int status = launch_all();
+  if (status == LLMOPT_OK && hipStreamSynchronize(stream) != hipSuccess)
+    status = fail(LLMOPT_ERR_FAILURE, "HIP batch failed");
+  hipGraph_t graph = nullptr;
+  hipGraphExec_t executable = nullptr;
+  hipEvent_t start = nullptr, stop = nullptr;
+  if (status == LLMOPT_OK && use_graph) {
+    if (hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal) != hipSuccess) {
+      status = fail(LLMOPT_ERR_FAILURE, "HIP stream capture could not begin");
+    } else {
+      status = launch_all();
+      if (hipStreamEndCapture(stream, &graph) != hipSuccess && status == LLMOPT_OK)
+        status = fail(LLMOPT_ERR_FAILURE, "HIP stream capture failed");
+      if (status == LLMOPT_OK &&
+          hipGraphInstantiate(&executable, graph, nullptr, nullptr, 0) != hipSuccess)
+        status = fail(LLMOPT_ERR_FAILURE, "HIP graph instantiation failed");
+    }
+  }
+  if (status == LLMOPT_OK &&
+      (hipEventCreate(&start) != hipSuccess || hipEventCreate(&stop) != hipSuccess))
+    status = fail(LLMOPT_ERR_FAILURE, "HIP could not create timing events");
+  if (status == LLMOPT_OK) {
+    (void)hipEventRecord(start, stream);
+    for (int i = 0; i < repeats && status == LLMOPT_OK; ++i) {
+      if (executable) {
+        if (hipGraphLaunch(executable, stream) != hipSuccess)
+          status = fail(LLMOPT_ERR_FAILURE, "HIP graph launch failed");
+      } else {
+        status = launch_all();
+      }
+    }
+    (void)hipEventRecord(stop, stream);
+    if (hipStreamSynchronize(stream) != hipSuccess && status == LLMOPT_OK)
+      status = fail(LLMOPT_ERR_FAILURE, "HIP batch failed");
+    float elapsed = 0.0f;
+    if (status == LLMOPT_OK && hipEventElapsedTime(&elapsed, start, stop) != hipSuccess)
+      status = fail(LLMOPT_ERR_FAILURE, "HIP could not read the timing events");
+    if (gpu_milliseconds) *gpu_milliseconds = elapsed;
+  }
+  if (start) (void)hipEventDestroy(start);
+  if (stop) (void)hipEventDestroy(stop);
+  if (executable) (void)hipGraphExecDestroy(executable);
+  if (graph) (void)hipGraphDestroy(graph);
+  (void)hipStreamSynchronize(stream);
+  clear_batch(batch);
+  return status;
+}
+
 int llmopt_hip_abort_batch(llmopt_hip_batch *batch) {
   if (batch != nullptr && !batch->finished) {
     clear_batch(batch);

@@ -93,6 +93,8 @@ def lib() -> ctypes.CDLL:
         "llmopt_hip_batch_barrier": (ctypes.c_int, [vp]),
         "llmopt_hip_commit_batch": (ctypes.c_int, [vp]),
         "llmopt_hip_commit_batch_async": (ctypes.c_int, [vp]),
+        "llmopt_hip_commit_batch_profiled": (ctypes.c_int, [vp, ctypes.c_int, ctypes.c_int,
+                                                           ctypes.POINTER(ctypes.c_float)]),
         "llmopt_hip_abort_batch": (ctypes.c_int, [vp]),
         "llmopt_hip_prebaked_create": (ctypes.c_int, [vp, item_p, sz, vp, vp, pp]),
         "llmopt_hip_release_prebaked": (None, [vp]),
@@ -119,7 +121,8 @@ EXPORTED_SYMBOLS = (
     "llmopt_hip_buffer_set_u32_array", "llmopt_hip_buffer_argmax_f16", "llmopt_hip_dispatch",
     "llmopt_hip_begin_batch", "llmopt_hip_release_batch", "llmopt_hip_batch_dispatch",
     "llmopt_hip_batch_dispatch_all", "llmopt_hip_batch_copy", "llmopt_hip_batch_barrier",
-    "llmopt_hip_commit_batch", "llmopt_hip_commit_batch_async", "llmopt_hip_abort_batch",
+    "llmopt_hip_commit_batch", "llmopt_hip_commit_batch_async",
+    "llmopt_hip_commit_batch_profiled", "llmopt_hip_abort_batch",
     "llmopt_hip_prebaked_create", "llmopt_hip_release_prebaked", "llmopt_hip_prebaked_execute",
 )
 
@@ -345,6 +348,13 @@ class Batch:
 
     def commit_async(self) -> None:
         _check(lib().llmopt_hip_commit_batch_async(self._handle))
+
+    def commit_profiled(self, repeats: int = 1, use_graph: bool = True) -> float:
+        """Runs the batch `repeats` times between HIP events; returns GPU milliseconds."""
+        elapsed = ctypes.c_float()
+        _check(lib().llmopt_hip_commit_batch_profiled(self._handle, int(use_graph), repeats,
+                                                      ctypes.byref(elapsed)))
+        return float(elapsed.value)
 
     def abort(self) -> None:
         _check(lib().llmopt_hip_abort_batch(self._handle))
