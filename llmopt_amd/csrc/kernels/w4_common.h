@@ -57,6 +57,22 @@ __device__ __forceinline__ W4Pairs w4_decode_pairs(uint32_t word) {
   return out;
 }
 
+// Same decode without the subtraction: the pairs hold q + 1032 (p04, p26) and
+// q + 72 (p15, p37).  (w ^ 0x88888888) & mask | magic equals
+// (w & mask) ^ (magic | (0x88888888 & mask)) because the magic bits lie outside
+// the mask, so each pair costs one three-input bit operation.  A dot product
+// with these is corrected afterwards by 1032 * sum(x at K offsets 0,4,2,6) +
+// 72 * sum(x at K offsets 1,5,3,7), which does not depend on the weight row.
+__device__ __forceinline__ W4Pairs w4_decode_biased(uint32_t word) {
+  const uint32_t hi = word >> 8;
+  W4Pairs out;
+  out.p04 = as_h2((word & 0x000F000Fu) ^ 0x64086408u);
+  out.p15 = as_h2((word & 0x00F000F0u) ^ 0x54805480u);
+  out.p26 = as_h2((hi & 0x000F000Fu) ^ 0x64086408u);
+  out.p37 = as_h2((hi & 0x00F000F0u) ^ 0x54805480u);
+  return out;
+}
+
 // Rearranges 8 consecutive fp16 activations (x0..x7) into the pair order of
 // w4_decode_pairs: {(x0,x4), (x1,x5), (x2,x6), (x3,x7)}.
 __device__ __forceinline__ uint4 pair_order(uint4 x) {

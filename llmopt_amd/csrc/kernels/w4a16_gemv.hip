@@ -12,6 +12,7 @@
 // llmopt_w4a16_dual_swiglu_f16_g64* / llmopt_w4a16_down_add_f16_g64*
 // (lib/metal_w4a16_source.ml:8-966) for m <= 8.
 #include <algorithm>
+#include <cstdlib>
 
 #include "kernels.h"
 #include "kernels_internal.h"
@@ -42,19 +43,78 @@ struct GemvParams {
   uint32_t addend_stride;
 };
 
-// M: activation rows held per lane, R: weight rows per wave, XLDS: activation
-// staged once per workgroup in LDS (pair order), DUAL: rows [0,R/2) are gate
-// rows and [R/2,R) the matching up rows; the output is silu(gate)*up.
-template <int M, int R, bool XLDS, bool DUAL>
+// M: activation rows held per lane, R: weight rows per wave and tile, U: K
+// chunks (2048 K values each) per work item, XLDS: activation staged once per
+// workgroup in LDS (pair order), DUAL: rows [0,R/2) are gate rows and [R/2,R)
+// the matching up rows; the output is silu(gate)*up.
+//
+// The grid is persistent: every wave walks row tiles gw, gw + W, gw + 2W, ...
+// (gw = global wave index) and, inside a tile, items of U chunks.  The weight
+// segments and scales of the next item are loaded into registers before the
+// current item is decoded, so HBM latency overlaps the VALU work.
+template <int M, int R, int U, bool XLDS, bool DUAL>
 __global__ __launch_bounds__(kThreads) void w4a16_gemv_kernel(GemvParams p) {
   extern __shared__ uint4 x_lds[];
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  // wave-uniform values are forced into scalar registers: tile indices, row
+  // pointers and the matrix selection then cost no vector work
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const uint32_t K = p.k;
-  const uint32_t segs = K >> 5;             // 16-byte weight segments per row
+  const uint32_t segs = K >> 5;              // 16-byte weight segments per row
   const uint32_t chunks = (segs + 63) >> 6;  // wave-wide steps over K
-  constexpr int C = DUAL ? R / 2 : R;        // output columns per wave
+  const uint32_t items_per_tile = (chunks + U - 1) / U;
+  constexpr int C = DUAL ? R / 2 : R;  // output columns per tile
 
+  const uint32_t wave_count = gridDim.x * kWaves;
+  const uint32_t first_tile = blockIdx.x * kWaves + wave;
+
+  // Raw loaded registers only: nothing here may be touched before the item is
+  // consumed, or the compiler has to wait for the loads right after issuing them.
+  struct Item {
+    u32x4_t w[R][U];
+    uint16_t s[R][U];
+  };
+
+  auto tile_rows = [&](uint32_t tile, const u32x4_t *(&wrow)[R], const uint16_t *(&srow)[R]) {
+    uint32_t which = 0;
+    if (!DUAL) {
+      if (p.nseg > 1 && tile >= p.seg[1].tile_begin) which = 1;
+      if (p.nseg > 2 && tile >= p.seg[2].tile_begin) which = 2;
+    }
+    const GemvSegment &sg = p.seg[which];
+    const uint32_t col0 = (tile - sg.tile_begin) * C;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+      const uint32_t col = min(col0 + (uint32_t)(DUAL ? r % C : r), sg.n - 1);
+      const GemvSegment &src = DUAL ? p.seg[r / C] : sg;
+      wrow[r] = reinterpret_cast<const u32x4_t *>(src.w + (size_t)col * (K >> 1));
+      srow[r] = src.s + (size_t)col * (K >> 6);
+    }
+  };
+
+  auto load_item = [&](uint32_t tile, uint32_t item, Item &out) {
+    const u32x4_t *wrow[R];
+    const uint16_t *srow[R];
+    tile_rows(tile, wrow, srow);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t seg = (item * U + u) * 64 + lane;
+      const uint32_t safe = seg < segs ? seg : 0;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        out.w[r][u] = __builtin_nontemporal_load(wrow[r] + safe);
+        out.s[r][u] = srow[r][safe >> 1];
+      }
+    }
+  };
+
+  // first weights are in flight while the activation is staged
+  Item item_a, item_b;
+  const bool has_work = first_tile < p.tiles;
+  if (has_work) load_item(first_tile, 0, item_a);
+
+  // Bias correction of w4_decode_biased per (m, chunk, lane), after the vectors.
+  float *corr_lds = reinterpret_cast<float *>(x_lds + (size_t)M * chunks * 256);
   if (XLDS) {
     // LDS layout [m][chunk][j][lane] of uint4: the j-th 8-K block of every
     // lane's segment is contiguous across lanes (conflict-free b128 reads).
@@ -69,73 +129,50 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemv_kernel(GemvParams p) {
       x_lds[((m * chunks + (seg >> 6)) * 4 + j) * 64 + (seg & 63)] = value;
     }
     __syncthreads();
-  }
-
-  for (uint32_t tile = blockIdx.x; tile < p.tiles; tile += gridDim.x) {
-    uint32_t which = 0;
-    if (!DUAL) {
-      if (p.nseg > 1 && tile >= p.seg[1].tile_begin) which = 1;
-      if (p.nseg > 2 && tile >= p.seg[2].tile_begin) which = 2;
-    }
-    const GemvSegment &sg = p.seg[which];
-    const uint32_t n = sg.n;
-    const uint32_t col0 = (tile - sg.tile_begin) * (kWaves * C) + wave * C;
-    if (col0 >= n) continue;  // whole wave idle (wave-uniform)
-
-    const u32x4_t *wrow[R];
-    const uint16_t *srow[R];
+    for (uint32_t i = threadIdx.x; i < (uint32_t)M * chunks * 64; i += kThreads) {
+      const uint32_t mc = i >> 6, ln = i & 63;  // mc = m * chunks + chunk
+      float sum_a = 0.0f, sum_b = 0.0f;
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-      const uint32_t col = min(col0 + (uint32_t)(DUAL ? r % C : r), n - 1);
-      const GemvSegment &src = DUAL ? p.seg[r / C] : sg;
-      wrow[r] = reinterpret_cast<const u32x4_t *>(src.w + (size_t)col * (K >> 1));
-      srow[r] = src.s + (size_t)col * (K >> 6);
-    }
-
-    float acc[R][M];
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-#pragma unroll
-      for (int m = 0; m < M; ++m) acc[r][m] = 0.0f;
-
-    u32x4_t w_cur[R];
-    float s_cur[R];
-    auto load_chunk = [&](uint32_t c, u32x4_t(&wv)[R], float(&sv)[R]) {
-      const uint32_t seg = c * 64 + lane;
-      const bool ok = seg < segs;
-      const uint32_t safe = ok ? seg : 0;
-#pragma unroll
-      for (int r = 0; r < R; ++r) {
-        wv[r] = __builtin_nontemporal_load(wrow[r] + safe);
-        sv[r] = half_bits_to_float(srow[r][safe >> 1]);
-        if (!ok) {
-          wv[r] = u32x4_t{0, 0, 0, 0};  // q = 0
-          sv[r] = 0.0f;
-        }
+      for (int j = 0; j < 4; ++j) {
+        const uint4 v = x_lds[(mc * 4 + j) * 64 + ln];
+        const h2_t a0 = as_h2(v.x), b0 = as_h2(v.y), a1 = as_h2(v.z), b1 = as_h2(v.w);
+        sum_a += ((float)a0[0] + (float)a0[1]) + ((float)a1[0] + (float)a1[1]);
+        sum_b += ((float)b0[0] + (float)b0[1]) + ((float)b1[0] + (float)b1[1]);
       }
-    };
-    load_chunk(0, w_cur, s_cur);
+      corr_lds[i] = 1032.0f * sum_a + 72.0f * sum_b;
+    }
+    __syncthreads();
+  }
+  if (!has_work) return;
 
-    for (uint32_t c = 0; c < chunks; ++c) {
-      u32x4_t w_next[R];
-      float s_next[R];
-      if (c + 1 < chunks) load_chunk(c + 1, w_next, s_next);
+  float acc[R][M];
+#pragma unroll
+  for (int r = 0; r < R; ++r)
+#pragma unroll
+    for (int m = 0; m < M; ++m) acc[r][m] = 0.0f;
 
+  // Decodes one item into acc; when it is the last item of its tile, reduces
+  // across the wave and stores.
+  auto consume = [&](uint32_t tile, uint32_t item, const Item &cur) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t c = item * U + u;
       const uint32_t seg = c * 64 + lane;
-      const uint32_t safe = seg < segs ? seg : 0;
+      const bool ok = seg < segs;  // a segment past the row end contributes scale 0
+      const uint32_t safe = ok ? seg : 0;
+      const uint32_t c_safe = c < chunks ? c : 0;
       float part[R][M];
 #pragma unroll
       for (int r = 0; r < R; ++r)
 #pragma unroll
         for (int m = 0; m < M; ++m) part[r][m] = 0.0f;
-
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
         uint4 xp[M];
 #pragma unroll
         for (int m = 0; m < M; ++m) {
           if (XLDS) {
-            xp[m] = x_lds[((m * chunks + c) * 4 + j) * 64 + lane];
+            xp[m] = x_lds[((m * chunks + c_safe) * 4 + j) * 64 + lane];
           } else {
             const uint32_t row = (uint32_t)m < p.m ? m : 0;
             xp[m] = pair_order(
@@ -144,8 +181,7 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemv_kernel(GemvParams p) {
         }
 #pragma unroll
         for (int r = 0; r < R; ++r) {
-          const uint32_t word = w_cur[r][j];
-          const W4Pairs q = w4_decode_pairs(word);
+          const W4Pairs q = XLDS ? w4_decode_biased(cur.w[r][u][j]) : w4_decode_pairs(cur.w[r][u][j]);
 #pragma unroll
           for (int m = 0; m < M; ++m) {
             float a = part[r][m];
@@ -158,48 +194,86 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemv_kernel(GemvParams p) {
         }
       }
 #pragma unroll
+      for (int m = 0; m < M; ++m) {
+        const float correction = XLDS ? corr_lds[(m * chunks + c_safe) * 64 + lane] : 0.0f;
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+          acc[r][m] = fmaf(part[r][m] - correction, ok ? half_bits_to_float(cur.s[r][u]) : 0.0f,
+                           acc[r][m]);
+      }
+    }
+
+    if (item + 1 == items_per_tile) {
+      uint32_t which = 0;
+      if (!DUAL) {
+        if (p.nseg > 1 && tile >= p.seg[1].tile_begin) which = 1;
+        if (p.nseg > 2 && tile >= p.seg[2].tile_begin) which = 2;
+      }
+      const GemvSegment &sg = p.seg[which];
+      const uint32_t n = sg.n;
+      const uint32_t col0 = (tile - sg.tile_begin) * C;
+      float total[R][M];
+#pragma unroll
       for (int r = 0; r < R; ++r)
 #pragma unroll
-        for (int m = 0; m < M; ++m) acc[r][m] = fmaf(part[r][m], s_cur[r], acc[r][m]);
-
-      if (c + 1 < chunks) {
-#pragma unroll
-        for (int r = 0; r < R; ++r) {
-          w_cur[r] = w_next[r];
-          s_cur[r] = s_next[r];
-        }
-      }
-    }
-
-    // wave reduction; the result is uniform, lane 0 stores
-    float total[R][M];
-#pragma unroll
-    for (int r = 0; r < R; ++r)
-#pragma unroll
-      for (int m = 0; m < M; ++m) total[r][m] = wave_sum(acc[r][m]);
-
-    if (lane == 0) {
-#pragma unroll
-      for (int cidx = 0; cidx < C; ++cidx) {
-        const uint32_t col = col0 + cidx;
-        if (col >= n) break;
-#pragma unroll
         for (int m = 0; m < M; ++m) {
-          if ((uint32_t)m >= p.m) break;
-          float value;
-          if (DUAL) {
-            const float gate = total[cidx][m];
-            const float up = total[cidx + C][m];
-            value = gate / (1.0f + __expf(-gate)) * up;
-          } else {
-            value = total[cidx][m];
-            if (p.has_addend)
-              value += half_bits_to_float(p.addend[(size_t)m * p.addend_stride + col]);
+          total[r][m] = wave_sum(acc[r][m]);
+          acc[r][m] = 0.0f;
+        }
+      if (lane == 0) {
+#pragma unroll
+        for (int cidx = 0; cidx < C; ++cidx) {
+          const uint32_t col = col0 + cidx;
+          if (col >= n) break;
+#pragma unroll
+          for (int m = 0; m < M; ++m) {
+            if ((uint32_t)m >= p.m) break;
+            float value;
+            if (DUAL) {
+              const float gate = total[cidx][m];
+              const float up = total[cidx + C][m];
+              value = gate / (1.0f + __expf(-gate)) * up;
+            } else {
+              value = total[cidx][m];
+              if (p.has_addend)
+                value += half_bits_to_float(p.addend[(size_t)m * p.addend_stride + col]);
+            }
+            sg.y[(size_t)m * n + col] = float_to_half_bits(value);
           }
-          sg.y[(size_t)m * n + col] = float_to_half_bits(value);
         }
       }
     }
+  };
+
+  auto advance = [&](uint32_t &tile, uint32_t &item) {
+    if (++item == items_per_tile) {
+      item = 0;
+      tile += wave_count;
+    }
+  };
+
+  // Ping-pong between two register sets: the next item's loads are issued
+  // before the current item is decoded.  The prefetch is unconditional (past
+  // the end it re-reads the current item) so that no branch skips the loads:
+  // with a skipped path the compiler must assume the shorter load queue and
+  // waits for the fresh loads before decoding the old ones.
+  uint32_t tile = first_tile, item = 0;
+  while (true) {
+    uint32_t next_tile = tile, next_item = item;
+    advance(next_tile, next_item);
+    bool more = next_tile < p.tiles;
+    load_item(more ? next_tile : tile, more ? next_item : item, item_b);
+    consume(tile, item, item_a);
+    if (!more) break;
+    tile = next_tile;
+    item = next_item;
+    advance(next_tile, next_item);
+    more = next_tile < p.tiles;
+    load_item(more ? next_tile : tile, more ? next_item : item, item_a);
+    consume(tile, item, item_b);
+    if (!more) break;
+    tile = next_tile;
+    item = next_item;
   }
 }
 
@@ -220,22 +294,35 @@ int device_compute_units() {
 
 namespace {
 
-template <int M, int R, bool DUAL>
-hipError_t launch_variant(const GemvParams &p, hipStream_t stream) {
+template <int M, int R, int U, bool DUAL>
+hipError_t launch_variant(GemvParams &p, hipStream_t stream) {
+  // a tile is R weight rows (DUAL: R/2 gate rows + the matching R/2 up rows)
+  constexpr int C = DUAL ? R / 2 : R;
+  uint32_t tiles = 0;
+  const uint32_t count = DUAL ? 1 : p.nseg;
+  for (uint32_t i = 0; i < count; ++i) {
+    p.seg[i].tile_begin = tiles;
+    tiles += (p.seg[i].n + C - 1) / C;
+  }
+  if (DUAL) p.seg[1].tile_begin = 0;
+  p.tiles = tiles;
+
   const uint32_t segs = p.k >> 5;
   const uint32_t chunks = (segs + 63) >> 6;
-  const size_t lds_bytes = (size_t)M * chunks * 256 * sizeof(uint4);
+  // activation vectors (pair order) + one float of bias correction per (m, chunk, lane)
+  const size_t lds_bytes = (size_t)M * chunks * 256 * sizeof(uint4) + (size_t)M * chunks * 64 * sizeof(float);
   const bool use_lds = lds_bytes <= 64 * 1024;
   const int cus = device_compute_units();
-  int per_cu = 4;
-  if (use_lds && lds_bytes > 0)
-    per_cu = (int)std::min<size_t>(4, std::max<size_t>(1, (size_t)(160 * 1024) / lds_bytes));
-  const uint32_t blocks = std::min<uint32_t>(p.tiles, (uint32_t)(cus * per_cu));
+  int per_cu = 2;  // 8 waves per CU, each with two work items of weights in flight
+  if (use_lds && lds_bytes > 80 * 1024) per_cu = 1;
+  if (const char *tune = getenv("LLMOPT_TUNE_GEMV_BLOCKS")) per_cu = atoi(tune);
+  const uint32_t wanted = (tiles + kWaves - 1) / kWaves;
+  const uint32_t blocks = std::max<uint32_t>(1, std::min<uint32_t>(wanted, (uint32_t)(cus * per_cu)));
   if (use_lds) {
-    hipLaunchKernelGGL((w4a16_gemv_kernel<M, R, true, DUAL>), dim3(blocks), dim3(kThreads),
+    hipLaunchKernelGGL((w4a16_gemv_kernel<M, R, U, true, DUAL>), dim3(blocks), dim3(kThreads),
                        lds_bytes, stream, p);
   } else {
-    hipLaunchKernelGGL((w4a16_gemv_kernel<M, R, false, DUAL>), dim3(blocks), dim3(kThreads), 0,
+    hipLaunchKernelGGL((w4a16_gemv_kernel<M, R, U, false, DUAL>), dim3(blocks), dim3(kThreads), 0,
                        stream, p);
   }
   return hipGetLastError();
@@ -243,32 +330,10 @@ hipError_t launch_variant(const GemvParams &p, hipStream_t stream) {
 
 template <bool DUAL>
 hipError_t launch_by_rows(GemvParams &p, hipStream_t stream) {
-  // tiles depend on the columns a workgroup covers: kWaves * C
-  auto finish = [&](int columns_per_wave) {
-    uint32_t tiles = 0;
-    const uint32_t per_tile = kWaves * columns_per_wave;
-    const uint32_t count = DUAL ? 1 : p.nseg;
-    for (uint32_t i = 0; i < count; ++i) {
-      p.seg[i].tile_begin = tiles;
-      tiles += (p.seg[i].n + per_tile - 1) / per_tile;
-    }
-    if (DUAL) p.seg[1].tile_begin = 0;
-    p.tiles = tiles;
-  };
-  if (p.m <= 1) {
-    finish(DUAL ? 2 : 4);
-    return launch_variant<1, 4, DUAL>(p, stream);
-  }
-  if (p.m <= 2) {
-    finish(DUAL ? 2 : 4);
-    return launch_variant<2, 4, DUAL>(p, stream);
-  }
-  if (p.m <= 4) {
-    finish(DUAL ? 1 : 2);
-    return launch_variant<4, 2, DUAL>(p, stream);
-  }
-  finish(DUAL ? 1 : 2);
-  return launch_variant<8, 2, DUAL>(p, stream);
+  if (p.m <= 1) return launch_variant<1, 2, 2, DUAL>(p, stream);
+  if (p.m <= 2) return launch_variant<2, 2, 2, DUAL>(p, stream);
+  if (p.m <= 4) return launch_variant<4, 2, 1, DUAL>(p, stream);
+  return launch_variant<8, 2, 1, DUAL>(p, stream);
 }
 
 __global__ void w4_dequant_f32_kernel(const uint8_t *weight, const uint16_t *scale, float *out,
