@@ -29,15 +29,13 @@ struct GemvSegment {
   const uint16_t *s;
   uint16_t *y;
   uint32_t n;
-  uint32_t tile_begin;  // first tile index of this matrix
 };
 
 struct GemvParams {
   const uint16_t *x;
   uint32_t m, k;
-  GemvSegment seg[3];
-  uint32_t nseg;
-  uint32_t tiles;
+  // blockIdx.y selects the matrix (QKV: three of them; DUAL: seg0 = gate, seg1 = up)
+  GemvSegment seg0, seg1, seg2;
   const uint16_t *addend;
   uint32_t has_addend;
   uint32_t addend_stride;
@@ -59,6 +57,8 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemv_kernel(GemvParams p) {
   // wave-uniform values are forced into scalar registers: tile indices, row
   // pointers and the matrix selection then cost no vector work
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const GemvSegment sg = blockIdx.y == 0 ? p.seg0 : blockIdx.y == 1 ? p.seg1 : p.seg2;
+  const uint32_t tiles = (sg.n + (DUAL ? R / 2 : R) - 1) / (DUAL ? R / 2 : R);
   const uint32_t K = p.k;
   const uint32_t segs = K >> 5;              // 16-byte weight segments per row
   const uint32_t chunks = (segs + 63) >> 6;  // wave-wide steps over K
@@ -76,19 +76,13 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemv_kernel(GemvParams p) {
   };
 
   auto tile_rows = [&](uint32_t tile, const u32x4_t *(&wrow)[R], const uint16_t *(&srow)[R]) {
-    uint32_t which = 0;
-    if (!DUAL) {
-      if (p.nseg > 1 && tile >= p.seg[1].tile_begin) which = 1;
-      if (p.nseg > 2 && tile >= p.seg[2].tile_begin) which = 2;
-    }
-    const GemvSegment &sg = p.seg[which];
-    const uint32_t col0 = (tile - sg.tile_begin) * C;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
-      const uint32_t col = min(col0 + (uint32_t)(DUAL ? r % C : r), sg.n - 1);
-      const GemvSegment &src = DUAL ? p.seg[r / C] : sg;
-      wrow[r] = reinterpret_cast<const u32x4_t *>(src.w + (size_t)col * (K >> 1));
-      srow[r] = src.s + (size_t)col * (K >> 6);
+      const uint32_t col = min(tile * C + (uint32_t)(DUAL ? r % C : r), sg.n - 1);
+      const uint8_t *w = DUAL && r >= C ? p.seg1.w : sg.w;
+      const uint16_t *sc = DUAL && r >= C ? p.seg1.s : sg.s;
+      wrow[r] = reinterpret_cast<const u32x4_t *>(w + (size_t)col * (K >> 1));
+      srow[r] = sc + (size_t)col * (K >> 6);
     }
   };
 
@@ -110,7 +104,7 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemv_kernel(GemvParams p) {
 
   // first weights are in flight while the activation is staged
   Item item_a, item_b;
-  const bool has_work = first_tile < p.tiles;
+  const bool has_work = first_tile < tiles;
   if (has_work) load_item(first_tile, 0, item_a);
 
   // Bias correction of w4_decode_biased per (m, chunk, lane), after the vectors.
@@ -204,14 +198,8 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemv_kernel(GemvParams p) {
     }
 
     if (item + 1 == items_per_tile) {
-      uint32_t which = 0;
-      if (!DUAL) {
-        if (p.nseg > 1 && tile >= p.seg[1].tile_begin) which = 1;
-        if (p.nseg > 2 && tile >= p.seg[2].tile_begin) which = 2;
-      }
-      const GemvSegment &sg = p.seg[which];
       const uint32_t n = sg.n;
-      const uint32_t col0 = (tile - sg.tile_begin) * C;
+      const uint32_t col0 = tile * C;
       float total[R][M];
 #pragma unroll
       for (int r = 0; r < R; ++r)
@@ -261,14 +249,14 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemv_kernel(GemvParams p) {
   while (true) {
     uint32_t next_tile = tile, next_item = item;
     advance(next_tile, next_item);
-    bool more = next_tile < p.tiles;
+    bool more = next_tile < tiles;
     load_item(more ? next_tile : tile, more ? next_item : item, item_b);
     consume(tile, item, item_a);
     if (!more) break;
     tile = next_tile;
     item = next_item;
     advance(next_tile, next_item);
-    more = next_tile < p.tiles;
+    more = next_tile < tiles;
     load_item(more ? next_tile : tile, more ? next_item : item, item_a);
     consume(tile, item, item_b);
     if (!more) break;
@@ -295,17 +283,10 @@ int device_compute_units() {
 namespace {
 
 template <int M, int R, int U, bool DUAL>
-hipError_t launch_variant(GemvParams &p, hipStream_t stream) {
+hipError_t launch_variant(const GemvParams &p, uint32_t matrices, uint32_t max_n, hipStream_t stream) {
   // a tile is R weight rows (DUAL: R/2 gate rows + the matching R/2 up rows)
   constexpr int C = DUAL ? R / 2 : R;
-  uint32_t tiles = 0;
-  const uint32_t count = DUAL ? 1 : p.nseg;
-  for (uint32_t i = 0; i < count; ++i) {
-    p.seg[i].tile_begin = tiles;
-    tiles += (p.seg[i].n + C - 1) / C;
-  }
-  if (DUAL) p.seg[1].tile_begin = 0;
-  p.tiles = tiles;
+  const uint32_t tiles = (max_n + C - 1) / C;  // of the largest matrix
 
   const uint32_t segs = p.k >> 5;
   const uint32_t chunks = (segs + 63) >> 6;
@@ -319,21 +300,21 @@ hipError_t launch_variant(GemvParams &p, hipStream_t stream) {
   const uint32_t wanted = (tiles + kWaves - 1) / kWaves;
   const uint32_t blocks = std::max<uint32_t>(1, std::min<uint32_t>(wanted, (uint32_t)(cus * per_cu)));
   if (use_lds) {
-    hipLaunchKernelGGL((w4a16_gemv_kernel<M, R, U, true, DUAL>), dim3(blocks), dim3(kThreads),
+    hipLaunchKernelGGL((w4a16_gemv_kernel<M, R, U, true, DUAL>), dim3(blocks, matrices), dim3(kThreads),
                        lds_bytes, stream, p);
   } else {
-    hipLaunchKernelGGL((w4a16_gemv_kernel<M, R, U, false, DUAL>), dim3(blocks), dim3(kThreads), 0,
+    hipLaunchKernelGGL((w4a16_gemv_kernel<M, R, U, false, DUAL>), dim3(blocks, matrices), dim3(kThreads), 0,
                        stream, p);
   }
   return hipGetLastError();
 }
 
 template <bool DUAL>
-hipError_t launch_by_rows(GemvParams &p, hipStream_t stream) {
-  if (p.m <= 1) return launch_variant<1, 2, 2, DUAL>(p, stream);
-  if (p.m <= 2) return launch_variant<2, 2, 2, DUAL>(p, stream);
-  if (p.m <= 4) return launch_variant<4, 2, 1, DUAL>(p, stream);
-  return launch_variant<8, 2, 1, DUAL>(p, stream);
+hipError_t launch_by_rows(const GemvParams &p, uint32_t matrices, uint32_t max_n, hipStream_t stream) {
+  if (p.m <= 1) return launch_variant<1, 2, 2, DUAL>(p, matrices, max_n, stream);
+  if (p.m <= 2) return launch_variant<2, 2, 2, DUAL>(p, matrices, max_n, stream);
+  if (p.m <= 4) return launch_variant<4, 2, 1, DUAL>(p, matrices, max_n, stream);
+  return launch_variant<8, 2, 1, DUAL>(p, matrices, max_n, stream);
 }
 
 __global__ void w4_dequant_f32_kernel(const uint8_t *weight, const uint16_t *scale, float *out,
@@ -359,12 +340,11 @@ hipError_t launch_w4a16_gemv_linear(const W4LinearArgs &a, hipStream_t stream) {
   p.x = a.x;
   p.m = a.m;
   p.k = a.k;
-  p.seg[0] = {a.w.weight, a.w.scale, a.y, a.n, 0};
-  p.nseg = 1;
+  p.seg0 = {a.w.weight, a.w.scale, a.y, a.n};
   p.addend = a.addend;
   p.has_addend = a.has_addend;
   p.addend_stride = a.addend_row_stride;
-  return launch_by_rows<false>(p, stream);
+  return launch_by_rows<false>(p, 1, a.n, stream);
 }
 
 hipError_t launch_w4a16_gemv_qkv(const W4QkvArgs &a, hipStream_t stream) {
@@ -372,9 +352,10 @@ hipError_t launch_w4a16_gemv_qkv(const W4QkvArgs &a, hipStream_t stream) {
   p.x = a.x;
   p.m = a.m;
   p.k = a.k;
-  for (int i = 0; i < 3; ++i) p.seg[i] = {a.w[i].weight, a.w[i].scale, a.y[i], a.n[i], 0};
-  p.nseg = 3;
-  return launch_by_rows<false>(p, stream);
+  p.seg0 = {a.w[0].weight, a.w[0].scale, a.y[0], a.n[0]};
+  p.seg1 = {a.w[1].weight, a.w[1].scale, a.y[1], a.n[1]};
+  p.seg2 = {a.w[2].weight, a.w[2].scale, a.y[2], a.n[2]};
+  return launch_by_rows<false>(p, 3, std::max(a.n[0], std::max(a.n[1], a.n[2])), stream);
 }
 
 hipError_t launch_w4a16_gemv_dual_swiglu(const W4DualSwigluArgs &a, hipStream_t stream) {
@@ -382,10 +363,9 @@ hipError_t launch_w4a16_gemv_dual_swiglu(const W4DualSwigluArgs &a, hipStream_t 
   p.x = a.x;
   p.m = a.m;
   p.k = a.k;
-  p.seg[0] = {a.gate.weight, a.gate.scale, a.product, a.n, 0};
-  p.seg[1] = {a.up.weight, a.up.scale, a.product, a.n, 0};
-  p.nseg = 2;
-  return launch_by_rows<true>(p, stream);
+  p.seg0 = {a.gate.weight, a.gate.scale, a.product, a.n};
+  p.seg1 = {a.up.weight, a.up.scale, a.product, a.n};
+  return launch_by_rows<true>(p, 1, a.n, stream);
 }
 
 hipError_t launch_w4_dequant_f32(const W4Matrix &w, float *out, uint32_t n, uint32_t k,
