@@ -117,5 +117,7 @@ hipError_t launch_q8_attention(const Q8AttentionArgs &args, hipStream_t stream);
 
 // The largest m the streaming GEMV path takes; above it the MFMA GEMM runs.
 constexpr uint32_t kGemvMaxRows = 8;
+// Up to this m the GEMV uses v_dot2 on the vector ALUs, above it the matrix cores.
+constexpr uint32_t kGemvDotRows = 4;
 
 }  // namespace llmopt
