@@ -95,6 +95,7 @@ struct Q8AttentionArgs {
   const uint16_t *current_key;    // f16 [b, kvh, q, D]
   const uint16_t *current_value;  // f16 [b, kvh, q, D]
   const uint8_t *pool;
+  size_t pool_bytes;  // 0 if unknown; below 4 GiB enables 32-bit slot offsets
   const uint32_t *slots;
   const uint8_t *mask;  // may be null
   uint16_t *output;     // f16 token-major [b, q, h, D]

@@ -30,9 +30,8 @@
 namespace llmopt {
 namespace {
 
-constexpr int kSplitThreads = 256;
-constexpr int kSplitWaves = 4;
-constexpr int kChunkTokens = 256;  // tokens per workgroup
+constexpr int kSplitMaxWaves = 4;   // KV heads per workgroup (one wave each)
+constexpr int kChunkTokens = 128;   // context tokens per workgroup
 constexpr int kTileTokens = 16;    // tokens per MFMA tile
 
 __device__ __forceinline__ float q8_scale_at(const uint8_t *token, uint32_t token_elements,
@@ -45,6 +44,13 @@ __device__ __forceinline__ void int8x4_to_h2(uint32_t biased, h2_t &lo, h2_t &hi
   const h2_t offset = {(_Float16)1152.0f, (_Float16)1152.0f};  // 1024 + 128
   lo = as_h2(__builtin_amdgcn_perm(0x64646464u, biased, 0x04010400u)) - offset;
   hi = as_h2(__builtin_amdgcn_perm(0x64646464u, biased, 0x04030402u)) - offset;
+}
+
+// Same without the subtraction: exact integers q + 1152.  Used for K, where the
+// bias becomes a per-head constant 1152 * sum_d(Q[d]) subtracted from the score.
+__device__ __forceinline__ void int8x4_to_h2_biased(uint32_t biased, h2_t &lo, h2_t &hi) {
+  lo = as_h2(__builtin_amdgcn_perm(0x64646464u, biased, 0x04010400u));
+  hi = as_h2(__builtin_amdgcn_perm(0x64646464u, biased, 0x04030402u));
 }
 
 __device__ __forceinline__ float shfl_xor_f32(float value, int mask) {
@@ -63,26 +69,30 @@ __device__ __forceinline__ size_t partial_floats(uint32_t heads_per_kv) {
   return 32 + (size_t)heads_per_kv * D;
 }
 
-template <int D>
-__global__ __launch_bounds__(kSplitThreads) void q8_attention_split_kernel(Q8AttentionArgs a,
+// OFF32: the pool is smaller than 4 GiB, so slot byte offsets fit 32 bits and the
+// loads can use a scalar base plus a 32-bit vector offset.
+template <int D, bool OFF32>
+__global__ __launch_bounds__(kSplitMaxWaves * 64) void q8_attention_split_kernel(Q8AttentionArgs a,
                                                                            uint32_t chunks_max) {
   constexpr int GROUPS = D / 64;      // scale groups per head
   constexpr int KLOADS = GROUPS;      // 16-byte K loads per lane per tile
   constexpr int VBLOCKS = D / 16;     // PV MFMAs (16 head_dim rows each)
-  __shared__ float merge_lds[kSplitWaves][32 + 16 * D];
-
+  // One wave per KV head; the waves of a workgroup walk the same tokens, so the
+  // cache lines of a token (its heads are adjacent in the pool slot, and all
+  // its scales share one line) are fetched into one CU instead of eight XCDs.
   const uint32_t chunk = blockIdx.x;
-  const uint32_t kv_head = blockIdx.y;
   const uint32_t batch = blockIdx.z;
   const uint32_t lane = threadIdx.x & 63;
-  const uint32_t wave = threadIdx.x >> 6;
+  const uint32_t kv_head =
+      blockIdx.y * kSplitMaxWaves + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  if (kv_head >= a.kv_heads) return;  // whole wave; no workgroup barriers below
   const uint32_t col = lane & 15;  // query head within the group / token / d-row
   const uint32_t quad = lane >> 4;
   const uint32_t heads_per_kv = a.query_heads / a.kv_heads;
 
   const uint32_t past = a.past_lengths ? a.past_lengths[batch] : a.past_length;
   const uint32_t chunk_begin = chunk * kChunkTokens;
-  if (chunk_begin >= past) return;  // whole workgroup (uniform)
+  if (chunk_begin >= past) return;
   const uint32_t *slots = a.slot_offsets ? a.slots + a.slot_offsets[batch] : a.slots;
   const uint32_t last_token = past - 1;
 
@@ -102,6 +112,23 @@ __global__ __launch_bounds__(kSplitThreads) void q8_attention_split_kernel(Q8Att
       }
   }
 
+  // 1152 * sum_d Q[head][d] per scale group: the constant the biased K decode
+  // adds to every score of this head
+  float key_bias[GROUPS];
+#pragma unroll
+  for (int g = 0; g < GROUPS; ++g) {
+    float sum = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sum += (float)q_frag[g][j][e];
+    sum += shfl_xor_f32(sum, 16);
+    sum += shfl_xor_f32(sum, 32);
+    key_bias[g] = 1152.0f * sum;
+  }
+  // softmax runs in base 2: exp(x) = exp2(x * log2(e))
+  const float score_scale = a.scale * 1.4426950408889634f;
+
   const uint32_t key_base = a.key_offset + kv_head * D;
   const uint32_t value_base = a.value_offset + kv_head * D;
   const uint32_t key_scale_index = (a.key_offset >> 6) + kv_head * GROUPS;
@@ -113,34 +140,76 @@ __global__ __launch_bounds__(kSplitThreads) void q8_attention_split_kernel(Q8Att
 #pragma unroll
   for (int v = 0; v < VBLOCKS; ++v) out_acc[v] = f4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
-  // waves interleave 16-token tiles of the chunk
-  for (uint32_t tile = wave; tile < kChunkTokens / kTileTokens; tile += kSplitWaves) {
+  // Loaded-but-untouched registers of one 16-token tile.  Nothing in here may be
+  // used before the tile is processed, or the loads are waited for at once.
+  struct TileSlots {
+    uint32_t key;       // slot of token (tile0 + col)
+    uint32_t value[4];  // slots of tokens (tile0 + quad*4 + i)
+  };
+  struct TileRaw {
+    u32x4_t k[KLOADS];          // lane (token = col, quad): 16 head_dim values per group
+    uint32_t v[4][GROUPS];      // lane (d-row = col, quad): tokens quad*4 + i
+    uint32_t k_scale[4];        // D = 128: both group scales of the token in one dword
+    uint32_t v_scale[4];        // D = 64: the single scale in the low half
+  };
+  // D = 128 reads the two adjacent fp16 scales of a (token, head) as one dword;
+  // the scale index is even because every segment offset is a multiple of 128.
+  auto load_slots = [&](uint32_t tile, TileSlots &out) __attribute__((always_inline)) {
     const uint32_t token0 = chunk_begin + tile * kTileTokens;
-    if (token0 >= past) break;  // wave-uniform
-
-    // ---- K: lane (token = col, quad) holds 16 head_dim values per group ----
-    const uint32_t key_token = min(token0 + col, last_token);
-    const uint8_t *key_slot = a.pool + (size_t)slots[key_token] * a.token_stride;
-    u32x4_t k_raw[KLOADS];
+    out.key = slots[min(token0 + col, last_token)];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) out.value[i] = slots[min(token0 + quad * 4 + i, last_token)];
+  };
+  // With OFF32 every address is the scalar pool base plus one 32-bit lane offset
+  // and a compile-time displacement, so a load needs no 64-bit vector add.
+  auto load_raw = [&](const TileSlots &where, TileRaw &out) __attribute__((always_inline)) {
+    if (OFF32) {
+      const uint32_t key_offset = where.key * a.token_stride + key_base + quad * 16;
+#pragma unroll
+      for (int g = 0; g < KLOADS; ++g)
+        out.k[g] = *reinterpret_cast<const u32x4_t *>(a.pool + key_offset + g * 64);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t slot_offset = where.value[i] * a.token_stride;
+        const uint32_t value_offset = slot_offset + value_base + col * 4;
+#pragma unroll
+        for (int g = 0; g < GROUPS; ++g)
+          out.v[i][g] = *reinterpret_cast<const uint32_t *>(a.pool + value_offset + g * 64);
+        const uint32_t key_scale_offset = slot_offset + a.token_elements + 2 * key_scale_index;
+        const uint32_t value_scale_offset = slot_offset + a.token_elements + 2 * value_scale_index;
+        if (GROUPS == 2) {
+          out.k_scale[i] = *reinterpret_cast<const uint32_t *>(a.pool + key_scale_offset);
+          out.v_scale[i] = *reinterpret_cast<const uint32_t *>(a.pool + value_scale_offset);
+        } else {
+          out.k_scale[i] = *reinterpret_cast<const uint16_t *>(a.pool + key_scale_offset);
+          out.v_scale[i] = *reinterpret_cast<const uint16_t *>(a.pool + value_scale_offset);
+        }
+      }
+      return;
+    }
+    const uint8_t *key_slot = a.pool + (size_t)where.key * a.token_stride;
 #pragma unroll
     for (int g = 0; g < KLOADS; ++g)
-      k_raw[g] = *reinterpret_cast<const u32x4_t *>(key_slot + key_base + g * 64 + quad * 16);
-
-    // ---- V and scales: lane (d-row = col, quad) holds tokens quad*4 + i ----
-    uint32_t v_raw[4][GROUPS];
-    float k_scale[4][GROUPS], v_scale[4][GROUPS];
+      out.k[g] = *reinterpret_cast<const u32x4_t *>(key_slot + key_base + g * 64 + quad * 16);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      const uint32_t token = min(token0 + quad * 4 + i, last_token);
-      const uint8_t *slot = a.pool + (size_t)slots[token] * a.token_stride;
+      const uint8_t *slot = a.pool + (size_t)where.value[i] * a.token_stride;
 #pragma unroll
-      for (int g = 0; g < GROUPS; ++g) {
-        v_raw[i][g] = *reinterpret_cast<const uint32_t *>(slot + value_base + g * 64 + col * 4);
-        k_scale[i][g] = q8_scale_at(slot, a.token_elements, key_scale_index + g);
-        v_scale[i][g] = q8_scale_at(slot, a.token_elements, value_scale_index + g);
+      for (int g = 0; g < GROUPS; ++g)
+        out.v[i][g] = *reinterpret_cast<const uint32_t *>(slot + value_base + g * 64 + col * 4);
+      const uint8_t *scales = slot + a.token_elements;
+      if (GROUPS == 2) {
+        out.k_scale[i] = *reinterpret_cast<const uint32_t *>(scales + 2 * key_scale_index);
+        out.v_scale[i] = *reinterpret_cast<const uint32_t *>(scales + 2 * value_scale_index);
+      } else {
+        out.k_scale[i] = *reinterpret_cast<const uint16_t *>(scales + 2 * key_scale_index);
+        out.v_scale[i] = *reinterpret_cast<const uint16_t *>(scales + 2 * value_scale_index);
       }
     }
+  };
 
+  auto process = [&](uint32_t tile, const TileRaw &raw) __attribute__((always_inline)) {
+    const uint32_t token0 = chunk_begin + tile * kTileTokens;
     // ---- scores S^T[token][head] = sum_g k_scale[token][g] * (K_g . Q_g) ----
     f4_t score = f4_t{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
@@ -149,33 +218,35 @@ __global__ __launch_bounds__(kSplitThreads) void q8_attention_split_kernel(Q8Att
 #pragma unroll
       for (int j = 0; j < 2; ++j) {
         h2_t h0, h1, h2, h3;
-        int8x4_to_h2(k_raw[g][2 * j] ^ 0x80808080u, h0, h1);
-        int8x4_to_h2(k_raw[g][2 * j + 1] ^ 0x80808080u, h2, h3);
+        int8x4_to_h2_biased(raw.k[g][2 * j] ^ 0x80808080u, h0, h1);
+        int8x4_to_h2_biased(raw.k[g][2 * j + 1] ^ 0x80808080u, h2, h3);
         const h8_t k_frag = {h0[0], h0[1], h1[0], h1[1], h2[0], h2[1], h3[0], h3[1]};
         part = __builtin_amdgcn_mfma_f32_16x16x32_f16(k_frag, q_frag[g][j], part, 0, 0, 0);
       }
 #pragma unroll
-      for (int i = 0; i < 4; ++i) score[i] = fmaf(part[i], k_scale[i][g], score[i]);
+      for (int i = 0; i < 4; ++i)
+        score[i] = fmaf(part[i] - key_bias[g],
+                        half_bits_to_float((uint16_t)(raw.k_scale[i] >> (16 * g))), score[i]);
     }
     float tile_max = -INFINITY;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const bool valid = token0 + quad * 4 + i < past;
-      score[i] = valid ? score[i] * a.scale : -INFINITY;
+      score[i] = valid ? score[i] * score_scale : -INFINITY;
       tile_max = fmaxf(tile_max, score[i]);
     }
     tile_max = fmaxf(tile_max, shfl_xor_f32(tile_max, 16));
     tile_max = fmaxf(tile_max, shfl_xor_f32(tile_max, 32));
     // the first token of the tile is valid, so tile_max is finite
     const float new_max = fmaxf(running_max, tile_max);
-    const float alpha = __expf(running_max - new_max);  // exp(-inf) = 0 on the first tile
+    const float alpha = __builtin_amdgcn_exp2f(running_max - new_max);  // 0 on the first tile
     running_max = new_max;
 
     float p[4];
     float tile_sum = 0.0f;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      p[i] = __expf(score[i] - new_max);
+      p[i] = __builtin_amdgcn_exp2f(score[i] - new_max);
       tile_sum += p[i];
     }
     running_sum = running_sum * alpha + tile_sum;
@@ -193,9 +264,10 @@ __global__ __launch_bounds__(kSplitThreads) void q8_attention_split_kernel(Q8Att
     for (int g = 0; g < GROUPS; ++g) {
       h4_t p_frag;
 #pragma unroll
-      for (int i = 0; i < 4; ++i) p_frag[i] = (_Float16)(p[i] * v_scale[i][g]);
-      const uint32_t a0 = v_raw[0][g] ^ 0x80808080u, a1 = v_raw[1][g] ^ 0x80808080u;
-      const uint32_t a2 = v_raw[2][g] ^ 0x80808080u, a3 = v_raw[3][g] ^ 0x80808080u;
+      for (int i = 0; i < 4; ++i)
+        p_frag[i] = (_Float16)(p[i] * half_bits_to_float((uint16_t)(raw.v_scale[i] >> (16 * g))));
+      const uint32_t a0 = raw.v[0][g] ^ 0x80808080u, a1 = raw.v[1][g] ^ 0x80808080u;
+      const uint32_t a2 = raw.v[2][g] ^ 0x80808080u, a3 = raw.v[3][g] ^ 0x80808080u;
       const uint32_t t01_lo = __builtin_amdgcn_perm(a1, a0, 0x05010400u);
       const uint32_t t01_hi = __builtin_amdgcn_perm(a1, a0, 0x07030602u);
       const uint32_t t23_lo = __builtin_amdgcn_perm(a3, a2, 0x05010400u);
@@ -213,94 +285,143 @@ __global__ __launch_bounds__(kSplitThreads) void q8_attention_split_kernel(Q8Att
             __builtin_amdgcn_mfma_f32_16x16x16f16(v_frag, p_frag, out_acc[g * 4 + jj], 0, 0, 0);
       }
     }
+  };
+
+  // The wave walks the 16-token tiles of the chunk.  Slot indices run two tiles
+  // ahead and the K/V bytes one tile ahead of the arithmetic; requests past the
+  // last tile are clamped to valid tokens and never used.
+  const uint32_t chunk_tiles = (min(past - chunk_begin, (uint32_t)kChunkTokens) + kTileTokens - 1) / kTileTokens;
+  {
+    TileSlots slots_a, slots_b;
+    TileRaw raw_a, raw_b;
+    load_slots(0, slots_a);
+    load_slots(1, slots_b);
+    load_raw(slots_a, raw_a);
+    // Loads return in issue order, so the small slot loads go out before the
+    // K/V loads of the same step: waiting for a slot then never waits for a
+    // younger K/V request.
+    for (uint32_t tile = 0; tile < chunk_tiles; tile += 2) {
+      load_slots(tile + 2, slots_a);
+      load_raw(slots_b, raw_b);
+      process(tile, raw_a);
+      if (tile + 1 >= chunk_tiles) break;
+      load_slots(tile + 3, slots_b);
+      load_raw(slots_a, raw_a);
+      process(tile + 1, raw_b);
+    }
   }
 
-  // ---- merge the 4 waves, write one partial per (batch, kv_head, chunk) ----
+  // ---- one partial per (batch, kv_head, chunk), straight from registers ----
   // out_acc[g*4+jj][i] is O[head = col][d = g*64 + 4*(quad*4 + i) + jj].
   running_sum += shfl_xor_f32(running_sum, 16);
   running_sum += shfl_xor_f32(running_sum, 32);
-  float *mine = merge_lds[wave];
-  if (quad == 0) {
-    mine[col] = running_max;
-    mine[16 + col] = running_sum;
-  }
-#pragma unroll
-  for (int v = 0; v < VBLOCKS; ++v)
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const uint32_t d = (v >> 2) * 64 + 4 * (quad * 4 + i) + (v & 3);
-      mine[32 + col * D + d] = out_acc[v][i];
-    }
-  __syncthreads();
-
   float *partial = reinterpret_cast<float *>(a.workspace) +
                    (((size_t)batch * a.kv_heads + kv_head) * chunks_max + chunk) *
                        partial_floats<D>(heads_per_kv);
-  for (uint32_t index = threadIdx.x; index < heads_per_kv * D; index += kSplitThreads) {
-    const uint32_t head = index / D;
-    float best = -INFINITY;
-#pragma unroll
-    for (int w = 0; w < kSplitWaves; ++w) best = fmaxf(best, merge_lds[w][head]);
-    float sum = 0.0f, value = 0.0f;
-#pragma unroll
-    for (int w = 0; w < kSplitWaves; ++w) {
-      const float wave_max_value = merge_lds[w][head];
-      const float weight = wave_max_value == -INFINITY ? 0.0f : __expf(wave_max_value - best);
-      sum += merge_lds[w][16 + head] * weight;
-      value += merge_lds[w][32 + index] * weight;
+  if (col < heads_per_kv) {
+    if (quad == 0) {
+      partial[col] = running_max;
+      partial[16 + col] = running_sum;
     }
-    partial[32 + index] = value;
-    if (index == head * D) {
-      partial[head] = best;
-      partial[16 + head] = sum;
-    }
+#pragma unroll
+    for (int v = 0; v < VBLOCKS; ++v)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t d = (v >> 2) * 64 + 4 * (quad * 4 + i) + (v & 3);
+        partial[32 + col * D + d] = out_acc[v][i];
+      }
   }
 }
 
-// One workgroup of D threads per (batch, query head): folds the chunk partials
-// and the current token (fp16 K/V) into the output row.
+constexpr int kMaxSplitChunks = 1024;  // merge kernel keeps one weight per chunk in LDS
+
+constexpr int kMergeSlices = 4;  // chunk slices summed in parallel per output row
+
+// One workgroup of kMergeSlices * D threads per (batch, query head): folds the
+// chunk partials and the current token (fp16 K/V) into the output row.  Phase 1
+// finds the global maximum and the per-chunk weights exp2(max_c - max) in
+// parallel over chunks; phase 2 is an independent-load weighted sum over a
+// quarter of the chunks per thread, finished through LDS.
 template <int D>
-__global__ __launch_bounds__(D) void q8_attention_merge_kernel(Q8AttentionArgs a,
-                                                               uint32_t chunks_max) {
-  __shared__ float reduce_lds[D / 64];
+__global__ __launch_bounds__(kMergeSlices *D) void q8_attention_merge_kernel(Q8AttentionArgs a,
+                                                                             uint32_t chunks_max) {
+  constexpr int THREADS = kMergeSlices * D;
+  constexpr int WAVES = THREADS / 64;
+  __shared__ float reduce_lds[3][WAVES];
+  __shared__ float weight_lds[kMaxSplitChunks];
+  __shared__ float slice_lds[kMergeSlices][D];
   const uint32_t head = blockIdx.x;
   const uint32_t batch = blockIdx.y;
-  const uint32_t d = threadIdx.x;
+  const uint32_t tid = threadIdx.x;
+  const uint32_t d = tid % D;
+  const uint32_t slice = tid / D;
   const uint32_t heads_per_kv = a.query_heads / a.kv_heads;
   const uint32_t kv_head = head / heads_per_kv;
   const uint32_t local_head = head - kv_head * heads_per_kv;
   const uint32_t past = a.past_lengths ? a.past_lengths[batch] : a.past_length;
   const uint32_t chunks = (past + kChunkTokens - 1) / kChunkTokens;
-
-  // score of the current token
-  const float q = half_bits_to_float(a.query[((size_t)batch * a.query_heads + head) * D + d]);
-  const size_t current = ((size_t)batch * a.kv_heads + kv_head) * D + d;
-  float dot = wave_sum(q * half_bits_to_float(a.current_key[current]));
-  if ((d & 63) == 0) reduce_lds[d >> 6] = dot;
-  __syncthreads();
-  float score = 0.0f;
-#pragma unroll
-  for (int w = 0; w < D / 64; ++w) score += reduce_lds[w];
-  score *= a.scale;
-
-  float best = score;
-  float denominator = 1.0f;
-  float value = half_bits_to_float(a.current_value[current]);
+  const size_t stride = partial_floats<D>(heads_per_kv);
   const float *partial = reinterpret_cast<const float *>(a.workspace) +
-                         ((size_t)batch * a.kv_heads + kv_head) * chunks_max *
-                             partial_floats<D>(heads_per_kv);
-  for (uint32_t c = 0; c < chunks; ++c, partial += partial_floats<D>(heads_per_kv)) {
-    const float chunk_max = partial[local_head];
-    const float chunk_sum = partial[16 + local_head];
-    const float chunk_value = partial[32 + local_head * D + d];
-    const float new_best = fmaxf(best, chunk_max);
-    const float keep = __expf(best - new_best);
-    const float take = __expf(chunk_max - new_best);
-    denominator = denominator * keep + chunk_sum * take;
-    value = value * keep + chunk_value * take;
-    best = new_best;
+                         ((size_t)batch * a.kv_heads + kv_head) * chunks_max * stride;
+
+  // score of the current token (slice 0 holds the dot product) and the largest chunk maximum
+  const size_t current = ((size_t)batch * a.kv_heads + kv_head) * D + d;
+  float dot = 0.0f;
+  if (slice == 0)
+    dot = half_bits_to_float(a.query[((size_t)batch * a.query_heads + head) * D + d]) *
+          half_bits_to_float(a.current_key[current]);
+  dot = wave_sum(dot);
+  float chunk_best = -INFINITY;
+  for (uint32_t c = tid; c < chunks; c += THREADS)
+    chunk_best = fmaxf(chunk_best, partial[c * stride + local_head]);
+  chunk_best = wave_max(chunk_best);
+  if ((tid & 63) == 0) {
+    reduce_lds[0][tid >> 6] = dot;
+    reduce_lds[1][tid >> 6] = chunk_best;
   }
-  a.output[((size_t)batch * a.query_heads + head) * D + d] = float_to_half_bits(value / denominator);
+  __syncthreads();
+  float score = 0.0f, best = -INFINITY;
+#pragma unroll
+  for (int w = 0; w < WAVES; ++w) {
+    score += reduce_lds[0][w];
+    best = fmaxf(best, reduce_lds[1][w]);
+  }
+  score *= a.scale * 1.4426950408889634f;  // the partial maxima are in base-2 units
+  best = fmaxf(best, score);
+
+  // weights and denominator
+  float denominator_part = 0.0f;
+  for (uint32_t c = tid; c < chunks; c += THREADS) {
+    const float weight = __builtin_amdgcn_exp2f(partial[c * stride + local_head] - best);
+    weight_lds[c] = weight;
+    denominator_part += weight * partial[c * stride + 16 + local_head];
+  }
+  denominator_part = wave_sum(denominator_part);
+  if ((tid & 63) == 0) reduce_lds[2][tid >> 6] = denominator_part;
+  __syncthreads();
+  const float current_weight = __builtin_amdgcn_exp2f(score - best);
+  float denominator = current_weight;
+#pragma unroll
+  for (int w = 0; w < WAVES; ++w) denominator += reduce_lds[2][w];
+
+  float value = slice == 0 ? current_weight * half_bits_to_float(a.current_value[current]) : 0.0f;
+  const float *column = partial + 32 + local_head * D + d;
+  uint32_t c = slice;
+  for (; c + 3 * kMergeSlices < chunks; c += 4 * kMergeSlices) {
+    const float v0 = column[(c + 0 * kMergeSlices) * stride], v1 = column[(c + 1 * kMergeSlices) * stride];
+    const float v2 = column[(c + 2 * kMergeSlices) * stride], v3 = column[(c + 3 * kMergeSlices) * stride];
+    value += weight_lds[c] * v0 + weight_lds[c + kMergeSlices] * v1 +
+             weight_lds[c + 2 * kMergeSlices] * v2 + weight_lds[c + 3 * kMergeSlices] * v3;
+  }
+  for (; c < chunks; c += kMergeSlices) value += weight_lds[c] * column[c * stride];
+  slice_lds[slice][d] = value;
+  __syncthreads();
+  if (slice == 0) {
+    float total = 0.0f;
+#pragma unroll
+    for (int s = 0; s < kMergeSlices; ++s) total += slice_lds[s][d];
+    a.output[((size_t)batch * a.query_heads + head) * D + d] = float_to_half_bits(total / denominator);
+  }
 }
 
 // ---- row-serial kernel (every other configuration) ---------------------------
@@ -402,6 +523,9 @@ bool use_split_path(const Q8AttentionArgs &a) {
   // 16-byte K loads and 4-byte V loads from pool slots
   if (a.token_stride % 16 != 0 || a.key_offset % 16 != 0 || a.value_offset % 4 != 0) return false;
   if (a.token_elements % 2 != 0) return false;
+  // D = 128 reads the two group scales of a head as one aligned dword
+  if (a.head_dim == 128 && (a.key_offset % 128 != 0 || a.value_offset % 128 != 0)) return false;
+  if (a.max_past_length > (uint32_t)kChunkTokens * kMaxSplitChunks) return false;
   return a.max_past_length >= 64;  // short contexts: one launch of the row kernel is cheaper
 }
 
@@ -422,14 +546,23 @@ hipError_t launch_q8_attention(const Q8AttentionArgs &a, hipStream_t stream) {
     const uint32_t chunks = split_chunks(a);
     if (a.workspace == nullptr || a.workspace_bytes < q8_attention_workspace_bytes(a))
       return hipErrorInvalidValue;
-    const dim3 grid(chunks, a.kv_heads, a.batches);
+    const uint32_t waves = std::min<uint32_t>(a.kv_heads, kSplitMaxWaves);
+    const dim3 grid(chunks, (a.kv_heads + kSplitMaxWaves - 1) / kSplitMaxWaves, a.batches);
+    const dim3 block(waves * 64);
     const dim3 merge_grid(a.query_heads, a.batches);
+    const bool small_pool = a.pool_bytes > 0 && a.pool_bytes <= 0xffffffffull;
     if (a.head_dim == 128) {
-      hipLaunchKernelGGL(q8_attention_split_kernel<128>, grid, dim3(kSplitThreads), 0, stream, a, chunks);
-      hipLaunchKernelGGL(q8_attention_merge_kernel<128>, merge_grid, dim3(128), 0, stream, a, chunks);
+      if (small_pool)
+        hipLaunchKernelGGL((q8_attention_split_kernel<128, true>), grid, block, 0, stream, a, chunks);
+      else
+        hipLaunchKernelGGL((q8_attention_split_kernel<128, false>), grid, block, 0, stream, a, chunks);
+      hipLaunchKernelGGL(q8_attention_merge_kernel<128>, merge_grid, dim3(kMergeSlices * 128), 0, stream, a, chunks);
     } else {
-      hipLaunchKernelGGL(q8_attention_split_kernel<64>, grid, dim3(kSplitThreads), 0, stream, a, chunks);
-      hipLaunchKernelGGL(q8_attention_merge_kernel<64>, merge_grid, dim3(64), 0, stream, a, chunks);
+      if (small_pool)
+        hipLaunchKernelGGL((q8_attention_split_kernel<64, true>), grid, block, 0, stream, a, chunks);
+      else
+        hipLaunchKernelGGL((q8_attention_split_kernel<64, false>), grid, block, 0, stream, a, chunks);
+      hipLaunchKernelGGL(q8_attention_merge_kernel<64>, merge_grid, dim3(kMergeSlices * 64), 0, stream, a, chunks);
     }
     return hipGetLastError();
   }

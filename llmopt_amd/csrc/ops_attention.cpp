@@ -194,6 +194,7 @@ int paged_attention(llmopt_hip_context *context, const DispatchRecord &record, b
   args.current_key = reinterpret_cast<const uint16_t *>(record.buffers[1].device);
   args.current_value = reinterpret_cast<const uint16_t *>(record.buffers[2].device);
   args.pool = record.buffers[3].device;
+  args.pool_bytes = record.buffers[3].length;
   args.slots = reinterpret_cast<const uint32_t *>(record.buffers[4].device);
   args.mask = masked ? record.buffers[5].device : nullptr;
   args.output = reinterpret_cast<uint16_t *>(record.buffers[6].device);
