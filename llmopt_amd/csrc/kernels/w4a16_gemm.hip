@@ -26,11 +26,10 @@
 namespace llmopt {
 namespace {
 
-constexpr int BM = 128;
-constexpr int BN = 128;
-constexpr int BK = 64;             // one scale group per K step
+constexpr int BK = 64;              // one scale group per K step
 constexpr int LDS_STRIDE = BK + 8;  // halfs; 144-byte rows keep b128 reads conflict-free
-constexpr int kThreads = 256;
+constexpr int kWaves = 8;           // 4 (m) x 2 (n) waves, two per SIMD
+constexpr int kThreads = kWaves * 64;
 
 struct GemmParams {
   const uint16_t *x;
@@ -51,17 +50,26 @@ __device__ __forceinline__ f16x_t zero_tile() {
   return z;
 }
 
-template <bool DUAL>
+// Each wave owns WM x WN MFMA tiles of 32 x 32 outputs; the workgroup tile is
+// (4 * WM * 32) x (2 * WN * 32).  DUAL computes gate and up tiles of the same
+// outputs and stores silu(gate) * up.
+template <int WM, int WN, bool DUAL>
 __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
   constexpr int NW = DUAL ? 2 : 1;  // weight matrices per tile
-  __shared__ __attribute__((aligned(16))) _Float16 x_lds[BM * LDS_STRIDE];
-  __shared__ __attribute__((aligned(16))) _Float16 w_lds[NW][BN * LDS_STRIDE];
-  __shared__ float s_lds[NW][BN];
+  constexpr int BM = 4 * WM * 32;
+  constexpr int BN = 2 * WN * 32;
+  constexpr int X_VECTORS = BM * BK / 8 / kThreads;    // 16-byte activation vectors per thread
+  constexpr int W_VECTORS = (BN * BK / 32 + kThreads - 1) / kThreads;  // 32-nibble vectors per thread
+  static_assert(BM * BK / 8 % kThreads == 0, "activation tile must divide over the threads");
+  extern __shared__ __attribute__((aligned(16))) unsigned char gemm_lds[];
+  _Float16 *x_lds = reinterpret_cast<_Float16 *>(gemm_lds);
+  _Float16 *w_lds = x_lds + BM * LDS_STRIDE;            // [NW][BN * LDS_STRIDE]
+  float *s_lds = reinterpret_cast<float *>(w_lds + NW * BN * LDS_STRIDE);  // [NW][BN]
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
-  const int wave_m = wave >> 1;  // 2 x 2 waves, 64 x 64 outputs each
+  const int wave_m = wave >> 1;
   const int wave_n = wave & 1;
 
   // XCD-aware tile order: workgroups are handed to the 8 XCDs round-robin, so
@@ -76,70 +84,72 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
   const uint32_t n0 = tile_n * BN;
   const uint32_t K = p.k;
 
-  // global -> register staging assignments
-  // x: 128 rows x 8 vectors of 8 halfs; thread covers rows (tid/8) + 32*i, vector tid%8
+  // global -> register staging: x rows (tid/8) + 64*i, vector tid%8;
+  // w row (tid/2) + 256*i, half tid%2
   const uint32_t x_vec = tid & 7;
   const uint32_t x_row = tid >> 3;
-  // w: 128 rows x 2 vectors of 32 nibbles; thread covers row tid/2, half tid%2
   const uint32_t w_row = tid >> 1;
   const uint32_t w_half = tid & 1;
 
-  uint4 x_reg[4];
-  u32x4_t w_reg[NW];
-  float s_reg[NW];
+  uint4 x_reg[X_VECTORS];
+  u32x4_t w_reg[NW][W_VECTORS];
+  uint16_t s_reg[NW][W_VECTORS];
 
-  auto load_global = [&](uint32_t k0) {
+  auto load_global = [&](uint32_t k0) __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const uint32_t row = m0 + x_row + 32 * i;
-      x_reg[i] = row < p.m
-                     ? reinterpret_cast<const uint4 *>(p.x + (size_t)row * K + k0)[x_vec]
-                     : make_uint4(0, 0, 0, 0);
+    for (int i = 0; i < X_VECTORS; ++i) {
+      const uint32_t row = min(m0 + x_row + 64 * i, p.m - 1);  // rows past m are never stored
+      x_reg[i] = reinterpret_cast<const uint4 *>(p.x + (size_t)row * K + k0)[x_vec];
     }
-    const uint32_t col = n0 + w_row;
 #pragma unroll
-    for (int v = 0; v < NW; ++v) {
-      if (col < p.n) {
-        w_reg[v] = reinterpret_cast<const u32x4_t *>(p.w[v] + (size_t)col * (K >> 1) + (k0 >> 1))[w_half];
-        s_reg[v] = half_bits_to_float(p.s[v][(size_t)col * (K >> 6) + (k0 >> 6)]);
-      } else {
-        w_reg[v] = u32x4_t{0, 0, 0, 0};
-        s_reg[v] = 0.0f;
+    for (int i = 0; i < W_VECTORS; ++i) {
+      const uint32_t local = w_row + 256 * i;
+      const uint32_t col = min(n0 + local, p.n - 1);  // columns past n are never stored
+#pragma unroll
+      for (int v = 0; v < NW; ++v) {
+        w_reg[v][i] = reinterpret_cast<const u32x4_t *>(p.w[v] + (size_t)col * (K >> 1) + (k0 >> 1))[w_half];
+        s_reg[v][i] = p.s[v][(size_t)col * (K >> 6) + (k0 >> 6)];
       }
     }
   };
 
-  auto store_lds = [&]() {
+  auto store_lds = [&]() __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-      *reinterpret_cast<uint4 *>(&x_lds[(x_row + 32 * i) * LDS_STRIDE + x_vec * 8]) =
-          pair_order(x_reg[i]);
+    for (int i = 0; i < X_VECTORS; ++i)
+      *reinterpret_cast<uint4 *>(&x_lds[(x_row + 64 * i) * LDS_STRIDE + x_vec * 8]) = pair_order(x_reg[i]);
 #pragma unroll
-    for (int v = 0; v < NW; ++v) {
+    for (int i = 0; i < W_VECTORS; ++i) {
+      const uint32_t local = w_row + 256 * i;
+      if (BN % 256 != 0 && local >= (uint32_t)BN) continue;
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const W4Pairs q = w4_decode_pairs(w_reg[v][j]);
-        uint4 packed;
-        packed.x = as_u32(q.p04);
-        packed.y = as_u32(q.p15);
-        packed.z = as_u32(q.p26);
-        packed.w = as_u32(q.p37);
-        *reinterpret_cast<uint4 *>(&w_lds[v][w_row * LDS_STRIDE + w_half * 32 + j * 8]) = packed;
+      for (int v = 0; v < NW; ++v) {
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const W4Pairs q = w4_decode_pairs(w_reg[v][i][j]);
+          uint4 packed;
+          packed.x = as_u32(q.p04);
+          packed.y = as_u32(q.p15);
+          packed.z = as_u32(q.p26);
+          packed.w = as_u32(q.p37);
+          *reinterpret_cast<uint4 *>(&w_lds[(v * BN + local) * LDS_STRIDE + w_half * 32 + j * 8]) = packed;
+        }
+        if (w_half == 0) s_lds[v * BN + local] = half_bits_to_float(s_reg[v][i]);
       }
-      if (w_half == 0) s_lds[v][w_row] = s_reg[v];
     }
   };
 
-  f16x_t acc[NW][2][2];
+  f16x_t acc[NW][WM][WN];
 #pragma unroll
   for (int v = 0; v < NW; ++v)
 #pragma unroll
-    for (int a = 0; a < 2; ++a)
+    for (int a = 0; a < WM; ++a)
 #pragma unroll
-      for (int b = 0; b < 2; ++b) acc[v][a][b] = zero_tile();
+      for (int b = 0; b < WN; ++b) acc[v][a][b] = zero_tile();
 
   const int frag_row = lane & 31;  // operand row (A) / column (B) inside a 32-wide tile
   const int frag_k = (lane >> 5) * 8;
+  const int row_base = wave_m * WM * 32;
+  const int col_base = wave_n * WN * 32;
 
   load_global(0);
   for (uint32_t k0 = 0; k0 < K; k0 += BK) {
@@ -148,49 +158,48 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
     __syncthreads();
     if (k0 + BK < K) load_global(k0 + BK);
 
-    f16x_t part[NW][2][2];
+    h8_t a_frag[WM][BK / 16];
 #pragma unroll
-    for (int ks = 0; ks < BK / 16; ++ks) {
-      h8_t a_frag[2];
+    for (int a = 0; a < WM; ++a)
 #pragma unroll
-      for (int a = 0; a < 2; ++a)
-        a_frag[a] = *reinterpret_cast<const h8_t *>(
-            &x_lds[(wave_m * 64 + a * 32 + frag_row) * LDS_STRIDE + ks * 16 + frag_k]);
+      for (int ks = 0; ks < BK / 16; ++ks)
+        a_frag[a][ks] = *reinterpret_cast<const h8_t *>(
+            &x_lds[(row_base + a * 32 + frag_row) * LDS_STRIDE + ks * 16 + frag_k]);
 #pragma unroll
-      for (int v = 0; v < NW; ++v) {
+    for (int v = 0; v < NW; ++v) {
 #pragma unroll
-        for (int b = 0; b < 2; ++b) {
-          const h8_t b_frag = *reinterpret_cast<const h8_t *>(
-              &w_lds[v][(wave_n * 64 + b * 32 + frag_row) * LDS_STRIDE + ks * 16 + frag_k]);
+      for (int b = 0; b < WN; ++b) {
+        h8_t b_frag[BK / 16];
 #pragma unroll
-          for (int a = 0; a < 2; ++a)
-            part[v][a][b] = __builtin_amdgcn_mfma_f32_32x32x16_f16(
-                a_frag[a], b_frag, ks == 0 ? zero_tile() : part[v][a][b], 0, 0, 0);
+        for (int ks = 0; ks < BK / 16; ++ks)
+          b_frag[ks] = *reinterpret_cast<const h8_t *>(
+              &w_lds[(v * BN + col_base + b * 32 + frag_row) * LDS_STRIDE + ks * 16 + frag_k]);
+        const float scale = s_lds[v * BN + col_base + b * 32 + frag_row];
+#pragma unroll
+        for (int a = 0; a < WM; ++a) {
+          // one 64-wide scale group: four chained MFMAs into a temporary tile,
+          // then acc += temporary * float(scale) in fp32
+          f16x_t part = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_frag[a][0], b_frag[0], zero_tile(), 0, 0, 0);
+#pragma unroll
+          for (int ks = 1; ks < BK / 16; ++ks)
+            part = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_frag[a][ks], b_frag[ks], part, 0, 0, 0);
+#pragma unroll
+          for (int i = 0; i < 16; ++i) acc[v][a][b][i] = fmaf(part[i], scale, acc[v][a][b][i]);
         }
       }
     }
-#pragma unroll
-    for (int v = 0; v < NW; ++v)
-#pragma unroll
-      for (int b = 0; b < 2; ++b) {
-        const float scale = s_lds[v][wave_n * 64 + b * 32 + frag_row];
-#pragma unroll
-        for (int a = 0; a < 2; ++a)
-#pragma unroll
-          for (int i = 0; i < 16; ++i) acc[v][a][b][i] = fmaf(part[v][a][b][i], scale, acc[v][a][b][i]);
-      }
   }
 
   // epilogue: lane owns column col, rows (i/4)*8 + (lane/32)*4 + i%4 of each tile
 #pragma unroll
-  for (int b = 0; b < 2; ++b) {
-    const uint32_t col = n0 + wave_n * 64 + b * 32 + frag_row;
+  for (int b = 0; b < WN; ++b) {
+    const uint32_t col = n0 + col_base + b * 32 + frag_row;
     if (col >= p.n) continue;
 #pragma unroll
-    for (int a = 0; a < 2; ++a) {
+    for (int a = 0; a < WM; ++a) {
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
-        const uint32_t row = m0 + wave_m * 64 + a * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3);
+        const uint32_t row = m0 + row_base + a * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3);
         if (row >= p.m) continue;
         float value;
         if (DUAL) {
@@ -208,13 +217,37 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
   }
 }
 
-template <bool DUAL>
-hipError_t launch_gemm(GemmParams &p, hipStream_t stream) {
+template <int WM, int WN, bool DUAL>
+hipError_t launch_tile(GemmParams &p, hipStream_t stream) {
+  constexpr int NW = DUAL ? 2 : 1;
+  constexpr int BM = 4 * WM * 32;
+  constexpr int BN = 2 * WN * 32;
+  constexpr size_t lds_bytes =
+      (size_t)(BM + NW * BN) * LDS_STRIDE * sizeof(_Float16) + (size_t)NW * BN * sizeof(float);
+  static bool configured = false;
+  if (!configured) {
+    hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(&w4a16_gemm_kernel<WM, WN, DUAL>),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+    if (status != hipSuccess) return status;
+    configured = true;
+  }
   p.tiles_m = (p.m + BM - 1) / BM;
   p.tiles_n = (p.n + BN - 1) / BN;
   const uint32_t blocks = p.tiles_m * p.tiles_n;
-  hipLaunchKernelGGL((w4a16_gemm_kernel<DUAL>), dim3(blocks), dim3(kThreads), 0, stream, p);
+  hipLaunchKernelGGL((w4a16_gemm_kernel<WM, WN, DUAL>), dim3(blocks), dim3(kThreads), lds_bytes, stream, p);
   return hipGetLastError();
+}
+
+template <bool DUAL>
+hipError_t launch_gemm(GemmParams &p, hipStream_t stream) {
+  if (DUAL) return launch_tile<2, 2, true>(p, stream);  // 256 x 128, two accumulator sets
+  // 256 x 256 when that still gives every CU a tile, otherwise 128 x 256 / 128 x 128
+  const int cus = device_compute_units();
+  const uint64_t big = (uint64_t)((p.m + 255) / 256) * ((p.n + 255) / 256);
+  if (big >= (uint64_t)cus) return launch_tile<2, 4, false>(p, stream);
+  const uint64_t mid = (uint64_t)((p.m + 127) / 128) * ((p.n + 255) / 256);
+  if (mid >= (uint64_t)cus) return launch_tile<1, 4, false>(p, stream);
+  return launch_tile<1, 2, false>(p, stream);
 }
 
 }  // namespace
