@@ -296,7 +296,6 @@ hipError_t launch_variant(const GemvParams &p, uint32_t matrices, uint32_t max_n
   const int cus = device_compute_units();
   int per_cu = 2;  // 8 waves per CU, each with two work items of weights in flight
   if (use_lds && lds_bytes > 80 * 1024) per_cu = 1;
-  if (const char *tune = getenv("LLMOPT_TUNE_GEMV_BLOCKS")) per_cu = atoi(tune);
   const uint32_t wanted = (tiles + kWaves - 1) / kWaves;
   const uint32_t blocks = std::max<uint32_t>(1, std::min<uint32_t>(wanted, (uint32_t)(cus * per_cu)));
   if (use_lds) {
