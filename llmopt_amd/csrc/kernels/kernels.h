@@ -26,7 +26,17 @@ struct W4LinearArgs {
   uint32_t addend_row_stride;
   uint16_t *y;  // f16 [m, n]
   uint32_t m, n, k;
+  // Optional scratch for the decode path when m x k exceeds the LDS budget and the
+  // K range is split over workgroups: fp32 partial sums and one arrival counter per
+  // 16-row tile (zero before the first launch; the kernel leaves them zero).
+  void *workspace;
+  size_t workspace_bytes;
+  uint32_t *counters;
+  uint32_t counter_count;
 };
+
+// Bytes of workspace the decode path wants for this shape (0 when it does not split K).
+size_t w4a16_gemv_workspace_bytes(uint32_t m, uint32_t n, uint32_t k);
 
 // Three projections of one activation in one launch
 // (llmopt_w4a16_qkv_linear_f16_g64*, lib/metal_w4a16_source.ml:218-480).
@@ -119,6 +129,6 @@ hipError_t launch_q8_attention(const Q8AttentionArgs &args, hipStream_t stream);
 // The largest m the streaming GEMV path takes; above it the MFMA GEMM runs.
 constexpr uint32_t kGemvMaxRows = 8;
 // Up to this m the GEMV uses v_dot2 on the vector ALUs, above it the matrix cores.
-constexpr uint32_t kGemvDotRows = 4;
+constexpr uint32_t kGemvDotRows = 2;
 
 }  // namespace llmopt

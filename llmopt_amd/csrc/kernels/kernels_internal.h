@@ -13,7 +13,7 @@ hipError_t launch_w4a16_gemv_linear(const W4LinearArgs &args, hipStream_t stream
 hipError_t launch_w4a16_gemv_qkv(const W4QkvArgs &args, hipStream_t stream);
 hipError_t launch_w4a16_gemv_dual_swiglu(const W4DualSwigluArgs &args, hipStream_t stream);
 
-// 3 <= m <= 8: matrix-core GEMV
+// kGemvDotRows < m <= kGemvMaxRows: matrix-core GEMV
 hipError_t launch_w4a16_gemv_mfma_linear(const W4LinearArgs &args, hipStream_t stream);
 hipError_t launch_w4a16_gemv_mfma_qkv(const W4QkvArgs &args, hipStream_t stream);
 hipError_t launch_w4a16_gemv_mfma_dual_swiglu(const W4DualSwigluArgs &args, hipStream_t stream);

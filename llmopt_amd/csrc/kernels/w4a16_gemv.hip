@@ -86,14 +86,16 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemv_kernel(GemvParams p) {
     }
   };
 
-  auto load_item = [&](uint32_t tile, uint32_t item, Item &out) {
+  // `real` = false is the prefetch past the last item: still issued (see the
+  // main loop) but every lane reads segment 0 of the rows, one line per row.
+  auto load_item = [&](uint32_t tile, uint32_t item, bool real, Item &out) {
     const u32x4_t *wrow[R];
     const uint16_t *srow[R];
     tile_rows(tile, wrow, srow);
 #pragma unroll
     for (int u = 0; u < U; ++u) {
       const uint32_t seg = (item * U + u) * 64 + lane;
-      const uint32_t safe = seg < segs ? seg : 0;
+      const uint32_t safe = (real && seg < segs) ? seg : 0;
 #pragma unroll
       for (int r = 0; r < R; ++r) {
         out.w[r][u] = __builtin_nontemporal_load(wrow[r] + safe);
@@ -105,7 +107,7 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemv_kernel(GemvParams p) {
   // first weights are in flight while the activation is staged
   Item item_a, item_b;
   const bool has_work = first_tile < tiles;
-  if (has_work) load_item(first_tile, 0, item_a);
+  if (has_work) load_item(first_tile, 0, true, item_a);
 
   // Bias correction of w4_decode_biased per (m, chunk, lane), after the vectors.
   float *corr_lds = reinterpret_cast<float *>(x_lds + (size_t)M * chunks * 256);
@@ -242,7 +244,7 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemv_kernel(GemvParams p) {
 
   // Ping-pong between two register sets: the next item's loads are issued
   // before the current item is decoded.  The prefetch is unconditional (past
-  // the end it re-reads the current item) so that no branch skips the loads:
+  // the end it reads one line per row) so that no branch skips the loads:
   // with a skipped path the compiler must assume the shorter load queue and
   // waits for the fresh loads before decoding the old ones.
   uint32_t tile = first_tile, item = 0;
@@ -250,14 +252,14 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemv_kernel(GemvParams p) {
     uint32_t next_tile = tile, next_item = item;
     advance(next_tile, next_item);
     bool more = next_tile < tiles;
-    load_item(more ? next_tile : tile, more ? next_item : item, item_b);
+    load_item(more ? next_tile : tile, next_item, more, item_b);
     consume(tile, item, item_a);
     if (!more) break;
     tile = next_tile;
     item = next_item;
     advance(next_tile, next_item);
     more = next_tile < tiles;
-    load_item(more ? next_tile : tile, more ? next_item : item, item_a);
+    load_item(more ? next_tile : tile, next_item, more, item_a);
     consume(tile, item, item_b);
     if (!more) break;
     tile = next_tile;

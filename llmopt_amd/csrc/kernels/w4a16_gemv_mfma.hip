@@ -1,25 +1,34 @@
-// W4A16 decode GEMV for 5 <= M <= 8 activation rows on gfx950, using the matrix
-// cores for the contraction.
+// W4A16 decode GEMV for 1 <= M <= 8 activation rows on gfx950 with the
+// contraction on the matrix cores.
 //
-// With more than four activation rows the v_dot2 path of w4a16_gemv.hip becomes VALU
-// bound (4 dot instructions per row per weight dword).  Here one
-// v_mfma_f32_32x32x16_f16 contracts four independent 8(m) x 8(n) x 16(k)
-// blocks at once: matrix columns 8q..8q+7 are 8 weight rows in scale group
-// g0 + q (q = 0..3) and the activation occupies A rows 8q..8q+7 with the K
-// values of that same group; the off-diagonal blocks are not used.  Every lane
-// therefore loads one 16-byte weight segment that lies inside a single 64-wide
-// scale group (so the fp16 group scale is one scalar per lane, applied in fp32
-// to the accumulator), and each wave-wide load covers 8 rows x 128 contiguous
-// bytes; a wave takes two adjacent steps, i.e. 256 contiguous bytes per row.
+// One v_mfma_f32_16x16x32_f16 multiplies a 16(m) x 32(k) activation block with
+// a 32(k) x 16(n) weight block.  Lane (c = lane % 16, h = lane / 16) supplies
+// the B operand of weight row c: the 8 K values of dword j of the 16 bytes it
+// loaded at byte offset 16 h of a 128-wide K block.  Lanes h = 0,1 therefore
+// hold the first 64-wide scale group of the block and lanes h = 2,3 the second.
+// The activation is laid out block-diagonally: A rows 0..7 are x rows 0..7 for
+// K quarters 0,1 and zero for quarters 2,3, A rows 8..15 the other way round.
+// D rows 0..7 then hold the partial sums of the first scale group and rows
+// 8..15 those of the second, and the D registers of a lane (rows 4 h .. 4 h + 3,
+// column c) belong to exactly the scale group of the weights that lane loaded:
+// the fp16 group scale is one scalar per lane, applied in fp32 to the 4
+// accumulators.
 //
-// A workgroup of 4 waves owns one 8-row tile; the waves split the K steps
-// (256 K values each) and are reduced through LDS at the end.  The activation
-// is staged through LDS in chunks of 2048 K values in the operand order of the
-// nibble decode.
+// The nibbles are decoded to fp16 with a bias (q + 1032 or q + 72, one bit
+// operation per pair of nibbles).  The bias is removed by starting the MFMA
+// accumulation of a scale group from -(1032 sum x_even_pairs + 72 sum
+// x_odd_pairs), computed once per workgroup while the activation is staged to
+// LDS in the operand order of the decode.
 //
-// Same arithmetic contract as llmopt_w4a16_linear_f16_g64_m4 / _m8,
-// llmopt_w4a16_qkv_linear_f16_g64_m4, llmopt_w4a16_dual_swiglu_f16_g64_m4 and
-// llmopt_w4a16_down_add_f16_g64_m4 (lib/metal_w4a16_source.ml:42-966).
+// A workgroup of 8 waves streams tiles of 16 weight rows; its waves split the
+// K range of the tile in steps of 256 and are reduced through LDS.  When M x K
+// does not fit the LDS budget the K range is split over blockIdx.y as well:
+// the slices leave fp32 partial sums in a workspace and the last workgroup to
+// arrive at a tile (an atomic counter per tile) adds them in slice order.
+//
+// Same arithmetic contract as llmopt_w4a16_linear_f16_g64{,_m4,_m8},
+// llmopt_w4a16_qkv_linear_f16_g64*, llmopt_w4a16_dual_swiglu_f16_g64* and
+// llmopt_w4a16_down_add_f16_g64* (lib/metal_w4a16_source.ml:8-966).
 #include <algorithm>
 
 #include "kernels.h"
@@ -29,14 +38,13 @@
 namespace llmopt {
 namespace {
 
-constexpr int kWaves = 4;
+constexpr int kWaves = 8;
 constexpr int kThreads = kWaves * 64;
-constexpr int MP = 8;                 // activation rows held (padded)
-constexpr int TN = 8;                 // weight rows per workgroup tile
-constexpr int KC = 2048;              // K values staged per chunk
-constexpr int kStepsPerChunk = KC / 256;
-constexpr int kStepsPerWave = kStepsPerChunk / kWaves;  // 2: one per ping-pong buffer
-static_assert(kStepsPerWave == 2, "the ping-pong below assumes two steps per wave and chunk");
+constexpr int TN = 16;        // weight rows per tile
+constexpr int kStepK = 256;   // K values one wave consumes per step
+constexpr int kZeroVectors = 20;  // per activation row: covers every operand offset of a step
+template <bool DUAL>
+constexpr int kReduceSlots = DUAL ? 1 : 2;  // DUAL keeps two sets of partial sums per tile
 
 struct MfmaMatrix {
   const uint8_t *w;
@@ -48,146 +56,236 @@ struct MfmaMatrix {
 struct MfmaGemvParams {
   const uint16_t *x;
   uint32_t m, k;
-  MfmaMatrix mat0, mat1, mat2;  // blockIdx.y selects (DUAL: mat0 = gate, mat1 = up)
+  MfmaMatrix mat0, mat1, mat2;  // blockIdx.z selects (DUAL: mat0 = gate, mat1 = up)
   const uint16_t *addend;
   uint32_t has_addend;
   uint32_t addend_stride;
+  uint32_t k_slice;    // K values per blockIdx.y slice, a multiple of 256
+  float *partials;     // [gridDim.y][8][n] fp32, used when gridDim.y > 1
+  uint32_t *counters;  // one per tile, zero between launches
 };
 
-template <bool DUAL>
+// MP = activation rows held in LDS (1, 2, 4 or 8, >= m)
+template <int MP, bool DUAL>
 __global__ __launch_bounds__(kThreads) void w4a16_gemv_mfma_kernel(MfmaGemvParams p) {
   constexpr int NW = DUAL ? 2 : 1;
+  constexpr int SPI = DUAL ? 1 : 2;      // steps per work item: 64 bytes per lane in flight per item
+  constexpr int RS = kReduceSlots<DUAL>;  // tiles finished between two workgroup reductions
   extern __shared__ uint4 lds[];
-  uint4 *x_lds = lds;                                                    // KC * MP / 8 vectors
-  float *red_lds = reinterpret_cast<float *>(lds + (size_t)KC * MP / 8);  // [NW][waves][MP][TN]
 
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const uint32_t c = lane & 31;   // matrix column: weight row r of group quarter q
-  const uint32_t kq = lane >> 5;  // which 8-wide K block of an MFMA this lane holds
-  const uint32_t q = c >> 3;      // scale group within the step
-  const uint32_t r = c & 7;       // weight row within the tile / activation row
-  const MfmaMatrix mat = DUAL ? p.mat0 : (blockIdx.y == 0 ? p.mat0 : blockIdx.y == 1 ? p.mat1 : p.mat2);
+  const uint32_t c = lane & 15;  // weight row of the tile (B column, D column)
+  const uint32_t h = lane >> 4;  // K quarter of the B operand; D rows 4h..4h+3
+  const MfmaMatrix mat = DUAL ? p.mat0 : (blockIdx.z == 0 ? p.mat0 : blockIdx.z == 1 ? p.mat1 : p.mat2);
+  const uint32_t tiles = (mat.n + TN - 1) / TN;
+  if (blockIdx.x >= tiles) return;  // a shorter matrix of a QKV launch (whole workgroup)
+
   const uint32_t K = p.k;
-  const uint32_t groups = K >> 6;
-  const uint32_t steps = (groups + 3) >> 2;
-  const uint32_t chunks = (K + KC - 1) / KC;
-  const uint32_t n0 = blockIdx.x * TN;
-  if (n0 >= mat.n) return;  // a shorter matrix of a QKV launch (whole workgroup)
-  const uint32_t row = min(n0 + r, mat.n - 1);
+  const uint32_t groups_total = K >> 6;
+  const uint32_t k_begin = blockIdx.y * p.k_slice;
+  const uint32_t k_len = min(p.k_slice, K - k_begin);
+  const uint32_t groups = k_len >> 6;  // scale groups of this slice
+  const uint32_t steps = (k_len + kStepK - 1) / kStepK;
+  const uint32_t items_per_tile = (steps + kWaves * SPI - 1) / (kWaves * SPI);  // per wave
 
-  const uint8_t *wrow[NW];
-  const uint16_t *srow[NW];
-  wrow[0] = mat.w + (size_t)row * (K >> 1);
-  srow[0] = mat.s + (size_t)row * groups;
-  if (DUAL) {
-    wrow[NW - 1] = p.mat1.w + (size_t)row * (K >> 1);
-    srow[NW - 1] = p.mat1.s + (size_t)row * groups;
-  }
+  // LDS: zero vectors | x in operand order | -bias correction | wave partial sums | flags
+  const uint32_t x_vectors = steps * 32 * MP;
+  uint4 *x_lds = lds + kZeroVectors * MP;
+  float *corr_lds = reinterpret_cast<float *>(x_lds + x_vectors);  // [steps*4][8]
+  float *red_lds = corr_lds + steps * 4 * 8;                       // [RS][NW][waves][8][16]
+  uint32_t *flag_lds = reinterpret_cast<uint32_t *>(red_lds + RS * NW * kWaves * 8 * TN);  // [RS]
 
-  struct Item {  // raw loaded registers only (see w4a16_gemv.hip)
-    u32x4_t w[NW];
-    uint16_t s[NW];
+  struct Item {  // raw loaded registers only: conversions at the load would serialise the prefetch
+    u32x4_t w[NW][SPI][2];
+    uint16_t s[NW][SPI][2];
   };
-  auto load_step = [&](uint32_t step, Item &out) __attribute__((always_inline)) {
-    const uint32_t g = min(step * 4 + q, groups - 1);
+  // item `index` of a tile covers steps (wave + index*kWaves)*SPI .. +SPI-1
+  // `real` = false is the prefetch past the last item: it stays unconditional
+  // (a skipped load would make the compiler wait for the whole load queue) but
+  // every lane reads the first 16 bytes of the matrix, one cache line per wave.
+  auto load_item = [&](uint32_t tile, uint32_t index, bool real, Item &out) __attribute__((always_inline)) {
+    const uint32_t row = min(tile * TN + c, mat.n - 1);
+    const uint32_t step0 = (wave + index * kWaves) * SPI;
 #pragma unroll
-    for (int v = 0; v < NW; ++v) {
-      out.w[v] = __builtin_nontemporal_load(
-          reinterpret_cast<const u32x4_t *>(wrow[v] + (size_t)g * 32 + kq * 16));
-      out.s[v] = srow[v][g];
-    }
-  };
-
-  // The useful block of a lane's tile is registers 4q..4q+3 (rows 8q + kq*4 + i);
-  // all 16 are accumulated and the block is picked at the end.
-  f16x_t acc[NW];
+    for (int u = 0; u < SPI; ++u) {
 #pragma unroll
-  for (int v = 0; v < NW; ++v)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) acc[v][i] = 0.0f;
-
-  auto consume = [&](uint32_t step, uint32_t chunk, const Item &cur) __attribute__((always_inline)) {
-    const uint32_t g = step * 4 + q;
-    const bool ok = g < groups;
-    const uint32_t g_local = min(g, groups - 1) - chunk * (KC / 64);
-    h8_t a_frag[4];
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-      a_frag[j] = __builtin_bit_cast(h8_t, x_lds[((g_local * 4 + j) * 2 + kq) * MP + r]);
-#pragma unroll
-    for (int v = 0; v < NW; ++v) {
-      f16x_t tile;
-#pragma unroll
-      for (int i = 0; i < 16; ++i) tile[i] = 0.0f;
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const W4Pairs w = w4_decode_pairs(cur.w[v][j]);
-        uint4 packed;
-        packed.x = as_u32(w.p04);
-        packed.y = as_u32(w.p15);
-        packed.z = as_u32(w.p26);
-        packed.w = as_u32(w.p37);
-        tile = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_frag[j], __builtin_bit_cast(h8_t, packed), tile, 0, 0, 0);
+      for (int t = 0; t < 2; ++t) {
+        // clamped past the end of the slice (the scale is zeroed when consumed)
+        const uint32_t g = min((step0 + u) * 4 + 2 * t + (h >> 1), groups - 1);
+        const size_t w_off = real ? (size_t)row * (K >> 1) + (k_begin >> 1) + g * 32 + (h & 1) * 16 : 0;
+        const size_t s_off = real ? (size_t)row * groups_total + (k_begin >> 6) + g : 0;
+        out.w[0][u][t] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(mat.w + w_off));
+        out.s[0][u][t] = mat.s[s_off];
+        if (DUAL) {
+          out.w[NW - 1][u][t] =
+              __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(p.mat1.w + w_off));
+          out.s[NW - 1][u][t] = p.mat1.s[s_off];
+        }
       }
-      const float scale = ok ? half_bits_to_float(cur.s[v]) : 0.0f;
-#pragma unroll
-      for (int i = 0; i < 16; ++i) acc[v][i] = fmaf(tile[i], scale, acc[v][i]);
     }
   };
 
-  // this wave's steps in chunk ch are ch*8 + 2*wave and the next one
+  // first loads go out before the activation is staged
   Item item_a, item_b;
-  load_step(min(2 * wave, steps - 1), item_a);
-  for (uint32_t chunk = 0; chunk < chunks; ++chunk) {
-    // stage x[:, chunk*KC .. +KC) in operand order: vector index
-    // ((g_local*4 + j)*2 + kq)*MP + m holds K block g*64 + kq*32 + j*8 of row m
-    for (uint32_t i = threadIdx.x; i < (uint32_t)MP * (KC / 8); i += kThreads) {
-      const uint32_t m = i / (KC / 8);
-      const uint32_t kk = i - m * (KC / 8);
-      const uint32_t k0 = chunk * KC + kk * 8;
-      uint4 value = make_uint4(0, 0, 0, 0);
-      if (m < p.m && k0 < K)
-        value = pair_order(*reinterpret_cast<const uint4 *>(p.x + (size_t)m * K + k0));
-      x_lds[(((kk >> 3) * 4 + (kk & 3)) * 2 + ((kk >> 2) & 1)) * MP + m] = value;
-    }
-    __syncthreads();
-    const uint32_t step_a = chunk * kStepsPerChunk + 2 * wave;
-    const uint32_t step_b = step_a + 1;
-    const uint32_t step_c = step_a + kStepsPerChunk;  // first step of the next chunk
-    load_step(min(step_b, steps - 1), item_b);
-    if (step_a < steps) consume(step_a, chunk, item_a);
-    load_step(min(step_c, steps - 1), item_a);
-    if (step_b < steps) consume(step_b, chunk, item_b);
-    __syncthreads();  // every wave is done with this chunk of x
-  }
+  load_item(blockIdx.x, 0, true, item_a);
 
-  // pick the lane's block, add the four group quarters of each weight row
-  // (8, 16 and 24 lanes apart), then reduce the waves through LDS
+  // ---- stage x[:, k_begin .. k_begin + steps*256) and the bias correction ----
+  for (uint32_t i = threadIdx.x; i < kZeroVectors * MP; i += kThreads) lds[i] = make_uint4(0, 0, 0, 0);
+  {
+    constexpr int UNROLL = 4;  // independent loads in flight per thread
+    const uint32_t padded = (x_vectors + 63) & ~63u;
+    for (uint32_t base = threadIdx.x; base < padded; base += kThreads * UNROLL) {
+      uint4 value[UNROLL];
 #pragma unroll
-  for (int v = 0; v < NW; ++v) {
+      for (int u = 0; u < UNROLL; ++u) {
+        const uint32_t i = base + u * kThreads;
+        const uint32_t m = i & (MP - 1);
+        const uint32_t kb = i / MP;  // block of 8 K values within the slice
+        value[u] = make_uint4(0, 0, 0, 0);
+        if (m < p.m && kb * 8 < k_len)
+          value[u] = *reinterpret_cast<const uint4 *>(p.x + (size_t)m * K + k_begin + kb * 8);
+      }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      float mine = q == 0 ? acc[v][i] : q == 1 ? acc[v][4 + i] : q == 2 ? acc[v][8 + i] : acc[v][12 + i];
-      mine += __builtin_bit_cast(
-          float, __builtin_amdgcn_ds_bpermute((int)((lane ^ 8) << 2), __builtin_bit_cast(int, mine)));
-      mine += __builtin_bit_cast(
-          float, __builtin_amdgcn_ds_bpermute((int)((lane ^ 16) << 2), __builtin_bit_cast(int, mine)));
-      if (q == 0) red_lds[((v * kWaves + wave) * MP + kq * 4 + i) * TN + r] = mine;
+      for (int u = 0; u < UNROLL; ++u) {
+        const uint32_t i = base + u * kThreads;
+        if (i >= padded) break;  // uniform per wave: padded is a multiple of 64
+        const uint32_t m = i & (MP - 1);
+        const uint32_t kb = i / MP;
+        const uint4 ordered = pair_order(value[u]);
+        if (i < x_vectors) x_lds[i] = ordered;
+        // pairs .x and .z meet weights decoded as q + 1032, pairs .y and .w as q + 72
+        const h2_t a = as_h2(ordered.x), b = as_h2(ordered.y), cc = as_h2(ordered.z), d = as_h2(ordered.w);
+        float bias = 1032.0f * (((float)a[0] + (float)a[1]) + ((float)cc[0] + (float)cc[1])) +
+                     72.0f * (((float)b[0] + (float)b[1]) + ((float)d[0] + (float)d[1]));
+        // the 8 blocks of a scale group sit MP lanes apart
+        bias += __shfl_xor(bias, MP);
+        bias += __shfl_xor(bias, 2 * MP);
+        bias += __shfl_xor(bias, 4 * MP);
+        if ((kb & 7) == 0 && i < x_vectors) corr_lds[(kb >> 3) * 8 + m] = -bias;
+      }
+    }
+    if (MP < 8) {
+      // rows MP..7 of the correction are read (their D rows are never used): keep them finite
+      for (uint32_t i = threadIdx.x; i < steps * 4 * 8; i += kThreads)
+        if ((i & 7) >= MP) corr_lds[i] = 0.0f;
     }
   }
   __syncthreads();
-  if (threadIdx.x < MP * TN) {
-    const uint32_t m = threadIdx.x / TN, col_in_tile = threadIdx.x % TN;
-    const uint32_t col = n0 + col_in_tile;
-    if (m < p.m && col < mat.n) {
-      float total[NW];
+
+  // operand addressing: lanes off the block diagonal read the zero vectors
+  const bool on_diagonal = (c >= 8) == (h >= 2);
+  const uint32_t m_of_lane = (c & 7) & (MP - 1);
+  const uint32_t a_base = on_diagonal ? (kZeroVectors + h * 4) * MP + m_of_lane : 0;  // in vectors
+  const uint32_t a_step = on_diagonal ? 32 * MP : 0;
+  const uint32_t corr_base = (h >> 1) * 8 + (h & 1) * 4;
+
+  f4_t acc[NW];
+#pragma unroll
+  for (int v = 0; v < NW; ++v) acc[v] = f4_t{0.0f, 0.0f, 0.0f, 0.0f};
+
+  auto consume = [&](uint32_t index, const Item &cur) __attribute__((always_inline)) {
+    const uint32_t step0 = (wave + index * kWaves) * SPI;
+#pragma unroll
+    for (int u = 0; u < SPI; ++u) {
+      const uint32_t step = step0 + u;
+      const uint32_t step_l = min(step, steps - 1);
+      const uint4 *a_ptr = lds + a_base + a_step * step_l;
+      const float *corr_ptr = corr_lds + corr_base + step_l * 32;
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        const bool ok = step * 4 + 2 * t + (h >> 1) < groups;
+        const f4_t start = *reinterpret_cast<const f4_t *>(corr_ptr + t * 16);
+        h8_t a_frag[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) a_frag[j] = __builtin_bit_cast(h8_t, a_ptr[(t * 16 + j) * MP]);
+#pragma unroll
+        for (int v = 0; v < NW; ++v) {
+          f4_t tile = start;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const W4Pairs w = w4_decode_biased(cur.w[v][u][t][j]);
+            uint4 packed;
+            packed.x = as_u32(w.p04);
+            packed.y = as_u32(w.p15);
+            packed.z = as_u32(w.p26);
+            packed.w = as_u32(w.p37);
+            tile = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_frag[j], __builtin_bit_cast(h8_t, packed), tile, 0,
+                                                          0, 0);
+          }
+          const float scale = ok ? half_bits_to_float(cur.s[v][u][t]) : 0.0f;
+#pragma unroll
+          for (int i = 0; i < 4; ++i) acc[v][i] = fmaf(tile[i], scale, acc[v][i]);
+        }
+      }
+    }
+  };
+
+  // A finished tile leaves the wave's partial sums in a reduction slot; the
+  // workgroup reduces RS tiles at a time.
+  uint32_t pending = 0;        // tiles waiting in the slots (uniform)
+  uint32_t pending_first = 0;  // tile index of slot 0; slot s holds pending_first + s*gridDim.x
+  auto park_tile = [&](uint32_t tile) __attribute__((always_inline)) {
+    if (pending == 0) pending_first = tile;
+    float *slot = red_lds + pending * (NW * kWaves * 8 * TN);
+    // the two scale-group halves of a column sit 32 lanes apart
+#pragma unroll
+    for (int v = 0; v < NW; ++v) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float total = acc[v][i] + __shfl_xor(acc[v][i], 32);
+        if (h < 2) slot[((v * kWaves + wave) * 8 + h * 4 + i) * TN + c] = total;
+        acc[v][i] = 0.0f;
+      }
+    }
+    ++pending;
+  };
+  auto flush = [&]() __attribute__((always_inline)) {
+    __syncthreads();
+    const uint32_t slot_index = threadIdx.x >> 7;  // 128 outputs per tile
+    const uint32_t in_slot = threadIdx.x & 127;
+    const uint32_t m = in_slot >> 4, col_in_tile = in_slot & 15;
+    const uint32_t tile = pending_first + slot_index * gridDim.x;
+    const uint32_t col = tile * TN + col_in_tile;
+    const bool active = slot_index < pending;
+    const bool writer = active && m < p.m && col < mat.n;
+    float total[NW];
+    if (active) {
+      const float *slot = red_lds + slot_index * (NW * kWaves * 8 * TN);
 #pragma unroll
       for (int v = 0; v < NW; ++v) {
         total[v] = 0.0f;
 #pragma unroll
-        for (int w = 0; w < kWaves; ++w) total[v] += red_lds[((v * kWaves + w) * MP + m) * TN + col_in_tile];
+        for (int w = 0; w < kWaves; ++w) total[v] += slot[((v * kWaves + w) * 8 + m) * TN + col_in_tile];
       }
+    }
+    bool store = writer;
+    if (!DUAL && gridDim.y > 1) {
+      // K split over workgroups: leave the partial sum where every CU sees it
+      // (device-scope stores and loads, no cache write-back needed); the last
+      // workgroup to arrive at a tile adds the slices in order.
+      if (writer)
+        __hip_atomic_store(p.partials + ((size_t)blockIdx.y * 8 + m) * mat.n + col, total[0], __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+      __syncthreads();  // waits for the stores of every wave
+      if (active && in_slot == 0) {
+        const uint32_t arrived =
+            __hip_atomic_fetch_add(p.counters + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const bool last = arrived == gridDim.y - 1;
+        if (last) __hip_atomic_store(p.counters + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        flag_lds[slot_index] = last ? 1u : 0u;
+      }
+      __syncthreads();
+      store = writer && flag_lds[slot_index] != 0;
+      if (store) {
+        float sum = 0.0f;
+        for (uint32_t slice = 0; slice < gridDim.y; ++slice)
+          sum += __hip_atomic_load(p.partials + ((size_t)slice * 8 + m) * mat.n + col, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+        total[0] = sum;
+      }
+    }
+    if (store) {
       float value;
       if (DUAL) {
         value = total[0] / (1.0f + __expf(-total[0])) * total[NW - 1];
@@ -197,19 +295,112 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemv_mfma_kernel(MfmaGemvParam
       }
       mat.y[(size_t)m * mat.n + col] = float_to_half_bits(value);
     }
+    __syncthreads();  // the slots are free again
+    pending = 0;
+  };
+
+  // Items of this wave: for each tile of the workgroup, items 0 .. items_per_tile-1.
+  // Ping-pong between two register sets with an unconditional prefetch.
+  auto advance = [&](uint32_t &tile, uint32_t &index) {
+    if (++index == items_per_tile) {
+      index = 0;
+      tile += gridDim.x;
+    }
+  };
+  uint32_t tile = blockIdx.x, index = 0;
+  while (true) {
+    uint32_t next_tile = tile, next_index = index;
+    advance(next_tile, next_index);
+    bool more = next_tile < tiles;
+    load_item(next_tile, next_index, more, item_b);
+    consume(index, item_a);
+    if (index == items_per_tile - 1) {
+      park_tile(tile);
+      if (pending == RS || !more) flush();
+    }
+    if (!more) break;
+    tile = next_tile;
+    index = next_index;
+    advance(next_tile, next_index);
+    more = next_tile < tiles;
+    load_item(next_tile, next_index, more, item_a);
+    consume(index, item_b);
+    if (index == items_per_tile - 1) {
+      park_tile(tile);
+      if (pending == RS || !more) flush();
+    }
+    if (!more) break;
+    tile = next_tile;
+    index = next_index;
   }
 }
 
-template <bool DUAL>
-hipError_t launch(const MfmaGemvParams &p, uint32_t matrices, uint32_t max_n, hipStream_t stream) {
-  constexpr int NW = DUAL ? 2 : 1;
-  const size_t lds_bytes = (size_t)KC * MP * 2 + (size_t)NW * kWaves * MP * TN * sizeof(float);
-  const dim3 grid((max_n + TN - 1) / TN, matrices);
-  hipLaunchKernelGGL((w4a16_gemv_mfma_kernel<DUAL>), grid, dim3(kThreads), lds_bytes, stream, p);
+constexpr size_t kLdsBudget = 79 * 1024;  // two workgroups per CU (160 KB)
+
+size_t lds_bytes_for(uint32_t mp, uint32_t steps, int nw) {
+  const int slots = nw == 2 ? kReduceSlots<true> : kReduceSlots<false>;
+  return (size_t)(kZeroVectors * mp + steps * 32 * mp) * 16 + (size_t)steps * 4 * 8 * 4 +
+         (size_t)slots * nw * kWaves * 8 * TN * 4 + 16;
+}
+
+struct Plan {
+  uint32_t mp, slices, k_slice;
+  size_t lds_bytes;
+};
+
+Plan make_plan(uint32_t m, uint32_t k, int nw, bool may_split) {
+  Plan plan;
+  plan.mp = m <= 1 ? 1 : m <= 2 ? 2 : m <= 4 ? 4 : 8;
+  const uint32_t steps_total = (k + kStepK - 1) / kStepK;
+  plan.slices = 1;
+  if (may_split) {
+    while (plan.slices < steps_total &&
+           lds_bytes_for(plan.mp, (steps_total + plan.slices - 1) / plan.slices, nw) > kLdsBudget)
+      ++plan.slices;
+  }
+  const uint32_t steps = (steps_total + plan.slices - 1) / plan.slices;
+  plan.k_slice = steps * kStepK;
+  plan.slices = (k + plan.k_slice - 1) / plan.k_slice;
+  plan.lds_bytes = lds_bytes_for(plan.mp, steps, nw);
+  return plan;
+}
+
+template <int MP, bool DUAL>
+hipError_t launch_instance(const MfmaGemvParams &p, dim3 grid, size_t lds_bytes, hipStream_t stream) {
+  static bool configured = false;  // per instantiation; the attribute is per device function
+  if (!configured) {
+    hipError_t status = hipFuncSetAttribute(
+        reinterpret_cast<const void *>(&w4a16_gemv_mfma_kernel<MP, DUAL>),
+        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    if (status != hipSuccess) return status;
+    configured = true;
+  }
+  hipLaunchKernelGGL((w4a16_gemv_mfma_kernel<MP, DUAL>), grid, dim3(kThreads), lds_bytes, stream, p);
   return hipGetLastError();
 }
 
+template <bool DUAL>
+hipError_t launch(MfmaGemvParams p, uint32_t matrices, uint32_t max_n, const Plan &plan, hipStream_t stream) {
+  p.k_slice = plan.k_slice;
+  const uint32_t tiles = (max_n + TN - 1) / TN;
+  const uint32_t per_cu = plan.lds_bytes <= kLdsBudget ? 2 : 1;
+  const uint32_t resident = (uint32_t)device_compute_units() * per_cu;
+  const uint32_t blocks = std::max<uint32_t>(1, std::min<uint32_t>(tiles, resident / (plan.slices * matrices)));
+  const dim3 grid(blocks, plan.slices, matrices);
+  switch (plan.mp) {
+    case 1: return launch_instance<1, DUAL>(p, grid, plan.lds_bytes, stream);
+    case 2: return launch_instance<2, DUAL>(p, grid, plan.lds_bytes, stream);
+    case 4: return launch_instance<4, DUAL>(p, grid, plan.lds_bytes, stream);
+    default: return launch_instance<8, DUAL>(p, grid, plan.lds_bytes, stream);
+  }
+}
+
 }  // namespace
+
+size_t w4a16_gemv_workspace_bytes(uint32_t m, uint32_t n, uint32_t k) {
+  const Plan plan = make_plan(m, k, 1, true);
+  return plan.slices > 1 ? (size_t)plan.slices * 8 * n * sizeof(float) : 0;
+}
 
 hipError_t launch_w4a16_gemv_mfma_linear(const W4LinearArgs &a, hipStream_t stream) {
   MfmaGemvParams p = {};
@@ -222,7 +413,14 @@ hipError_t launch_w4a16_gemv_mfma_linear(const W4LinearArgs &a, hipStream_t stre
   p.addend = a.addend;
   p.has_addend = a.has_addend;
   p.addend_stride = a.addend_row_stride;
-  return launch<false>(p, 1, a.n, stream);
+  const uint32_t tiles = (a.n + TN - 1) / TN;
+  const bool may_split = a.workspace != nullptr && a.counters != nullptr && tiles <= a.counter_count &&
+                         a.workspace_bytes >= w4a16_gemv_workspace_bytes(a.m, a.n, a.k);
+  const Plan plan = make_plan(a.m, a.k, 1, may_split);
+  if (plan.lds_bytes > 160 * 1024) return hipErrorInvalidValue;
+  p.partials = static_cast<float *>(a.workspace);
+  p.counters = a.counters;
+  return launch<false>(p, 1, a.n, plan, stream);
 }
 
 hipError_t launch_w4a16_gemv_mfma_qkv(const W4QkvArgs &a, hipStream_t stream) {
@@ -233,7 +431,9 @@ hipError_t launch_w4a16_gemv_mfma_qkv(const W4QkvArgs &a, hipStream_t stream) {
   p.mat0 = {a.w[0].weight, a.w[0].scale, a.y[0], a.n[0]};
   p.mat1 = {a.w[1].weight, a.w[1].scale, a.y[1], a.n[1]};
   p.mat2 = {a.w[2].weight, a.w[2].scale, a.y[2], a.n[2]};
-  return launch<false>(p, 3, std::max(a.n[0], std::max(a.n[1], a.n[2])), stream);
+  const Plan plan = make_plan(a.m, a.k, 1, false);
+  if (plan.lds_bytes > 160 * 1024) return hipErrorInvalidValue;
+  return launch<false>(p, 3, std::max(a.n[0], std::max(a.n[1], a.n[2])), plan, stream);
 }
 
 hipError_t launch_w4a16_gemv_mfma_dual_swiglu(const W4DualSwigluArgs &a, hipStream_t stream) {
@@ -244,7 +444,9 @@ hipError_t launch_w4a16_gemv_mfma_dual_swiglu(const W4DualSwigluArgs &a, hipStre
   p.mat0 = {a.gate.weight, a.gate.scale, a.product, a.n};
   p.mat1 = {a.up.weight, a.up.scale, a.product, a.n};
   p.mat2 = p.mat0;
-  return launch<true>(p, 1, a.n, stream);
+  const Plan plan = make_plan(a.m, a.k, 2, false);
+  if (plan.lds_bytes > 160 * 1024) return hipErrorInvalidValue;
+  return launch<true>(p, 1, a.n, plan, stream);
 }
 
 }  // namespace llmopt

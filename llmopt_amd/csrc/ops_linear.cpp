@@ -34,6 +34,20 @@ int launched(hipError_t status, const char *name) {
   return LLMOPT_OK;
 }
 
+// Scratch for the decode path when it splits K over workgroups (m x k beyond
+// the LDS budget); none is needed for most shapes.
+int attach_linear_scratch(llmopt_hip_context *context, W4LinearArgs *args) {
+  if (args->m > kGemvMaxRows) return LLMOPT_OK;
+  const size_t bytes = w4a16_gemv_workspace_bytes(args->m, args->n, args->k);
+  if (bytes == 0) return LLMOPT_OK;
+  args->workspace = context_workspace(context, bytes);
+  if (args->workspace == nullptr) return LLMOPT_ERR_FAILURE;
+  args->workspace_bytes = bytes;
+  args->counters = context_counters(context, &args->counter_count);
+  if (args->counters == nullptr) return LLMOPT_ERR_FAILURE;
+  return LLMOPT_OK;
+}
+
 // W4A16Params {u32 m, n, k, has_bias, bias_row_stride}  (lib/metal_w4a16_source.ml:7)
 // buffers: input, packed_weight, scale, bias_or_scale, output.
 int w4a16_linear(llmopt_hip_context *context, const DispatchRecord &record) {
@@ -59,6 +73,7 @@ int w4a16_linear(llmopt_hip_context *context, const DispatchRecord &record) {
   args.m = m;
   args.n = n;
   args.k = k;
+  if (int status = attach_linear_scratch(context, &args)) return status;
   return launched(launch_w4a16_linear(args, context->stream), record.name.c_str());
 }
 
@@ -131,6 +146,7 @@ int w4a16_down_add(llmopt_hip_context *context, const DispatchRecord &record) {
   args.m = m;
   args.n = k;
   args.k = n;
+  if (int status = attach_linear_scratch(context, &args)) return status;
   return launched(launch_w4a16_linear(args, context->stream), record.name.c_str());
 }
 

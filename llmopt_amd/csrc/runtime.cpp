@@ -125,6 +125,24 @@ void *context_workspace(llmopt_hip_context *context, size_t bytes) {
   return block;
 }
 
+uint32_t *context_counters(llmopt_hip_context *context, uint32_t *count) {
+  constexpr uint32_t kCounters = 16384;
+  if (context->counters == nullptr) {
+    void *block = nullptr;
+    hipError_t status = hipMalloc(&block, kCounters * sizeof(uint32_t));
+    if (status == hipSuccess) status = hipMemset(block, 0, kCounters * sizeof(uint32_t));
+    if (status != hipSuccess) {
+      if (block) (void)hipFree(block);
+      fail_hip(status, "HIP could not allocate the tile counters");
+      return nullptr;
+    }
+    context->counters = static_cast<uint32_t *>(block);
+    context->counter_count = kCounters;
+  }
+  *count = context->counter_count;
+  return context->counters;
+}
+
 static int positive_size(int64_t value, const char *name) {
   if (value <= 0) return fail(LLMOPT_ERR_INVALID, "HIP %s must be positive", name);
   return LLMOPT_OK;
@@ -254,6 +272,7 @@ void llmopt_hip_release_context(llmopt_hip_context *context) {
   (void)hipSetDevice(context->device);
   if (context->stream) (void)hipStreamSynchronize(context->stream);
   if (context->workspace) (void)hipFree(context->workspace);
+  if (context->counters) (void)hipFree(context->counters);
   if (context->owns_stream && context->stream) (void)hipStreamDestroy(context->stream);
   delete context;
 }

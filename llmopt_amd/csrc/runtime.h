@@ -45,6 +45,10 @@ struct llmopt_hip_context : llmopt::RefCounted {
   // on the context's single stream.
   void *workspace = nullptr;
   size_t workspace_bytes = 0;
+  // Arrival counters of kernels that split one output tile over several
+  // workgroups; zeroed once, every kernel leaves them zero.
+  uint32_t *counters = nullptr;
+  uint32_t counter_count = 0;
 };
 
 struct llmopt_hip_buffer : llmopt::RefCounted {
@@ -103,6 +107,9 @@ float param_f32(const DispatchRecord &record, size_t byte_offset);
 // Returns device scratch of at least `bytes` (256-byte aligned) or nullptr
 // with the error set.
 void *context_workspace(llmopt_hip_context *context, size_t bytes);
+// Returns the context's zero-initialised arrival counters (allocated on first
+// use) or nullptr with the error set.
+uint32_t *context_counters(llmopt_hip_context *context, uint32_t *count);
 
 void retain(RefCounted *object);
 // Returns true when the caller dropped the last reference.
