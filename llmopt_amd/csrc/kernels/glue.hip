@@ -1,0 +1,277 @@
+// Small decode-step kernels around the W4A16 linears and the Q8 attention:
+// RMSNorm, rotate-half RoPE for Q and K, fp16 embedding gather, broadcasting
+// fp16 add, byte copy and the two-step argmax of the LM head.  All of them move
+// a few kilobytes per launch at decode sizes and are launch-latency bound; they
+// are written for clarity, one wave per row where a row reduction is needed.
+#include <algorithm>
+
+#include "kernels.h"
+#include "w4_common.h"
+
+namespace llmopt {
+namespace {
+
+constexpr int kRowWaves = 4;  // rows (waves) per workgroup of the row kernels
+
+template <typename In>
+__device__ __forceinline__ float load_as_float(const In *p, size_t i);
+template <>
+__device__ __forceinline__ float load_as_float<uint16_t>(const uint16_t *p, size_t i) {
+  return half_bits_to_float(p[i]);
+}
+template <>
+__device__ __forceinline__ float load_as_float<float>(const float *p, size_t i) {
+  return p[i];
+}
+
+// lib/metal_normalization_source.ml:70-91 and lib/metal_w4a16_source.ml:496-526
+template <typename In, bool WEIGHT_FIRST>
+__global__ __launch_bounds__(kRowWaves * 64) void rms_norm_kernel(const In *input, const uint16_t *weight,
+                                                                  uint16_t *output, uint32_t rows,
+                                                                  uint32_t width, float epsilon) {
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t row = blockIdx.x * kRowWaves + (threadIdx.x >> 6);
+  if (row >= rows) return;  // whole wave
+  const size_t base = (size_t)row * width;
+  float square_sum = 0.0f;
+  for (uint32_t col = lane; col < width; col += 64) {
+    const float value = load_as_float(input, base + col);
+    square_sum += value * value;
+  }
+  square_sum = wave_sum(square_sum);
+  const float inverse = rsqrtf(square_sum / (float)width + epsilon);
+  for (uint32_t col = lane; col < width; col += 64) {
+    const float value = load_as_float(input, base + col);
+    const float w = half_bits_to_float(weight[col]);
+    output[base + col] = float_to_half_bits(WEIGHT_FIRST ? value * w * inverse : value * inverse * w);
+  }
+}
+
+// lib/metal_normalization_source.ml:765-802
+__global__ __launch_bounds__(kRowWaves * 64) void rotary_qk_kernel(RotaryQkArgs a) {
+#pragma clang fp contract(off)  // every product and the sum round to half separately
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t row = blockIdx.x * kRowWaves + (threadIdx.x >> 6);
+  const uint32_t total_rows = a.batches * (a.q_heads + a.k_heads) * a.tokens;
+  if (row >= total_rows) return;
+  const uint32_t q_rows = a.batches * a.q_heads * a.tokens;
+  const bool is_q = row < q_rows;
+  const uint32_t local_row = is_q ? row : row - q_rows;
+  const uint32_t heads = is_q ? a.q_heads : a.k_heads;
+  const uint32_t batch = local_row / (heads * a.tokens);
+  const uint32_t head_token = local_row % (heads * a.tokens);
+  const uint32_t head = head_token / a.tokens;
+  const uint32_t token = head_token % a.tokens;
+  const size_t input_base = ((size_t)(batch * a.tokens + token) * heads + head) * a.width;
+  const _Float16 *input = reinterpret_cast<const _Float16 *>(is_q ? a.q_input : a.k_input);
+  _Float16 *output = reinterpret_cast<_Float16 *>(is_q ? a.q_output : a.k_output);
+  const _Float16 *cosine = reinterpret_cast<const _Float16 *>(a.cosine);
+  const _Float16 *sine = reinterpret_cast<const _Float16 *>(a.sine);
+  const uint32_t trig_batch = a.trig_batches == 1 ? 0 : batch;
+  const size_t trig_base = (size_t)(trig_batch * a.tokens + token) * a.width;
+  const size_t output_base = (size_t)local_row * a.width;
+  for (uint32_t col = lane; col < a.width; col += 64) {
+    const uint32_t rotated_col = col < a.half_dimension ? col + a.half_dimension : col - a.half_dimension;
+    _Float16 rotated = input[input_base + rotated_col];
+    if (col < a.half_dimension) rotated = -rotated;
+    const _Float16 direct = input[input_base + col] * cosine[trig_base + col];
+    const _Float16 turned = rotated * sine[trig_base + col];
+    output[output_base + col] = direct + turned;
+  }
+}
+
+// lib/metal_tensor_source.ml:306-320
+__global__ void embedding_kernel(EmbeddingArgs a) {
+  const size_t gid = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const size_t count = (size_t)a.tokens * a.width;
+  if (gid >= count) return;
+  const uint32_t token = (uint32_t)(gid / a.width);
+  const uint32_t dimension = (uint32_t)(gid % a.width);
+  const int64_t index = a.indices[token];
+  a.output[gid] =
+      (index >= 0 && index < (int64_t)a.vocabulary) ? a.weight[(size_t)index * a.width + dimension] : (uint16_t)0;
+}
+
+// llmopt_pointwise_offset, lib/metal_tensor_source.ml:1014-1028
+__device__ __forceinline__ uint32_t pointwise_offset(uint32_t gid, const PointwiseArgs &a, bool is_left) {
+  uint32_t remaining = gid, offset = 0, stride = 1;
+  for (int axis = (int)a.rank - 1; axis >= 0; --axis) {
+    const uint32_t output_dimension = a.output_shape[axis];
+    const uint32_t coordinate = remaining % output_dimension;
+    remaining /= output_dimension;
+    const uint32_t input_dimension = is_left ? a.left_shape[axis] : a.right_shape[axis];
+    offset += (input_dimension == 1 ? 0 : coordinate) * stride;
+    stride *= input_dimension;
+  }
+  return offset;
+}
+
+__global__ void add_f16_kernel(PointwiseArgs a) {
+  const uint32_t gid = blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= a.count) return;
+  const _Float16 left = a.left_scalar
+                            ? (_Float16)a.left_f32
+                            : reinterpret_cast<const _Float16 *>(a.left)[pointwise_offset(gid, a, true)];
+  const _Float16 right = a.right_scalar
+                             ? (_Float16)a.right_f32
+                             : reinterpret_cast<const _Float16 *>(a.right)[pointwise_offset(gid, a, false)];
+  reinterpret_cast<_Float16 *>(a.output)[gid] = left + right;
+}
+
+// both operands have the output's shape: 8 halves per thread
+__global__ void add_f16_same_shape_kernel(const uint4 *left, const uint4 *right, uint4 *output,
+                                          uint32_t vectors) {
+  const uint32_t gid = blockIdx.x * blockDim.x + threadIdx.x;
+  if (gid >= vectors) return;
+  const uint4 l = left[gid], r = right[gid];
+  uint4 out;
+  out.x = as_u32(as_h2(l.x) + as_h2(r.x));
+  out.y = as_u32(as_h2(l.y) + as_h2(r.y));
+  out.z = as_u32(as_h2(l.z) + as_h2(r.z));
+  out.w = as_u32(as_h2(l.w) + as_h2(r.w));
+  output[gid] = out;
+}
+
+__global__ void copy_vectors_kernel(const u32x4_t *source, u32x4_t *destination, size_t vectors) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < vectors; i += stride)
+    destination[i] = __builtin_nontemporal_load(source + i);
+}
+
+__global__ void copy_bytes_kernel(const uint8_t *source, uint8_t *destination, size_t bytes) {
+  const size_t stride = (size_t)gridDim.x * blockDim.x;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < bytes; i += stride)
+    destination[i] = source[i];
+}
+
+struct Candidate {
+  float value;
+  uint32_t index;
+};
+
+__device__ __forceinline__ bool better(float value, uint32_t index, float best_value, uint32_t best_index) {
+  return value > best_value || (value == best_value && index < best_index);
+}
+
+// thread t of row `blockIdx.x` scans columns t, t + 256, ...
+__global__ __launch_bounds__(256) void argmax_candidates_kernel(const float *logits, Candidate *candidates,
+                                                               uint32_t n) {
+  const uint32_t row = blockIdx.x;
+  float best_value = -3.402823466e+38f;
+  uint32_t best_index = 0;
+  for (uint32_t col = threadIdx.x; col < n; col += 256) {
+    const float value = logits[(size_t)row * n + col];
+    if (better(value, col, best_value, best_index)) {
+      best_value = value;
+      best_index = col;
+    }
+  }
+  candidates[row * 256 + threadIdx.x] = {best_value, best_index};
+}
+
+// lib/metal_w4a16_source.ml:1287-1315
+__global__ __launch_bounds__(256) void argmax_reduce_kernel(const Candidate *candidates, uint32_t *token_ids) {
+  __shared__ float best_values[256];
+  __shared__ uint32_t best_indices[256];
+  const uint32_t row = blockIdx.x, tid = threadIdx.x;
+  best_values[tid] = candidates[row * 256 + tid].value;
+  best_indices[tid] = candidates[row * 256 + tid].index;
+  __syncthreads();
+  for (uint32_t width = 128; width > 0; width >>= 1) {
+    if (tid < width && better(best_values[tid + width], best_indices[tid + width], best_values[tid],
+                              best_indices[tid])) {
+      best_values[tid] = best_values[tid + width];
+      best_indices[tid] = best_indices[tid + width];
+    }
+    __syncthreads();
+  }
+  if (tid == 0) token_ids[row] = best_indices[0];
+}
+
+}  // namespace
+
+hipError_t launch_rms_norm(const RmsNormArgs &a, hipStream_t stream) {
+  const dim3 grid((a.rows + kRowWaves - 1) / kRowWaves), block(kRowWaves * 64);
+  if (a.input_f32) {
+    const float *in = static_cast<const float *>(a.input);
+    if (a.weight_first)
+      hipLaunchKernelGGL((rms_norm_kernel<float, true>), grid, block, 0, stream, in, a.weight, a.output, a.rows,
+                         a.width, a.epsilon);
+    else
+      hipLaunchKernelGGL((rms_norm_kernel<float, false>), grid, block, 0, stream, in, a.weight, a.output,
+                         a.rows, a.width, a.epsilon);
+  } else {
+    const uint16_t *in = static_cast<const uint16_t *>(a.input);
+    if (a.weight_first)
+      hipLaunchKernelGGL((rms_norm_kernel<uint16_t, true>), grid, block, 0, stream, in, a.weight, a.output,
+                         a.rows, a.width, a.epsilon);
+    else
+      hipLaunchKernelGGL((rms_norm_kernel<uint16_t, false>), grid, block, 0, stream, in, a.weight, a.output,
+                         a.rows, a.width, a.epsilon);
+  }
+  return hipGetLastError();
+}
+
+hipError_t launch_rotary_qk(const RotaryQkArgs &a, hipStream_t stream) {
+  const uint32_t rows = a.batches * (a.q_heads + a.k_heads) * a.tokens;
+  hipLaunchKernelGGL(rotary_qk_kernel, dim3((rows + kRowWaves - 1) / kRowWaves), dim3(kRowWaves * 64), 0,
+                     stream, a);
+  return hipGetLastError();
+}
+
+hipError_t launch_embedding(const EmbeddingArgs &a, hipStream_t stream) {
+  const size_t count = (size_t)a.tokens * a.width;
+  hipLaunchKernelGGL(embedding_kernel, dim3((uint32_t)((count + 255) / 256)), dim3(256), 0, stream, a);
+  return hipGetLastError();
+}
+
+hipError_t launch_add_f16(const PointwiseArgs &a, hipStream_t stream) {
+  bool same_shape = !a.left_scalar && !a.right_scalar && a.count % 8 == 0;
+  for (uint32_t axis = 0; axis < a.rank && same_shape; ++axis)
+    same_shape = a.left_shape[axis] == a.output_shape[axis] && a.right_shape[axis] == a.output_shape[axis];
+  const auto aligned = [](const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; };
+  if (same_shape && aligned(a.left) && aligned(a.right) && aligned(a.output)) {
+    const uint32_t vectors = a.count / 8;
+    hipLaunchKernelGGL(add_f16_same_shape_kernel, dim3((vectors + 255) / 256), dim3(256), 0, stream,
+                       reinterpret_cast<const uint4 *>(a.left), reinterpret_cast<const uint4 *>(a.right),
+                       reinterpret_cast<uint4 *>(a.output), vectors);
+  } else {
+    hipLaunchKernelGGL(add_f16_kernel, dim3((a.count + 255) / 256), dim3(256), 0, stream, a);
+  }
+  return hipGetLastError();
+}
+
+hipError_t launch_copy_bytes(void *destination, const void *source, size_t bytes, hipStream_t stream) {
+  if (bytes == 0) return hipSuccess;
+  const bool vector_ok = ((reinterpret_cast<uintptr_t>(destination) | reinterpret_cast<uintptr_t>(source)) & 15) == 0;
+  const size_t vectors = vector_ok ? bytes / 16 : 0;
+  if (vectors > 0) {
+    const size_t wanted = (vectors + 255) / 256;
+    const uint32_t blocks = (uint32_t)std::min<size_t>(wanted, 8192);
+    hipLaunchKernelGGL(copy_vectors_kernel, dim3(blocks), dim3(256), 0, stream,
+                       static_cast<const u32x4_t *>(source), static_cast<u32x4_t *>(destination), vectors);
+  }
+  const size_t done = vectors * 16;
+  if (done < bytes) {
+    const size_t rest = bytes - done;
+    const uint32_t blocks = (uint32_t)std::min<size_t>((rest + 255) / 256, 8192);
+    hipLaunchKernelGGL(copy_bytes_kernel, dim3(blocks), dim3(256), 0, stream,
+                       static_cast<const uint8_t *>(source) + done, static_cast<uint8_t *>(destination) + done, rest);
+  }
+  return hipGetLastError();
+}
+
+hipError_t launch_argmax_candidates(const float *logits, void *candidates, uint32_t rows, uint32_t n,
+                                    hipStream_t stream) {
+  hipLaunchKernelGGL(argmax_candidates_kernel, dim3(rows), dim3(256), 0, stream, logits,
+                     static_cast<Candidate *>(candidates), n);
+  return hipGetLastError();
+}
+
+hipError_t launch_argmax_reduce(const void *candidates, uint32_t *token_ids, uint32_t rows, hipStream_t stream) {
+  hipLaunchKernelGGL(argmax_reduce_kernel, dim3(rows), dim3(256), 0, stream,
+                     static_cast<const Candidate *>(candidates), token_ids);
+  return hipGetLastError();
+}
+
+}  // namespace llmopt

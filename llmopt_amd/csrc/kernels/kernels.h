@@ -24,8 +24,11 @@ struct W4LinearArgs {
   const uint16_t *addend;  // may be null when has_addend == 0
   uint32_t has_addend;
   uint32_t addend_row_stride;
-  uint16_t *y;  // f16 [m, n]
+  uint16_t *y;  // f16 [m, n]; may be null when only y_f32 is wanted
   uint32_t m, n, k;
+  // Optional float32 copy of the output before rounding to half (decode path
+  // only, m <= kGemvMaxRows): the LM head takes its argmax over these.
+  float *y_f32;
   // Optional scratch for the decode path when m x k exceeds the LDS budget and the
   // K range is split over workgroups: fp32 partial sums and one arrival counter per
   // 16-row tile (zero before the first launch; the kernel leaves them zero).
@@ -125,6 +128,64 @@ struct Q8AttentionArgs {
 // row-serial kernel is used).
 size_t q8_attention_workspace_bytes(const Q8AttentionArgs &args);
 hipError_t launch_q8_attention(const Q8AttentionArgs &args, hipStream_t stream);
+
+// ---- decode glue ---------------------------------------------------------------
+
+// out[row, i] = half(x[row, i] * rsqrt(mean(x[row]^2) + eps) * w[i]), one wave per row.
+// weight_first selects the fp32 product order of llmopt_w4a16_swiglu_rms_*
+// (x * w * inverse, lib/metal_w4a16_source.ml:525) instead of that of
+// llmopt_rms_norm_f16_simd (x * inverse * w, lib/metal_normalization_source.ml:90).
+struct RmsNormArgs {
+  const void *input;  // f16 or f32 [rows, width]
+  bool input_f32;
+  const uint16_t *weight;  // f16 [width]
+  uint16_t *output;        // f16 [rows, width]
+  uint32_t rows, width;
+  float epsilon;
+  bool weight_first;
+};
+hipError_t launch_rms_norm(const RmsNormArgs &args, hipStream_t stream);
+
+// llmopt_rotary_qk_f16_simd_h64 (lib/metal_normalization_source.ml:765-802):
+// token-major [b, t, heads, width] in, head-major [b, heads, t, width] out,
+// rotate-half with every product and the sum rounded to half.
+struct RotaryQkArgs {
+  const uint16_t *q_input, *k_input, *cosine, *sine;
+  uint16_t *q_output, *k_output;
+  uint32_t batches, tokens, q_heads, k_heads, width, half_dimension, trig_batches;
+};
+hipError_t launch_rotary_qk(const RotaryQkArgs &args, hipStream_t stream);
+
+// llmopt_embedding_f16 (lib/metal_tensor_source.ml:306-320): row gather, rows
+// outside [0, vocabulary) give zeros.
+struct EmbeddingArgs {
+  const int64_t *indices;
+  const uint16_t *weight;
+  uint16_t *output;
+  uint32_t tokens, vocabulary, width;
+};
+hipError_t launch_embedding(const EmbeddingArgs &args, hipStream_t stream);
+
+// PointwiseParams of llmopt_add_f16 (lib/metal_tensor_source.ml:1007-1032): numpy-style
+// broadcasting over up to 8 axes, or a scalar operand.
+struct PointwiseArgs {
+  const uint16_t *left, *right;
+  uint16_t *output;
+  uint32_t count, rank, left_scalar, right_scalar;
+  uint32_t output_shape[8], left_shape[8], right_shape[8];
+  float left_f32, right_f32;
+};
+hipError_t launch_add_f16(const PointwiseArgs &args, hipStream_t stream);
+
+hipError_t launch_copy_bytes(void *destination, const void *source, size_t bytes, hipStream_t stream);
+
+// Argmax over float32 logits [rows, n] in two steps with the reference's
+// candidate layout (W4A16LmHeadCandidate {f32 value, u32 index}, 256 per row,
+// lib/metal_w4a16_source.ml:1287-1319); ties go to the lowest index.
+hipError_t launch_argmax_candidates(const float *logits, void *candidates, uint32_t rows, uint32_t n,
+                                    hipStream_t stream);
+hipError_t launch_argmax_reduce(const void *candidates, uint32_t *token_ids, uint32_t rows,
+                                hipStream_t stream);
 
 // The largest m the streaming GEMV path takes; above it the MFMA GEMM runs.
 constexpr uint32_t kGemvMaxRows = 8;

@@ -39,6 +39,7 @@ struct GemvParams {
   const uint16_t *addend;
   uint32_t has_addend;
   uint32_t addend_stride;
+  float *y_f32;  // optional float32 copy of seg0's output (same indexing), may be null
 };
 
 // M: activation rows held per lane, R: weight rows per wave and tile, U: K
@@ -228,7 +229,8 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemv_kernel(GemvParams p) {
               if (p.has_addend)
                 value += half_bits_to_float(p.addend[(size_t)m * p.addend_stride + col]);
             }
-            sg.y[(size_t)m * n + col] = float_to_half_bits(value);
+            if (sg.y != nullptr) sg.y[(size_t)m * n + col] = float_to_half_bits(value);
+            if (!DUAL && p.y_f32 != nullptr) p.y_f32[(size_t)m * n + col] = value;
           }
         }
       }
@@ -347,6 +349,7 @@ hipError_t launch_w4a16_gemv_linear(const W4LinearArgs &a, hipStream_t stream) {
   p.addend = a.addend;
   p.has_addend = a.has_addend;
   p.addend_stride = a.addend_row_stride;
+  p.y_f32 = a.y_f32;
   return launch_by_rows<false>(p, 1, a.n, stream);
 }
 

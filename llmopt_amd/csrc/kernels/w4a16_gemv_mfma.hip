@@ -63,6 +63,7 @@ struct MfmaGemvParams {
   uint32_t k_slice;    // K values per blockIdx.y slice, a multiple of 256
   float *partials;     // [gridDim.y][8][n] fp32, used when gridDim.y > 1
   uint32_t *counters;  // one per tile, zero between launches
+  float *y_f32;        // optional float32 copy of mat0's output, may be null
 };
 
 // MP = activation rows held in LDS (1, 2, 4 or 8, >= m)
@@ -293,7 +294,8 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemv_mfma_kernel(MfmaGemvParam
         value = total[0];
         if (p.has_addend) value += half_bits_to_float(p.addend[(size_t)m * p.addend_stride + col]);
       }
-      mat.y[(size_t)m * mat.n + col] = float_to_half_bits(value);
+      if (mat.y != nullptr) mat.y[(size_t)m * mat.n + col] = float_to_half_bits(value);
+      if (!DUAL && p.y_f32 != nullptr) p.y_f32[(size_t)m * mat.n + col] = value;
     }
     __syncthreads();  // the slots are free again
     pending = 0;
@@ -420,6 +422,7 @@ hipError_t launch_w4a16_gemv_mfma_linear(const W4LinearArgs &a, hipStream_t stre
   if (plan.lds_bytes > 160 * 1024) return hipErrorInvalidValue;
   p.partials = static_cast<float *>(a.workspace);
   p.counters = a.counters;
+  p.y_f32 = a.y_f32;
   return launch<false>(p, 1, a.n, plan, stream);
 }
 

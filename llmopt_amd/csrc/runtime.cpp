@@ -4,6 +4,8 @@
 // on them.
 #include "runtime.h"
 
+#include "kernels/kernels.h"
+
 #include <fcntl.h>
 #include <stdio.h>
 #include <string.h>
@@ -508,8 +510,7 @@ int llmopt_hip_buffer_copy(llmopt_hip_buffer *source, llmopt_hip_buffer *destina
     return fail(LLMOPT_ERR_INVALID, "HIP copy requires equal buffer lengths");
   if (int status = use_device(source->context)) return status;
   hipStream_t stream = source->context->stream;
-  LLMOPT_HIP_TRY(hipMemcpyAsync(destination->device, source->device, source->length,
-                                hipMemcpyDeviceToDevice, stream),
+  LLMOPT_HIP_TRY(launch_copy_bytes(destination->device, source->device, source->length, stream),
                  "HIP buffer copy failed");
   LLMOPT_HIP_TRY(hipStreamSynchronize(stream), "HIP buffer copy failed");
   return LLMOPT_OK;
@@ -668,8 +669,8 @@ static int submit_batch(llmopt_hip_batch *batch, bool wait) {
   int status = LLMOPT_OK;
   for (BatchOp &op : batch->ops) {
     if (op.is_copy) {
-      if (hipMemcpyAsync(op.destination->device, op.source->device, op.source->length,
-                         hipMemcpyDeviceToDevice, context->stream) != hipSuccess)
+      if (launch_copy_bytes(op.destination->device, op.source->device, op.source->length, context->stream) !=
+          hipSuccess)
         status = fail(LLMOPT_ERR_FAILURE, "HIP batched copy failed");
     } else {
       status = launch_record(context, op.record);
@@ -700,8 +701,8 @@ int llmopt_hip_commit_batch_profiled(llmopt_hip_batch *batch, int use_graph, int
   auto launch_all = [&]() -> int {
     for (BatchOp &op : batch->ops) {
       if (op.is_copy) {
-        if (hipMemcpyAsync(op.destination->device, op.source->device, op.source->length,
-                           hipMemcpyDeviceToDevice, stream) != hipSuccess)
+        if (launch_copy_bytes(op.destination->device, op.source->device, op.source->length, stream) !=
+            hipSuccess)
           return fail(LLMOPT_ERR_FAILURE, "HIP batched copy failed");
       } else if (int status = launch_record(context, op.record)) {
         return status;
