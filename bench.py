@@ -219,6 +219,48 @@ def bench_attention(runtime):
             "tokens_per_s": round(batches / (us * 1e-6), 1)}
 
 
+def bench_decode_step(runtime, batches=(1, 8, 32), context=2048):
+    """C5: one decode step of the 30-layer model (hidden 576, 9/3 heads of 64, MLP 1536,
+    vocabulary 49152), every sequence with `context` tokens in the Q8 pool, replayed as a
+    HIP graph.  tokens/s = batch / step time."""
+    from llmopt_amd.decode_step import DecodeConfig, DecodeStep, random_weights
+    rng = np.random.default_rng(SEED + 3)
+    config = DecodeConfig()
+    weights = random_weights(config, rng)
+    stride, elements = config.token_stride, config.token_elements
+    # one sequence's worth of pool content, reused for every sequence
+    block = np.empty((context, stride), dtype=np.uint8)
+    block[:, :elements] = np.clip(np.rint(rng.standard_normal((context, elements)) * 38.0), -127, 127) \
+        .astype(np.int8).view(np.uint8)
+    block[:, elements:] = rng.uniform(0.02, 0.035, size=(context, elements // 64)).astype(np.float16) \
+        .view(np.uint8).reshape(context, -1)
+    results = []
+    for batch in batches:
+        capacity = batch * (context + 1)
+        pool = runtime.create_buffer(capacity * stride)
+        for sequence in range(batch):
+            pool.write(block, offset=sequence * (context + 1) * stride)
+        slots = np.concatenate([np.arange(context, dtype=np.uint32) + sequence * (context + 1)
+                                for sequence in range(batch)])
+        offsets = np.arange(batch, dtype=np.uint32) * context
+        new_slots = np.arange(batch, dtype=np.uint32) * (context + 1) + context
+        step = DecodeStep(runtime, config, weights, batch, pool, runtime.buffer_of_bytes(slots), offsets,
+                          [context] * batch, new_slots, [context] * batch)
+        step.run(rng.integers(0, config.vocabulary, batch))  # first-use allocations
+        graph = runtime.begin_batch()
+        step.record(graph)
+        repeats = 20
+        ms = graph.commit_profiled(repeats=repeats, use_graph=True) / repeats
+        moved = step.weight_bytes() + step.kv_bytes()
+        results.append({"batch": batch, "context": context, "launches": len(step.dispatches),
+                        "ms_per_step": round(ms, 4), "tokens_per_s": round(batch / (ms * 1e-3), 1),
+                        "weight_bytes": step.weight_bytes(), "kv_bytes": step.kv_bytes(),
+                        "GBps": round(moved / (ms * 1e-3) / 1e9, 1),
+                        "hbm_frac": round(moved / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)})
+        del step, pool
+    return results
+
+
 def cpu_baseline(passes=2):
     """The C oracle (a port of lib/cpu.ml's w4a16_linear, lib/cpu.ml:128-152) on ONE host
     core: `passes` passes over the whole 12-case GEMV sweep at full size (about 15 s of
@@ -267,6 +309,7 @@ def main():
     if not args.skip_extras:
         extras["prefill_gemm"] = bench_gemm(runtime)
         extras["q8_attention"] = bench_attention(runtime)
+        extras["decode_step"] = bench_decode_step(runtime)
     line = {
         "metric": "W4A16 GEMV HBM GB/s (% peak); Q8 attn decode tokens/s; prefill MFMA %",
         "value": round(value, 1),

@@ -83,6 +83,10 @@ struct Q8PackArgs {
   uint32_t heads, head_dim;
   uint32_t token_elements, token_stride;
   uint32_t source_items, source_offset;
+  // Extension for batched decode: the sources are [items, heads, head_dim]
+  // (one new token per sequence, as the K/V projections leave them) instead of
+  // head-major; source_items / source_offset are then unused.
+  uint32_t item_major;
 };
 
 struct Q8UnpackArgs {

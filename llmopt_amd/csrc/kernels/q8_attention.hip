@@ -22,6 +22,7 @@
 //    serial over keys with an online softmax.  Covers everything else (mask,
 //    window, several query tokens, other head sizes).
 #include <algorithm>
+#include <type_traits>
 
 #include "kernels.h"
 #include "kernels_internal.h"
@@ -71,7 +72,7 @@ __device__ __forceinline__ size_t partial_floats(uint32_t heads_per_kv) {
 
 // OFF32: the pool is smaller than 4 GiB, so slot byte offsets fit 32 bits and the
 // loads can use a scalar base plus a 32-bit vector offset.
-template <int D, bool OFF32>
+template <int D, bool OFF32, bool A16>
 __global__ __launch_bounds__(kSplitMaxWaves * 64) void q8_attention_split_kernel(Q8AttentionArgs a,
                                                                            uint32_t chunks_max) {
   constexpr int GROUPS = D / 64;      // scale groups per head
@@ -162,12 +163,16 @@ __global__ __launch_bounds__(kSplitMaxWaves * 64) void q8_attention_split_kernel
   };
   // With OFF32 every address is the scalar pool base plus one 32-bit lane offset
   // and a compile-time displacement, so a load needs no 64-bit vector add.
+  // A16 = false: pool slots are only 4-byte aligned (a token stride that is not a
+  // multiple of 16, e.g. 11880 bytes); the key loads then carry that alignment.
+  typedef uint32_t unaligned_u32x4_t __attribute__((ext_vector_type(4), aligned(4)));
+  using KeyVector = typename std::conditional<A16, u32x4_t, unaligned_u32x4_t>::type;
   auto load_raw = [&](const TileSlots &where, TileRaw &out) __attribute__((always_inline)) {
     if (OFF32) {
       const uint32_t key_offset = where.key * a.token_stride + key_base + quad * 16;
 #pragma unroll
       for (int g = 0; g < KLOADS; ++g)
-        out.k[g] = *reinterpret_cast<const u32x4_t *>(a.pool + key_offset + g * 64);
+        out.k[g] = *reinterpret_cast<const KeyVector *>(a.pool + key_offset + g * 64);
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
         const uint32_t slot_offset = where.value[i] * a.token_stride;
@@ -190,7 +195,7 @@ __global__ __launch_bounds__(kSplitMaxWaves * 64) void q8_attention_split_kernel
     const uint8_t *key_slot = a.pool + (size_t)where.key * a.token_stride;
 #pragma unroll
     for (int g = 0; g < KLOADS; ++g)
-      out.k[g] = *reinterpret_cast<const u32x4_t *>(key_slot + key_base + g * 64 + quad * 16);
+      out.k[g] = *reinterpret_cast<const KeyVector *>(key_slot + key_base + g * 64 + quad * 16);
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const uint8_t *slot = a.pool + (size_t)where.value[i] * a.token_stride;
@@ -520,8 +525,9 @@ bool use_split_path(const Q8AttentionArgs &a) {
   if (a.head_dim != 64 && a.head_dim != 128) return false;
   if (a.kv_heads == 0 || a.query_heads % a.kv_heads != 0) return false;
   if (a.query_heads / a.kv_heads > 16) return false;
-  // 16-byte K loads and 4-byte V loads from pool slots
-  if (a.token_stride % 16 != 0 || a.key_offset % 16 != 0 || a.value_offset % 4 != 0) return false;
+  // 4-byte aligned K and V loads from pool slots (16-byte aligned K loads when the stride allows)
+  if (a.token_stride % 4 != 0 || a.key_offset % 4 != 0 || a.value_offset % 4 != 0) return false;
+  if ((reinterpret_cast<uintptr_t>(a.pool) & 3) != 0) return false;
   if (a.token_elements % 2 != 0) return false;
   // D = 128 reads the two group scales of a head as one aligned dword
   if (a.head_dim == 128 && (a.key_offset % 128 != 0 || a.value_offset % 128 != 0)) return false;
@@ -551,19 +557,24 @@ hipError_t launch_q8_attention(const Q8AttentionArgs &a, hipStream_t stream) {
     const dim3 block(waves * 64);
     const dim3 merge_grid(a.query_heads, a.batches);
     const bool small_pool = a.pool_bytes > 0 && a.pool_bytes <= 0xffffffffull;
-    if (a.head_dim == 128) {
-      if (small_pool)
-        hipLaunchKernelGGL((q8_attention_split_kernel<128, true>), grid, block, 0, stream, a, chunks);
+    const bool aligned16 = a.token_stride % 16 == 0 && a.key_offset % 16 == 0 &&
+                           (reinterpret_cast<uintptr_t>(a.pool) & 15) == 0;
+    const auto launch_split = [&](auto dim_tag) {
+      constexpr int D = decltype(dim_tag)::value;
+      if (small_pool && aligned16)
+        hipLaunchKernelGGL((q8_attention_split_kernel<D, true, true>), grid, block, 0, stream, a, chunks);
+      else if (small_pool)
+        hipLaunchKernelGGL((q8_attention_split_kernel<D, true, false>), grid, block, 0, stream, a, chunks);
+      else if (aligned16)
+        hipLaunchKernelGGL((q8_attention_split_kernel<D, false, true>), grid, block, 0, stream, a, chunks);
       else
-        hipLaunchKernelGGL((q8_attention_split_kernel<128, false>), grid, block, 0, stream, a, chunks);
-      hipLaunchKernelGGL(q8_attention_merge_kernel<128>, merge_grid, dim3(kMergeSlices * 128), 0, stream, a, chunks);
-    } else {
-      if (small_pool)
-        hipLaunchKernelGGL((q8_attention_split_kernel<64, true>), grid, block, 0, stream, a, chunks);
-      else
-        hipLaunchKernelGGL((q8_attention_split_kernel<64, false>), grid, block, 0, stream, a, chunks);
-      hipLaunchKernelGGL(q8_attention_merge_kernel<64>, merge_grid, dim3(kMergeSlices * 64), 0, stream, a, chunks);
-    }
+        hipLaunchKernelGGL((q8_attention_split_kernel<D, false, false>), grid, block, 0, stream, a, chunks);
+      hipLaunchKernelGGL(q8_attention_merge_kernel<D>, merge_grid, dim3(kMergeSlices * D), 0, stream, a, chunks);
+    };
+    if (a.head_dim == 128)
+      launch_split(std::integral_constant<int, 128>{});
+    else
+      launch_split(std::integral_constant<int, 64>{});
     return hipGetLastError();
   }
   const uint32_t q_len = a.query_length == 0 ? 1 : a.query_length;

@@ -29,9 +29,9 @@ __global__ __launch_bounds__(256) void q8_pack_kernel(Q8PackArgs a) {
   const uint32_t local_group = logical_group - item * segment_groups;
   const uint32_t head = local_group / groups_per_head;
   const uint32_t group_in_head = local_group - head * groups_per_head;
-  const size_t source_index =
-      ((size_t)head * a.source_items + a.source_offset + item) * a.head_dim +
-      (size_t)group_in_head * 64 + lane;
+  const size_t source_row =
+      a.item_major ? (size_t)item * a.heads + head : (size_t)head * a.source_items + a.source_offset + item;
+  const size_t source_index = source_row * a.head_dim + (size_t)group_in_head * 64 + lane;
   const size_t slot_base = (size_t)a.slots[item] * a.token_stride;
   int8_t *values = reinterpret_cast<int8_t *>(a.pool + slot_base);
   uint16_t *scales = reinterpret_cast<uint16_t *>(a.pool + slot_base + a.token_elements);

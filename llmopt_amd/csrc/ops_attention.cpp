@@ -61,7 +61,7 @@ int cache_pack(llmopt_hip_context *context, const DispatchRecord &record) {
 
 // AttentionCachePairParams, 11 x u32 (lib/metal_cache_source.ml:22-34).
 // buffers: key_source, value_source, slots, pool.
-int cache_pack_pair(llmopt_hip_context *context, const DispatchRecord &record) {
+int cache_pack_pair_layout(llmopt_hip_context *context, const DispatchRecord &record, bool item_major) {
   if (int status = require_buffer_count(record, 4)) return status;
   if (int status = require_parameter_bytes(record, 44)) return status;
   Q8PackArgs args = {};
@@ -75,6 +75,11 @@ int cache_pack_pair(llmopt_hip_context *context, const DispatchRecord &record) {
   args.token_stride = param_u32(record, 32);
   args.source_items = param_u32(record, 36);
   args.source_offset = param_u32(record, 40);
+  args.item_major = item_major ? 1 : 0;
+  if (item_major) {
+    args.source_items = args.items;
+    args.source_offset = 0;
+  }
   if (int status = check_cache_geometry(record.name.c_str(), args.heads, args.head_dim, group_size,
                                         args.token_elements, args.token_stride))
     return status;
@@ -94,6 +99,16 @@ int cache_pack_pair(llmopt_hip_context *context, const DispatchRecord &record) {
   args.slots = reinterpret_cast<const uint32_t *>(record.buffers[2].device);
   args.pool = record.buffers[3].device;
   return launched(launch_q8_pack(args, true, context->stream), record.name.c_str());
+}
+
+int cache_pack_pair(llmopt_hip_context *context, const DispatchRecord &record) {
+  return cache_pack_pair_layout(context, record, false);
+}
+
+// Extension (no reference kernel): the same pair quantiser for one new token of
+// each of `items` sequences, sources laid out [items, heads, head_dim].
+int cache_pack_pair_batched(llmopt_hip_context *context, const DispatchRecord &record) {
+  return cache_pack_pair_layout(context, record, true);
 }
 
 // buffers: pool, slots, destination; AttentionCacheParams.
@@ -228,6 +243,7 @@ void register_cache_kernels(std::vector<KernelEntryPoint> &table) {
   table.push_back({"llmopt_cache_pack_attention_q8", cache, cache_pack});
   table.push_back({"llmopt_cache_pack_attention_q8_simd", cache, cache_pack});
   table.push_back({"llmopt_cache_pack_attention_q8_pair_simd", cache, cache_pack_pair});
+  table.push_back({"llmopt_cache_pack_attention_q8_pair_batched", cache, cache_pack_pair_batched});
   table.push_back({"llmopt_cache_unpack_attention_q8", cache, cache_unpack});
   table.push_back({"llmopt_cache_unpack_attention_q8_vec4", cache, cache_unpack});
 }

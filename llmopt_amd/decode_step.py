@@ -1,0 +1,225 @@
+"""One decode step of a W4A16 / Q8-KV transformer as a list of kernel dispatches.
+
+The host-side counterpart of what the reference's schedule executor encodes
+for a decode step (lib/metal_schedule_executor.ml via lib/metal_dispatch_*.ml):
+per layer RMSNorm, fused QKV projection, RoPE on Q and K, Q8 pack of the new
+K/V, paged Q8 attention, output projection with the residual as addend, and
+the three-launch SwiGLU FFN; then the LM-head argmax.  Every entry is
+(kernel name, buffers, parameter block, grid, threadgroup) in the reference's
+buffer order, ready for Batch.dispatch or a Prebaked plan.
+
+Sequences of a batch have their own context lengths and slot tables, which the
+batched attention / pack entry points take as two extra buffers.
+"""
+from __future__ import annotations
+
+import math
+import struct
+from dataclasses import dataclass
+
+import numpy as np
+
+from .native import Buffer, Runtime
+
+
+def u32s(*values) -> bytes:
+    """Metal_parameters.u32s (lib/metal_parameters.ml:14-22)."""
+    return struct.pack("<%dI" % len(values), *values)
+
+
+def linear_grid(columns: int) -> int:
+    """linear_f16_grid (lib/metal_dispatch_common.ml:64-70)."""
+    return ((columns + 7) // 8) * 8 * 32
+
+
+@dataclass(frozen=True)
+class DecodeConfig:
+    hidden: int = 576
+    q_heads: int = 9
+    kv_heads: int = 3
+    head_dim: int = 64
+    mlp: int = 1536
+    layers: int = 30
+    vocabulary: int = 49152
+    epsilon: float = 1e-5
+    rope_theta: float = 10000.0
+
+    @property
+    def layer_elements(self) -> int:
+        return 2 * self.kv_heads * self.head_dim
+
+    @property
+    def token_elements(self) -> int:
+        return self.layers * self.layer_elements
+
+    @property
+    def token_stride(self) -> int:
+        """Kv_cache.Layout bytes per token: int8 values + one f16 scale per 64 (lib/kv_cache.ml:126-166)."""
+        return self.token_elements + 2 * (self.token_elements // 64)
+
+
+def rope_rows(config: DecodeConfig, positions) -> tuple[np.ndarray, np.ndarray]:
+    """cos / sin rows for the given positions, duplicated into both halves
+    (Serving_rope_table.create, lib/serving_rope_table.ml:156-172): the angle is
+    f32(inv_freq * f32(position)), cos/sin in f64 -> f32 -> f16."""
+    d = config.head_dim
+    inv_freq = (config.rope_theta ** (-np.arange(0, d, 2, dtype=np.float64) / d)).astype(np.float32)
+    angle = (inv_freq[None, :] * np.asarray(positions, dtype=np.float32)[:, None]).astype(np.float32)
+    cos = np.cos(angle.astype(np.float64)).astype(np.float32).astype(np.float16)
+    sin = np.sin(angle.astype(np.float64)).astype(np.float32).astype(np.float16)
+    return np.concatenate([cos, cos], axis=1), np.concatenate([sin, sin], axis=1)
+
+
+def random_w4(rng, n: int, k: int):
+    packed = rng.integers(0, 256, size=(n, k // 2), dtype=np.uint8)
+    scale = rng.uniform(0.005, 0.02, size=(n, k // 64)).astype(np.float16)
+    return packed, scale
+
+
+def random_weights(config: DecodeConfig, rng) -> dict:
+    """Random-init weights in the reference's formats (host arrays)."""
+    h, kv = config.hidden, config.kv_heads * config.head_dim
+    layers = []
+    for _ in range(config.layers):
+        layers.append({
+            "attn_norm": rng.uniform(0.5, 1.5, h).astype(np.float16),
+            "q": random_w4(rng, config.q_heads * config.head_dim, h),
+            "k": random_w4(rng, kv, h),
+            "v": random_w4(rng, kv, h),
+            "o": random_w4(rng, h, config.q_heads * config.head_dim),
+            "ffn_norm": rng.uniform(0.5, 1.5, h).astype(np.float16),
+            "gate": random_w4(rng, config.mlp, h),
+            "up": random_w4(rng, config.mlp, h),
+            "down": random_w4(rng, h, config.mlp),
+        })
+    return {
+        "embedding": (rng.standard_normal((config.vocabulary, h)) * 0.5).astype(np.float16),
+        "layers": layers,
+        "final_norm": rng.uniform(0.5, 1.5, h).astype(np.float16),
+        "lm_head": random_w4(rng, config.vocabulary, h),
+    }
+
+
+class DecodeStep:
+    """Device buffers and the dispatch list of one decode step for `batch` sequences."""
+
+    def __init__(self, runtime: Runtime, config: DecodeConfig, weights: dict, batch: int, pool: Buffer,
+                 slots: Buffer, slot_offsets, past_lengths, new_slots, positions):
+        self.runtime, self.config, self.batch = runtime, config, batch
+        b = runtime.buffer_of_bytes
+        c = config
+        h = c.hidden
+        self.pool, self.slots = pool, slots
+        self.tokens = b(np.zeros(batch, dtype=np.int64))
+        self.token_ids = b(np.zeros(batch, dtype=np.uint32))
+        self.past_lengths = b(np.asarray(past_lengths, dtype=np.uint32))
+        self.slot_offsets = b(np.asarray(slot_offsets, dtype=np.uint32))
+        self.new_slots = b(np.asarray(new_slots, dtype=np.uint32))
+        cos, sin = rope_rows(c, positions)
+        self.cos, self.sin = b(cos), b(sin)
+        self.max_past = int(max(past_lengths))
+        self.device = {
+            "embedding": b(weights["embedding"]),
+            "final_norm": b(weights["final_norm"]),
+            "lm_head": tuple(b(a) for a in weights["lm_head"]),
+            "layers": [{key: (tuple(b(a) for a in value) if isinstance(value, tuple) else b(value))
+                        for key, value in layer.items()} for layer in weights["layers"]],
+        }
+        create = runtime.create_buffer
+        q_bytes, kv_bytes = batch * c.q_heads * c.head_dim * 2, batch * c.kv_heads * c.head_dim * 2
+        self.work = {
+            "x": [create(batch * h * 2), create(batch * h * 2)],
+            "normed": create(batch * h * 2),
+            "q": create(q_bytes), "k": create(kv_bytes), "v": create(kv_bytes),
+            "q_rot": create(q_bytes), "k_rot": create(kv_bytes),
+            "attention": create(q_bytes),
+            "product": create(batch * c.mlp * 2),
+        }
+        self.dispatches = self._build()
+
+    def _linear_entry(self, columns_of_one_row: int):
+        """Kernel name suffix and grid of the reference's m = 1 / m > 1 choice
+        (lib/metal_dispatch_linear.ml:349-395, 938-982)."""
+        m = self.batch
+        if m == 1:
+            return "", (linear_grid(columns_of_one_row), 1, 1)
+        return "_m4", (linear_grid(((m + 3) // 4) * columns_of_one_row), 1, 1)
+
+    def _build(self) -> list[tuple]:
+        c, m, w = self.config, self.batch, self.work
+        h, qd, kvd = c.hidden, c.q_heads * c.head_dim, c.kv_heads * c.head_dim
+        group = (256, 1, 1)
+        out: list[tuple] = []
+        count = m * h
+        out.append(("llmopt_embedding_f16", [self.tokens, self.device["embedding"], w["x"][0]],
+                    u32s(m, c.vocabulary, h), (((count + 255) // 256) * 256, 1, 1), group))
+        rows_grid = (((m + 7) // 8) * 256, 1, 1)
+        rope_rows_total = m * (c.q_heads + c.kv_heads)
+        for index, layer in enumerate(self.device["layers"]):
+            x_in, x_mid = w["x"][0], w["x"][1]
+            key_offset = index * c.layer_elements
+            value_offset = key_offset + kvd
+            out.append(("llmopt_rms_norm_f16_simd", [x_in, layer["attn_norm"], w["normed"]],
+                        struct.pack("<IIf", m, h, c.epsilon), rows_grid, group))
+            suffix, grid = self._linear_entry(qd + 2 * kvd)
+            out.append(("llmopt_w4a16_qkv_linear_f16_g64" + suffix,
+                        [w["normed"], *layer["q"], *layer["k"], *layer["v"], w["q"], w["k"], w["v"]],
+                        u32s(m, h, qd, kvd, kvd), grid, group))
+            out.append(("llmopt_rotary_qk_f16_simd_h64",
+                        [w["q"], w["k"], self.cos, self.sin, w["q_rot"], w["k_rot"]],
+                        u32s(m, 1, c.q_heads, c.kv_heads, c.head_dim, c.head_dim // 2, m),
+                        (((rope_rows_total + 7) // 8) * 256, 1, 1), group))
+            out.append(("llmopt_cache_pack_attention_q8_pair_batched",
+                        [w["k_rot"], w["v"], self.new_slots, self.pool],
+                        u32s(m, key_offset, value_offset, c.kv_heads, c.head_dim, 64, c.token_elements,
+                             c.token_elements // 64, c.token_stride, m, 0),
+                        (m * c.kv_heads * 32, 1, 1), group))
+            attention_params = struct.pack(
+                "<12IfIII", m, c.q_heads, c.kv_heads, 0, c.head_dim, 0, 0, c.token_elements, key_offset,
+                value_offset, 64, c.token_stride, 1.0 / math.sqrt(c.head_dim), 1, 0, 0)
+            attention_params += struct.pack("<I", self.max_past)
+            out.append(("llmopt_attention_q8_paged_batched",
+                        [w["q_rot"], w["k_rot"], w["v"], self.pool, self.slots, self.slots, w["attention"],
+                         self.past_lengths, self.slot_offsets],
+                        attention_params, (((m * c.q_heads + 7) // 8) * 256, 1, 1), group))
+            suffix, grid = self._linear_entry(h)
+            out.append(("llmopt_w4a16_linear_f16_g64" + suffix,
+                        [w["attention"], *layer["o"], x_in, x_mid], u32s(m, h, qd, 1, h), grid, group))
+            ffn_params = u32s(m, c.mlp, h) + struct.pack("<f", c.epsilon)
+            out.append(("llmopt_w4a16_swiglu_rms_f16_g64", [x_mid, layer["ffn_norm"], w["normed"]],
+                        ffn_params, (m * 256, 1, 1), group))
+            suffix, grid = self._linear_entry(c.mlp)
+            out.append(("llmopt_w4a16_dual_swiglu_f16_g64" + suffix,
+                        [w["normed"], *layer["gate"], *layer["up"], w["product"]], ffn_params, grid, group))
+            suffix, grid = self._linear_entry(h)
+            out.append(("llmopt_w4a16_down_add_f16_g64" + suffix,
+                        [w["product"], *layer["down"], x_mid, x_in], ffn_params, grid, group))
+        out.append(("llmopt_w4a16_lm_head_argmax_f16",
+                    [w["x"][0], self.device["final_norm"], *self.device["lm_head"], self.token_ids],
+                    u32s(m, c.vocabulary, h) + struct.pack("<f", c.epsilon), (m * 256, 1, 1), group))
+        return out
+
+    def record(self, batch) -> None:
+        for name, buffers, parameters, grid, group in self.dispatches:
+            batch.dispatch(name, buffers, parameters, grid=grid, group=group)
+
+    def run(self, tokens) -> np.ndarray:
+        """One eager step: returns the next token id of every sequence."""
+        self.tokens.write(np.asarray(tokens, dtype=np.int64))
+        batch = self.runtime.begin_batch()
+        self.record(batch)
+        batch.commit()
+        return self.token_ids.numpy(np.uint32, (self.batch,))
+
+    def weight_bytes(self) -> int:
+        """Algorithmic weight bytes one step streams (packed weights + scales, the LM head included)."""
+        c = self.config
+        h, qd, kvd = c.hidden, c.q_heads * c.head_dim, c.kv_heads * c.head_dim
+        w4 = lambda n, k: n * k // 2 + 2 * n * (k // 64)
+        layer = w4(qd, h) + 2 * w4(kvd, h) + w4(h, qd) + 2 * w4(c.mlp, h) + w4(h, c.mlp)
+        return c.layers * layer + w4(c.vocabulary, h)
+
+    def kv_bytes(self) -> int:
+        """Algorithmic KV-cache bytes one step reads: every past token's whole pool slot."""
+        total = int(self.past_lengths.numpy(np.uint32).sum())
+        return total * self.config.token_stride

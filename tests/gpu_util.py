@@ -18,7 +18,7 @@ def w4_case(rng, m, n, k, bias=False):
     return x, packed, scale, b
 
 
-def assert_close_to_oracle(actual_f16, expected_f32, what=""):
+def assert_close_to_oracle(actual_f16, expected_f32, what="", rel_l2_tol=REL_L2_TOL):
     actual = np.asarray(actual_f16, dtype=np.float32).reshape(-1)
     expected = np.asarray(expected_f32, dtype=np.float32).reshape(-1)
     assert actual.shape == expected.shape, (what, actual.shape, expected.shape)
@@ -28,7 +28,7 @@ def assert_close_to_oracle(actual_f16, expected_f32, what=""):
     rel_l2 = float(np.sqrt(np.sum(difference ** 2))) / max(norm, 1e-30)
     rms = norm / np.sqrt(max(1, expected.size))
     max_abs = float(np.max(np.abs(difference))) if difference.size else 0.0
-    assert rel_l2 <= REL_L2_TOL, f"{what}: rel-L2 {rel_l2:.3e} > {REL_L2_TOL}"
+    assert rel_l2 <= rel_l2_tol, f"{what}: rel-L2 {rel_l2:.3e} > {rel_l2_tol}"
     assert max_abs <= MAX_ABS_RMS_TOL * rms + 1e-6, \
         f"{what}: max-abs {max_abs:.3e} > {MAX_ABS_RMS_TOL} x RMS {rms:.3e}"
     return rel_l2, max_abs

@@ -207,6 +207,27 @@ def test_decode_attention_shared_slots(runtime, b, h, kvh, dim, past):
     assert_close_to_oracle(out, expected, f"paged b{b} h{h}/{kvh} d{dim} past{past}")
 
 
+@pytest.mark.parametrize("kvh,dim,layers,layer", [(3, 64, 3, 1), (1, 128, 3, 2), (3, 64, 30, 17)])
+def test_decode_attention_slots_not_16_byte_aligned(runtime, kvh, dim, layers, layer):
+    """Token strides that are not a multiple of 16 (e.g. 11880 bytes for 30 layers of 3 x 64)."""
+    rng = np.random.default_rng(layers * 100 + dim)
+    past, group = 700, 3
+    pool, slots, _, te, stride, ko, vo = build_pool(rng, kvh, dim, [past], layers=layers, layer=layer)
+    assert stride % 16 != 0
+    h = kvh * group
+    query = rng.standard_normal((2, h, 1, dim)).astype(np.float16)
+    ck = rng.standard_normal((2, kvh, 1, dim)).astype(np.float16)
+    cv = rng.standard_normal((2, kvh, 1, dim)).astype(np.float16)
+    params = PagedParams(batches=2, query_heads=h, kv_heads=kvh, past_length=past, head_dim=dim,
+                         mask_batches=0, mask_heads=0, token_elements=te, key_offset=ko,
+                         value_offset=vo, group_size=64, token_stride=stride,
+                         scale=1.0 / math.sqrt(dim), query_length=1, mask_dtype=0, window=0)
+    name = "llmopt_attention_q8_paged_simd_generic" if dim == 128 else "llmopt_attention_q8_paged_simd_h64_gqa3"
+    out = run_paged(runtime, name, query, ck, cv, pool, slots, None, params)
+    expected = oracle.paged_attention_q8(query, ck, cv, pool, slots, None, params)
+    assert_close_to_oracle(out, expected, f"unaligned stride {stride}")
+
+
 def test_decode_attention_per_sequence_lengths(runtime):
     """The batched extension: ragged contexts, one slot table per sequence."""
     rng = np.random.default_rng(99)
