@@ -219,7 +219,7 @@ def bench_attention(runtime):
             "tokens_per_s": round(batches / (us * 1e-6), 1)}
 
 
-def bench_decode_step(runtime, batches=(1, 8, 32), context=2048):
+def bench_decode_step(runtime, batches=(1, 8, 32), context=2048, use_graph=True):
     """C5: one decode step of the 30-layer model (hidden 576, 9/3 heads of 64, MLP 1536,
     vocabulary 49152), every sequence with `context` tokens in the Q8 pool, replayed as a
     HIP graph.  tokens/s = batch / step time."""
@@ -250,7 +250,7 @@ def bench_decode_step(runtime, batches=(1, 8, 32), context=2048):
         graph = runtime.begin_batch()
         step.record(graph)
         repeats = 20
-        ms = graph.commit_profiled(repeats=repeats, use_graph=True) / repeats
+        ms = graph.commit_profiled(repeats=repeats, use_graph=use_graph) / repeats
         moved = step.weight_bytes() + step.kv_bytes()
         results.append({"batch": batch, "context": context, "launches": len(step.dispatches),
                         "ms_per_step": round(ms, 4), "tokens_per_s": round(batch / (ms * 1e-3), 1),
@@ -259,6 +259,43 @@ def bench_decode_step(runtime, batches=(1, 8, 32), context=2048):
                         "hbm_frac": round(moved / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)})
         del step, pool
     return results
+
+
+def pmc_probe(runtime):
+    """A short run for hardware counters (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE): four plain
+    64 MiB device-to-device copies, whose bytes are known, then the headline GEMV (M = 1,
+    K = 4096, N = 14336) over 16 distinct weight copies.  The copy calibrates the counters."""
+    rng = np.random.default_rng(SEED)
+    copy_bytes = 64 << 20
+    source = runtime.buffer_of_bytes(rng.integers(0, 256, copy_bytes, dtype=np.uint8))
+    destination = runtime.create_buffer(copy_bytes)
+    for _ in range(4):
+        source.copy_to(destination)
+    k, n = 4096, 14336
+    x, packed, scale = w4_inputs(rng, 1, n, k)
+    bx, out = runtime.buffer_of_bytes(x), runtime.create_buffer(n * 2)
+    weights = [(runtime.buffer_of_bytes(packed), runtime.buffer_of_bytes(scale)) for _ in range(COPIES)]
+    batch = runtime.begin_batch()
+    for bw, bs in weights:
+        record_linear(batch, 1, n, k, bx, bw, bs, out)
+    batch.commit()
+    return {"copy_kernel": "copy_vectors_kernel", "copy_bytes_read": copy_bytes, "copy_bytes_written": copy_bytes,
+            "copy_launches": 4, "gemv_kernel": "w4a16_gemv_kernel<1, 2, 1, true, false>",
+            "gemv_launches": COPIES, "gemv_algorithmic_bytes": gemv_bytes(1, k, n)}
+
+
+def measured_traffic():
+    """HBM bytes per launch of the headline kernel, measured with rocprofv3 hardware counters
+    (FETCH_SIZE and WRITE_SIZE, each calibrated on a plain copy) and kept with the profile
+    summaries; None when the summary is not there."""
+    path = os.path.join(ROOT, "profiles", "w4a16_gemv_m1_k4096_n14336_hbm_traffic.txt")
+    try:
+        for line in open(path):
+            if line.startswith("traffic_bytes_per_launch:"):
+                return int(line.split(":")[1])
+    except OSError:
+        pass
+    return None
 
 
 def cpu_baseline(passes=2):
@@ -290,13 +327,23 @@ def main():
     parser.add_argument("--steps", type=int, default=64)
     parser.add_argument("--warmup", type=int, default=16)
     parser.add_argument("--skip-extras", action="store_true")
+    parser.add_argument("--extras", default="gemm,attention,decode",
+                        help="comma-separated subset of gemm, attention, decode")
     parser.add_argument("--skip-cpu", action="store_true")
+    parser.add_argument("--decode-eager", action="store_true",
+                        help="launch the decode step from the host instead of replaying a HIP graph")
+    parser.add_argument("--pmc-probe", action="store_true",
+                        help="only the calibration copy and the headline GEMV, for rocprofv3 --pmc")
     args = parser.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this hot path has no multi-GPU part; run with --gpus 1")
 
     from llmopt_amd.native import Runtime
     runtime = Runtime()
+    if args.pmc_probe:
+        print(json.dumps(pmc_probe(runtime)))
+        runtime.close()
+        return
     gemv = bench_gemv(runtime, args.steps, args.warmup)
     headline = next(c for c in gemv["cases"] if (c["m"], c["k"], c["n"]) == (1, 4096, 14336))
     # the K steps replayed as one HIP graph, timed by HIP events on the launch stream
@@ -306,10 +353,13 @@ def main():
                   round(gemv["bytes_per_step"] / (gemv["ms_per_step"] * 1e-3) / 1e9, 1),
               "gemv_eager_host_launch_ms_per_step": round(gemv["ms_per_step"], 4),
               "device": runtime.device_name(), "seed": SEED}
-    if not args.skip_extras:
+    wanted = set() if args.skip_extras else set(filter(None, args.extras.split(",")))
+    if "gemm" in wanted:
         extras["prefill_gemm"] = bench_gemm(runtime)
+    if "attention" in wanted:
         extras["q8_attention"] = bench_attention(runtime)
-        extras["decode_step"] = bench_decode_step(runtime)
+    if "decode" in wanted:
+        extras["decode_step"] = bench_decode_step(runtime, use_graph=not args.decode_eager)
     line = {
         "metric": "W4A16 GEMV HBM GB/s (% peak); Q8 attn decode tokens/s; prefill MFMA %",
         "value": round(value, 1),
@@ -329,7 +379,7 @@ def main():
                    "bytes_per_step": gemv["bytes_per_step"]},
         "roofline": {"bound": "hbm", "kernel": "w4a16_gemv_kernel<M=1,R=4> at K=4096 N=14336",
                      "achieved": headline["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": headline["hbm_frac"], "traffic": None,
+                     "frac": headline["hbm_frac"], "traffic": measured_traffic(),
                      "bytes_per_launch": headline["bytes"], "us_per_launch": headline["us_per_launch"]},
         "cpu_baseline": None if args.skip_cpu else cpu_baseline(),
         "extras": extras,

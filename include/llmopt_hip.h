@@ -6,10 +6,9 @@
  * (`external ... = "caml_llmopt_metal_*"`, implemented for Apple GPUs in
  * native/ocaml_metal_stubs.m).  Every entry point below names the reference
  * symbol it stands in for.  The OCaml-value calling convention of the
- * reference is not part of this header: a thin CAMLprim shim (shown in
- * INTEGRATION.md) unpacks OCaml values, calls these functions and turns a
- * non-zero status into `Failure` / `Invalid_argument` carrying
- * llmopt_hip_last_error().
+ * reference is not part of this header: a thin CAMLprim shim unpacks OCaml
+ * values, calls these functions and turns a non-zero status into `Failure` /
+ * `Invalid_argument` carrying llmopt_hip_last_error().
  *
  * Conventions
  *  - Every function returns LLMOPT_OK (0) or a negative status; the message of
