@@ -61,9 +61,9 @@ def test_null_handles_are_rejected_not_dereferenced(library):
     status = library.llmopt_hip_has_function(None, b"llmopt_w4a16_linear_f16_g64")
     assert status < 0
     assert b"finalized" in library.llmopt_hip_last_error() or b"null" in library.llmopt_hip_last_error().lower()
-    library.llmopt_hip_buffer_length.argtypes = [ctypes.c_void_p, ctypes.POINTER(ctypes.c_uint64)]
-    length = ctypes.c_uint64(0)
-    assert library.llmopt_hip_buffer_length(None, ctypes.byref(length)) < 0
+    library.llmopt_hip_buffer_length.argtypes = [ctypes.c_void_p]
+    library.llmopt_hip_buffer_length.restype = ctypes.c_int64
+    assert library.llmopt_hip_buffer_length(None) < 0
     library.llmopt_hip_commit_batch.argtypes = [ctypes.c_void_p]
     assert library.llmopt_hip_commit_batch(None) < 0
 
