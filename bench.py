@@ -261,7 +261,7 @@ def bench_decode_step(runtime, batches=(1, 8, 32), context=2048, use_graph=True)
     return results
 
 
-def pmc_probe(runtime):
+def pmc_probe(runtime, m=1):
     """A short run for hardware counters (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE): four plain
     64 MiB device-to-device copies, whose bytes are known, then the headline GEMV (M = 1,
     K = 4096, N = 14336) over 16 distinct weight copies.  The copy calibrates the counters."""
@@ -272,16 +272,16 @@ def pmc_probe(runtime):
     for _ in range(4):
         source.copy_to(destination)
     k, n = 4096, 14336
-    x, packed, scale = w4_inputs(rng, 1, n, k)
-    bx, out = runtime.buffer_of_bytes(x), runtime.create_buffer(n * 2)
+    x, packed, scale = w4_inputs(rng, m, n, k)
+    bx, out = runtime.buffer_of_bytes(x), runtime.create_buffer(m * n * 2)
     weights = [(runtime.buffer_of_bytes(packed), runtime.buffer_of_bytes(scale)) for _ in range(COPIES)]
     batch = runtime.begin_batch()
     for bw, bs in weights:
-        record_linear(batch, 1, n, k, bx, bw, bs, out)
+        record_linear(batch, m, n, k, bx, bw, bs, out)
     batch.commit()
     return {"copy_kernel": "copy_vectors_kernel", "copy_bytes_read": copy_bytes, "copy_bytes_written": copy_bytes,
             "copy_launches": 4, "gemv_kernel": "w4a16_gemv_kernel<1, 2, 1, true, false>",
-            "gemv_launches": COPIES, "gemv_algorithmic_bytes": gemv_bytes(1, k, n)}
+            "gemv_rows": m, "gemv_launches": COPIES, "gemv_algorithmic_bytes": gemv_bytes(m, k, n)}
 
 
 def measured_traffic():
@@ -332,6 +332,7 @@ def main():
     parser.add_argument("--skip-cpu", action="store_true")
     parser.add_argument("--decode-eager", action="store_true",
                         help="launch the decode step from the host instead of replaying a HIP graph")
+    parser.add_argument("--pmc-rows", type=int, default=1, help="activation rows of the --pmc-probe GEMV")
     parser.add_argument("--pmc-probe", action="store_true",
                         help="only the calibration copy and the headline GEMV, for rocprofv3 --pmc")
     args = parser.parse_args()
@@ -341,7 +342,7 @@ def main():
     from llmopt_amd.native import Runtime
     runtime = Runtime()
     if args.pmc_probe:
-        print(json.dumps(pmc_probe(runtime)))
+        print(json.dumps(pmc_probe(runtime, args.pmc_rows)))
         runtime.close()
         return
     gemv = bench_gemv(runtime, args.steps, args.warmup)

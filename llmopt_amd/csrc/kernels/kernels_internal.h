@@ -14,6 +14,9 @@ hipError_t launch_w4a16_gemv_qkv(const W4QkvArgs &args, hipStream_t stream);
 hipError_t launch_w4a16_gemv_dual_swiglu(const W4DualSwigluArgs &args, hipStream_t stream);
 
 // kGemvDotRows < m <= kGemvMaxRows: matrix-core GEMV
+// true when K does not fit one workgroup (more than 16 ranges of 256): only the plain
+// linear can then run (it splits K over workgroups and needs scratch)
+bool w4a16_gemv_mfma_needs_split(uint32_t k);
 hipError_t launch_w4a16_gemv_mfma_linear(const W4LinearArgs &args, hipStream_t stream);
 hipError_t launch_w4a16_gemv_mfma_qkv(const W4QkvArgs &args, hipStream_t stream);
 hipError_t launch_w4a16_gemv_mfma_dual_swiglu(const W4DualSwigluArgs &args, hipStream_t stream);

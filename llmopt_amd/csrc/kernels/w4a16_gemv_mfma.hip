@@ -1,30 +1,39 @@
-// W4A16 decode GEMV for 1 <= M <= 8 activation rows on gfx950 with the
-// contraction on the matrix cores.
+// W4A16 decode GEMV for a few activation rows (M <= 8) on gfx950 with the
+// contraction on the matrix cores and the activation held in registers.
 //
-// One v_mfma_f32_16x16x32_f16 multiplies a 16(m) x 32(k) activation block with
-// a 32(k) x 16(n) weight block.  Lane (c = lane % 16, h = lane / 16) supplies
-// the B operand of weight row c: the 8 K values of dword j of the 16 bytes it
-// loaded at byte offset 16 h of a 128-wide K block.  Lanes h = 0,1 therefore
-// hold the first 64-wide scale group of the block and lanes h = 2,3 the second.
-// The activation is laid out block-diagonally: A rows 0..7 are x rows 0..7 for
-// K quarters 0,1 and zero for quarters 2,3, A rows 8..15 the other way round.
-// D rows 0..7 then hold the partial sums of the first scale group and rows
-// 8..15 those of the second, and the D registers of a lane (rows 4 h .. 4 h + 3,
-// column c) belong to exactly the scale group of the weights that lane loaded:
-// the fp16 group scale is one scalar per lane, applied in fp32 to the 4
-// accumulators.
+// Work split.  A wave owns one 256-wide K range for the whole kernel; the waves
+// of a workgroup cover the K extent (16 waves = 4096) and, when K is short,
+// several tiles side by side.  A workgroup walks tiles of 16 weight rows; per
+// tile a wave reads its 16 rows x 128 bytes, multiplies them with its own
+// activation fragment and leaves an 8 x 16 partial sum in LDS; the workgroup
+// adds the partial sums of its K ranges every few tiles.  K extents beyond one
+// workgroup are split over blockIdx.y: the slices leave fp32 partial sums in a
+// workspace and the last workgroup to arrive at a tile (an atomic counter per
+// tile) adds them in slice order.
 //
-// The nibbles are decoded to fp16 with a bias (q + 1032 or q + 72, one bit
-// operation per pair of nibbles).  The bias is removed by starting the MFMA
-// accumulation of a scale group from -(1032 sum x_even_pairs + 72 sum
-// x_odd_pairs), computed once per workgroup while the activation is staged to
-// LDS in the operand order of the decode.
+// Matrix operands.  One v_mfma_f32_16x16x32_f16 multiplies a 16(m) x 32(k)
+// activation block with a 32(k) x 16(n) weight block.  Lane (c = lane % 16,
+// h = lane / 16) supplies the B operand of weight row c: the 8 K values of
+// dword j of the 16-byte chunk h of a 64-byte half step.  Chunks 0,1 lie in one
+// 64-wide scale group, chunks 2,3 in the next, so the activation is laid out
+// block-diagonally: A rows 0..7 are x rows 0..7 for chunks 0,1 and zero for
+// chunks 2,3, A rows 8..15 the other way round.  D rows 0..7 / 8..15 are then
+// the partial sums of the two scale groups, and the 4 D registers of a lane
+// (rows 4h..4h+3, column c) belong to the scale group of the weights that lane
+// holds: the fp16 group scale is one scalar per lane, applied in fp32.
 //
-// A workgroup of 8 waves streams tiles of 16 weight rows; its waves split the
-// K range of the tile in steps of 256 and are reduced through LDS.  When M x K
-// does not fit the LDS budget the K range is split over blockIdx.y as well:
-// the slices leave fp32 partial sums in a workspace and the last workgroup to
-// arrive at a tile (an atomic counter per tile) adds them in slice order.
+// Loads.  In operand order a lane quad would touch four weight rows (four
+// cache lines) per load.  The loads therefore use a row-major lane order (lane
+// = 4 row + chunk: a quad reads 64 contiguous bytes) and four ds_bpermute_b32
+// per load move the dwords to the operand lanes; the scales travel the same way.
+// The activation fragment is requested first and then a ring of tiles, so that
+// all of a workgroup's weights are in flight from the start and a tile can be
+// multiplied as soon as it has arrived (loads return in order).
+//
+// Decode.  Nibbles become fp16 with a bias (q + 1032 or q + 72, one bit
+// operation per pair of nibbles); the bias is removed by starting every MFMA
+// chain from -(x . bias pattern), which one extra MFMA chain per wave computes
+// once from the resident activation fragment.
 //
 // Same arithmetic contract as llmopt_w4a16_linear_f16_g64{,_m4,_m8},
 // llmopt_w4a16_qkv_linear_f16_g64*, llmopt_w4a16_dual_swiglu_f16_g64* and
@@ -38,13 +47,11 @@
 namespace llmopt {
 namespace {
 
-constexpr int kWaves = 8;
-constexpr int kThreads = kWaves * 64;
-constexpr int TN = 16;        // weight rows per tile
-constexpr int kStepK = 256;   // K values one wave consumes per step
-constexpr int kZeroVectors = 20;  // per activation row: covers every operand offset of a step
-template <bool DUAL>
-constexpr int kReduceSlots = DUAL ? 1 : 2;  // DUAL keeps two sets of partial sums per tile
+constexpr int TN = 16;         // weight rows per tile
+constexpr int kStepK = 256;    // K values per wave
+constexpr int kMaxWaves = 16;  // per workgroup
+constexpr uint32_t kXRowBytes = 33 * 16;           // 32 pieces of 8 activation values + padding
+constexpr uint32_t kXStageBytes = 9 * kXRowBytes;  // per wave: 8 rows and a zero row
 
 struct MfmaMatrix {
   const uint8_t *w;
@@ -61,348 +68,322 @@ struct MfmaGemvParams {
   uint32_t has_addend;
   uint32_t addend_stride;
   uint32_t k_slice;    // K values per blockIdx.y slice, a multiple of 256
+  uint32_t waves_k;    // waves along K (each 256 wide)
+  uint32_t waves_t;    // tiles processed side by side
   float *partials;     // [gridDim.y][8][n] fp32, used when gridDim.y > 1
   uint32_t *counters;  // one per tile, zero between launches
   float *y_f32;        // optional float32 copy of mat0's output, may be null
 };
 
-// MP = activation rows held in LDS (1, 2, 4 or 8, >= m)
-template <int MP, bool DUAL>
-__global__ __launch_bounds__(kThreads) void w4a16_gemv_mfma_kernel(MfmaGemvParams p) {
+// NB = tiles in flight per wave (= tiles between two workgroup reductions)
+template <int NB, bool DUAL>
+__global__ __launch_bounds__(kMaxWaves * 64) void w4a16_gemv_mfma_kernel(MfmaGemvParams p) {
   constexpr int NW = DUAL ? 2 : 1;
-  constexpr int SPI = DUAL ? 1 : 2;      // steps per work item: 64 bytes per lane in flight per item
-  constexpr int RS = kReduceSlots<DUAL>;  // tiles finished between two workgroup reductions
-  extern __shared__ uint4 lds[];
+  extern __shared__ float red_lds[];  // partial sums [NB][waves_t][NW][waves_k][8][16] | flags | activation staging
 
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const uint32_t c = lane & 15;  // weight row of the tile (B column, D column)
-  const uint32_t h = lane >> 4;  // K quarter of the B operand; D rows 4h..4h+3
+  const uint32_t wk = wave % p.waves_k;  // K range of this wave
+  const uint32_t wt = wave / p.waves_k;  // tile lane of this wave
   const MfmaMatrix mat = DUAL ? p.mat0 : (blockIdx.z == 0 ? p.mat0 : blockIdx.z == 1 ? p.mat1 : p.mat2);
   const uint32_t tiles = (mat.n + TN - 1) / TN;
-  if (blockIdx.x >= tiles) return;  // a shorter matrix of a QKV launch (whole workgroup)
+  const uint32_t tile_groups = (tiles + p.waves_t - 1) / p.waves_t;
+  if (blockIdx.x >= tile_groups) return;  // a shorter matrix of a QKV launch (whole workgroup)
+  const uint32_t rounds = (tile_groups - blockIdx.x + gridDim.x - 1) / gridDim.x;
 
   const uint32_t K = p.k;
   const uint32_t groups_total = K >> 6;
-  const uint32_t k_begin = blockIdx.y * p.k_slice;
-  const uint32_t k_len = min(p.k_slice, K - k_begin);
-  const uint32_t groups = k_len >> 6;  // scale groups of this slice
-  const uint32_t steps = (k_len + kStepK - 1) / kStepK;
-  const uint32_t items_per_tile = (steps + kWaves * SPI - 1) / (kWaves * SPI);  // per wave
+  const uint32_t slice_end = min(K, (blockIdx.y + 1) * p.k_slice);
+  const uint32_t k0 = blockIdx.y * p.k_slice + wk * kStepK;  // first K value of this wave
+  const uint32_t valid_groups = k0 >= slice_end ? 0 : min(4u, (slice_end - k0) >> 6);
 
-  // LDS: zero vectors | x in operand order | -bias correction | wave partial sums | flags
-  const uint32_t x_vectors = steps * 32 * MP;
-  uint4 *x_lds = lds + kZeroVectors * MP;
-  float *corr_lds = reinterpret_cast<float *>(x_lds + x_vectors);  // [steps*4][8]
-  float *red_lds = corr_lds + steps * 4 * 8;                       // [RS][NW][waves][8][16]
-  uint32_t *flag_lds = reinterpret_cast<uint32_t *>(red_lds + RS * NW * kWaves * 8 * TN);  // [RS]
+  // ---- lane roles -----------------------------------------------------------------
+  // operand order: weight row c, chunk h
+  const uint32_t c = lane & 15, h = lane >> 4;
+  // load order: weight row lane / 4, chunk lane % 4 (a quad reads 64 contiguous bytes)
+  const uint32_t load_row = lane >> 2, load_chunk = lane & 3;
+  const uint32_t weight_source = (4 * c + h) * 4;  // byte address for ds_bpermute
 
-  struct Item {  // raw loaded registers only: conversions at the load would serialise the prefetch
-    u32x4_t w[NW][SPI][2];
-    uint16_t s[NW][SPI][2];
+  struct Raw {  // loaded-but-untouched registers of one tile
+    u32x4_t w[NW][2];
+    uint32_t s[NW];
   };
-  // item `index` of a tile covers steps (wave + index*kWaves)*SPI .. +SPI-1
-  // `real` = false is the prefetch past the last item: it stays unconditional
-  // (a skipped load would make the compiler wait for the whole load queue) but
-  // every lane reads the first 16 bytes of the matrix, one cache line per wave.
-  auto load_item = [&](uint32_t tile, uint32_t index, bool real, Item &out) __attribute__((always_inline)) {
-    const uint32_t row = min(tile * TN + c, mat.n - 1);
-    const uint32_t step0 = (wave + index * kWaves) * SPI;
+  // Loads that have nothing to fetch (past the last tile, a wave without K range)
+  // stay unconditional - a skipped load would make the compiler wait for the
+  // whole load queue - and read 16 bytes that are this wave's own, so the idle
+  // loads of different waves do not meet on one cache line.
+  const size_t idle_row = min(blockIdx.x * p.waves_t * TN, mat.n - 1);
+  const size_t idle_w_off = idle_row * (K >> 1) + (min(k0, K - 64) >> 1);
+  const size_t idle_s_off = idle_row * groups_total + (min(k0, K - 64) >> 6);
+  const uint32_t last_group = valid_groups > 0 ? valid_groups - 1 : 0;
+  auto load_tile = [&](uint32_t round, Raw &out) __attribute__((always_inline)) {
+    const uint32_t tile = (blockIdx.x + round * gridDim.x) * p.waves_t + wt;
+    // bitwise on purpose: short-circuit evaluation would turn the loads into branches
+    const bool real = (round < rounds) & (tile < tiles) & (valid_groups > 0);
+    const uint32_t row = min(tile * TN + load_row, mat.n - 1);
 #pragma unroll
-    for (int u = 0; u < SPI; ++u) {
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        // clamped past the end of the slice (the scale is zeroed when consumed)
-        const uint32_t g = min((step0 + u) * 4 + 2 * t + (h >> 1), groups - 1);
-        const size_t w_off = real ? (size_t)row * (K >> 1) + (k_begin >> 1) + g * 32 + (h & 1) * 16 : 0;
-        const size_t s_off = real ? (size_t)row * groups_total + (k_begin >> 6) + g : 0;
-        out.w[0][u][t] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(mat.w + w_off));
-        out.s[0][u][t] = mat.s[s_off];
-        if (DUAL) {
-          out.w[NW - 1][u][t] =
-              __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(p.mat1.w + w_off));
-          out.s[NW - 1][u][t] = p.mat1.s[s_off];
-        }
-      }
+    for (int t = 0; t < 2; ++t) {
+      const uint32_t g = min(2u * t + (load_chunk >> 1), last_group);  // clamped; its scale is zeroed later
+      const size_t w_off =
+          real ? (size_t)row * (K >> 1) + (k0 >> 1) + g * 32 + (load_chunk & 1) * 16 : idle_w_off + t * 16;
+      out.w[0][t] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(mat.w + w_off));
+      if (DUAL)
+        out.w[NW - 1][t] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(p.mat1.w + w_off));
     }
+    // scale of (row lane / 4, group lane % 4): a quad reads 8 contiguous bytes
+    const size_t s_off = real ? (size_t)row * groups_total + (k0 >> 6) + min(load_chunk, last_group) : idle_s_off;
+    out.s[0] = mat.s[s_off];
+    if (DUAL) out.s[NW - 1] = p.mat1.s[s_off];
   };
 
-  // first loads go out before the activation is staged
-  Item item_a, item_b;
-  load_item(blockIdx.x, 0, true, item_a);
-
-  // ---- stage x[:, k_begin .. k_begin + steps*256) and the bias correction ----
-  for (uint32_t i = threadIdx.x; i < kZeroVectors * MP; i += kThreads) lds[i] = make_uint4(0, 0, 0, 0);
+  // ---- activation fragment of this wave's K range, in registers ----------------------
+  // A operand of lane (row r = lane % 16, quarter h): x row r % 8 if the row half
+  // matches the chunk half, else zero.
+  // The 8 rows x 256 values are read row-major (half a wave reads 512 contiguous
+  // bytes of one row), rearranged into the decoder's pair order and passed through
+  // a wave-private LDS area (rows padded to 33 pieces: conflict-free 16-byte reads
+  // down the rows) to reach the operand lanes.  Row 8 of the area is zero: it serves
+  // the lanes off the block diagonal.
+  h8_t a_frag[2][4];
+  const uint32_t slot_floats = NW * p.waves_k * 8 * TN;  // partial sums of one tile
+  uint32_t *flag_lds = reinterpret_cast<uint32_t *>(red_lds + NB * p.waves_t * slot_floats);
+  uint8_t *x_stage = reinterpret_cast<uint8_t *>(flag_lds + ((NB * p.waves_t + 3) & ~3u)) + wave * kXStageBytes;
+  uint4 x_loaded[4];  // requested before the weights: loads return in order
+  const uint32_t x_piece = lane & 31;
   {
-    constexpr int UNROLL = 4;  // independent loads in flight per thread
-    const uint32_t padded = (x_vectors + 63) & ~63u;
-    for (uint32_t base = threadIdx.x; base < padded; base += kThreads * UNROLL) {
-      uint4 value[UNROLL];
 #pragma unroll
-      for (int u = 0; u < UNROLL; ++u) {
-        const uint32_t i = base + u * kThreads;
-        const uint32_t m = i & (MP - 1);
-        const uint32_t kb = i / MP;  // block of 8 K values within the slice
-        value[u] = make_uint4(0, 0, 0, 0);
-        if (m < p.m && kb * 8 < k_len)
-          value[u] = *reinterpret_cast<const uint4 *>(p.x + (size_t)m * K + k_begin + kb * 8);
-      }
-#pragma unroll
-      for (int u = 0; u < UNROLL; ++u) {
-        const uint32_t i = base + u * kThreads;
-        if (i >= padded) break;  // uniform per wave: padded is a multiple of 64
-        const uint32_t m = i & (MP - 1);
-        const uint32_t kb = i / MP;
-        const uint4 ordered = pair_order(value[u]);
-        if (i < x_vectors) x_lds[i] = ordered;
-        // pairs .x and .z meet weights decoded as q + 1032, pairs .y and .w as q + 72
-        const h2_t a = as_h2(ordered.x), b = as_h2(ordered.y), cc = as_h2(ordered.z), d = as_h2(ordered.w);
-        float bias = 1032.0f * (((float)a[0] + (float)a[1]) + ((float)cc[0] + (float)cc[1])) +
-                     72.0f * (((float)b[0] + (float)b[1]) + ((float)d[0] + (float)d[1]));
-        // the 8 blocks of a scale group sit MP lanes apart
-        bias += __shfl_xor(bias, MP);
-        bias += __shfl_xor(bias, 2 * MP);
-        bias += __shfl_xor(bias, 4 * MP);
-        if ((kb & 7) == 0 && i < x_vectors) corr_lds[(kb >> 3) * 8 + m] = -bias;
-      }
-    }
-    if (MP < 8) {
-      // rows MP..7 of the correction are read (their D rows are never used): keep them finite
-      for (uint32_t i = threadIdx.x; i < steps * 4 * 8; i += kThreads)
-        if ((i & 7) >= MP) corr_lds[i] = 0.0f;
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t row = 2 * i + (lane >> 5);
+      const uint32_t kk = k0 + x_piece * 8;
+      x_loaded[i] =
+          *reinterpret_cast<const uint4 *>(p.x + (size_t)min(row, p.m - 1) * K + min(kk, K - 8));
     }
   }
-  __syncthreads();
-
-  // operand addressing: lanes off the block diagonal read the zero vectors
-  const bool on_diagonal = (c >= 8) == (h >= 2);
-  const uint32_t m_of_lane = (c & 7) & (MP - 1);
-  const uint32_t a_base = on_diagonal ? (kZeroVectors + h * 4) * MP + m_of_lane : 0;  // in vectors
-  const uint32_t a_step = on_diagonal ? 32 * MP : 0;
-  const uint32_t corr_base = (h >> 1) * 8 + (h & 1) * 4;
-
-  f4_t acc[NW];
+  // all tiles of the ring go out next
+  Raw ring[NB];
 #pragma unroll
-  for (int v = 0; v < NW; ++v) acc[v] = f4_t{0.0f, 0.0f, 0.0f, 0.0f};
-
-  auto consume = [&](uint32_t index, const Item &cur) __attribute__((always_inline)) {
-    const uint32_t step0 = (wave + index * kWaves) * SPI;
+  for (int b = 0; b < NB; ++b) load_tile(b, ring[b]);
+  {
 #pragma unroll
-    for (int u = 0; u < SPI; ++u) {
-      const uint32_t step = step0 + u;
-      const uint32_t step_l = min(step, steps - 1);
-      const uint4 *a_ptr = lds + a_base + a_step * step_l;
-      const float *corr_ptr = corr_lds + corr_base + step_l * 32;
-#pragma unroll
-      for (int t = 0; t < 2; ++t) {
-        const bool ok = step * 4 + 2 * t + (h >> 1) < groups;
-        const f4_t start = *reinterpret_cast<const f4_t *>(corr_ptr + t * 16);
-        h8_t a_frag[4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j) a_frag[j] = __builtin_bit_cast(h8_t, a_ptr[(t * 16 + j) * MP]);
-#pragma unroll
-        for (int v = 0; v < NW; ++v) {
-          f4_t tile = start;
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const W4Pairs w = w4_decode_biased(cur.w[v][u][t][j]);
-            uint4 packed;
-            packed.x = as_u32(w.p04);
-            packed.y = as_u32(w.p15);
-            packed.z = as_u32(w.p26);
-            packed.w = as_u32(w.p37);
-            tile = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_frag[j], __builtin_bit_cast(h8_t, packed), tile, 0,
-                                                          0, 0);
-          }
-          const float scale = ok ? half_bits_to_float(cur.s[v][u][t]) : 0.0f;
-#pragma unroll
-          for (int i = 0; i < 4; ++i) acc[v][i] = fmaf(tile[i], scale, acc[v][i]);
-        }
-      }
+    for (int i = 0; i < 4; ++i) {
+      const uint32_t row = 2 * i + (lane >> 5);
+      const bool keep = (row < p.m) & (k0 + x_piece * 8 < slice_end);
+      const uint4 ordered = pair_order(x_loaded[i]);
+      uint4 value;
+      value.x = keep ? ordered.x : 0u;
+      value.y = keep ? ordered.y : 0u;
+      value.z = keep ? ordered.z : 0u;
+      value.w = keep ? ordered.w : 0u;
+      *reinterpret_cast<uint4 *>(x_stage + row * kXRowBytes + x_piece * 16) = value;
     }
-  };
+    if (lane < 33) *reinterpret_cast<uint4 *>(x_stage + 8 * kXRowBytes + lane * 16) = make_uint4(0, 0, 0, 0);
+    __builtin_amdgcn_wave_barrier();  // the LDS unit serves one wave's accesses in order
+    const bool on_diagonal = (c >= 8) == (h >= 2);
+    const uint8_t *mine = x_stage + (on_diagonal ? (c & 7) : 8) * kXRowBytes + (on_diagonal ? h * 64 : 0);
+#pragma unroll
+    for (int t = 0; t < 2; ++t)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        a_frag[t][j] = __builtin_bit_cast(h8_t, *reinterpret_cast<const uint4 *>(mine + (t * 16 + j) * 16));
+  }
+  // -(x . decode bias) per half step: pairs (k0,k4) and (k2,k6) carry 1032, (k1,k5) and (k3,k7) carry 72
+  f4_t start[2];
+  {
+    const h8_t bias = {(_Float16)1032.0f, (_Float16)1032.0f, (_Float16)72.0f, (_Float16)72.0f,
+                       (_Float16)1032.0f, (_Float16)1032.0f, (_Float16)72.0f, (_Float16)72.0f};
+#pragma unroll
+    for (int t = 0; t < 2; ++t) {
+      f4_t sum = f4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) sum = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_frag[t][j], bias, sum, 0, 0, 0);
+      start[t] = -sum;
+    }
+  }
 
-  // A finished tile leaves the wave's partial sums in a reduction slot; the
-  // workgroup reduces RS tiles at a time.
-  uint32_t pending = 0;        // tiles waiting in the slots (uniform)
-  uint32_t pending_first = 0;  // tile index of slot 0; slot s holds pending_first + s*gridDim.x
-  auto park_tile = [&](uint32_t tile) __attribute__((always_inline)) {
-    if (pending == 0) pending_first = tile;
-    float *slot = red_lds + pending * (NW * kWaves * 8 * TN);
-    // the two scale-group halves of a column sit 32 lanes apart
+  // Multiplies one tile by the fragment and leaves the wave's partial sums in reduction slot `slot`.
+  auto consume = [&](const Raw &raw, uint32_t slot) __attribute__((always_inline)) {
+    float *out = red_lds + (slot * p.waves_t + wt) * slot_floats;
 #pragma unroll
     for (int v = 0; v < NW; ++v) {
+      f4_t acc = f4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int t = 0; t < 2; ++t) {
+        uint32_t words[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          words[j] = (uint32_t)__builtin_amdgcn_ds_bpermute((int)weight_source, (int)raw.w[v][t][j]);
+        const uint32_t group = 2 * t + (h >> 1);
+        const uint32_t scale_bits =
+            (uint32_t)__builtin_amdgcn_ds_bpermute((int)((4 * c + group) * 4), (int)raw.s[v]);
+        f4_t tile = start[t];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const W4Pairs w = w4_decode_biased(words[j]);
+          uint4 packed;
+          packed.x = as_u32(w.p04);
+          packed.y = as_u32(w.p15);
+          packed.z = as_u32(w.p26);
+          packed.w = as_u32(w.p37);
+          tile = __builtin_amdgcn_mfma_f32_16x16x32_f16(a_frag[t][j], __builtin_bit_cast(h8_t, packed), tile, 0, 0, 0);
+        }
+        const float scale = group < valid_groups ? half_bits_to_float((uint16_t)scale_bits) : 0.0f;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[i] = fmaf(tile[i], scale, acc[i]);
+      }
+      // the two scale groups of a column sit 32 lanes apart
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const float total = acc[v][i] + __shfl_xor(acc[v][i], 32);
-        if (h < 2) slot[((v * kWaves + wave) * 8 + h * 4 + i) * TN + c] = total;
-        acc[v][i] = 0.0f;
+        const float total = acc[i] + __shfl_xor(acc[i], 32);
+        if (h < 2) out[((v * p.waves_k + wk) * 8 + h * 4 + i) * TN + c] = total;
       }
     }
-    ++pending;
   };
-  auto flush = [&]() __attribute__((always_inline)) {
+
+  // Adds the K ranges of the tiles parked in slots [0, count) and stores them.
+  auto flush = [&](uint32_t first_round, uint32_t count) __attribute__((always_inline)) {
     __syncthreads();
-    const uint32_t slot_index = threadIdx.x >> 7;  // 128 outputs per tile
-    const uint32_t in_slot = threadIdx.x & 127;
-    const uint32_t m = in_slot >> 4, col_in_tile = in_slot & 15;
-    const uint32_t tile = pending_first + slot_index * gridDim.x;
-    const uint32_t col = tile * TN + col_in_tile;
-    const bool active = slot_index < pending;
-    const bool writer = active && m < p.m && col < mat.n;
-    float total[NW];
-    if (active) {
-      const float *slot = red_lds + slot_index * (NW * kWaves * 8 * TN);
+    const uint32_t outputs = count * p.waves_t * 8 * TN;
+    const bool split = !DUAL && gridDim.y > 1;
+    for (uint32_t base = 0; base < outputs; base += blockDim.x) {  // uniform trip count
+      const uint32_t o = base + threadIdx.x;
+      const bool in_range = o < outputs;
+      const uint32_t slot_tile = o >> 7;  // slot * waves_t + tile lane
+      const uint32_t slot = slot_tile / p.waves_t, lane_t = slot_tile - slot * p.waves_t;
+      const uint32_t m = (o >> 4) & 7, col_in_tile = o & 15;
+      const uint32_t tile = (blockIdx.x + (first_round + slot) * gridDim.x) * p.waves_t + lane_t;
+      const uint32_t col = tile * TN + col_in_tile;
+      const bool writer = in_range && tile < tiles && m < p.m && col < mat.n;
+      float total[NW];
 #pragma unroll
-      for (int v = 0; v < NW; ++v) {
-        total[v] = 0.0f;
+      for (int v = 0; v < NW; ++v) total[v] = 0.0f;
+      if (in_range) {
+        const float *in = red_lds + slot_tile * slot_floats;
 #pragma unroll
-        for (int w = 0; w < kWaves; ++w) total[v] += slot[((v * kWaves + w) * 8 + m) * TN + col_in_tile];
+        for (int v = 0; v < NW; ++v)
+          for (uint32_t w = 0; w < p.waves_k; ++w) total[v] += in[((v * p.waves_k + w) * 8 + m) * TN + col_in_tile];
       }
-    }
-    bool store = writer;
-    if (!DUAL && gridDim.y > 1) {
-      // K split over workgroups: leave the partial sum where every CU sees it
-      // (device-scope stores and loads, no cache write-back needed); the last
-      // workgroup to arrive at a tile adds the slices in order.
-      if (writer)
-        __hip_atomic_store(p.partials + ((size_t)blockIdx.y * 8 + m) * mat.n + col, total[0], __ATOMIC_RELAXED,
-                           __HIP_MEMORY_SCOPE_AGENT);
-      __syncthreads();  // waits for the stores of every wave
-      if (active && in_slot == 0) {
-        const uint32_t arrived =
-            __hip_atomic_fetch_add(p.counters + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        const bool last = arrived == gridDim.y - 1;
-        if (last) __hip_atomic_store(p.counters + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        flag_lds[slot_index] = last ? 1u : 0u;
+      bool store = writer;
+      if (split) {
+        // K split over workgroups: leave the partial sum where every CU sees it
+        // (device-scope stores and loads, no cache write-back needed); the last
+        // workgroup to arrive at a tile adds the slices in order.
+        if (writer)
+          __hip_atomic_store(p.partials + ((size_t)blockIdx.y * 8 + m) * mat.n + col, total[0], __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_AGENT);
+        __syncthreads();  // waits for the stores of every wave
+        if (in_range && (o & 127) == 0 && tile < tiles) {
+          const uint32_t arrived =
+              __hip_atomic_fetch_add(p.counters + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          const bool last = arrived == gridDim.y - 1;
+          if (last) __hip_atomic_store(p.counters + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+          flag_lds[slot_tile] = last ? 1u : 0u;
+        }
+        __syncthreads();
+        store = writer && flag_lds[slot_tile] != 0;
+        if (store) {
+          float sum = 0.0f;
+          for (uint32_t slice = 0; slice < gridDim.y; ++slice)
+            sum += __hip_atomic_load(p.partials + ((size_t)slice * 8 + m) * mat.n + col, __ATOMIC_RELAXED,
+                                     __HIP_MEMORY_SCOPE_AGENT);
+          total[0] = sum;
+        }
+        __syncthreads();  // the flags are free again
       }
-      __syncthreads();
-      store = writer && flag_lds[slot_index] != 0;
       if (store) {
-        float sum = 0.0f;
-        for (uint32_t slice = 0; slice < gridDim.y; ++slice)
-          sum += __hip_atomic_load(p.partials + ((size_t)slice * 8 + m) * mat.n + col, __ATOMIC_RELAXED,
-                                   __HIP_MEMORY_SCOPE_AGENT);
-        total[0] = sum;
+        float value;
+        if (DUAL) {
+          value = total[0] / (1.0f + __expf(-total[0])) * total[NW - 1];
+        } else {
+          value = total[0];
+          if (p.has_addend) value += half_bits_to_float(p.addend[(size_t)m * p.addend_stride + col]);
+        }
+        if (mat.y != nullptr) mat.y[(size_t)m * mat.n + col] = float_to_half_bits(value);
+        if (!DUAL && p.y_f32 != nullptr) p.y_f32[(size_t)m * mat.n + col] = value;
       }
-    }
-    if (store) {
-      float value;
-      if (DUAL) {
-        value = total[0] / (1.0f + __expf(-total[0])) * total[NW - 1];
-      } else {
-        value = total[0];
-        if (p.has_addend) value += half_bits_to_float(p.addend[(size_t)m * p.addend_stride + col]);
-      }
-      if (mat.y != nullptr) mat.y[(size_t)m * mat.n + col] = float_to_half_bits(value);
-      if (!DUAL && p.y_f32 != nullptr) p.y_f32[(size_t)m * mat.n + col] = value;
     }
     __syncthreads();  // the slots are free again
-    pending = 0;
   };
 
-  // Items of this wave: for each tile of the workgroup, items 0 .. items_per_tile-1.
-  // Ping-pong between two register sets with an unconditional prefetch.
-  auto advance = [&](uint32_t &tile, uint32_t &index) {
-    if (++index == items_per_tile) {
-      index = 0;
-      tile += gridDim.x;
+  // ---- tiles: NB per pass, each buffer refilled as soon as it has been consumed ------
+  for (uint32_t first = 0; first < rounds; first += NB) {
+    const bool refill = first + NB < rounds;  // nothing is loaded after the last pass
+#pragma unroll
+    for (int b = 0; b < NB; ++b) {
+      consume(ring[b], b);
+      if (refill) load_tile(first + NB + b, ring[b]);
     }
-  };
-  uint32_t tile = blockIdx.x, index = 0;
-  while (true) {
-    uint32_t next_tile = tile, next_index = index;
-    advance(next_tile, next_index);
-    bool more = next_tile < tiles;
-    load_item(next_tile, next_index, more, item_b);
-    consume(index, item_a);
-    if (index == items_per_tile - 1) {
-      park_tile(tile);
-      if (pending == RS || !more) flush();
-    }
-    if (!more) break;
-    tile = next_tile;
-    index = next_index;
-    advance(next_tile, next_index);
-    more = next_tile < tiles;
-    load_item(next_tile, next_index, more, item_a);
-    consume(index, item_b);
-    if (index == items_per_tile - 1) {
-      park_tile(tile);
-      if (pending == RS || !more) flush();
-    }
-    if (!more) break;
-    tile = next_tile;
-    index = next_index;
+    flush(first, min((uint32_t)NB, rounds - first));
   }
-}
-
-constexpr size_t kLdsBudget = 79 * 1024;  // two workgroups per CU (160 KB)
-
-size_t lds_bytes_for(uint32_t mp, uint32_t steps, int nw) {
-  const int slots = nw == 2 ? kReduceSlots<true> : kReduceSlots<false>;
-  return (size_t)(kZeroVectors * mp + steps * 32 * mp) * 16 + (size_t)steps * 4 * 8 * 4 +
-         (size_t)slots * nw * kWaves * 8 * TN * 4 + 16;
 }
 
 struct Plan {
-  uint32_t mp, slices, k_slice;
+  uint32_t slices, k_slice, waves_k, waves_t, blocks, ring;
   size_t lds_bytes;
 };
 
-Plan make_plan(uint32_t m, uint32_t k, int nw, bool may_split) {
+Plan make_plan(uint32_t k, uint32_t max_n, uint32_t matrices, bool dual) {
   Plan plan;
-  plan.mp = m <= 1 ? 1 : m <= 2 ? 2 : m <= 4 ? 4 : 8;
   const uint32_t steps_total = (k + kStepK - 1) / kStepK;
-  plan.slices = 1;
-  if (may_split) {
-    while (plan.slices < steps_total &&
-           lds_bytes_for(plan.mp, (steps_total + plan.slices - 1) / plan.slices, nw) > kLdsBudget)
-      ++plan.slices;
-  }
-  const uint32_t steps = (steps_total + plan.slices - 1) / plan.slices;
-  plan.k_slice = steps * kStepK;
+  plan.slices = (steps_total + kMaxWaves - 1) / kMaxWaves;
+  plan.waves_k = (steps_total + plan.slices - 1) / plan.slices;
+  plan.k_slice = plan.waves_k * kStepK;
   plan.slices = (k + plan.k_slice - 1) / plan.k_slice;
-  plan.lds_bytes = lds_bytes_for(plan.mp, steps, nw);
+  const uint32_t tiles = (max_n + TN - 1) / TN;
+  const uint32_t cus = (uint32_t)device_compute_units();
+  // short K: several tiles side by side in one workgroup, once there are more tiles than CUs
+  const uint32_t room = std::max<uint32_t>(1, kMaxWaves / plan.waves_k);
+  plan.waves_t = std::max<uint32_t>(1, std::min<uint32_t>(room, tiles * plan.slices * matrices / cus));
+  const uint32_t tile_groups = (tiles + plan.waves_t - 1) / plan.waves_t;
+  const uint32_t waves = plan.waves_k * plan.waves_t;
+  const uint32_t per_cu = waves <= 4 ? 4 : waves <= 8 ? 2 : 1;
+  const uint32_t resident = std::max<uint32_t>(1, cus * per_cu / (plan.slices * matrices));
+  plan.blocks = std::min(tile_groups, resident);
+  // tiles in flight per wave: all of a workgroup's tiles when they are few
+  const uint32_t rounds = (tile_groups + plan.blocks - 1) / plan.blocks;
+  plan.ring = rounds <= 1 ? 1 : (rounds <= 2 || dual) ? 2 : 4;
+  const int nw = dual ? 2 : 1;
+  plan.lds_bytes = (size_t)plan.ring * plan.waves_t * nw * plan.waves_k * 8 * TN * sizeof(float) +
+                   (size_t)((plan.ring * plan.waves_t + 3) & ~3u) * sizeof(uint32_t) + (size_t)waves * kXStageBytes;
   return plan;
 }
 
-template <int MP, bool DUAL>
-hipError_t launch_instance(const MfmaGemvParams &p, dim3 grid, size_t lds_bytes, hipStream_t stream) {
-  static bool configured = false;  // per instantiation; the attribute is per device function
+template <int NB, bool DUAL>
+hipError_t launch_ring(const MfmaGemvParams &p, uint32_t matrices, const Plan &plan, hipStream_t stream) {
+  static bool configured = false;  // the attribute is per device function
   if (!configured) {
-    hipError_t status = hipFuncSetAttribute(
-        reinterpret_cast<const void *>(&w4a16_gemv_mfma_kernel<MP, DUAL>),
-        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(&w4a16_gemv_mfma_kernel<NB, DUAL>),
+                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     if (status != hipSuccess) return status;
     configured = true;
   }
-  hipLaunchKernelGGL((w4a16_gemv_mfma_kernel<MP, DUAL>), grid, dim3(kThreads), lds_bytes, stream, p);
+  const dim3 grid(plan.blocks, plan.slices, matrices);
+  hipLaunchKernelGGL((w4a16_gemv_mfma_kernel<NB, DUAL>), grid, dim3(plan.waves_k * plan.waves_t * 64),
+                     plan.lds_bytes, stream, p);
   return hipGetLastError();
 }
 
 template <bool DUAL>
-hipError_t launch(MfmaGemvParams p, uint32_t matrices, uint32_t max_n, const Plan &plan, hipStream_t stream) {
+hipError_t launch(MfmaGemvParams p, uint32_t matrices, const Plan &plan, hipStream_t stream) {
   p.k_slice = plan.k_slice;
-  const uint32_t tiles = (max_n + TN - 1) / TN;
-  const uint32_t per_cu = plan.lds_bytes <= kLdsBudget ? 2 : 1;
-  const uint32_t resident = (uint32_t)device_compute_units() * per_cu;
-  const uint32_t blocks = std::max<uint32_t>(1, std::min<uint32_t>(tiles, resident / (plan.slices * matrices)));
-  const dim3 grid(blocks, plan.slices, matrices);
-  switch (plan.mp) {
-    case 1: return launch_instance<1, DUAL>(p, grid, plan.lds_bytes, stream);
-    case 2: return launch_instance<2, DUAL>(p, grid, plan.lds_bytes, stream);
-    case 4: return launch_instance<4, DUAL>(p, grid, plan.lds_bytes, stream);
-    default: return launch_instance<8, DUAL>(p, grid, plan.lds_bytes, stream);
-  }
+  p.waves_k = plan.waves_k;
+  p.waves_t = plan.waves_t;
+  if (plan.lds_bytes > 160 * 1024) return hipErrorInvalidValue;
+  if (plan.ring == 1) return launch_ring<1, DUAL>(p, matrices, plan, stream);
+  if (plan.ring == 2) return launch_ring<2, DUAL>(p, matrices, plan, stream);
+  if constexpr (DUAL) return hipErrorInvalidValue;
+  else return launch_ring<4, false>(p, matrices, plan, stream);
 }
 
 }  // namespace
 
 size_t w4a16_gemv_workspace_bytes(uint32_t m, uint32_t n, uint32_t k) {
-  const Plan plan = make_plan(m, k, 1, true);
-  return plan.slices > 1 ? (size_t)plan.slices * 8 * n * sizeof(float) : 0;
+  (void)m;
+  const uint32_t steps_total = (k + kStepK - 1) / kStepK;
+  const uint32_t slices = (steps_total + kMaxWaves - 1) / kMaxWaves;
+  return slices > 1 ? (size_t)slices * 8 * n * sizeof(float) : 0;
 }
+
+bool w4a16_gemv_mfma_needs_split(uint32_t k) { return (k + kStepK - 1) / kStepK > (uint32_t)kMaxWaves; }
 
 hipError_t launch_w4a16_gemv_mfma_linear(const W4LinearArgs &a, hipStream_t stream) {
   MfmaGemvParams p = {};
@@ -415,15 +396,17 @@ hipError_t launch_w4a16_gemv_mfma_linear(const W4LinearArgs &a, hipStream_t stre
   p.addend = a.addend;
   p.has_addend = a.has_addend;
   p.addend_stride = a.addend_row_stride;
-  const uint32_t tiles = (a.n + TN - 1) / TN;
-  const bool may_split = a.workspace != nullptr && a.counters != nullptr && tiles <= a.counter_count &&
-                         a.workspace_bytes >= w4a16_gemv_workspace_bytes(a.m, a.n, a.k);
-  const Plan plan = make_plan(a.m, a.k, 1, may_split);
-  if (plan.lds_bytes > 160 * 1024) return hipErrorInvalidValue;
+  const Plan plan = make_plan(a.k, a.n, 1, false);
+  if (plan.slices > 1) {
+    const uint32_t tiles = (a.n + TN - 1) / TN;
+    if (a.workspace == nullptr || a.counters == nullptr || tiles > a.counter_count ||
+        a.workspace_bytes < w4a16_gemv_workspace_bytes(a.m, a.n, a.k))
+      return hipErrorInvalidValue;
+  }
   p.partials = static_cast<float *>(a.workspace);
   p.counters = a.counters;
   p.y_f32 = a.y_f32;
-  return launch<false>(p, 1, a.n, plan, stream);
+  return launch<false>(p, 1, plan, stream);
 }
 
 hipError_t launch_w4a16_gemv_mfma_qkv(const W4QkvArgs &a, hipStream_t stream) {
@@ -434,9 +417,9 @@ hipError_t launch_w4a16_gemv_mfma_qkv(const W4QkvArgs &a, hipStream_t stream) {
   p.mat0 = {a.w[0].weight, a.w[0].scale, a.y[0], a.n[0]};
   p.mat1 = {a.w[1].weight, a.w[1].scale, a.y[1], a.n[1]};
   p.mat2 = {a.w[2].weight, a.w[2].scale, a.y[2], a.n[2]};
-  const Plan plan = make_plan(a.m, a.k, 1, false);
-  if (plan.lds_bytes > 160 * 1024) return hipErrorInvalidValue;
-  return launch<false>(p, 3, std::max(a.n[0], std::max(a.n[1], a.n[2])), plan, stream);
+  const Plan plan = make_plan(a.k, std::max(a.n[0], std::max(a.n[1], a.n[2])), 3, false);
+  if (plan.slices > 1) return hipErrorInvalidValue;  // callers check w4a16_gemv_mfma_needs_split
+  return launch<false>(p, 3, plan, stream);
 }
 
 hipError_t launch_w4a16_gemv_mfma_dual_swiglu(const W4DualSwigluArgs &a, hipStream_t stream) {
@@ -447,9 +430,9 @@ hipError_t launch_w4a16_gemv_mfma_dual_swiglu(const W4DualSwigluArgs &a, hipStre
   p.mat0 = {a.gate.weight, a.gate.scale, a.product, a.n};
   p.mat1 = {a.up.weight, a.up.scale, a.product, a.n};
   p.mat2 = p.mat0;
-  const Plan plan = make_plan(a.m, a.k, 2, false);
-  if (plan.lds_bytes > 160 * 1024) return hipErrorInvalidValue;
-  return launch<true>(p, 1, a.n, plan, stream);
+  const Plan plan = make_plan(a.k, a.n, 1, true);
+  if (plan.slices > 1) return hipErrorInvalidValue;
+  return launch<true>(p, 1, plan, stream);
 }
 
 }  // namespace llmopt
