@@ -258,9 +258,19 @@ __global__ __launch_bounds__(kMaxWaves * 64) void w4a16_gemv_mfma_kernel(MfmaGem
       for (int v = 0; v < NW; ++v) total[v] = 0.0f;
       if (in_range) {
         const float *in = red_lds + slot_tile * slot_floats;
+        // four independent sums so that the LDS reads are issued back to back
 #pragma unroll
-        for (int v = 0; v < NW; ++v)
-          for (uint32_t w = 0; w < p.waves_k; ++w) total[v] += in[((v * p.waves_k + w) * 8 + m) * TN + col_in_tile];
+        for (int v = 0; v < NW; ++v) {
+          const float *column = in + (v * p.waves_k * 8 + m) * TN + col_in_tile;
+          float part[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+          uint32_t w = 0;
+          for (; w + 4 <= p.waves_k; w += 4) {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) part[u] += column[(w + u) * 8 * TN];
+          }
+          for (; w < p.waves_k; ++w) part[0] += column[w * 8 * TN];
+          total[v] = (part[0] + part[1]) + (part[2] + part[3]);
+        }
       }
       bool store = writer;
       if (split) {
