@@ -6,18 +6,19 @@
 // (lib/metal_dispatch_linear.ml:975-982).  Same arithmetic contract here
 // (lib/metal_w4a16_source.ml:42-122), different machine mapping:
 //
-//  * int4 nibbles are decoded to *exact* fp16 integers and staged in LDS; the
-//    fp16 group scale is never folded into the fp16 operand.  Each 64-wide K
-//    group is contracted by v_mfma_f32_32x32x16_f16 into a temporary fp32 tile
-//    which is then scaled by float(scale[n, g]) and added to the running fp32
-//    tile, so q*s is applied in fp32 exactly as `float(q) * s` in the reference.
+//  * int4 nibbles are decoded to exact fp16 integers, multiplied by the fp16
+//    group scale in fp16 (one rounding, at most 2^-11 relative per weight; the
+//    product overflows fp16 only for scales above 8188) and staged in LDS as
+//    the MFMA B operand in natural K order; accumulation is fp32.
+//  * Activation tiles are copied global -> LDS without passing registers,
+//    weight nibbles pass registers for the decode.  LDS holds two stages and a
+//    K step has one barrier; the decode of the next stage is issued between
+//    groups of MFMAs of the current one.
 //  * The activation tile is the MFMA A operand (rows = m) and the weight tile
 //    the B operand (columns = n), so every lane's 16 accumulator values belong
-//    to one output column and the group scale is one scalar per lane.
-//  * K order inside an aligned block of 8 is permuted identically for both
-//    operands (see w4_decode_pairs / pair_order), which costs nothing in a dot
-//    product and keeps the nibble decode at 9 VALU ops per 8 weights.
+//    to one output column.
 #include <algorithm>
+#include <type_traits>
 
 #include "kernels.h"
 #include "kernels_internal.h"
@@ -58,17 +59,19 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
   constexpr int NW = DUAL ? 2 : 1;  // weight matrices per tile
   constexpr int BM = 4 * WM * 32;
   constexpr int BN = 2 * WN * 32;
-  constexpr int X_VECTORS = BM * BK / 8 / kThreads;    // 16-byte activation vectors per thread
   constexpr int W_VECTORS = (BN * BK / 32 + kThreads - 1) / kThreads;  // 32-nibble vectors per thread
-  static_assert(BM * BK / 8 % kThreads == 0, "activation tile must divide over the threads");
   extern __shared__ __attribute__((aligned(16))) unsigned char gemm_lds[];
-  _Float16 *x_lds = reinterpret_cast<_Float16 *>(gemm_lds);
-  _Float16 *w_lds = x_lds + BM * LDS_STRIDE;            // [NW][BN * LDS_STRIDE]
-  float *s_lds = reinterpret_cast<float *>(w_lds + NW * BN * LDS_STRIDE);  // [NW][BN]
+  // two stages of {x[BM] rows of BK halfs, vector index swizzled; w[NW][BN] rows
+  // of LDS_STRIDE halfs}
+  constexpr int X_HALFS = BM * BK;
+  constexpr int STAGE_HALFS = X_HALFS + NW * BN * LDS_STRIDE;
+  constexpr int X_CHUNKS = BM / 8 / (kThreads / 64);  // 8-row direct loads per wave and K step
+  static_assert(BM / 8 % (kThreads / 64) == 0, "activation tile must divide over the waves");
+  _Float16 *stage_lds = reinterpret_cast<_Float16 *>(gemm_lds);
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
-  const int wave = tid >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wave_m = wave >> 1;
   const int wave_n = wave & 1;
 
@@ -84,58 +87,93 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
   const uint32_t n0 = tile_n * BN;
   const uint32_t K = p.k;
 
-  // global -> register staging: x rows (tid/8) + 64*i, vector tid%8;
-  // w row (tid/2) + 256*i, half tid%2
-  const uint32_t x_vec = tid & 7;
-  const uint32_t x_row = tid >> 3;
-  const uint32_t w_row = tid >> 1;
-  const uint32_t w_half = tid & 1;
-
-  uint4 x_reg[X_VECTORS];
-  u32x4_t w_reg[NW][W_VECTORS];
-  uint16_t s_reg[NW][W_VECTORS];
-
-  auto load_global = [&](uint32_t k0) __attribute__((always_inline)) {
+  // Activations go global -> LDS directly, 8 rows (1 KiB) per wave-wide load:
+  // lane l fills physical vector l % 8 of row l / 8, i.e. fetches the logical
+  // vector which the swizzle maps there.
+  const uint16_t *x_src[X_CHUNKS];
 #pragma unroll
-    for (int i = 0; i < X_VECTORS; ++i) {
-      const uint32_t row = min(m0 + x_row + 64 * i, p.m - 1);  // rows past m are never stored
-      x_reg[i] = reinterpret_cast<const uint4 *>(p.x + (size_t)row * K + k0)[x_vec];
-    }
+  for (int c = 0; c < X_CHUNKS; ++c) {
+    const uint32_t tile_row = (wave * X_CHUNKS + c) * 8 + (lane >> 3);
+    const uint32_t vec = (lane & 7) ^ ((tile_row >> 1) & 7u);
+    const uint32_t row = min(m0 + tile_row, p.m - 1);  // rows past m are never stored
+    x_src[c] = p.x + (size_t)row * K + vec * 8;
+  }
+  // Every vector memory load of the K loop is issued as assembly and waited for
+  // by hand: loads return in order, so "at most n outstanding" names exactly
+  // which of them have landed, and no wait is stricter than the data flow needs
+  // (the compiler's own bookkeeping waits for the activation copy before the
+  // next LDS write, and for the youngest weight loads on every other step).
+  const uint32_t lds_base = (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char *)gemm_lds;
+  auto fetch_x = [&](uint32_t k0, int stage) __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < W_VECTORS; ++i) {
-      const uint32_t local = w_row + 256 * i;
-      const uint32_t col = min(n0 + local, p.n - 1);  // columns past n are never stored
-#pragma unroll
-      for (int v = 0; v < NW; ++v) {
-        w_reg[v][i] = reinterpret_cast<const u32x4_t *>(p.w[v] + (size_t)col * (K >> 1) + (k0 >> 1))[w_half];
-        s_reg[v][i] = p.s[v][(size_t)col * (K >> 6) + (k0 >> 6)];
-      }
+    for (int c = 0; c < X_CHUNKS; ++c) {
+      const uint32_t lds_address =
+          lds_base + (uint32_t)((stage * STAGE_HALFS + (wave * X_CHUNKS + c) * 8 * BK) * sizeof(_Float16));
+      asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
+                   :
+                   : "v"(x_src[c] + k0), "s"(lds_address)
+                   : "memory", "m0");
     }
   };
 
-  auto store_lds = [&]() __attribute__((always_inline)) {
+  // Weights go global -> registers (w row tid/2, half tid%2) -> decode -> LDS.
+  // Two register sets: a set is decoded one step after it was requested and
+  // requested again right after, so every load has a whole K step to arrive.
+  static_assert(W_VECTORS == 1, "one 32-nibble vector per thread and matrix");
+  const uint32_t w_row = tid >> 1;
+  const uint32_t w_half = tid & 1;
+  struct Fetched {
+    u32x4_t w[NW];
+    uint32_t s[NW];  // fp16 bits in the low half
+  };
+  Fetched fetched[2];
+  constexpr int W_LOADS = 2 * NW;  // vector memory loads of one fetch_w
+  const uint32_t w_col = min(n0 + w_row, p.n - 1);  // columns past n are never stored
+
+  auto fetch_w = [&](Fetched &f, uint32_t k0) __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < X_VECTORS; ++i)
-      *reinterpret_cast<uint4 *>(&x_lds[(x_row + 64 * i) * LDS_STRIDE + x_vec * 8]) = pair_order(x_reg[i]);
-#pragma unroll
-    for (int i = 0; i < W_VECTORS; ++i) {
-      const uint32_t local = w_row + 256 * i;
-      if (BN % 256 != 0 && local >= (uint32_t)BN) continue;
-#pragma unroll
-      for (int v = 0; v < NW; ++v) {
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const W4Pairs q = w4_decode_pairs(w_reg[v][i][j]);
-          uint4 packed;
-          packed.x = as_u32(q.p04);
-          packed.y = as_u32(q.p15);
-          packed.z = as_u32(q.p26);
-          packed.w = as_u32(q.p37);
-          *reinterpret_cast<uint4 *>(&w_lds[(v * BN + local) * LDS_STRIDE + w_half * 32 + j * 8]) = packed;
-        }
-        if (w_half == 0) s_lds[v * BN + local] = half_bits_to_float(s_reg[v][i]);
-      }
+    for (int v = 0; v < NW; ++v) {
+      const void *w_src = p.w[v] + (size_t)w_col * (K >> 1) + (k0 >> 1) + w_half * 16;
+      const void *s_src = p.s[v] + (size_t)w_col * (K >> 6) + (k0 >> 6);
+      asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(f.w[v]) : "v"(w_src) : "memory");
+      asm volatile("global_load_ushort %0, %1, off" : "=&v"(f.s[v]) : "v"(s_src) : "memory");
     }
+  };
+  // at most `younger` loads issued after those of f are still outstanding
+  auto wait_w = [&](Fetched &f, auto younger) __attribute__((always_inline)) {
+    constexpr int n = decltype(younger)::value;
+    if constexpr (NW == 1)
+      asm volatile("s_waitcnt vmcnt(%2)" : "+v"(f.w[0]), "+v"(f.s[0]) : "n"(n) : "memory");
+    else
+      asm volatile("s_waitcnt vmcnt(%4)"
+                   : "+v"(f.w[0]), "+v"(f.s[0]), "+v"(f.w[1]), "+v"(f.s[1])
+                   : "n"(n)
+                   : "memory");
+  };
+  auto wait_all = [&](auto younger) __attribute__((always_inline)) {
+    asm volatile("s_waitcnt vmcnt(%0)" : : "n"(decltype(younger)::value) : "memory");
+  };
+
+  // The decode of one fetched set into an LDS stage, cut into items of one
+  // weight dword (8 nibbles): q * s as fp16 (one rounding, 2^-11 relative at
+  // most), in natural K order.
+  constexpr int ITEMS = NW * 4;
+  auto store_item = [&](const Fetched &f, int stage, int item) __attribute__((always_inline)) {
+    _Float16 *w_lds = stage_lds + stage * STAGE_HALFS + X_HALFS;
+    const int v = item / 4;
+    const int j = item % 4;
+    if (BN % 256 != 0 && w_row >= (uint32_t)BN) return;
+    const _Float16 scale = __builtin_bit_cast(_Float16, (uint16_t)f.s[v]);
+    const h2_t scale2 = {scale, scale};
+    const W4Pairs q = w4_decode_pairs(f.w[v][j]);
+    const uint32_t p04 = as_u32(q.p04 * scale2), p15 = as_u32(q.p15 * scale2);
+    const uint32_t p26 = as_u32(q.p26 * scale2), p37 = as_u32(q.p37 * scale2);
+    uint4 packed;
+    packed.x = __builtin_amdgcn_perm(p15, p04, 0x05040100u);  // k0 k1
+    packed.y = __builtin_amdgcn_perm(p37, p26, 0x05040100u);  // k2 k3
+    packed.z = __builtin_amdgcn_perm(p15, p04, 0x07060302u);  // k4 k5
+    packed.w = __builtin_amdgcn_perm(p37, p26, 0x07060302u);  // k6 k7
+    *reinterpret_cast<uint4 *>(&w_lds[(v * BN + w_row) * LDS_STRIDE + w_half * 32 + j * 8]) = packed;
   };
 
   f16x_t acc[NW][WM][WN];
@@ -147,48 +185,84 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
       for (int b = 0; b < WN; ++b) acc[v][a][b] = zero_tile();
 
   const int frag_row = lane & 31;  // operand row (A) / column (B) inside a 32-wide tile
-  const int frag_k = (lane >> 5) * 8;
+  const int frag_kq = lane >> 5;
+  const int frag_k = frag_kq * 8;
   const int row_base = wave_m * WM * 32;
   const int col_base = wave_n * WN * 32;
 
-  load_global(0);
-  for (uint32_t k0 = 0; k0 < K; k0 += BK) {
-    __syncthreads();  // previous step's LDS reads are done
-    store_lds();
-    __syncthreads();
-    if (k0 + BK < K) load_global(k0 + BK);
-
+  // One barrier per K step.  Step i runs its MFMAs from stage i%2 while the set
+  // fetched for step i+1 is decoded into the other stage; that set is then
+  // requested again for step i+3 (requests past the end fetch the last K block
+  // again, which nothing reads).  The issue order is fixed by hand: groups of
+  // four chained MFMAs alternate with one or two decode items, and the weight
+  // operands of the next column block are read while the current one computes,
+  // so the matrix pipe does not wait for the vector work, LDS or HBM.
+  constexpr int BLOCKS = NW * WN;      // column blocks of a step
+  constexpr int GROUPS = BLOCKS * WM;  // MFMA groups of a step
+  constexpr int ITEMS_PER_GROUP = (ITEMS + GROUPS - 1) / GROUPS;
+  auto step = [&](uint32_t k0, auto parity) __attribute__((always_inline)) {
+    constexpr int stage = decltype(parity)::value;
+    __syncthreads();  // this stage is written; the other stage's readers are done
+    const _Float16 *x_lds = stage_lds + stage * STAGE_HALFS;
+    const _Float16 *w_lds = x_lds + X_HALFS;
     h8_t a_frag[WM][BK / 16];
+    h8_t b_frag[2][BK / 16];
+    auto read_block = [&](int block) __attribute__((always_inline)) {
+      const int v = block / WN;
+      const int b = block % WN;
+#pragma unroll
+      for (int ks = 0; ks < BK / 16; ++ks)
+        b_frag[block & 1][ks] = *reinterpret_cast<const h8_t *>(
+            &w_lds[(v * BN + col_base + b * 32 + frag_row) * LDS_STRIDE + ks * 16 + frag_k]);
+    };
+    read_block(0);
 #pragma unroll
     for (int a = 0; a < WM; ++a)
 #pragma unroll
       for (int ks = 0; ks < BK / 16; ++ks)
         a_frag[a][ks] = *reinterpret_cast<const h8_t *>(
-            &x_lds[(row_base + a * 32 + frag_row) * LDS_STRIDE + ks * 16 + frag_k]);
+            &x_lds[(row_base + a * 32 + frag_row) * BK +
+                   (((ks * 2 + frag_kq) ^ (((row_base + a * 32 + frag_row) >> 1) & 7)) << 3)]);
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int v = 0; v < NW; ++v) {
+    for (int block = 0; block < BLOCKS; ++block) {
+      const int v = block / WN;
+      const int b = block % WN;
 #pragma unroll
-      for (int b = 0; b < WN; ++b) {
-        h8_t b_frag[BK / 16];
+      for (int a = 0; a < WM; ++a) {
 #pragma unroll
         for (int ks = 0; ks < BK / 16; ++ks)
-          b_frag[ks] = *reinterpret_cast<const h8_t *>(
-              &w_lds[(v * BN + col_base + b * 32 + frag_row) * LDS_STRIDE + ks * 16 + frag_k]);
-        const float scale = s_lds[v * BN + col_base + b * 32 + frag_row];
+          acc[v][a][b] =
+              __builtin_amdgcn_mfma_f32_32x32x16_f16(a_frag[a][ks], b_frag[block & 1][ks], acc[v][a][b], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (a == 0 && block + 1 < BLOCKS) read_block(block + 1);
+        const int group = block * WM + a;
+        if (group == 0) wait_w(fetched[stage ^ 1], std::integral_constant<int, W_LOADS>{});
 #pragma unroll
-        for (int a = 0; a < WM; ++a) {
-          // one 64-wide scale group: four chained MFMAs into a temporary tile,
-          // then acc += temporary * float(scale) in fp32
-          f16x_t part = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_frag[a][0], b_frag[0], zero_tile(), 0, 0, 0);
-#pragma unroll
-          for (int ks = 1; ks < BK / 16; ++ks)
-            part = __builtin_amdgcn_mfma_f32_32x32x16_f16(a_frag[a][ks], b_frag[ks], part, 0, 0, 0);
-#pragma unroll
-          for (int i = 0; i < 16; ++i) acc[v][a][b][i] = fmaf(part[i], scale, acc[v][a][b][i]);
-        }
+        for (int n = 0; n < ITEMS_PER_GROUP; ++n)
+          if (group * ITEMS_PER_GROUP + n < ITEMS)
+            store_item(fetched[stage ^ 1], stage ^ 1, group * ITEMS_PER_GROUP + n);
+        if (group == 0) fetch_x(min(k0 + BK, K - BK), stage ^ 1);
+        __builtin_amdgcn_sched_barrier(0);
       }
     }
+    fetch_w(fetched[stage ^ 1], min(k0 + 3 * BK, K - BK));
+    __builtin_amdgcn_sched_barrier(0);
+    wait_all(std::integral_constant<int, W_LOADS>{});  // the activation copy has landed
+  };
+
+  fetch_x(0, 0);
+  fetch_w(fetched[0], 0);
+  fetch_w(fetched[1], min((uint32_t)BK, K - BK));
+  wait_w(fetched[0], std::integral_constant<int, W_LOADS>{});
+#pragma unroll
+  for (int item = 0; item < ITEMS; ++item) store_item(fetched[0], 0, item);
+  fetch_w(fetched[0], min(2u * BK, K - BK));
+  for (uint32_t k0 = 0; k0 < K; k0 += 2 * BK) {
+    step(k0, std::integral_constant<int, 0>{});
+    if (k0 + BK < K) step(k0 + BK, std::integral_constant<int, 1>{});
   }
+  wait_all(std::integral_constant<int, 0>{});  // the surplus requests still target live registers
 
   // epilogue: lane owns column col, rows (i/4)*8 + (lane/32)*4 + i%4 of each tile
 #pragma unroll
@@ -223,7 +297,7 @@ hipError_t launch_tile(GemmParams &p, hipStream_t stream) {
   constexpr int BM = 4 * WM * 32;
   constexpr int BN = 2 * WN * 32;
   constexpr size_t lds_bytes =
-      (size_t)(BM + NW * BN) * LDS_STRIDE * sizeof(_Float16) + (size_t)NW * BN * sizeof(float);
+      2 * ((size_t)BM * BK + (size_t)NW * BN * LDS_STRIDE) * sizeof(_Float16);
   static bool configured = false;
   if (!configured) {
     hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(&w4a16_gemm_kernel<WM, WN, DUAL>),
