@@ -72,9 +72,11 @@ __device__ __forceinline__ size_t partial_floats(uint32_t heads_per_kv) {
 
 // OFF32: the pool is smaller than 4 GiB, so slot byte offsets fit 32 bits and the
 // loads can use a scalar base plus a 32-bit vector offset.
+// Three waves per SIMD: left alone the register allocator takes 209 registers
+// (two waves), and the kernel is bound by the latency of each wave's requests.
 template <int D, bool OFF32, bool A16>
-__global__ __launch_bounds__(kSplitMaxWaves * 64) void q8_attention_split_kernel(Q8AttentionArgs a,
-                                                                           uint32_t chunks_max) {
+__global__ __launch_bounds__(kSplitMaxWaves * 64) __attribute__((amdgpu_waves_per_eu(3, 3))) void
+q8_attention_split_kernel(Q8AttentionArgs a, uint32_t chunks_max) {
   constexpr int GROUPS = D / 64;      // scale groups per head
   constexpr int KLOADS = GROUPS;      // 16-byte K loads per lane per tile
   constexpr int VBLOCKS = D / 16;     // PV MFMAs (16 head_dim rows each)
@@ -95,7 +97,9 @@ __global__ __launch_bounds__(kSplitMaxWaves * 64) void q8_attention_split_kernel
   const uint32_t chunk_begin = chunk * kChunkTokens;
   if (chunk_begin >= past) return;
   const uint32_t *slots = a.slot_offsets ? a.slots + a.slot_offsets[batch] : a.slots;
-  const uint32_t last_token = past - 1;
+  // requests that run ahead of the arithmetic stop at the chunk's last token:
+  // what lies beyond belongs to another workgroup and would be fetched twice
+  const uint32_t last_token = min(chunk_begin + (uint32_t)kChunkTokens, past) - 1;
 
   // B operand of the score MFMAs: Q[head = col][d], zero for columns >= G.
   h8_t q_frag[GROUPS][2];
