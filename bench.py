@@ -124,11 +124,32 @@ def bench_gemv(runtime, steps, warmup):
             ms = batch.commit_profiled(repeats=repeats, use_graph=True)
             us = ms * 1e3 / (repeats * COPIES)
             gbs = gemv_bytes(m, k, n) / (us * 1e-6) / 1e9
+            # warm: the same weight copy every launch (31 MB stays in the 256 MB Infinity Cache)
+            batch = runtime.begin_batch()
+            bw, bs = weights[(k, n)][0]
+            for _ in range(COPIES):
+                record_linear(batch, m, n, k, activations[(m, k)], bw, bs, outputs[(m, n)])
+            warm_us = batch.commit_profiled(repeats=repeats, use_graph=True) * 1e3 / (repeats * COPIES)
             cases.append({"m": m, "k": k, "n": n, "bytes": gemv_bytes(m, k, n),
                           "us_per_launch": round(us, 3), "GBps": round(gbs, 1),
-                          "hbm_frac": round(gbs / HBM_PEAK_GBS, 4)})
+                          "hbm_frac": round(gbs / HBM_PEAK_GBS, 4),
+                          "warm_us_per_launch": round(warm_us, 3),
+                          "warm_GBps": round(gemv_bytes(m, k, n) / (warm_us * 1e-6) / 1e9, 1)})
+
+    # C1: the 1 x 576 -> 1536 projection of the 30-layer model (474 KB: launch/latency-bound)
+    k, n = 576, 1536
+    _, packed, scale = w4_inputs(rng, 1, n, k)
+    c1_weights = [(runtime.buffer_of_bytes(packed), runtime.buffer_of_bytes(scale)) for _ in range(COPIES)]
+    c1_x = runtime.buffer_of_bytes(rng.standard_normal((1, k)).astype(np.float16))
+    c1_out = runtime.create_buffer(n * 2)
+    batch = runtime.begin_batch()
+    for bw, bs in c1_weights:
+        record_linear(batch, 1, n, k, c1_x, bw, bs, c1_out)
+    c1_us = batch.commit_profiled(repeats=8, use_graph=True) * 1e3 / (8 * COPIES)
+    c1 = {"m": 1, "k": k, "n": n, "bytes": gemv_bytes(1, k, n), "us_per_launch": round(c1_us, 3),
+          "GBps": round(gemv_bytes(1, k, n) / (c1_us * 1e-6) / 1e9, 1)}
     return {"bytes_per_step": bytes_per_step, "ms_per_step": ms_per_step,
-            "graph_ms_per_step": graph_ms_per_step, "cases": cases}
+            "graph_ms_per_step": graph_ms_per_step, "cases": cases, "c1": c1}
 
 
 def bench_gemm(runtime):
@@ -349,7 +370,7 @@ def main():
     headline = next(c for c in gemv["cases"] if (c["m"], c["k"], c["n"]) == (1, 4096, 14336))
     # the K steps replayed as one HIP graph, timed by HIP events on the launch stream
     value = gemv["bytes_per_step"] / (gemv["graph_ms_per_step"] * 1e-3) / 1e9
-    extras = {"gemv_cases": gemv["cases"],
+    extras = {"gemv_cases": gemv["cases"], "gemv_c1_1x576x1536": gemv["c1"],
               "gemv_eager_host_launch_GBps":
                   round(gemv["bytes_per_step"] / (gemv["ms_per_step"] * 1e-3) / 1e9, 1),
               "gemv_eager_host_launch_ms_per_step": round(gemv["ms_per_step"], 4),
