@@ -240,6 +240,31 @@ def bench_attention(runtime):
             "tokens_per_s": round(batches / (us * 1e-6), 1)}
 
 
+def bench_prefill_attention(runtime):
+    """Dense causal fp16 attention of a prefill (the step that fills the KV cache): 32/8 heads of
+    128 at 2048 and 8192 tokens, and the 30-layer model's 9/3 heads of 64 at 2048."""
+    rng = np.random.default_rng(SEED + 4)
+    results = []
+    for heads, kv_heads, dim, length in ((32, 8, 128, 2048), (32, 8, 128, 8192), (9, 3, 64, 2048)):
+        query = runtime.buffer_of_bytes(rng.standard_normal((1, heads, length, dim)).astype(np.float16))
+        key = runtime.buffer_of_bytes(rng.standard_normal((1, kv_heads, length, dim)).astype(np.float16))
+        value = runtime.buffer_of_bytes(rng.standard_normal((1, kv_heads, length, dim)).astype(np.float16))
+        out = runtime.create_buffer(heads * length * dim * 2)
+        params = struct.pack("<8IfIIIII", 1, heads, length, length, dim, 0, 0, 1, 1.0 / math.sqrt(dim),
+                             kv_heads, 1, 0, 0, 0)
+        batch = runtime.begin_batch()
+        for _ in range(4):
+            batch.dispatch(f"llmopt_attention_f16_simd_h{dim}", [query, key, value, query, out], params,
+                           grid=(heads * ((length + 31) // 32) * 128, 1, 1), group=(128, 1, 1))
+        repeats = 3
+        us = batch.commit_profiled(repeats=repeats, use_graph=True) * 1e3 / (repeats * 4)
+        flops = 4.0 * heads * dim * (length * (length + 1) / 2)  # QK^T and PV over the causal half
+        results.append({"heads": heads, "kv_heads": kv_heads, "head_dim": dim, "tokens": length,
+                        "us_per_launch": round(us, 2), "TFLOPs": round(flops / (us * 1e-6) / 1e12, 1),
+                        "mfma_frac": round(flops / (us * 1e-6) / 1e12 / MFMA_F16_PEAK_TFLOPS, 4)})
+    return results
+
+
 def bench_decode_step(runtime, batches=(1, 8, 32), context=2048, use_graph=True):
     """C5: one decode step of the 30-layer model (hidden 576, 9/3 heads of 64, MLP 1536,
     vocabulary 49152), every sequence with `context` tokens in the Q8 pool, replayed as a
@@ -348,8 +373,8 @@ def main():
     parser.add_argument("--steps", type=int, default=64)
     parser.add_argument("--warmup", type=int, default=16)
     parser.add_argument("--skip-extras", action="store_true")
-    parser.add_argument("--extras", default="gemm,attention,decode",
-                        help="comma-separated subset of gemm, attention, decode")
+    parser.add_argument("--extras", default="gemm,attention,prefill_attention,decode",
+                        help="comma-separated subset of gemm, attention, prefill_attention, decode")
     parser.add_argument("--skip-cpu", action="store_true")
     parser.add_argument("--decode-eager", action="store_true",
                         help="launch the decode step from the host instead of replaying a HIP graph")
@@ -380,6 +405,8 @@ def main():
         extras["prefill_gemm"] = bench_gemm(runtime)
     if "attention" in wanted:
         extras["q8_attention"] = bench_attention(runtime)
+    if "prefill_attention" in wanted:
+        extras["prefill_attention"] = bench_prefill_attention(runtime)
     if "decode" in wanted:
         extras["decode_step"] = bench_decode_step(runtime, use_graph=not args.decode_eager)
     line = {

@@ -106,6 +106,15 @@ int llmopt_op_paged_attention_q8(llmopt_op_context *context,
 /* ---- pure helpers (no GPU) --------------------------------------------------- */
 
 /* Paged_attention_tactic.kernel_name (lib/metal_dispatch_common.ml:41-57). */
+/* dispatch_attention ctx st ~config ~query ~key ~value ~mask ~output
+ * (lib/metal_dispatch_attention.ml:6-102): dense fp16 attention (prefill).  query [b,h,q,d],
+ * key [b,kvh,L,d], value [b,kvh,L,d] or [b,L,kvh,d], mask NULL or [mb,mh,q,L] (BOOL or F16),
+ * output [b,h,q,d], [b,q,h,d] or [b,q,h*d]; past_length = max(0, L - q). */
+int llmopt_op_attention(llmopt_op_context *context, double scale, int causal,
+                        const llmopt_op_value *query, const llmopt_op_value *key,
+                        const llmopt_op_value *value, const llmopt_op_value *mask,
+                        const llmopt_op_value *output);
+
 const char *llmopt_op_paged_attention_kernel_name(int experimental_gqa3_split8, int split8,
                                                   int64_t query_heads, int64_t kv_heads,
                                                   int64_t head_dimension);

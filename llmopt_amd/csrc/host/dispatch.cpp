@@ -429,6 +429,76 @@ int llmopt_op_paged_attention_q8(llmopt_op_context *context, const llmopt_op_pag
   return dispatch(context, name, "attention", buffers, parameters, grid);
 }
 
+// dispatch_attention (lib/metal_dispatch_attention.ml:6-102): dense fp16
+// attention, the prefill side of the KV cache.
+int llmopt_op_attention(llmopt_op_context *context, double scale, int causal, const llmopt_op_value *query,
+                        const llmopt_op_value *key, const llmopt_op_value *value, const llmopt_op_value *mask,
+                        const llmopt_op_value *output) {
+  if (context == nullptr) return fail(LLMOPT_ERR_FAILURE, "operator context has been finalized");
+  context->kernels.clear();
+  if (query == nullptr || key == nullptr || value == nullptr || output == nullptr)
+    return fail(LLMOPT_ERR_INVALID, "attention argument is null");
+  if (query->rank != 4) return fail(LLMOPT_ERR_FAILURE, "attention query must have rank four");
+  const int64_t batches = query->dims[0], heads = query->dims[1], query_length = query->dims[2],
+                head_dimension = query->dims[3];
+  if (key->rank != 4) return fail(LLMOPT_ERR_FAILURE, "attention key must have rank four");
+  const int64_t kv_heads = key->dims[1], key_length = key->dims[2];
+  int64_t token_first_value;
+  if (has_dims(*value, {batches, kv_heads, key_length, head_dimension}))
+    token_first_value = 0;  // also when kv_heads == key_length: head-major is tried first
+  else if (has_dims(*value, {batches, key_length, kv_heads, head_dimension}))
+    token_first_value = 1;
+  else
+    return fail(LLMOPT_ERR_FAILURE, "attention value must match key in head-major or token-major layout");
+  int64_t mask_batches = 0, mask_heads = 0, mask_dtype = 0;
+  const llmopt_op_value *mask_buffer = query;  // the query buffer fills the slot when there is no mask
+  if (mask != nullptr) {
+    if (mask->rank != 4) return fail(LLMOPT_ERR_FAILURE, "attention mask must have rank four");
+    if (mask->dtype == LLMOPT_BOOL)
+      mask_dtype = 1;
+    else if (mask->dtype == LLMOPT_F16)
+      mask_dtype = 2;
+    else
+      return fail(LLMOPT_ERR_FAILURE, "attention mask dtype %d is unsupported", mask->dtype);
+    mask_batches = mask->dims[0];
+    mask_heads = mask->dims[1];
+    mask_buffer = mask;
+  }
+  const int64_t token_first_output =
+      (has_dims(*output, {batches, query_length, heads * head_dimension}) ||
+       has_dims(*output, {batches, query_length, heads, head_dimension}))
+          ? 1
+          : 0;
+  std::vector<llmopt_hip_buffer *> buffers(5);
+  const llmopt_op_value *ordered[5] = {query, key, value, mask_buffer, output};
+  for (size_t i = 0; i < 5; ++i)
+    if (int status = find_value(ordered[i], &buffers[i])) return status;
+  const int64_t past_length = key_length > query_length ? key_length - query_length : 0;
+  Parameters parameters;  // Parameters.attention, lib/metal_parameters.ml:95-117
+  for (int64_t field : {batches, heads, query_length, key_length, head_dimension, mask_batches, mask_heads,
+                        (int64_t)(causal != 0 ? 1 : 0)})
+    parameters.u32(field);
+  parameters.f32(scale);
+  for (int64_t field : {kv_heads, token_first_output, past_length, token_first_value, mask_dtype})
+    parameters.u32(field);
+  // select_attention_kernel (lib/metal_dispatch_common.ml:166-189): the head-dimension entry
+  // when the package has it, else the portable one
+  char specialized[64];
+  snprintf(specialized, sizeof specialized, "llmopt_attention_f16_simd_h%lld", (long long)head_dimension);
+  const bool simd = head_dimension % 8 == 0 && llmopt_hip_has_function(context->library, specialized) == 1;
+  const char *name = simd ? specialized : "llmopt_attention_f16";
+  int64_t grid;
+  if (simd) {
+    const int64_t q_tiles = (query_length + 31) / 32;
+    const int64_t groups = batches * heads * q_tiles;
+    if (groups > kMaxInt / 128) return fail(LLMOPT_ERR_FAILURE, "Metal attention grid dimension overflows");
+    grid = groups * 128;
+  } else {
+    grid = batches * heads * query_length;
+  }
+  return dispatch(context, name, "attention", buffers, parameters, grid);
+}
+
 const char *llmopt_op_paged_attention_kernel_name(int experimental_gqa3_split8, int split8, int64_t query_heads,
                                                   int64_t kv_heads, int64_t head_dimension) {
   return paged_kernel_name(experimental_gqa3_split8 != 0, split8 != 0, query_heads, kv_heads, head_dimension);

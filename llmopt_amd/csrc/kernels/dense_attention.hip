@@ -1,0 +1,317 @@
+// Dense fp16 attention (prefill and any other non-paged attention) for gfx950.
+//
+// Contract: llmopt_attention_f16 / llmopt_attention_f16_simd_h<D>
+// (lib/metal_attention_source.ml:239-347, AttentionParams :251-256): query
+// [b, h, q, D] head-major, key [b, kvh, L, D] head-major, value head-major or
+// token-major [b, L, kvh, D], optional mask [mb, mh, q, L] (bool: nonzero
+// allowed; half: >= 0 allowed), causal limit key <= past_length + q, GQA
+// kv_head = head / (h / kvh), output head-major [b, h, q, D] or token-major
+// [b, q, h, D]; a row with no allowed key is zero.  Scores and softmax in fp32.
+//
+//  * dense_attention_mfma_kernel<D> (D = 64, 128): a wave owns 32 query rows of
+//    one head and walks the keys in tiles of 16 with an online softmax in base
+//    2.  S^T = K Q^T on v_mfma_f32_16x16x32_f16, so that a lane's four scores
+//    belong to one query row (its column) and feed, converted to fp16, the B
+//    operand of O^T = V^T P^T on v_mfma_f32_16x16x16f16 without any exchange
+//    between lanes; V tiles are transposed in registers (4 keys x 4 head_dim
+//    halfs per lane).  Key tiles past the causal limit of the wave's rows are
+//    skipped.
+//  * dense_attention_rows_kernel: one wave per output row, serial over the keys
+//    (any D up to 512, every option); the direct restatement.
+#include <algorithm>
+
+#include "kernels.h"
+#include "kernels_internal.h"
+#include "w4_common.h"
+
+namespace llmopt {
+namespace {
+
+__device__ __forceinline__ float lanes_xor_max(float value, int mask) {
+  const int lane = (int)(threadIdx.x & 63);
+  const float other = __builtin_bit_cast(
+      float, __builtin_amdgcn_ds_bpermute((lane ^ mask) << 2, __builtin_bit_cast(int, value)));
+  return fmaxf(value, other);
+}
+
+__device__ __forceinline__ float lanes_xor_sum(float value, int mask) {
+  const int lane = (int)(threadIdx.x & 63);
+  const float other = __builtin_bit_cast(
+      float, __builtin_amdgcn_ds_bpermute((lane ^ mask) << 2, __builtin_bit_cast(int, value)));
+  return value + other;
+}
+
+__device__ __forceinline__ bool mask_allows(const DenseAttentionArgs &a, uint32_t batch, uint32_t head,
+                                            uint32_t query_position, uint32_t key_position) {
+  const uint32_t mask_batch = a.mask_batches == 1 ? 0 : batch;
+  const uint32_t mask_head = a.mask_heads == 1 ? 0 : head;
+  const size_t index =
+      (((size_t)mask_batch * a.mask_heads + mask_head) * a.query_length + query_position) * a.key_length +
+      key_position;
+  if (a.mask_dtype == 2) return half_bits_to_float(reinterpret_cast<const uint16_t *>(a.mask)[index]) >= 0.0f;
+  return a.mask[index] != 0;
+}
+
+constexpr int kQueryTiles = 2;    // 16-row query tiles per wave
+constexpr int kWavesPerBlock = 4;  // consecutive 32-row slabs of one head
+
+template <int D>
+__global__ __launch_bounds__(kWavesPerBlock * 64) void dense_attention_mfma_kernel(DenseAttentionArgs a) {
+  constexpr int QSTEPS = D / 32;   // score MFMAs per tile pair
+  constexpr int VBLOCKS = D / 64;  // 64-wide head_dim blocks of the V transposes
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t wave = threadIdx.x >> 6;
+  const uint32_t col = lane & 15;
+  const uint32_t quad = lane >> 4;
+  const uint32_t head = blockIdx.y;
+  const uint32_t batch = blockIdx.z;
+  const uint32_t q0 = (blockIdx.x * kWavesPerBlock + wave) * (kQueryTiles * 16);
+  if (q0 >= a.query_length) return;  // whole wave; the kernel has no barriers
+  const uint32_t kv_heads = a.kv_heads > 0 ? a.kv_heads : a.heads;
+  const uint32_t kv_head = kv_heads < a.heads ? head / (a.heads / kv_heads) : head;
+  const bool masked = a.mask != nullptr && a.mask_batches > 0;
+  const uint32_t L = a.key_length;
+
+  // B operand of the score MFMAs: Q[row = col][d = j*32 + quad*8 ..], rows past the end repeat the last one
+  h8_t q_frag[kQueryTiles][QSTEPS];
+#pragma unroll
+  for (int t = 0; t < kQueryTiles; ++t) {
+    const uint32_t row = min(q0 + t * 16 + col, a.query_length - 1);
+    const uint16_t *q_row = a.query + (((size_t)batch * a.heads + head) * a.query_length + row) * D;
+#pragma unroll
+    for (int j = 0; j < QSTEPS; ++j)
+      q_frag[t][j] = __builtin_bit_cast(h8_t, *reinterpret_cast<const uint4 *>(q_row + j * 32 + quad * 8));
+  }
+
+  const uint16_t *key_base = a.key + ((size_t)batch * kv_heads + kv_head) * L * D;
+  const size_t value_row_stride = a.token_first_value ? (size_t)kv_heads * D : D;
+  const uint16_t *value_base = a.token_first_value
+                                   ? a.value + ((size_t)batch * L * kv_heads + kv_head) * D
+                                   : a.value + ((size_t)batch * kv_heads + kv_head) * L * D;
+
+  // softmax in base 2
+  const float score_scale = a.scale * 1.4426950408889634f;
+  float running_max[kQueryTiles], running_sum[kQueryTiles];  // per lane: row col of each tile; sum over this quad's keys
+  f4_t out_acc[kQueryTiles][VBLOCKS * 4];                    // O^T[d = blk*64 + 4*(quad*4+i) + jj][row col]
+#pragma unroll
+  for (int t = 0; t < kQueryTiles; ++t) {
+    running_max[t] = -INFINITY;
+    running_sum[t] = 0.0f;
+#pragma unroll
+    for (int v = 0; v < VBLOCKS * 4; ++v) out_acc[t][v] = f4_t{0.0f, 0.0f, 0.0f, 0.0f};
+  }
+
+  // keys this wave can need: all of them, or up to the causal limit of its last row
+  uint32_t key_end = L;
+  if (a.causal) {
+    const uint32_t last_row = min(q0 + kQueryTiles * 16, a.query_length) - 1;
+    key_end = min((uint64_t)L, (uint64_t)a.past_length + last_row + 1);
+  }
+
+  for (uint32_t key0 = 0; key0 < key_end; key0 += 16) {
+    // A operand: K[key = col][d = j*32 + quad*8 ..]; keys past the end repeat the last one (masked below)
+    h8_t k_frag[QSTEPS];
+    {
+      const uint16_t *k_row = key_base + (size_t)min(key0 + col, L - 1) * D;
+#pragma unroll
+      for (int j = 0; j < QSTEPS; ++j)
+        k_frag[j] = __builtin_bit_cast(h8_t, *reinterpret_cast<const uint4 *>(k_row + j * 32 + quad * 8));
+    }
+    // V: lane (c = col, quad) reads head_dim c*4 .. c*4+3 of keys quad*4 + i
+    uint2 v_raw[VBLOCKS][4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const uint16_t *v_row = value_base + (size_t)min(key0 + quad * 4 + i, L - 1) * value_row_stride;
+#pragma unroll
+      for (int blk = 0; blk < VBLOCKS; ++blk)
+        v_raw[blk][i] = *reinterpret_cast<const uint2 *>(v_row + blk * 64 + col * 4);
+    }
+    // 4 x 4 transposes: v_t[blk][jj] = V[keys quad*4 + 0..3][blk*64 + col*4 + jj], the A operand of PV
+    h4_t v_t[VBLOCKS][4];
+#pragma unroll
+    for (int blk = 0; blk < VBLOCKS; ++blk) {
+      const uint32_t lo01_a = __builtin_amdgcn_perm(v_raw[blk][1].x, v_raw[blk][0].x, 0x05040100u);
+      const uint32_t lo01_b = __builtin_amdgcn_perm(v_raw[blk][1].x, v_raw[blk][0].x, 0x07060302u);
+      const uint32_t lo23_a = __builtin_amdgcn_perm(v_raw[blk][3].x, v_raw[blk][2].x, 0x05040100u);
+      const uint32_t lo23_b = __builtin_amdgcn_perm(v_raw[blk][3].x, v_raw[blk][2].x, 0x07060302u);
+      const uint32_t hi01_a = __builtin_amdgcn_perm(v_raw[blk][1].y, v_raw[blk][0].y, 0x05040100u);
+      const uint32_t hi01_b = __builtin_amdgcn_perm(v_raw[blk][1].y, v_raw[blk][0].y, 0x07060302u);
+      const uint32_t hi23_a = __builtin_amdgcn_perm(v_raw[blk][3].y, v_raw[blk][2].y, 0x05040100u);
+      const uint32_t hi23_b = __builtin_amdgcn_perm(v_raw[blk][3].y, v_raw[blk][2].y, 0x07060302u);
+      v_t[blk][0] = __builtin_bit_cast(h4_t, make_uint2(lo01_a, lo23_a));
+      v_t[blk][1] = __builtin_bit_cast(h4_t, make_uint2(lo01_b, lo23_b));
+      v_t[blk][2] = __builtin_bit_cast(h4_t, make_uint2(hi01_a, hi23_a));
+      v_t[blk][3] = __builtin_bit_cast(h4_t, make_uint2(hi01_b, hi23_b));
+    }
+
+#pragma unroll
+    for (int t = 0; t < kQueryTiles; ++t) {
+      const uint32_t row = q0 + t * 16 + col;  // this lane's query row in tile t
+      // tiles that lie wholly past this tile's causal limit contribute nothing
+      if (a.causal && key0 > a.past_length + q0 + t * 16 + 15) continue;
+      f4_t score = f4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+      for (int j = 0; j < QSTEPS; ++j)
+        score = __builtin_amdgcn_mfma_f32_16x16x32_f16(k_frag[j], q_frag[t][j], score, 0, 0, 0);
+      float tile_max = -INFINITY;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const uint32_t key = key0 + quad * 4 + i;
+        bool allowed = key < L && row < a.query_length;
+        if (a.causal) allowed = allowed && key <= a.past_length + row;
+        if (masked && allowed) allowed = mask_allows(a, batch, head, row, key);
+        score[i] = allowed ? score[i] * score_scale : -INFINITY;
+        tile_max = fmaxf(tile_max, score[i]);
+      }
+      tile_max = lanes_xor_max(tile_max, 16);
+      tile_max = lanes_xor_max(tile_max, 32);
+      const float new_max = fmaxf(running_max[t], tile_max);
+      // no allowed key yet: keep every exponent finite (the probabilities are zero anyway)
+      const float reference = new_max == -INFINITY ? 0.0f : new_max;
+      const float alpha = __builtin_amdgcn_exp2f(running_max[t] - reference);  // 0 while running_max is -inf
+      running_max[t] = new_max;
+      h4_t p_frag;
+      float tile_sum = 0.0f;
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const float p = __builtin_amdgcn_exp2f(score[i] - reference);
+        tile_sum += p;
+        p_frag[i] = (_Float16)p;
+      }
+      running_sum[t] = running_sum[t] * alpha + tile_sum;
+      if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+        for (int v = 0; v < VBLOCKS * 4; ++v)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) out_acc[t][v][i] *= alpha;
+      }
+#pragma unroll
+      for (int blk = 0; blk < VBLOCKS; ++blk)
+#pragma unroll
+        for (int jj = 0; jj < 4; ++jj)
+          out_acc[t][blk * 4 + jj] =
+              __builtin_amdgcn_mfma_f32_16x16x16f16(v_t[blk][jj], p_frag, out_acc[t][blk * 4 + jj], 0, 0, 0);
+    }
+  }
+
+  // out_acc[t][blk*4 + jj][i] is O[row = q0 + t*16 + col][d = blk*64 + 4*(quad*4 + i) + jj]
+#pragma unroll
+  for (int t = 0; t < kQueryTiles; ++t) {
+    float total = lanes_xor_sum(running_sum[t], 16);
+    total = lanes_xor_sum(total, 32);
+    const uint32_t row = q0 + t * 16 + col;
+    if (row >= a.query_length) continue;
+    const float inverse = total != 0.0f ? 1.0f / total : 0.0f;
+    uint16_t *out_row = a.token_first_output
+                            ? a.output + (((size_t)batch * a.query_length + row) * a.heads + head) * D
+                            : a.output + (((size_t)batch * a.heads + head) * a.query_length + row) * D;
+#pragma unroll
+    for (int blk = 0; blk < VBLOCKS; ++blk)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        // the four jj of one (blk, i) are adjacent in head_dim: one 8-byte store
+        uint2 packed;
+        packed.x = (uint32_t)float_to_half_bits(out_acc[t][blk * 4 + 0][i] * inverse) |
+                   ((uint32_t)float_to_half_bits(out_acc[t][blk * 4 + 1][i] * inverse) << 16);
+        packed.y = (uint32_t)float_to_half_bits(out_acc[t][blk * 4 + 2][i] * inverse) |
+                   ((uint32_t)float_to_half_bits(out_acc[t][blk * 4 + 3][i] * inverse) << 16);
+        *reinterpret_cast<uint2 *>(out_row + blk * 64 + 4 * (quad * 4 + i)) = packed;
+      }
+  }
+}
+
+// ---- row-serial kernel (every other configuration) ---------------------------
+
+constexpr int kMaxFragments = 8;  // head_dim <= 512
+
+__global__ __launch_bounds__(256) void dense_attention_rows_kernel(DenseAttentionArgs a) {
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t row_index = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const uint32_t rows = a.batches * a.heads * a.query_length;
+  if (row_index >= rows) return;
+  const uint32_t query_position = row_index % a.query_length;
+  const uint32_t head = (row_index / a.query_length) % a.heads;
+  const uint32_t batch = row_index / (a.query_length * a.heads);
+  const uint32_t kv_heads = a.kv_heads > 0 ? a.kv_heads : a.heads;
+  const uint32_t kv_head = kv_heads < a.heads ? head / (a.heads / kv_heads) : head;
+  const uint32_t D = a.head_dim;
+  const uint32_t fragments = (D + 63) / 64;
+  const bool masked = a.mask != nullptr && a.mask_batches > 0;
+  const uint16_t *q_row = a.query + (size_t)row_index * D;
+
+  float q[kMaxFragments], result[kMaxFragments];
+#pragma unroll
+  for (int f = 0; f < kMaxFragments; ++f) {
+    result[f] = 0.0f;
+    const uint32_t d = f * 64 + lane;
+    q[f] = (uint32_t)f < fragments && d < D ? half_bits_to_float(q_row[d]) : 0.0f;
+  }
+  float maximum = -INFINITY, denominator = 0.0f;
+  for (uint32_t key_position = 0; key_position < a.key_length; ++key_position) {
+    if (a.causal && key_position > a.past_length + query_position) break;
+    if (masked && !mask_allows(a, batch, head, query_position, key_position)) continue;
+    const uint16_t *k_row = a.key + (((size_t)batch * kv_heads + kv_head) * a.key_length + key_position) * D;
+    const uint16_t *v_row =
+        a.token_first_value
+            ? a.value + (((size_t)batch * a.key_length + key_position) * kv_heads + kv_head) * D
+            : a.value + (((size_t)batch * kv_heads + kv_head) * a.key_length + key_position) * D;
+    float partial = 0.0f;
+    float value[kMaxFragments];
+#pragma unroll
+    for (int f = 0; f < kMaxFragments; ++f) {
+      if ((uint32_t)f >= fragments) break;
+      const uint32_t d = f * 64 + lane;
+      const bool inside = d < D;
+      partial += inside ? q[f] * half_bits_to_float(k_row[d]) : 0.0f;
+      value[f] = inside ? half_bits_to_float(v_row[d]) : 0.0f;
+    }
+    const float score = wave_sum(partial) * a.scale;
+    const float new_max = fmaxf(maximum, score);
+    const float alpha = __expf(maximum - new_max);  // 0 for the first allowed key
+    const float p = __expf(score - new_max);
+    denominator = denominator * alpha + p;
+#pragma unroll
+    for (int f = 0; f < kMaxFragments; ++f) {
+      if ((uint32_t)f >= fragments) break;
+      result[f] = result[f] * alpha + p * value[f];
+    }
+    maximum = new_max;
+  }
+  const float inverse = denominator != 0.0f ? 1.0f / denominator : 0.0f;
+  uint16_t *out_row =
+      a.token_first_output
+          ? a.output + (((size_t)batch * a.query_length + query_position) * a.heads + head) * D
+          : a.output + (size_t)row_index * D;
+#pragma unroll
+  for (int f = 0; f < kMaxFragments; ++f) {
+    if ((uint32_t)f >= fragments) break;
+    const uint32_t d = f * 64 + lane;
+    if (d < D) out_row[d] = float_to_half_bits(result[f] * inverse);
+  }
+}
+
+}  // namespace
+
+hipError_t launch_dense_attention(const DenseAttentionArgs &a, hipStream_t stream) {
+  const uint64_t rows = (uint64_t)a.batches * a.heads * a.query_length;
+  if (rows == 0) return hipSuccess;
+  if (a.key_length == 0 || a.head_dim == 0 || a.head_dim > 64 * kMaxFragments) return hipErrorInvalidValue;
+  const bool aligned = reinterpret_cast<uintptr_t>(a.query) % 16 == 0 && reinterpret_cast<uintptr_t>(a.key) % 16 == 0 &&
+                       reinterpret_cast<uintptr_t>(a.value) % 8 == 0 && reinterpret_cast<uintptr_t>(a.output) % 8 == 0;
+  if ((a.head_dim == 64 || a.head_dim == 128) && aligned && a.query_length >= 16 && a.heads <= 65535 &&
+      a.batches <= 65535) {
+    const uint32_t slab = kWavesPerBlock * kQueryTiles * 16;
+    const dim3 grid((a.query_length + slab - 1) / slab, a.heads, a.batches);
+    if (a.head_dim == 64)
+      hipLaunchKernelGGL(dense_attention_mfma_kernel<64>, grid, dim3(kWavesPerBlock * 64), 0, stream, a);
+    else
+      hipLaunchKernelGGL(dense_attention_mfma_kernel<128>, grid, dim3(kWavesPerBlock * 64), 0, stream, a);
+    return hipGetLastError();
+  }
+  const uint64_t blocks = (rows + 3) / 4;
+  if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
+  hipLaunchKernelGGL(dense_attention_rows_kernel, dim3((uint32_t)blocks), dim3(256), 0, stream, a);
+  return hipGetLastError();
+}
+
+}  // namespace llmopt

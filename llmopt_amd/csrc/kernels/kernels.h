@@ -133,6 +133,22 @@ struct Q8AttentionArgs {
 size_t q8_attention_workspace_bytes(const Q8AttentionArgs &args);
 hipError_t launch_q8_attention(const Q8AttentionArgs &args, hipStream_t stream);
 
+// ---- dense fp16 attention -------------------------------------------------------
+
+// llmopt_attention_f16 / llmopt_attention_f16_simd_h<D>
+// (lib/metal_attention_source.ml:239-347; AttentionParams :251-256).
+struct DenseAttentionArgs {
+  const uint16_t *query;  // f16 [b, h, q, D]
+  const uint16_t *key;    // f16 [b, kvh, L, D]
+  const uint16_t *value;  // f16 [b, kvh, L, D], or [b, L, kvh, D] with token_first_value
+  const uint8_t *mask;    // [mb, mh, q, L] bool or f16; null or mask_batches == 0: none
+  uint16_t *output;       // f16 [b, h, q, D], or [b, q, h, D] with token_first_output
+  uint32_t batches, heads, query_length, key_length, head_dim, mask_batches, mask_heads, causal;
+  float scale;
+  uint32_t kv_heads, token_first_output, past_length, token_first_value, mask_dtype;
+};
+hipError_t launch_dense_attention(const DenseAttentionArgs &args, hipStream_t stream);
+
 // ---- decode glue ---------------------------------------------------------------
 
 // out[row, i] = half(x[row, i] * rsqrt(mean(x[row]^2) + eps) * w[i]), one wave per row.

@@ -236,6 +236,63 @@ int paged_attention_batched(llmopt_hip_context *context, const DispatchRecord &r
   return paged_attention(context, record, true);
 }
 
+// AttentionParams, 14 x 4 bytes (lib/metal_attention_source.ml:251-256,
+// lib/metal_parameters.ml:95-117).  buffers: query, key, value, mask (the query
+// buffer again when there is no mask, lib/metal_dispatch_attention.ml:52-54),
+// output.
+int dense_attention(llmopt_hip_context *context, const DispatchRecord &record) {
+  if (int status = require_buffer_count(record, 5)) return status;
+  if (int status = require_parameter_bytes(record, 56)) return status;
+  DenseAttentionArgs args = {};
+  args.batches = param_u32(record, 0);
+  args.heads = param_u32(record, 4);
+  args.query_length = param_u32(record, 8);
+  args.key_length = param_u32(record, 12);
+  args.head_dim = param_u32(record, 16);
+  args.mask_batches = param_u32(record, 20);
+  args.mask_heads = param_u32(record, 24);
+  args.causal = param_u32(record, 28);
+  args.scale = param_f32(record, 32);
+  args.kv_heads = param_u32(record, 36);
+  args.token_first_output = param_u32(record, 40);
+  args.past_length = param_u32(record, 44);
+  args.token_first_value = param_u32(record, 48);
+  args.mask_dtype = param_u32(record, 52);
+  const char *name = record.name.c_str();
+  if (args.head_dim == 0 || args.head_dim > 512)
+    return fail(LLMOPT_ERR_INVALID, "%s supports head dimensions 1..512, got %u", name, args.head_dim);
+  const uint32_t kv_heads = args.kv_heads > 0 ? args.kv_heads : args.heads;
+  if (kv_heads == 0 || (kv_heads < args.heads && args.heads % kv_heads != 0) || kv_heads > args.heads)
+    return fail(LLMOPT_ERR_INVALID, "%s requires heads to be a multiple of kv_heads", name);
+  if (args.mask_batches > 0 && (args.mask_heads == 0 || (args.mask_dtype != 1 && args.mask_dtype != 2)))
+    return fail(LLMOPT_ERR_INVALID, "%s received an inconsistent mask description", name);
+  if (args.mask_batches > 1 && args.mask_batches != args.batches)
+    return fail(LLMOPT_ERR_INVALID, "%s mask batches must be 1 or the batch count", name);
+  if (args.mask_batches > 0 && args.mask_heads > 1 && args.mask_heads != args.heads)
+    return fail(LLMOPT_ERR_INVALID, "%s mask heads must be 1 or the head count", name);
+  const uint64_t rows = (uint64_t)args.batches * args.heads * args.query_length;
+  const uint64_t kv_elements = (uint64_t)args.batches * kv_heads * args.key_length * args.head_dim;
+  if (rows != 0 && args.key_length == 0)
+    return fail(LLMOPT_ERR_INVALID, "%s requires at least one key", name);
+  if (int status = require_buffer_size(record.buffers[0], rows * args.head_dim * 2, "attention query")) return status;
+  if (int status = require_buffer_size(record.buffers[1], kv_elements * 2, "attention key")) return status;
+  if (int status = require_buffer_size(record.buffers[2], kv_elements * 2, "attention value")) return status;
+  if (args.mask_batches > 0) {
+    const uint64_t mask_elements =
+        (uint64_t)args.mask_batches * args.mask_heads * args.query_length * args.key_length;
+    if (int status = require_buffer_size(record.buffers[3], mask_elements * (args.mask_dtype == 2 ? 2 : 1),
+                                         "attention mask"))
+      return status;
+    args.mask = record.buffers[3].device;
+  }
+  if (int status = require_buffer_size(record.buffers[4], rows * args.head_dim * 2, "attention output")) return status;
+  args.query = reinterpret_cast<const uint16_t *>(record.buffers[0].device);
+  args.key = reinterpret_cast<const uint16_t *>(record.buffers[1].device);
+  args.value = reinterpret_cast<const uint16_t *>(record.buffers[2].device);
+  args.output = reinterpret_cast<uint16_t *>(record.buffers[4].device);
+  return launched(launch_dense_attention(args, context->stream), name);
+}
+
 }  // namespace
 
 void register_cache_kernels(std::vector<KernelEntryPoint> &table) {
@@ -256,6 +313,12 @@ void register_attention_kernels(std::vector<KernelEntryPoint> &table) {
       "llmopt_attention_q8_paged_simd_h512",      "llmopt_attention_q8_paged_simd_h64_split8",
       "llmopt_attention_q8_paged_simd_h64_gqa3_split8"};
   for (const char *name : names) table.push_back({name, attention, paged_attention_reference});
+  // dense fp16 attention: the portable entry and the per-head-dimension ones
+  // the reference generates on demand (lib/metal_dispatch_common.ml:166-189)
+  static const char *const dense[] = {"llmopt_attention_f16",           "llmopt_attention_f16_simd_h64",
+                                      "llmopt_attention_f16_simd_h128", "llmopt_attention_f16_simd_h256",
+                                      "llmopt_attention_f16_simd_h512"};
+  for (const char *name : dense) table.push_back({name, attention, dense_attention});
   // Extension: per-sequence context lengths and slot tables in one launch.
   table.push_back({"llmopt_attention_q8_paged_batched", attention, paged_attention_batched});
 }

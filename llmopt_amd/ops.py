@@ -46,6 +46,7 @@ OPERATOR_SYMBOLS = (
     "llmopt_op_context_create", "llmopt_op_context_release", "llmopt_op_context_set_batch",
     "llmopt_op_last_kernels", "llmopt_op_w4a16_linear", "llmopt_op_w4a16_qkv_linear",
     "llmopt_op_w4a16_swiglu_ffn", "llmopt_op_w4a16_lm_head_argmax", "llmopt_op_paged_attention_q8",
+    "llmopt_op_attention",
     "llmopt_op_paged_attention_kernel_name", "llmopt_op_linear_f16_grid", "llmopt_op_simd_rows_grid",
     "llmopt_op_parameters_paged_attention_q8", "llmopt_op_kernel_operation",
 )
@@ -71,6 +72,7 @@ def _lib() -> ctypes.CDLL:
         handle.llmopt_op_w4a16_lm_head_argmax.argtypes = [vp, i64, i64, i64, dbl, values, sz, values, values, sz]
         handle.llmopt_op_paged_attention_q8.argtypes = [vp, ctypes.POINTER(_CPagedConfig), values, values,
                                                         values, values, values, values, sz, values]
+        handle.llmopt_op_attention.argtypes = [vp, dbl, ctypes.c_int, values, values, values, values, values]
         handle.llmopt_op_paged_attention_kernel_name.argtypes = [ctypes.c_int, ctypes.c_int, i64, i64, i64]
         handle.llmopt_op_paged_attention_kernel_name.restype = ctypes.c_char_p
         handle.llmopt_op_linear_f16_grid.argtypes = [i64]
@@ -180,6 +182,12 @@ class Operators:
         return self._done(_lib().llmopt_op_w4a16_lm_head_argmax(
             self._handle, m, n, k, float(epsilon), _values(values), len(values), _values([output]),
             _values(extra_outputs), len(extra_outputs)))
+
+    def attention(self, *, scale: float, causal: bool, query, key, value, mask, output) -> list[str]:
+        """dispatch_attention (lib/metal_dispatch_attention.ml:6-102): dense fp16 attention."""
+        return self._done(_lib().llmopt_op_attention(
+            self._handle, float(scale), int(bool(causal)), _values([query]), _values([key]), _values([value]),
+            _values([mask]) if mask is not None else None, _values([output])))
 
     def paged_attention_q8(self, *, config: dict, query, current_key, current_value, pool, slots, mask_values,
                            output) -> list[str]:

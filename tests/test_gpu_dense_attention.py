@@ -1,0 +1,239 @@
+"""GPU parity of dense fp16 attention (llmopt_attention_f16 and its per-head-dimension
+entries) against the CPU oracle and the reference's own smoke vectors."""
+import math
+import struct
+
+import numpy as np
+import pytest
+
+import oracle
+from tests.gpu_util import assert_close_to_oracle
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def runtime():
+    from llmopt_amd.native import Runtime
+    rt = Runtime()
+    yield rt
+    rt.close()
+
+
+def attention_params(batches, heads, query_length, key_length, head_dim, mask_batches, mask_heads, causal,
+                     scale, kv_heads, token_first_output=0, past_length=0, token_first_value=0,
+                     mask_dtype=0):
+    """Metal_parameters.attention (lib/metal_parameters.ml:95-117): 56 bytes."""
+    return struct.pack("<8IfIIIII", batches, heads, query_length, key_length, head_dim, mask_batches,
+                       mask_heads, 1 if causal else 0, scale, kv_heads, token_first_output, past_length,
+                       token_first_value, mask_dtype)
+
+
+def run(runtime, name, query, key, value, mask, params, out_shape):
+    b_query = runtime.buffer_of_bytes(query)
+    buffers = [b_query, runtime.buffer_of_bytes(key), runtime.buffer_of_bytes(value),
+               runtime.buffer_of_bytes(mask) if mask is not None else b_query]
+    out = runtime.create_buffer(int(np.prod(out_shape)) * 2)
+    # poison the output: rows the kernel must zero are then seen to be written
+    out.write(np.full(int(np.prod(out_shape)), 0x7e00, dtype=np.uint16))
+    rows = query.shape[0] * query.shape[1] * query.shape[2]
+    runtime.dispatch(name, buffers + [out], params, grid=(rows, 1, 1), group=(64, 1, 1))
+    return out.numpy(np.float16, out_shape)
+
+
+def expected(query, key, value, allowed, scale):
+    """Oracle (Cpu.attention semantics) with GQA expanded and every rule folded into one mask
+    [b, h, q, L] of allowed keys."""
+    b, h, q, d = query.shape
+    kvh = key.shape[1]
+    repeat = h // kvh
+    key_e = np.repeat(key, repeat, axis=1)
+    value_e = np.repeat(value, repeat, axis=1)
+    return oracle.attention(query, key_e, value_e, allowed.astype(np.float32), scale, causal=False)
+
+
+def test_reference_smoke_vector_2x2(runtime):
+    """bin/ocaml_metal_primitives_smoke.ml:221-228,382-383: Q = K = I, V = diag(10, 20),
+    bool mask [T, F; F, T], scale 1 -> the values themselves."""
+    bits = lambda *v: np.array(v, dtype=np.uint16).view(np.float16).reshape(1, 1, 2, 2)
+    query = bits(0x3c00, 0, 0, 0x3c00)
+    value = bits(0x4900, 0, 0, 0x4d00)
+    mask = np.array([1, 0, 0, 1], dtype=np.uint8)
+    params = attention_params(1, 1, 2, 2, 2, 1, 1, False, 1.0, 1, mask_dtype=1)
+    got = run(runtime, "llmopt_attention_f16", query, query, value, mask, params, (1, 1, 2, 2))
+    assert got.view(np.uint16).reshape(-1).tolist() == [0x4900, 0, 0, 0x4d00]
+
+
+def test_reference_smoke_vector_wide(runtime):
+    """bin/native_schedule_fixture.ml:278-294, bin/ocaml_metal_primitives_smoke.ml:229-237,384-386:
+    D = 256, two query heads on one KV head, f16 mask [0, -inf; 0, 0], token-major output
+    [1, 2, 512]: first token sees key 0 only (1.0), second the mean of 1.0 and 3.0."""
+    query = np.zeros((1, 2, 2, 256), dtype=np.float16)
+    key = np.zeros((1, 1, 2, 256), dtype=np.float16)
+    value = np.empty((1, 1, 2, 256), dtype=np.float16)
+    value[0, 0, 0] = 1.0
+    value[0, 0, 1] = 3.0
+    mask = np.array([0, 0xfc00, 0, 0], dtype=np.uint16)
+    params = attention_params(1, 2, 2, 2, 256, 1, 1, False, 1.0, 1, token_first_output=1, mask_dtype=2)
+    for name in ("llmopt_attention_f16_simd_h256", "llmopt_attention_f16"):
+        got = run(runtime, name, query, key, value, mask, params, (1, 2, 512))
+        bits = got.view(np.uint16).reshape(-1)
+        assert np.all(bits[:512] == 0x3c00) and np.all(bits[512:] == 0x4000), name
+
+
+@pytest.mark.parametrize("dim,heads,kv_heads,length", [(64, 9, 3, 200), (128, 8, 2, 150), (64, 2, 2, 33),
+                                                      (128, 4, 1, 512)])
+def test_causal_prefill_matches_oracle(runtime, dim, heads, kv_heads, length):
+    rng = np.random.default_rng(dim + length)
+    batches = 2
+    query = rng.standard_normal((batches, heads, length, dim)).astype(np.float16)
+    key = rng.standard_normal((batches, kv_heads, length, dim)).astype(np.float16)
+    value = rng.standard_normal((batches, kv_heads, length, dim)).astype(np.float16)
+    scale = 1.0 / math.sqrt(dim)
+    params = attention_params(batches, heads, length, length, dim, 0, 0, True, scale, kv_heads)
+    got = run(runtime, f"llmopt_attention_f16_simd_h{dim}", query, key, value, None, params,
+              (batches, heads, length, dim))
+    allowed = np.tril(np.ones((length, length), dtype=bool))[None, None]
+    want = expected(query, key, value, np.broadcast_to(allowed, (batches, heads, length, length)), scale)
+    assert_close_to_oracle(got, want, f"causal prefill D={dim} L={length}")
+
+
+@pytest.mark.parametrize("dim", [64, 128])
+def test_chunked_prefill_with_past_and_token_major_layouts(runtime, dim):
+    """A second prefill chunk: 40 new tokens after 100 cached ones, V and the output token-major."""
+    rng = np.random.default_rng(11 + dim)
+    batches, heads, kv_heads, new, past = 1, 6, 2, 40, 100
+    length = past + new
+    query = rng.standard_normal((batches, heads, new, dim)).astype(np.float16)
+    key = rng.standard_normal((batches, kv_heads, length, dim)).astype(np.float16)
+    value = rng.standard_normal((batches, kv_heads, length, dim)).astype(np.float16)
+    value_token_major = np.ascontiguousarray(value.transpose(0, 2, 1, 3))
+    scale = 0.11
+    params = attention_params(batches, heads, new, length, dim, 0, 0, True, scale, kv_heads,
+                              token_first_output=1, past_length=past, token_first_value=1)
+    got = run(runtime, f"llmopt_attention_f16_simd_h{dim}", query, key, value_token_major, None, params,
+              (batches, new, heads, dim))
+    allowed = (np.arange(length)[None, :] <= past + np.arange(new)[:, None])[None, None]
+    want = expected(query, key, value, np.broadcast_to(allowed, (batches, heads, new, length)), scale)
+    assert_close_to_oracle(got.transpose(0, 2, 1, 3), want, f"chunked prefill D={dim}")
+
+
+@pytest.mark.parametrize("mask_dtype", [1, 2])
+@pytest.mark.parametrize("dim", [64, 96])
+def test_masks_and_rows_without_keys(runtime, mask_dtype, dim):
+    """Random masks (bool / f16), broadcast over heads, one query row with no allowed key -> zeros.
+    D = 96 takes the row-serial kernel, D = 64 the matrix-core one."""
+    rng = np.random.default_rng(5 + mask_dtype + dim)
+    batches, heads, kv_heads, q_len, length = 2, 4, 4, 37, 70
+    query = rng.standard_normal((batches, heads, q_len, dim)).astype(np.float16)
+    key = rng.standard_normal((batches, kv_heads, length, dim)).astype(np.float16)
+    value = rng.standard_normal((batches, kv_heads, length, dim)).astype(np.float16)
+    allowed = rng.random((batches, 1, q_len, length)) < 0.6
+    allowed[1, 0, 5, :] = False
+    if mask_dtype == 1:
+        mask = allowed.astype(np.uint8)
+    else:
+        mask = np.where(allowed, 0.0, -np.inf).astype(np.float16)
+    scale = 1.0 / math.sqrt(dim)
+    params = attention_params(batches, heads, q_len, length, dim, batches, 1, False, scale, kv_heads,
+                              mask_dtype=mask_dtype)
+    name = f"llmopt_attention_f16_simd_h{dim}" if dim == 64 else "llmopt_attention_f16"
+    got = run(runtime, name, query, key, value, mask, params, (batches, heads, q_len, dim))
+    want = expected(query, key, value, np.broadcast_to(allowed, (batches, heads, q_len, length)), scale)
+    assert np.all(got[1, :, 5, :].view(np.uint16) == 0)
+    assert_close_to_oracle(got, want, f"masked attention dtype={mask_dtype} D={dim}")
+
+
+def test_single_query_row_and_tiny_shapes(runtime):
+    rng = np.random.default_rng(21)
+    for dim, q_len, length in ((64, 1, 17), (128, 3, 5), (8, 4, 9)):
+        query = rng.standard_normal((1, 2, q_len, dim)).astype(np.float16)
+        key = rng.standard_normal((1, 2, length, dim)).astype(np.float16)
+        value = rng.standard_normal((1, 2, length, dim)).astype(np.float16)
+        params = attention_params(1, 2, q_len, length, dim, 0, 0, False, 0.3, 2)
+        got = run(runtime, "llmopt_attention_f16", query, key, value, None, params, (1, 2, q_len, dim))
+        want = expected(query, key, value, np.ones((1, 2, q_len, length), dtype=bool), 0.3)
+        assert_close_to_oracle(got, want, f"tiny D={dim} q={q_len} L={length}")
+
+
+def test_softmax_shift_invariance_at_full_size(runtime):
+    """Prefill 2048 x 2048, D = 128: a property the oracle is too slow for.  With every key equal
+    the output is the running mean of V (closed form), whatever the scores are."""
+    rng = np.random.default_rng(77)
+    heads, kv_heads, length, dim = 4, 1, 2048, 128
+    query = rng.standard_normal((1, heads, length, dim)).astype(np.float16)
+    key = np.broadcast_to(rng.standard_normal((1, kv_heads, 1, dim)).astype(np.float16),
+                          (1, kv_heads, length, dim)).copy()
+    value = rng.standard_normal((1, kv_heads, length, dim)).astype(np.float16)
+    params = attention_params(1, heads, length, length, dim, 0, 0, True, 1.0 / math.sqrt(dim), kv_heads)
+    got = run(runtime, "llmopt_attention_f16_simd_h128", query, key, value, None, params,
+              (1, heads, length, dim))
+    running_mean = np.cumsum(value[0, 0].astype(np.float64), axis=0) / np.arange(1, length + 1)[:, None]
+    want = np.broadcast_to(running_mean[None, None], (1, heads, length, dim))
+    assert_close_to_oracle(got, want, "equal keys -> running mean of V")
+
+
+def test_prefill_then_q8_pack_then_paged_decode(runtime):
+    """The step on the other side of the KV cache: prefill attention over fp16 K/V, the same K/V
+    quantised into the pool (lib/serving_engine.ml:409-421), then one decode step over the pool.
+    The decode row must agree with dense attention over the dequantised cache (oracle) and, to
+    quantisation error, with dense attention over the fp16 K/V."""
+    from oracle import CacheParams, PagedParams
+    rng = np.random.default_rng(31)
+    heads, kv_heads, dim, length = 8, 2, 128, 96
+    token_elements = 2 * kv_heads * dim
+    stride = token_elements + 2 * (token_elements // 64)
+    key = rng.standard_normal((1, kv_heads, length, dim)).astype(np.float16)
+    value = rng.standard_normal((1, kv_heads, length, dim)).astype(np.float16)
+    slots = rng.permutation(length).astype(np.uint32)
+    pool = runtime.buffer_of_bytes(np.zeros(length * stride, dtype=np.uint8))
+    runtime.dispatch("llmopt_cache_pack_attention_q8_pair_simd",
+                     [runtime.buffer_of_bytes(key), runtime.buffer_of_bytes(value),
+                      runtime.buffer_of_bytes(slots), pool],
+                     struct.pack("<11I", length, 0, kv_heads * dim, kv_heads, dim, 64, token_elements,
+                                 token_elements // 64, stride, length, 0),
+                     grid=(length * kv_heads * 32, 1, 1), group=(256, 1, 1))
+    query = rng.standard_normal((1, heads, 1, dim)).astype(np.float16)
+    current_key = rng.standard_normal((1, kv_heads, 1, dim)).astype(np.float16)
+    current_value = rng.standard_normal((1, kv_heads, 1, dim)).astype(np.float16)
+    scale = 1.0 / math.sqrt(dim)
+    out = runtime.create_buffer(heads * dim * 2)
+    b_slots = runtime.buffer_of_bytes(slots)
+    runtime.dispatch("llmopt_attention_q8_paged_simd_generic",
+                     [runtime.buffer_of_bytes(query), runtime.buffer_of_bytes(current_key),
+                      runtime.buffer_of_bytes(current_value), pool, b_slots, b_slots, out],
+                     struct.pack("<12IfIII", 1, heads, kv_heads, length, dim, 0, 0, token_elements, 0,
+                                 kv_heads * dim, 64, stride, scale, 1, 0, 0),
+                     grid=(256, 1, 1), group=(256, 1, 1))
+    decode = out.numpy(np.float16, (1, 1, heads, dim))
+    host_pool = pool.numpy(np.uint8, (length * stride,))
+    paged = oracle.paged_attention_q8(
+        query, current_key, current_value, host_pool, slots, None,
+        PagedParams(batches=1, query_heads=heads, kv_heads=kv_heads, past_length=length, head_dim=dim,
+                    mask_batches=0, mask_heads=0, token_elements=token_elements, key_offset=0,
+                    value_offset=kv_heads * dim, group_size=64, token_stride=stride, scale=scale,
+                    query_length=1, mask_dtype=0, window=0))
+    assert_close_to_oracle(decode, paged, "decode over the packed prefill cache")
+    # dense attention of the same query over [prefill K/V ; current K/V] in fp16
+    all_key = np.concatenate([key, current_key], axis=2)
+    all_value = np.concatenate([value, current_value], axis=2)
+    params = attention_params(1, heads, 1, length + 1, dim, 0, 0, True, scale, kv_heads,
+                              token_first_output=1, past_length=length)
+    dense = run(runtime, "llmopt_attention_f16_simd_h128", query, all_key, all_value, None, params,
+                (1, 1, heads, dim))
+    difference = decode.astype(np.float64) - dense.astype(np.float64)
+    relative = np.linalg.norm(difference) / np.linalg.norm(dense.astype(np.float64))
+    assert relative < 2e-2, f"Q8 cache changes the decode row by {relative:.3e}"
+
+
+def test_rejects_bad_arguments(runtime):
+    query = np.zeros((1, 2, 4, 64), dtype=np.float16)
+    key = np.zeros((1, 2, 4, 64), dtype=np.float16)
+    good = attention_params(1, 2, 4, 4, 64, 0, 0, False, 1.0, 2)
+    with pytest.raises(Exception):
+        run(runtime, "llmopt_attention_f16", query, key[:, :, :2], key, None, good, (1, 2, 4, 64))
+    with pytest.raises(Exception):
+        run(runtime, "llmopt_attention_f16", query, key, key, None, good[:40], (1, 2, 4, 64))
+    bad_heads = attention_params(1, 2, 4, 4, 64, 0, 0, False, 1.0, 3)
+    with pytest.raises(Exception):
+        run(runtime, "llmopt_attention_f16", query, key, key, None, bad_heads, (1, 2, 4, 64))

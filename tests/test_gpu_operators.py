@@ -195,3 +195,50 @@ def test_dispatch_paged_attention_q8(runtime, operators, heads, kvh, dim, kernel
     arguments["query"] = Value(arguments["query"].buffer, F16, (batches, heads, dim))
     with pytest.raises(ops.LlmoptError, match=r"query must have shape \[b,h,q,d\]"):
         operators.paged_attention_q8(**arguments)
+
+
+@pytest.mark.parametrize("dim,kernel", [(64, "llmopt_attention_f16_simd_h64"), (128, "llmopt_attention_f16_simd_h128"),
+                                        (20, "llmopt_attention_f16")])
+def test_dispatch_attention(runtime, operators, dim, kernel):
+    """dispatch_attention: layouts read off the value shapes, past_length = L - q, kernel by head
+    dimension (lib/metal_dispatch_attention.ml:6-102, lib/metal_dispatch_common.ml:166-189)."""
+    rng = np.random.default_rng(dim)
+    batches, heads, kv_heads, q_len, length = 1, 4, 2, 24, 40
+    query = rng.standard_normal((batches, heads, q_len, dim)).astype(np.float16)
+    key = rng.standard_normal((batches, kv_heads, length, dim)).astype(np.float16)
+    value = rng.standard_normal((batches, kv_heads, length, dim)).astype(np.float16)
+    value_tm = np.ascontiguousarray(value.transpose(0, 2, 1, 3))
+    out = runtime.create_buffer(batches * q_len * heads * dim * 2)
+    scale = 1.0 / math.sqrt(dim)
+    kernels = operators.attention(
+        scale=scale, causal=True,
+        query=Value(runtime.buffer_of_bytes(query), F16, query.shape),
+        key=Value(runtime.buffer_of_bytes(key), F16, key.shape),
+        value=Value(runtime.buffer_of_bytes(value_tm), F16, value_tm.shape), mask=None,
+        output=Value(out, F16, (batches, q_len, heads * dim)))
+    assert kernels == [kernel]
+    got = out.numpy(np.float16, (batches, q_len, heads, dim)).transpose(0, 2, 1, 3)
+    allowed = (np.arange(length)[None, :] <= (length - q_len) + np.arange(q_len)[:, None])[None, None]
+    want = oracle.attention(query, np.repeat(key, 2, axis=1), np.repeat(value, 2, axis=1),
+                            np.broadcast_to(allowed, (batches, heads, q_len, length)).astype(np.float32), scale)
+    assert_close_to_oracle(got, want, f"dispatch_attention D={dim}")
+
+
+def test_dispatch_attention_errors(runtime, operators):
+    buffer = runtime.create_buffer(4096)
+    q = Value(buffer, F16, (1, 2, 4, 64))
+    with pytest.raises(ops.LlmoptError, match="attention query must have rank four"):
+        operators.attention(scale=1.0, causal=False, query=Value(buffer, F16, (2, 4, 64)), key=q, value=q,
+                            mask=None, output=q)
+    with pytest.raises(ops.LlmoptError, match="attention key must have rank four"):
+        operators.attention(scale=1.0, causal=False, query=q, key=Value(buffer, F16, (2, 4, 64)), value=q,
+                            mask=None, output=q)
+    with pytest.raises(ops.LlmoptError, match="attention value must match key in head-major or token-major layout"):
+        operators.attention(scale=1.0, causal=False, query=q, key=q, value=Value(buffer, F16, (1, 2, 3, 64)),
+                            mask=None, output=q)
+    with pytest.raises(ops.LlmoptError, match="attention mask must have rank four"):
+        operators.attention(scale=1.0, causal=False, query=q, key=q, value=q,
+                            mask=Value(buffer, BOOL, (4, 4)), output=q)
+    with pytest.raises(ops.LlmoptError, match="attention mask dtype"):
+        operators.attention(scale=1.0, causal=False, query=q, key=q, value=q,
+                            mask=Value(buffer, F32, (1, 1, 4, 4)), output=q)
