@@ -65,7 +65,9 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void dense_attention_mfma_kern
   const uint32_t quad = lane >> 4;
   const uint32_t head = blockIdx.y;
   const uint32_t batch = blockIdx.z;
-  const uint32_t q0 = (blockIdx.x * kWavesPerBlock + wave) * (kQueryTiles * 16);
+  // with a causal limit the last rows see the most keys: hand them out first
+  const uint32_t slab = a.causal ? gridDim.x - 1 - blockIdx.x : blockIdx.x;
+  const uint32_t q0 = (slab * kWavesPerBlock + wave) * (kQueryTiles * 16);
   if (q0 >= a.query_length) return;  // whole wave; the kernel has no barriers
   const uint32_t kv_heads = a.kv_heads > 0 ? a.kv_heads : a.heads;
   const uint32_t kv_head = kv_heads < a.heads ? head / (a.heads / kv_heads) : head;
@@ -154,14 +156,26 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void dense_attention_mfma_kern
       for (int j = 0; j < QSTEPS; ++j)
         score = __builtin_amdgcn_mfma_f32_16x16x32_f16(k_frag[j], q_frag[t][j], score, 0, 0, 0);
       float tile_max = -INFINITY;
+      // a tile of existing keys, all below the causal limit of the tile's first row, of
+      // existing rows and without a mask needs no per-score test
+      const bool interior = !masked && key0 + 16 <= L && q0 + t * 16 + 16 <= a.query_length &&
+                            (!a.causal || key0 + 15 <= a.past_length + q0 + t * 16);
+      if (interior) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const uint32_t key = key0 + quad * 4 + i;
-        bool allowed = key < L && row < a.query_length;
-        if (a.causal) allowed = allowed && key <= a.past_length + row;
-        if (masked && allowed) allowed = mask_allows(a, batch, head, row, key);
-        score[i] = allowed ? score[i] * score_scale : -INFINITY;
-        tile_max = fmaxf(tile_max, score[i]);
+        for (int i = 0; i < 4; ++i) {
+          score[i] *= score_scale;
+          tile_max = fmaxf(tile_max, score[i]);
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const uint32_t key = key0 + quad * 4 + i;
+          bool allowed = key < L && row < a.query_length;
+          if (a.causal) allowed = allowed && key <= a.past_length + row;
+          if (masked && allowed) allowed = mask_allows(a, batch, head, row, key);
+          score[i] = allowed ? score[i] * score_scale : -INFINITY;
+          tile_max = fmaxf(tile_max, score[i]);
+        }
       }
       tile_max = lanes_xor_max(tile_max, 16);
       tile_max = lanes_xor_max(tile_max, 32);
