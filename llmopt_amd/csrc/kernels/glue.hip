@@ -153,20 +153,74 @@ __device__ __forceinline__ bool better(float value, uint32_t index, float best_v
   return value > best_value || (value == best_value && index < best_index);
 }
 
-// thread t of row `blockIdx.x` scans columns t, t + 256, ...
-__global__ __launch_bounds__(256) void argmax_candidates_kernel(const float *logits, Candidate *candidates,
-                                                               uint32_t n) {
+// 256 (value, index) candidates per row, the record the reference's stage 1
+// hands to its reduce kernel (lib/metal_w4a16_source.ml:1256-1283; there one
+// candidate per threadgroup of columns, here candidate t is the best of columns
+// t, t + 256, ... - the reduce step only needs every column covered once and
+// ties resolved to the lowest index).  Four slices of 256 threads scan a quarter
+// of those columns each with several independent loads in flight, then meet in
+// LDS: a single thread per candidate would walk its 192 columns of a 49152-wide
+// vocabulary one load latency at a time.
+constexpr int kArgmaxSlices = 4;
+constexpr int kArgmaxUnroll = 4;
+
+__global__ __launch_bounds__(256 * kArgmaxSlices) void argmax_candidates_kernel(const float *logits,
+                                                                                Candidate *candidates,
+                                                                                uint32_t n) {
+  __shared__ float slice_values[kArgmaxSlices][256];
+  __shared__ uint32_t slice_indices[kArgmaxSlices][256];
   const uint32_t row = blockIdx.x;
+  const uint32_t t = threadIdx.x & 255;
+  const uint32_t slice = threadIdx.x >> 8;
+  const float *row_logits = logits + (size_t)row * n;
   float best_value = -3.402823466e+38f;
   uint32_t best_index = 0;
-  for (uint32_t col = threadIdx.x; col < n; col += 256) {
-    const float value = logits[(size_t)row * n + col];
-    if (better(value, col, best_value, best_index)) {
+  bool found = false;
+  const uint32_t step = 256 * kArgmaxSlices;
+  uint32_t col = t + 256 * slice;
+  // columns are visited in increasing order, so `>` alone keeps the lowest index among equals
+  for (; col + (kArgmaxUnroll - 1) * step < n; col += kArgmaxUnroll * step) {
+    float value[kArgmaxUnroll];
+#pragma unroll
+    for (int u = 0; u < kArgmaxUnroll; ++u) value[u] = row_logits[col + u * step];
+#pragma unroll
+    for (int u = 0; u < kArgmaxUnroll; ++u)
+      if (!found || value[u] > best_value) {
+        best_value = value[u];
+        best_index = col + u * step;
+        found = true;
+      }
+  }
+  for (; col < n; col += step) {
+    const float value = row_logits[col];
+    if (!found || value > best_value) {
       best_value = value;
       best_index = col;
+      found = true;
     }
   }
-  candidates[row * 256 + threadIdx.x] = {best_value, best_index};
+  // a slice that saw no column keeps (lowest float, index 0), which never beats a real column
+  // except against equal values at a higher index - impossible for index 0
+  slice_values[slice][t] = found ? best_value : -3.402823466e+38f;
+  slice_indices[slice][t] = found ? best_index : 0xffffffffu;
+  __syncthreads();
+  if (slice == 0) {
+    float value = slice_values[0][t];
+    uint32_t index = slice_indices[0][t];
+#pragma unroll
+    for (int other = 1; other < kArgmaxSlices; ++other)
+      if (slice_indices[other][t] != 0xffffffffu &&
+          (index == 0xffffffffu || better(slice_values[other][t], slice_indices[other][t], value, index))) {
+        value = slice_values[other][t];
+        index = slice_indices[other][t];
+      }
+    // a candidate with no column at all (n <= t): the reference's initial (lowest float, 0)
+    if (index == 0xffffffffu) {
+      value = -3.402823466e+38f;
+      index = 0;
+    }
+    candidates[row * 256 + t] = {value, index};
+  }
 }
 
 // lib/metal_w4a16_source.ml:1287-1315
@@ -263,7 +317,7 @@ hipError_t launch_copy_bytes(void *destination, const void *source, size_t bytes
 
 hipError_t launch_argmax_candidates(const float *logits, void *candidates, uint32_t rows, uint32_t n,
                                     hipStream_t stream) {
-  hipLaunchKernelGGL(argmax_candidates_kernel, dim3(rows), dim3(256), 0, stream, logits,
+  hipLaunchKernelGGL(argmax_candidates_kernel, dim3(rows), dim3(256 * kArgmaxSlices), 0, stream, logits,
                      static_cast<Candidate *>(candidates), n);
   return hipGetLastError();
 }
