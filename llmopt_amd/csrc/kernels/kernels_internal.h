@@ -17,6 +17,11 @@ hipError_t launch_w4a16_gemv_dual_swiglu(const W4DualSwigluArgs &args, hipStream
 // true when K does not fit one workgroup (more than 16 ranges of 256): only the plain
 // linear can then run (it splits K over workgroups and needs scratch)
 bool w4a16_gemv_mfma_needs_split(uint32_t k);
+// kGemvMaxRows < m <= 32 with small weights and a K one workgroup covers: the
+// same kernel once per group of 8 rows (the weights are re-read from L2), which
+// beats a handful of 128-wide GEMM tiles on 256 CUs.  `columns` = all outputs
+// of the launch (three matrices of a QKV launch, two of a SwiGLU pair).
+bool w4a16_gemv_mfma_row_groups_ok(uint32_t m, uint64_t columns, uint32_t k);
 hipError_t launch_w4a16_gemv_mfma_linear(const W4LinearArgs &args, hipStream_t stream);
 hipError_t launch_w4a16_gemv_mfma_qkv(const W4QkvArgs &args, hipStream_t stream);
 hipError_t launch_w4a16_gemv_mfma_dual_swiglu(const W4DualSwigluArgs &args, hipStream_t stream);

@@ -363,19 +363,23 @@ hipError_t launch_w4a16_linear(const W4LinearArgs &args, hipStream_t stream) {
   if (args.m <= kGemvDotRows) return launch_w4a16_gemv_linear(args, stream);
   if (args.m <= kGemvMaxRows && (!w4a16_gemv_mfma_needs_split(args.k) || args.workspace != nullptr))
     return launch_w4a16_gemv_mfma_linear(args, stream);
+  if (w4a16_gemv_mfma_row_groups_ok(args.m, args.n, args.k) && args.y_f32 == nullptr)
+    return launch_w4a16_gemv_mfma_linear(args, stream);
   return launch_w4a16_gemm_linear(args, stream);
 }
 
 hipError_t launch_w4a16_dual_swiglu(const W4DualSwigluArgs &args, hipStream_t stream) {
   if (args.m <= kGemvDotRows) return launch_w4a16_gemv_dual_swiglu(args, stream);
-  if (args.m <= kGemvMaxRows && !w4a16_gemv_mfma_needs_split(args.k))
+  if ((args.m <= kGemvMaxRows && !w4a16_gemv_mfma_needs_split(args.k)) ||
+      w4a16_gemv_mfma_row_groups_ok(args.m, 2ull * args.n, args.k))
     return launch_w4a16_gemv_mfma_dual_swiglu(args, stream);
   return launch_w4a16_gemm_dual_swiglu(args, stream);
 }
 
 hipError_t launch_w4a16_qkv(const W4QkvArgs &args, hipStream_t stream) {
   if (args.m <= kGemvDotRows) return launch_w4a16_gemv_qkv(args, stream);
-  if (args.m <= kGemvMaxRows && !w4a16_gemv_mfma_needs_split(args.k))
+  if ((args.m <= kGemvMaxRows && !w4a16_gemv_mfma_needs_split(args.k)) ||
+      w4a16_gemv_mfma_row_groups_ok(args.m, (uint64_t)args.n[0] + args.n[1] + args.n[2], args.k))
     return launch_w4a16_gemv_mfma_qkv(args, stream);
   // prefill: three GEMMs sharing the activation through L2
   for (int i = 0; i < 3; ++i) {

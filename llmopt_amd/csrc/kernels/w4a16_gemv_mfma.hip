@@ -73,6 +73,7 @@ struct MfmaGemvParams {
   float *partials;     // [gridDim.y][8][n] fp32, used when gridDim.y > 1
   uint32_t *counters;  // one per tile, zero between launches
   float *y_f32;        // optional float32 copy of mat0's output, may be null
+  uint32_t row_groups;  // > 1: blockIdx.y is a group of 8 activation rows instead of a K slice
 };
 
 // NB = tiles in flight per wave (= tiles between two workgroup reductions)
@@ -91,10 +92,15 @@ __global__ __launch_bounds__(kMaxWaves * 64) void w4a16_gemv_mfma_kernel(MfmaGem
   if (blockIdx.x >= tile_groups) return;  // a shorter matrix of a QKV launch (whole workgroup)
   const uint32_t rounds = (tile_groups - blockIdx.x + gridDim.x - 1) / gridDim.x;
 
+  // blockIdx.y: K slice (long K, at most 8 rows) or group of 8 activation rows (short K, up to 32 rows)
+  const uint32_t row0 = p.row_groups > 1 ? blockIdx.y * 8 : 0;
+  const uint32_t rows = min(8u, p.m - row0);
+  const uint32_t slice = p.row_groups > 1 ? 0 : blockIdx.y;
+  const uint32_t slices = p.row_groups > 1 ? 1 : gridDim.y;
   const uint32_t K = p.k;
   const uint32_t groups_total = K >> 6;
-  const uint32_t slice_end = min(K, (blockIdx.y + 1) * p.k_slice);
-  const uint32_t k0 = blockIdx.y * p.k_slice + wk * kStepK;  // first K value of this wave
+  const uint32_t slice_end = min(K, (slice + 1) * p.k_slice);
+  const uint32_t k0 = slice * p.k_slice + wk * kStepK;  // first K value of this wave
   const uint32_t valid_groups = k0 >= slice_end ? 0 : min(4u, (slice_end - k0) >> 6);
 
   // ---- lane roles -----------------------------------------------------------------
@@ -156,7 +162,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void w4a16_gemv_mfma_kernel(MfmaGem
       const uint32_t row = 2 * i + (lane >> 5);
       const uint32_t kk = k0 + x_piece * 8;
       x_loaded[i] =
-          *reinterpret_cast<const uint4 *>(p.x + (size_t)min(row, p.m - 1) * K + min(kk, K - 8));
+          *reinterpret_cast<const uint4 *>(p.x + (size_t)(row0 + min(row, rows - 1)) * K + min(kk, K - 8));
     }
   }
   // all tiles of the ring go out next
@@ -167,7 +173,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void w4a16_gemv_mfma_kernel(MfmaGem
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const uint32_t row = 2 * i + (lane >> 5);
-      const bool keep = (row < p.m) & (k0 + x_piece * 8 < slice_end);
+      const bool keep = (row < rows) & (k0 + x_piece * 8 < slice_end);
       const uint4 ordered = pair_order(x_loaded[i]);
       uint4 value;
       value.x = keep ? ordered.x : 0u;
@@ -243,7 +249,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void w4a16_gemv_mfma_kernel(MfmaGem
   auto flush = [&](uint32_t first_round, uint32_t count) __attribute__((always_inline)) {
     __syncthreads();
     const uint32_t outputs = count * p.waves_t * 8 * TN;
-    const bool split = !DUAL && gridDim.y > 1;
+    const bool split = !DUAL && slices > 1;
     for (uint32_t base = 0; base < outputs; base += blockDim.x) {  // uniform trip count
       const uint32_t o = base + threadIdx.x;
       const bool in_range = o < outputs;
@@ -252,7 +258,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void w4a16_gemv_mfma_kernel(MfmaGem
       const uint32_t m = (o >> 4) & 7, col_in_tile = o & 15;
       const uint32_t tile = (blockIdx.x + (first_round + slot) * gridDim.x) * p.waves_t + lane_t;
       const uint32_t col = tile * TN + col_in_tile;
-      const bool writer = in_range && tile < tiles && m < p.m && col < mat.n;
+      const bool writer = in_range && tile < tiles && m < rows && col < mat.n;
       float total[NW];
 #pragma unroll
       for (int v = 0; v < NW; ++v) total[v] = 0.0f;
@@ -278,13 +284,13 @@ __global__ __launch_bounds__(kMaxWaves * 64) void w4a16_gemv_mfma_kernel(MfmaGem
         // (device-scope stores and loads, no cache write-back needed); the last
         // workgroup to arrive at a tile adds the slices in order.
         if (writer)
-          __hip_atomic_store(p.partials + ((size_t)blockIdx.y * 8 + m) * mat.n + col, total[0], __ATOMIC_RELAXED,
+          __hip_atomic_store(p.partials + ((size_t)slice * 8 + m) * mat.n + col, total[0], __ATOMIC_RELAXED,
                              __HIP_MEMORY_SCOPE_AGENT);
         __syncthreads();  // waits for the stores of every wave
         if (in_range && (o & 127) == 0 && tile < tiles) {
           const uint32_t arrived =
               __hip_atomic_fetch_add(p.counters + tile, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-          const bool last = arrived == gridDim.y - 1;
+          const bool last = arrived == slices - 1;
           if (last) __hip_atomic_store(p.counters + tile, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
           flag_lds[slot_tile] = last ? 1u : 0u;
         }
@@ -292,8 +298,8 @@ __global__ __launch_bounds__(kMaxWaves * 64) void w4a16_gemv_mfma_kernel(MfmaGem
         store = writer && flag_lds[slot_tile] != 0;
         if (store) {
           float sum = 0.0f;
-          for (uint32_t slice = 0; slice < gridDim.y; ++slice)
-            sum += __hip_atomic_load(p.partials + ((size_t)slice * 8 + m) * mat.n + col, __ATOMIC_RELAXED,
+          for (uint32_t other = 0; other < slices; ++other)
+            sum += __hip_atomic_load(p.partials + ((size_t)other * 8 + m) * mat.n + col, __ATOMIC_RELAXED,
                                      __HIP_MEMORY_SCOPE_AGENT);
           total[0] = sum;
         }
@@ -305,10 +311,10 @@ __global__ __launch_bounds__(kMaxWaves * 64) void w4a16_gemv_mfma_kernel(MfmaGem
           value = total[0] / (1.0f + __expf(-total[0])) * total[NW - 1];
         } else {
           value = total[0];
-          if (p.has_addend) value += half_bits_to_float(p.addend[(size_t)m * p.addend_stride + col]);
+          if (p.has_addend) value += half_bits_to_float(p.addend[(size_t)(row0 + m) * p.addend_stride + col]);
         }
-        if (mat.y != nullptr) mat.y[(size_t)m * mat.n + col] = float_to_half_bits(value);
-        if (!DUAL && p.y_f32 != nullptr) p.y_f32[(size_t)m * mat.n + col] = value;
+        if (mat.y != nullptr) mat.y[(size_t)(row0 + m) * mat.n + col] = float_to_half_bits(value);
+        if (!DUAL && p.y_f32 != nullptr) p.y_f32[(size_t)(row0 + m) * mat.n + col] = value;
       }
     }
     __syncthreads();  // the slots are free again
@@ -366,7 +372,7 @@ hipError_t launch_ring(const MfmaGemvParams &p, uint32_t matrices, const Plan &p
     if (status != hipSuccess) return status;
     configured = true;
   }
-  const dim3 grid(plan.blocks, plan.slices, matrices);
+  const dim3 grid(plan.blocks, p.row_groups > 1 ? p.row_groups : plan.slices, matrices);
   hipLaunchKernelGGL((w4a16_gemv_mfma_kernel<NB, DUAL>), grid, dim3(plan.waves_k * plan.waves_t * 64),
                      plan.lds_bytes, stream, p);
   return hipGetLastError();
@@ -395,6 +401,10 @@ size_t w4a16_gemv_workspace_bytes(uint32_t m, uint32_t n, uint32_t k) {
 
 bool w4a16_gemv_mfma_needs_split(uint32_t k) { return (k + kStepK - 1) / kStepK > (uint32_t)kMaxWaves; }
 
+bool w4a16_gemv_mfma_row_groups_ok(uint32_t m, uint64_t columns, uint32_t k) {
+  return m > kGemvMaxRows && m <= 32 && !w4a16_gemv_mfma_needs_split(k) && columns * k / 2 <= (4u << 20);
+}
+
 hipError_t launch_w4a16_gemv_mfma_linear(const W4LinearArgs &a, hipStream_t stream) {
   MfmaGemvParams p = {};
   p.x = a.x;
@@ -406,8 +416,10 @@ hipError_t launch_w4a16_gemv_mfma_linear(const W4LinearArgs &a, hipStream_t stre
   p.addend = a.addend;
   p.has_addend = a.has_addend;
   p.addend_stride = a.addend_row_stride;
-  const Plan plan = make_plan(a.k, a.n, 1, false);
+  p.row_groups = (a.m + 7) / 8;
+  const Plan plan = make_plan(a.k, a.n, p.row_groups, false);
   if (plan.slices > 1) {
+    if (p.row_groups > 1) return hipErrorInvalidValue;  // callers check w4a16_gemv_mfma_row_groups_ok
     const uint32_t tiles = (a.n + TN - 1) / TN;
     if (a.workspace == nullptr || a.counters == nullptr || tiles > a.counter_count ||
         a.workspace_bytes < w4a16_gemv_workspace_bytes(a.m, a.n, a.k))
@@ -427,7 +439,8 @@ hipError_t launch_w4a16_gemv_mfma_qkv(const W4QkvArgs &a, hipStream_t stream) {
   p.mat0 = {a.w[0].weight, a.w[0].scale, a.y[0], a.n[0]};
   p.mat1 = {a.w[1].weight, a.w[1].scale, a.y[1], a.n[1]};
   p.mat2 = {a.w[2].weight, a.w[2].scale, a.y[2], a.n[2]};
-  const Plan plan = make_plan(a.k, std::max(a.n[0], std::max(a.n[1], a.n[2])), 3, false);
+  p.row_groups = (a.m + 7) / 8;
+  const Plan plan = make_plan(a.k, std::max(a.n[0], std::max(a.n[1], a.n[2])), 3 * p.row_groups, false);
   if (plan.slices > 1) return hipErrorInvalidValue;  // callers check w4a16_gemv_mfma_needs_split
   return launch<false>(p, 3, plan, stream);
 }
@@ -440,7 +453,8 @@ hipError_t launch_w4a16_gemv_mfma_dual_swiglu(const W4DualSwigluArgs &a, hipStre
   p.mat0 = {a.gate.weight, a.gate.scale, a.product, a.n};
   p.mat1 = {a.up.weight, a.up.scale, a.product, a.n};
   p.mat2 = p.mat0;
-  const Plan plan = make_plan(a.k, a.n, 1, true);
+  p.row_groups = (a.m + 7) / 8;
+  const Plan plan = make_plan(a.k, a.n, p.row_groups, true);
   if (plan.slices > 1) return hipErrorInvalidValue;
   return launch<true>(p, 1, plan, stream);
 }

@@ -88,9 +88,10 @@ def test_gemv_matches_oracle(runtime, m, n, k):
                            f"gemv+bias {m}x{n}x{k}")
 
 
-def test_gemv_residual_epilogue(runtime):
+@pytest.mark.parametrize("m", [4, 17])
+def test_gemv_residual_epilogue(runtime, m):
     rng = np.random.default_rng(5)
-    m, n, k = 4, 576, 1536
+    n, k = 576, 1536
     x, packed, scale, _ = w4_case(rng, m, n, k)
     residual = rng.standard_normal((m, n)).astype(np.float16)
     expected = oracle.add(oracle.w4a16_linear(x, packed, scale, None), residual.astype(np.float32))
@@ -98,7 +99,9 @@ def test_gemv_residual_epilogue(runtime):
                            "gemv+residual")
 
 
-GEMM_SHAPES = [(9, 64, 64), (16, 128, 128), (100, 29, 192), (128, 256, 512), (130, 300, 1024),
+# up to 32 rows with small weights run the matrix-core GEMV once per group of 8 rows
+GEMM_SHAPES = [(9, 64, 64), (16, 128, 128), (24, 576, 1536), (31, 100, 576), (32, 1536, 576),
+               (32, 96, 14336), (33, 64, 576), (100, 29, 192), (128, 256, 512), (130, 300, 1024),
                (512, 128, 4096)]
 
 
@@ -133,7 +136,7 @@ def qkv_params(m, k, nq, nk, nv):
     return u32s(m, k, nq, nk, nv)
 
 
-@pytest.mark.parametrize("m", [1, 4, 8, 40])
+@pytest.mark.parametrize("m", [1, 4, 8, 12, 32, 40])
 def test_qkv_linear(runtime, m):
     rng = np.random.default_rng(31 + m)
     k, sizes = 576, (576, 192, 192)
@@ -151,7 +154,7 @@ def test_qkv_linear(runtime, m):
                                oracle.w4a16_linear(x, packed, scale, None), f"qkv n={n}")
 
 
-@pytest.mark.parametrize("m", [1, 2, 4, 8, 48])
+@pytest.mark.parametrize("m", [1, 2, 4, 8, 9, 32, 48])
 def test_swiglu_ffn_chain(runtime, m):
     """dual-SwiGLU then down+residual, the two W4A16 stages of the reference's
     FFN macro-op; the intermediate product is rounded to f16 between stages
