@@ -378,6 +378,7 @@ def main():
     parser.add_argument("--skip-cpu", action="store_true")
     parser.add_argument("--decode-eager", action="store_true",
                         help="launch the decode step from the host instead of replaying a HIP graph")
+    parser.add_argument("--decode-batches", default="1,8,32", help="batch sizes of the decode-step extra")
     parser.add_argument("--pmc-rows", type=int, default=1, help="activation rows of the --pmc-probe GEMV")
     parser.add_argument("--pmc-probe", action="store_true",
                         help="only the calibration copy and the headline GEMV, for rocprofv3 --pmc")
@@ -408,7 +409,8 @@ def main():
     if "prefill_attention" in wanted:
         extras["prefill_attention"] = bench_prefill_attention(runtime)
     if "decode" in wanted:
-        extras["decode_step"] = bench_decode_step(runtime, use_graph=not args.decode_eager)
+        extras["decode_step"] = bench_decode_step(
+            runtime, batches=tuple(int(b) for b in args.decode_batches.split(",")), use_graph=not args.decode_eager)
     line = {
         "metric": "W4A16 GEMV HBM GB/s (% peak); Q8 attn decode tokens/s; prefill MFMA %",
         "value": round(value, 1),

@@ -47,6 +47,56 @@ __global__ __launch_bounds__(kRowWaves * 64) void rms_norm_kernel(const In *inpu
   }
 }
 
+// The same for f16 rows of up to 64 * 8 * kRmsVectors values, width a multiple
+// of 8: the row and the weights are requested once, 16 bytes per lane, all
+// loads in flight together, and stay in registers between the two passes (the
+// loop above walks the row one 2-byte load latency at a time, twice).
+constexpr int kRmsVectors = 4;
+
+template <bool WEIGHT_FIRST>
+__global__ __launch_bounds__(kRowWaves * 64) void rms_norm_f16_rows_kernel(const uint16_t *input,
+                                                                           const uint16_t *weight,
+                                                                           uint16_t *output, uint32_t rows,
+                                                                           uint32_t width, float epsilon) {
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t row = blockIdx.x * kRowWaves + (threadIdx.x >> 6);
+  if (row >= rows) return;  // whole wave
+  const uint32_t vectors = width / 8;
+  const uint4 *in = reinterpret_cast<const uint4 *>(input + (size_t)row * width);
+  const uint4 *w = reinterpret_cast<const uint4 *>(weight);
+  uint4 x_raw[kRmsVectors], w_raw[kRmsVectors];
+#pragma unroll
+  for (int v = 0; v < kRmsVectors; ++v) {
+    const uint32_t index = lane + 64 * v;
+    x_raw[v] = index < vectors ? in[index] : make_uint4(0, 0, 0, 0);
+    w_raw[v] = index < vectors ? w[index] : make_uint4(0, 0, 0, 0);
+  }
+  float square_sum = 0.0f;
+#pragma unroll
+  for (int v = 0; v < kRmsVectors; ++v) {
+    const h8_t x = __builtin_bit_cast(h8_t, x_raw[v]);
+#pragma unroll
+    for (int e = 0; e < 8; ++e) square_sum += (float)x[e] * (float)x[e];
+  }
+  square_sum = wave_sum(square_sum);
+  const float inverse = rsqrtf(square_sum / (float)width + epsilon);
+  uint4 *out = reinterpret_cast<uint4 *>(output + (size_t)row * width);
+#pragma unroll
+  for (int v = 0; v < kRmsVectors; ++v) {
+    const uint32_t index = lane + 64 * v;
+    if (index >= vectors) continue;
+    const h8_t x = __builtin_bit_cast(h8_t, x_raw[v]);
+    const h8_t g = __builtin_bit_cast(h8_t, w_raw[v]);
+    h8_t y;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+      const float value = (float)x[e], gain = (float)g[e];
+      y[e] = (_Float16)(WEIGHT_FIRST ? value * gain * inverse : value * inverse * gain);
+    }
+    out[index] = __builtin_bit_cast(uint4, y);
+  }
+}
+
 // lib/metal_normalization_source.ml:765-802
 __global__ __launch_bounds__(kRowWaves * 64) void rotary_qk_kernel(RotaryQkArgs a) {
 #pragma clang fp contract(off)  // every product and the sum round to half separately
@@ -256,6 +306,19 @@ hipError_t launch_rms_norm(const RmsNormArgs &a, hipStream_t stream) {
                          a.rows, a.width, a.epsilon);
   } else {
     const uint16_t *in = static_cast<const uint16_t *>(a.input);
+    const bool vector_rows = a.width % 8 == 0 && a.width <= 64 * 8 * kRmsVectors &&
+                             reinterpret_cast<uintptr_t>(in) % 16 == 0 &&
+                             reinterpret_cast<uintptr_t>(a.weight) % 16 == 0 &&
+                             reinterpret_cast<uintptr_t>(a.output) % 16 == 0;
+    if (vector_rows) {
+      if (a.weight_first)
+        hipLaunchKernelGGL((rms_norm_f16_rows_kernel<true>), grid, block, 0, stream, in, a.weight, a.output, a.rows,
+                           a.width, a.epsilon);
+      else
+        hipLaunchKernelGGL((rms_norm_f16_rows_kernel<false>), grid, block, 0, stream, in, a.weight, a.output, a.rows,
+                           a.width, a.epsilon);
+      return hipGetLastError();
+    }
     if (a.weight_first)
       hipLaunchKernelGGL((rms_norm_kernel<uint16_t, true>), grid, block, 0, stream, in, a.weight, a.output,
                          a.rows, a.width, a.epsilon);
