@@ -265,7 +265,7 @@ def bench_prefill_attention(runtime):
     return results
 
 
-def bench_decode_step(runtime, batches=(1, 8, 32), context=2048, use_graph=True):
+def bench_decode_step(runtime, batches=(1, 8, 32, 128), context=2048, use_graph=True):
     """C5: one decode step of the 30-layer model (hidden 576, 9/3 heads of 64, MLP 1536,
     vocabulary 49152), every sequence with `context` tokens in the Q8 pool, replayed as a
     HIP graph.  tokens/s = batch / step time."""
@@ -378,7 +378,7 @@ def main():
     parser.add_argument("--skip-cpu", action="store_true")
     parser.add_argument("--decode-eager", action="store_true",
                         help="launch the decode step from the host instead of replaying a HIP graph")
-    parser.add_argument("--decode-batches", default="1,8,32", help="batch sizes of the decode-step extra")
+    parser.add_argument("--decode-batches", default="1,8,32,128", help="batch sizes of the decode-step extra")
     parser.add_argument("--pmc-rows", type=int, default=1, help="activation rows of the --pmc-probe GEMV")
     parser.add_argument("--pmc-probe", action="store_true",
                         help="only the calibration copy and the headline GEMV, for rocprofv3 --pmc")

@@ -32,7 +32,7 @@ namespace llmopt {
 namespace {
 
 constexpr int kSplitMaxWaves = 4;   // KV heads per workgroup (one wave each)
-constexpr int kChunkTokens = 128;   // context tokens per workgroup
+constexpr int kMaxChunkTokens = 128;  // context tokens per workgroup: 128, or 64 / 32 when that leaves CUs idle
 constexpr int kTileTokens = 16;    // tokens per MFMA tile
 
 __device__ __forceinline__ float q8_scale_at(const uint8_t *token, uint32_t token_elements,
@@ -76,7 +76,7 @@ __device__ __forceinline__ size_t partial_floats(uint32_t heads_per_kv) {
 // (two waves), and the kernel is bound by the latency of each wave's requests.
 template <int D, bool OFF32, bool A16>
 __global__ __launch_bounds__(kSplitMaxWaves * 64) __attribute__((amdgpu_waves_per_eu(3, 3))) void
-q8_attention_split_kernel(Q8AttentionArgs a, uint32_t chunks_max) {
+q8_attention_split_kernel(Q8AttentionArgs a, uint32_t chunks_max, uint32_t chunk_tokens) {
   constexpr int GROUPS = D / 64;      // scale groups per head
   constexpr int KLOADS = GROUPS;      // 16-byte K loads per lane per tile
   constexpr int VBLOCKS = D / 16;     // PV MFMAs (16 head_dim rows each)
@@ -94,12 +94,12 @@ q8_attention_split_kernel(Q8AttentionArgs a, uint32_t chunks_max) {
   const uint32_t heads_per_kv = a.query_heads / a.kv_heads;
 
   const uint32_t past = a.past_lengths ? a.past_lengths[batch] : a.past_length;
-  const uint32_t chunk_begin = chunk * kChunkTokens;
+  const uint32_t chunk_begin = chunk * chunk_tokens;
   if (chunk_begin >= past) return;
   const uint32_t *slots = a.slot_offsets ? a.slots + a.slot_offsets[batch] : a.slots;
   // requests that run ahead of the arithmetic stop at the chunk's last token:
   // what lies beyond belongs to another workgroup and would be fetched twice
-  const uint32_t last_token = min(chunk_begin + (uint32_t)kChunkTokens, past) - 1;
+  const uint32_t last_token = min(chunk_begin + chunk_tokens, past) - 1;
 
   // B operand of the score MFMAs: Q[head = col][d], zero for columns >= G.
   h8_t q_frag[GROUPS][2];
@@ -299,7 +299,7 @@ q8_attention_split_kernel(Q8AttentionArgs a, uint32_t chunks_max) {
   // The wave walks the 16-token tiles of the chunk.  Slot indices run two tiles
   // ahead and the K/V bytes one tile ahead of the arithmetic; requests past the
   // last tile are clamped to valid tokens and never used.
-  const uint32_t chunk_tiles = (min(past - chunk_begin, (uint32_t)kChunkTokens) + kTileTokens - 1) / kTileTokens;
+  const uint32_t chunk_tiles = (min(past - chunk_begin, chunk_tokens) + kTileTokens - 1) / kTileTokens;
   {
     TileSlots slots_a, slots_b;
     TileRaw raw_a, raw_b;
@@ -353,7 +353,8 @@ constexpr int kMergeSlices = 4;  // chunk slices summed in parallel per output r
 // quarter of the chunks per thread, finished through LDS.
 template <int D>
 __global__ __launch_bounds__(kMergeSlices *D) void q8_attention_merge_kernel(Q8AttentionArgs a,
-                                                                             uint32_t chunks_max) {
+                                                                             uint32_t chunks_max,
+                                                                             uint32_t chunk_tokens) {
   constexpr int THREADS = kMergeSlices * D;
   constexpr int WAVES = THREADS / 64;
   __shared__ float reduce_lds[3][WAVES];
@@ -368,7 +369,7 @@ __global__ __launch_bounds__(kMergeSlices *D) void q8_attention_merge_kernel(Q8A
   const uint32_t kv_head = head / heads_per_kv;
   const uint32_t local_head = head - kv_head * heads_per_kv;
   const uint32_t past = a.past_lengths ? a.past_lengths[batch] : a.past_length;
-  const uint32_t chunks = (past + kChunkTokens - 1) / kChunkTokens;
+  const uint32_t chunks = (past + chunk_tokens - 1) / chunk_tokens;
   const size_t stride = partial_floats<D>(heads_per_kv);
   const float *partial = reinterpret_cast<const float *>(a.workspace) +
                          ((size_t)batch * a.kv_heads + kv_head) * chunks_max * stride;
@@ -535,12 +536,22 @@ bool use_split_path(const Q8AttentionArgs &a) {
   if (a.token_elements % 2 != 0) return false;
   // D = 128 reads the two group scales of a head as one aligned dword
   if (a.head_dim == 128 && (a.key_offset % 128 != 0 || a.value_offset % 128 != 0)) return false;
-  if (a.max_past_length > (uint32_t)kChunkTokens * kMaxSplitChunks) return false;
+  if (a.max_past_length > (uint32_t)kMaxChunkTokens * kMaxSplitChunks) return false;
   return a.max_past_length >= 64;  // short contexts: one launch of the row kernel is cheaper
 }
 
+// A wave is bound by the latency of its tiles, one after the other: when 128-token
+// chunks give fewer waves than the device holds, shorter chunks finish sooner.
+uint32_t split_chunk_tokens(const Q8AttentionArgs &a) {
+  const uint64_t waves = (uint64_t)a.batches * a.kv_heads * ((a.max_past_length + 127) / 128);
+  uint32_t tokens = waves >= 1024 ? 128 : waves >= 512 ? 64 : 32;
+  while ((a.max_past_length + tokens - 1) / tokens > (uint32_t)kMaxSplitChunks) tokens *= 2;
+  return tokens;
+}
+
 uint32_t split_chunks(const Q8AttentionArgs &a) {
-  return (a.max_past_length + kChunkTokens - 1) / kChunkTokens;
+  const uint32_t tokens = split_chunk_tokens(a);
+  return (a.max_past_length + tokens - 1) / tokens;
 }
 
 }  // namespace
@@ -554,6 +565,7 @@ size_t q8_attention_workspace_bytes(const Q8AttentionArgs &a) {
 hipError_t launch_q8_attention(const Q8AttentionArgs &a, hipStream_t stream) {
   if (use_split_path(a)) {
     const uint32_t chunks = split_chunks(a);
+    const uint32_t chunk_tokens = split_chunk_tokens(a);
     if (a.workspace == nullptr || a.workspace_bytes < q8_attention_workspace_bytes(a))
       return hipErrorInvalidValue;
     const uint32_t waves = std::min<uint32_t>(a.kv_heads, kSplitMaxWaves);
@@ -566,14 +578,15 @@ hipError_t launch_q8_attention(const Q8AttentionArgs &a, hipStream_t stream) {
     const auto launch_split = [&](auto dim_tag) {
       constexpr int D = decltype(dim_tag)::value;
       if (small_pool && aligned16)
-        hipLaunchKernelGGL((q8_attention_split_kernel<D, true, true>), grid, block, 0, stream, a, chunks);
+        hipLaunchKernelGGL((q8_attention_split_kernel<D, true, true>), grid, block, 0, stream, a, chunks, chunk_tokens);
       else if (small_pool)
-        hipLaunchKernelGGL((q8_attention_split_kernel<D, true, false>), grid, block, 0, stream, a, chunks);
+        hipLaunchKernelGGL((q8_attention_split_kernel<D, true, false>), grid, block, 0, stream, a, chunks, chunk_tokens);
       else if (aligned16)
-        hipLaunchKernelGGL((q8_attention_split_kernel<D, false, true>), grid, block, 0, stream, a, chunks);
+        hipLaunchKernelGGL((q8_attention_split_kernel<D, false, true>), grid, block, 0, stream, a, chunks, chunk_tokens);
       else
-        hipLaunchKernelGGL((q8_attention_split_kernel<D, false, false>), grid, block, 0, stream, a, chunks);
-      hipLaunchKernelGGL(q8_attention_merge_kernel<D>, merge_grid, dim3(kMergeSlices * D), 0, stream, a, chunks);
+        hipLaunchKernelGGL((q8_attention_split_kernel<D, false, false>), grid, block, 0, stream, a, chunks, chunk_tokens);
+      hipLaunchKernelGGL(q8_attention_merge_kernel<D>, merge_grid, dim3(kMergeSlices * D), 0, stream, a, chunks,
+                         chunk_tokens);
     };
     if (a.head_dim == 128)
       launch_split(std::integral_constant<int, 128>{});

@@ -402,7 +402,7 @@ size_t w4a16_gemv_workspace_bytes(uint32_t m, uint32_t n, uint32_t k) {
 bool w4a16_gemv_mfma_needs_split(uint32_t k) { return (k + kStepK - 1) / kStepK > (uint32_t)kMaxWaves; }
 
 bool w4a16_gemv_mfma_row_groups_ok(uint32_t m, uint64_t columns, uint32_t k) {
-  return m > kGemvMaxRows && m <= 32 && !w4a16_gemv_mfma_needs_split(k) && columns * k / 2 <= (4u << 20);
+  return m > kGemvMaxRows && m <= 128 && !w4a16_gemv_mfma_needs_split(k) && columns * k / 2 <= (4u << 20);
 }
 
 hipError_t launch_w4a16_gemv_mfma_linear(const W4LinearArgs &a, hipStream_t stream) {

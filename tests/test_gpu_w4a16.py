@@ -99,9 +99,9 @@ def test_gemv_residual_epilogue(runtime, m):
                            "gemv+residual")
 
 
-# up to 32 rows with small weights run the matrix-core GEMV once per group of 8 rows
+# up to 128 rows with small weights run the matrix-core GEMV once per group of 8 rows
 GEMM_SHAPES = [(9, 64, 64), (16, 128, 128), (24, 576, 1536), (31, 100, 576), (32, 1536, 576),
-               (32, 96, 14336), (33, 64, 576), (100, 29, 192), (128, 256, 512), (130, 300, 1024),
+               (32, 96, 14336), (33, 64, 576), (64, 576, 1536), (100, 29, 192), (128, 192, 576), (129, 64, 576), (128, 256, 512), (130, 300, 1024),
                (512, 128, 4096)]
 
 
@@ -136,7 +136,7 @@ def qkv_params(m, k, nq, nk, nv):
     return u32s(m, k, nq, nk, nv)
 
 
-@pytest.mark.parametrize("m", [1, 4, 8, 12, 32, 40])
+@pytest.mark.parametrize("m", [1, 4, 8, 12, 32, 40, 130])
 def test_qkv_linear(runtime, m):
     rng = np.random.default_rng(31 + m)
     k, sizes = 576, (576, 192, 192)
@@ -154,7 +154,7 @@ def test_qkv_linear(runtime, m):
                                oracle.w4a16_linear(x, packed, scale, None), f"qkv n={n}")
 
 
-@pytest.mark.parametrize("m", [1, 2, 4, 8, 9, 32, 48])
+@pytest.mark.parametrize("m", [1, 2, 4, 8, 9, 32, 48, 136])
 def test_swiglu_ffn_chain(runtime, m):
     """dual-SwiGLU then down+residual, the two W4A16 stages of the reference's
     FFN macro-op; the intermediate product is rounded to f16 between stages
