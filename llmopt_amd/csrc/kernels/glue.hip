@@ -47,6 +47,37 @@ __global__ __launch_bounds__(kRowWaves * 64) void rms_norm_kernel(const In *inpu
   }
 }
 
+// The LM head's normalisation (lib/metal_w4a16_source.ml:1038-1046 keeps
+// x * w * inverse in float32 and multiplies it with the dequantised weights).
+// The GEMV kernels take fp16 activations, so the float32 value v goes out as
+// two fp16 rows, hi = half(v) and lo = half(v - hi): W.hi + W.lo, accumulated
+// in float32, differs from W.v by 2^-22 relative instead of the 2^-11 of a
+// single fp16 row.  Output rows 2r (hi) and 2r + 1 (lo).
+template <typename In>
+__global__ __launch_bounds__(kRowWaves * 64) void rms_norm_split_kernel(const In *input, const uint16_t *weight,
+                                                                        uint16_t *output, uint32_t rows,
+                                                                        uint32_t width, float epsilon) {
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t row = blockIdx.x * kRowWaves + (threadIdx.x >> 6);
+  if (row >= rows) return;  // whole wave
+  const size_t base = (size_t)row * width;
+  float square_sum = 0.0f;
+  for (uint32_t col = lane; col < width; col += 64) {
+    const float value = load_as_float(input, base + col);
+    square_sum += value * value;
+  }
+  square_sum = wave_sum(square_sum);
+  const float inverse = rsqrtf(square_sum / (float)width + epsilon);
+  uint16_t *high = output + (size_t)(2 * row) * width;
+  uint16_t *low = high + width;
+  for (uint32_t col = lane; col < width; col += 64) {
+    const float value = load_as_float(input, base + col) * half_bits_to_float(weight[col]) * inverse;
+    const uint16_t high_bits = float_to_half_bits(value);
+    high[col] = high_bits;
+    low[col] = float_to_half_bits(value - half_bits_to_float(high_bits));
+  }
+}
+
 // The same for f16 rows of up to 64 * 8 * kRmsVectors values, width a multiple
 // of 8: the row and the weights are requested once, 16 bytes per lane, all
 // loads in flight together, and stay in registers between the two passes (the
@@ -214,15 +245,21 @@ __device__ __forceinline__ bool better(float value, uint32_t index, float best_v
 constexpr int kArgmaxSlices = 4;
 constexpr int kArgmaxUnroll = 4;
 
+// `pairs`: logits holds two rows per output row (the products with the hi and
+// the lo half of the activation, see rms_norm_split_kernel) whose sum is the
+// logit; `half_logits`, when not null, receives half(logit) [rows, n].
 __global__ __launch_bounds__(256 * kArgmaxSlices) void argmax_candidates_kernel(const float *logits,
                                                                                 Candidate *candidates,
-                                                                                uint32_t n) {
+                                                                                uint32_t n, bool pairs,
+                                                                                uint16_t *half_logits) {
   __shared__ float slice_values[kArgmaxSlices][256];
   __shared__ uint32_t slice_indices[kArgmaxSlices][256];
   const uint32_t row = blockIdx.x;
   const uint32_t t = threadIdx.x & 255;
   const uint32_t slice = threadIdx.x >> 8;
-  const float *row_logits = logits + (size_t)row * n;
+  const float *row_logits = logits + (size_t)row * n * (pairs ? 2 : 1);
+  const float *row_low = row_logits + n;  // read only with `pairs`
+  uint16_t *row_half = half_logits != nullptr ? half_logits + (size_t)row * n : nullptr;
   float best_value = -3.402823466e+38f;
   uint32_t best_index = 0;
   bool found = false;
@@ -230,9 +267,17 @@ __global__ __launch_bounds__(256 * kArgmaxSlices) void argmax_candidates_kernel(
   uint32_t col = t + 256 * slice;
   // columns are visited in increasing order, so `>` alone keeps the lowest index among equals
   for (; col + (kArgmaxUnroll - 1) * step < n; col += kArgmaxUnroll * step) {
-    float value[kArgmaxUnroll];
+    float value[kArgmaxUnroll], low[kArgmaxUnroll];
 #pragma unroll
-    for (int u = 0; u < kArgmaxUnroll; ++u) value[u] = row_logits[col + u * step];
+    for (int u = 0; u < kArgmaxUnroll; ++u) {
+      value[u] = row_logits[col + u * step];
+      low[u] = pairs ? row_low[col + u * step] : 0.0f;
+    }
+#pragma unroll
+    for (int u = 0; u < kArgmaxUnroll; ++u) {
+      value[u] += low[u];
+      if (row_half != nullptr) row_half[col + u * step] = float_to_half_bits(value[u]);
+    }
 #pragma unroll
     for (int u = 0; u < kArgmaxUnroll; ++u)
       if (!found || value[u] > best_value) {
@@ -242,7 +287,8 @@ __global__ __launch_bounds__(256 * kArgmaxSlices) void argmax_candidates_kernel(
       }
   }
   for (; col < n; col += step) {
-    const float value = row_logits[col];
+    const float value = row_logits[col] + (pairs ? row_low[col] : 0.0f);
+    if (row_half != nullptr) row_half[col] = float_to_half_bits(value);
     if (!found || value > best_value) {
       best_value = value;
       best_index = col;
@@ -378,10 +424,21 @@ hipError_t launch_copy_bytes(void *destination, const void *source, size_t bytes
   return hipGetLastError();
 }
 
-hipError_t launch_argmax_candidates(const float *logits, void *candidates, uint32_t rows, uint32_t n,
-                                    hipStream_t stream) {
+hipError_t launch_argmax_candidates(const float *logits, void *candidates, uint32_t rows, uint32_t n, bool pairs,
+                                    uint16_t *half_logits, hipStream_t stream) {
   hipLaunchKernelGGL(argmax_candidates_kernel, dim3(rows), dim3(256 * kArgmaxSlices), 0, stream, logits,
-                     static_cast<Candidate *>(candidates), n);
+                     static_cast<Candidate *>(candidates), n, pairs, half_logits);
+  return hipGetLastError();
+}
+
+hipError_t launch_rms_norm_split(const RmsNormArgs &a, hipStream_t stream) {
+  const dim3 grid((a.rows + kRowWaves - 1) / kRowWaves), block(kRowWaves * 64);
+  if (a.input_f32)
+    hipLaunchKernelGGL(rms_norm_split_kernel<float>, grid, block, 0, stream, static_cast<const float *>(a.input),
+                       a.weight, a.output, a.rows, a.width, a.epsilon);
+  else
+    hipLaunchKernelGGL(rms_norm_split_kernel<uint16_t>, grid, block, 0, stream,
+                       static_cast<const uint16_t *>(a.input), a.weight, a.output, a.rows, a.width, a.epsilon);
   return hipGetLastError();
 }
 

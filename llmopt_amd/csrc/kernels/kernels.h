@@ -165,6 +165,9 @@ struct RmsNormArgs {
   bool weight_first;
 };
 hipError_t launch_rms_norm(const RmsNormArgs &args, hipStream_t stream);
+// x * w * inverse kept to float32 accuracy as two fp16 rows per input row: output
+// [2 * rows, width], row 2r = half(v), row 2r + 1 = half(v - float(half(v))).
+hipError_t launch_rms_norm_split(const RmsNormArgs &args, hipStream_t stream);
 
 // llmopt_rotary_qk_f16_simd_h64 (lib/metal_normalization_source.ml:765-802):
 // token-major [b, t, heads, width] in, head-major [b, heads, t, width] out,
@@ -202,8 +205,10 @@ hipError_t launch_copy_bytes(void *destination, const void *source, size_t bytes
 // Argmax over float32 logits [rows, n] in two steps with the reference's
 // candidate layout (W4A16LmHeadCandidate {f32 value, u32 index}, 256 per row,
 // lib/metal_w4a16_source.ml:1287-1319); ties go to the lowest index.
-hipError_t launch_argmax_candidates(const float *logits, void *candidates, uint32_t rows, uint32_t n,
-                                    hipStream_t stream);
+// pairs: logits is [2 * rows, n], output row r = rows 2r + (2r + 1) (see launch_rms_norm_split);
+// half_logits, when not null, receives half(logit) [rows, n].
+hipError_t launch_argmax_candidates(const float *logits, void *candidates, uint32_t rows, uint32_t n, bool pairs,
+                                    uint16_t *half_logits, hipStream_t stream);
 hipError_t launch_argmax_reduce(const void *candidates, uint32_t *token_ids, uint32_t rows,
                                 hipStream_t stream);
 

@@ -171,11 +171,11 @@ int add_f16(llmopt_hip_context *context, const DispatchRecord &record) {
 
 // ---- LM head ------------------------------------------------------------------
 //
-// RMSNorm -> half, vocabulary GEMV with float32 logits, argmax with ties to the
-// lowest index.  The reference keeps the normalised activation in float32
-// (lib/metal_w4a16_source.ml:1038-1046); here it is rounded to half before the
-// GEMV like every other W4A16 input, which perturbs a logit by about 3e-4
-// relative and can change the winner only between near-tied logits.
+// RMSNorm, vocabulary GEMV with float32 logits, argmax with ties to the lowest
+// index.  The reference keeps the normalised activation in float32
+// (lib/metal_w4a16_source.ml:1038-1046); the GEMV kernels take fp16 rows, so the
+// float32 value travels as a hi and a lo fp16 row (2^-22 relative together) and
+// the two float32 products are added in the argmax kernel.
 //
 // W4A16LmHeadParams {u32 m, n, k; f32 epsilon}.
 // Buffers: input, norm_weight, weight, scale, result [, logits f16 [m, n]]
@@ -206,11 +206,13 @@ int lm_head(llmopt_hip_context *context, const DispatchRecord &record, LmHeadVar
   if (variant.extra)
     if (int status = require_buffer_size(record.buffers[5], (uint64_t)m * n * 2, "logits")) return status;
 
-  // workspace: normalised activation | float32 logits | candidates | GEMV scratch
-  const size_t normalized_bytes = round_up_256((size_t)m * k * 2);
-  const size_t logits_bytes = round_up_256((size_t)m * n * 4);
+  // workspace: normalised activation (hi and lo row per input row) | float32 partial logits
+  // [2m, n] | candidates | GEMV scratch
+  const uint32_t gemv_rows = 2 * m;
+  const size_t normalized_bytes = round_up_256((size_t)gemv_rows * k * 2);
+  const size_t logits_bytes = round_up_256((size_t)gemv_rows * n * 4);
   const size_t candidate_bytes = round_up_256((size_t)m * 256 * 8);
-  const size_t gemv_bytes = w4a16_gemv_workspace_bytes(std::min(m, kGemvMaxRows), n, k);
+  const size_t gemv_bytes = w4a16_gemv_workspace_bytes(std::min(gemv_rows, kGemvMaxRows), n, k);
   uint8_t *workspace = static_cast<uint8_t *>(
       context_workspace(context, normalized_bytes + logits_bytes + candidate_bytes + gemv_bytes));
   if (workspace == nullptr) return LLMOPT_ERR_FAILURE;
@@ -219,6 +221,8 @@ int lm_head(llmopt_hip_context *context, const DispatchRecord &record, LmHeadVar
   void *candidates = variant.stage1 ? static_cast<void *>(record.buffers[4].device)
                                     : static_cast<void *>(workspace + normalized_bytes + logits_bytes);
 
+  // input * weight * inverse (lib/metal_w4a16_source.ml:1043-1044) stays float32 there; here it
+  // goes through the fp16 GEMV as a hi and a lo row, whose float32 products are added again
   RmsNormArgs norm = {};
   norm.input = record.buffers[0].device;
   norm.input_f32 = variant.input_f32;
@@ -227,16 +231,15 @@ int lm_head(llmopt_hip_context *context, const DispatchRecord &record, LmHeadVar
   norm.rows = m;
   norm.width = k;
   norm.epsilon = epsilon;
-  norm.weight_first = true;  // input * weight * inverse, lib/metal_w4a16_source.ml:1043-1044
-  if (int status = launched(launch_rms_norm(norm, context->stream), name)) return status;
+  if (int status = launched(launch_rms_norm_split(norm, context->stream), name)) return status;
 
   // the decode GEMV keeps float32 results; more rows go through it in groups
-  for (uint32_t first = 0; first < m; first += kGemvMaxRows) {
-    const uint32_t rows = std::min(kGemvMaxRows, m - first);
+  for (uint32_t first = 0; first < gemv_rows; first += kGemvMaxRows) {
+    const uint32_t rows = std::min(kGemvMaxRows, gemv_rows - first);
     W4LinearArgs linear = {};
     linear.x = normalized + (size_t)first * k;
     linear.w = {record.buffers[2].device, as_f16(record.buffers[3])};
-    linear.y = variant.extra ? as_f16_out(record.buffers[5]) + (size_t)first * n : nullptr;
+    linear.y = nullptr;
     linear.y_f32 = logits + (size_t)first * n;
     linear.m = rows;
     linear.n = n;
@@ -249,7 +252,10 @@ int lm_head(llmopt_hip_context *context, const DispatchRecord &record, LmHeadVar
     }
     if (int status = launched(launch_w4a16_linear(linear, context->stream), name)) return status;
   }
-  if (int status = launched(launch_argmax_candidates(logits, candidates, m, n, context->stream), name)) return status;
+  uint16_t *half_logits = variant.extra ? as_f16_out(record.buffers[5]) : nullptr;
+  if (int status = launched(launch_argmax_candidates(logits, candidates, m, n, true, half_logits, context->stream),
+                            name))
+    return status;
   if (variant.stage1) return LLMOPT_OK;
   return launched(launch_argmax_reduce(candidates, reinterpret_cast<uint32_t *>(record.buffers[4].device), m,
                                        context->stream),

@@ -224,15 +224,15 @@ def run_lm_head(runtime, x, norm_weight, packed, scale, epsilon, extra=False, st
 
 
 def check_tokens(tokens, expected_logits):
-    """The chosen column must hold the oracle's maximum up to the path's tolerance
-    (the half-rounded normalised activation can reorder near-tied logits)."""
+    """The chosen column must hold the oracle's maximum; only logits closer than float32
+    accumulation can separate (1e-5 x RMS) may swap."""
     rms = float(np.sqrt(np.mean(expected_logits.astype(np.float64) ** 2)))
     for row, token in enumerate(tokens):
         best = float(expected_logits[row].max())
         assert 0 <= token < expected_logits.shape[1]
-        assert float(expected_logits[row, token]) >= best - 2e-2 * rms, (row, token)
+        assert float(expected_logits[row, token]) >= best - 1e-5 * rms, (row, token)
         margin = np.partition(expected_logits[row], -2)[-2]
-        if best - margin > 2e-2 * rms:
+        if best - margin > 1e-5 * rms:
             assert token == oracle.argmax(expected_logits[row])
 
 
