@@ -286,3 +286,60 @@ def test_row_kernel_features(runtime, b, h, kvh, dim, past, q_len, window, mask_
                     mask, params)
     expected = oracle.paged_attention_q8(query, ck, cv, pool, slots, mask, params)
     assert_close_to_oracle(out, expected, "row kernel")
+
+
+@pytest.mark.parametrize("batches", [16, 1])
+def test_decode_attention_full_size_closed_form(runtime, batches):
+    """BASELINE's attention configuration (32/8 heads of 128, contexts up to 8192 tokens, scattered
+    slots), far beyond what the oracle finishes in seconds.  Every cached key of a (sequence, KV head)
+    is the same vector, so all past scores of a row coincide and the output has a closed form:
+    (w_past * sum_t V_t + w_cur * v_cur) / (L * w_past + w_cur), evaluated here in float64 from the
+    dequantised pool.  Batch 16 takes 128-token chunks, batch 1 the 64-token ones."""
+    rng = np.random.default_rng(1234 + batches)
+    heads, kv_heads, dim = 32, 8, 128
+    lengths = rng.integers(512, 8193, size=batches).astype(np.uint32)
+    lengths[0] = 8192
+    token_elements, stride = layout(kv_heads, dim)
+    total = int(lengths.sum())
+    offsets = np.concatenate([[0], np.cumsum(lengths)[:-1]]).astype(np.uint32)
+    slots = rng.permutation(total).astype(np.uint32)
+    pool = np.zeros((total, stride), dtype=np.uint8)
+    key_q = rng.integers(-127, 128, size=(batches, kv_heads * dim), dtype=np.int8)
+    key_s = rng.uniform(0.01, 0.03, size=(batches, kv_heads * dim // 64)).astype(np.float16)
+    value_q = rng.integers(-127, 128, size=(total, kv_heads * dim), dtype=np.int8)
+    value_s = rng.uniform(0.01, 0.03, size=(total, kv_heads * dim // 64)).astype(np.float16)
+    sequence_of = np.repeat(np.arange(batches), lengths)
+    pool[slots, :kv_heads * dim] = key_q[sequence_of].view(np.uint8)
+    pool[slots, kv_heads * dim:token_elements] = value_q.view(np.uint8)
+    scales = np.concatenate([key_s[sequence_of], value_s], axis=1)
+    pool[slots, token_elements:] = scales.view(np.uint8).reshape(total, -1)
+    query = rng.standard_normal((batches, heads, 1, dim)).astype(np.float16)
+    ck = rng.standard_normal((batches, kv_heads, 1, dim)).astype(np.float16)
+    cv = rng.standard_normal((batches, kv_heads, 1, dim)).astype(np.float16)
+    scale = 1.0 / math.sqrt(dim)
+    params = PagedParams(batches=batches, query_heads=heads, kv_heads=kv_heads, past_length=0, head_dim=dim,
+                         mask_batches=0, mask_heads=0, token_elements=token_elements, key_offset=0,
+                         value_offset=kv_heads * dim, group_size=64, token_stride=stride, scale=scale,
+                         query_length=1, mask_dtype=0, window=0)
+    out = run_paged(runtime, "llmopt_attention_q8_paged_batched", query, ck, cv, pool.reshape(-1), slots, None,
+                    params, lengths=lengths, offsets=offsets)
+    value = value_q.astype(np.float64).reshape(total, kv_heads, dim // 64, 64) * \
+        value_s.astype(np.float64).reshape(total, kv_heads, dim // 64, 1)
+    value = value.reshape(total, kv_heads, dim)
+    key = (key_q.astype(np.float64).reshape(batches, kv_heads, dim // 64, 64) *
+           key_s.astype(np.float64).reshape(batches, kv_heads, dim // 64, 1)).reshape(batches, kv_heads, dim)
+    want = np.empty((batches, 1, heads, dim))
+    group = heads // kv_heads
+    for b in range(batches):
+        rows = slice(int(offsets[b]), int(offsets[b] + lengths[b]))
+        value_sum = value[rows].sum(axis=0)  # [kv_heads, dim]
+        for h in range(heads):
+            kvh = h // group
+            q = query[b, h, 0].astype(np.float64)
+            s_past = scale * float(q @ key[b, kvh])
+            s_cur = scale * float(q @ ck[b, kvh, 0].astype(np.float64))
+            top = max(s_past, s_cur)
+            w_past, w_cur = math.exp(s_past - top), math.exp(s_cur - top)
+            want[b, 0, h] = (w_past * value_sum[kvh] + w_cur * cv[b, kvh, 0].astype(np.float64)) / \
+                (int(lengths[b]) * w_past + w_cur)
+    assert_close_to_oracle(out, want, f"full-size closed form, batch {batches}")
