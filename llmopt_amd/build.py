@@ -24,6 +24,16 @@ COMMON = ["-O3", "-std=c++17", "-fPIC", "--offload-arch=gfx950",
           "-Wall", "-Wno-unused-function", "-fno-gpu-sanitize"]
 
 
+# Kernels whose MFMA accumulators are also rescaled by vector instructions (online softmax):
+# with the accumulators in AGPRs the compiler copies every one of them to a VGPR and back on
+# each loop iteration, so these files keep them in VGPRs.  (The GEMM kernels want the AGPRs:
+# their accumulators are touched by MFMAs only and the VGPRs are needed for everything else.)
+PER_FILE = {
+    "dense_attention.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+    "q8_attention.hip": ["-mllvm", "-amdgpu-mfma-vgpr-form=1"],
+}
+
+
 def sources() -> list[str]:
     found = sorted(glob.glob(os.path.join(CSRC, "*.cpp")))
     found += sorted(glob.glob(os.path.join(CSRC, "host", "*.cpp")))
@@ -40,10 +50,10 @@ def _headers() -> list[str]:
 def _compile(source: str, force: bool) -> str:
     rel = os.path.relpath(source, CSRC).replace(os.sep, "_")
     obj = os.path.join(BUILD, rel + ".o")
-    newest_dep = max(os.path.getmtime(p) for p in [source] + _headers())
+    newest_dep = max(os.path.getmtime(p) for p in [source, os.path.abspath(__file__)] + _headers())
     if not force and os.path.exists(obj) and os.path.getmtime(obj) >= newest_dep:
         return obj
-    command = ["hipcc", *COMMON, "-c", source, "-o", obj]
+    command = ["hipcc", *COMMON, *PER_FILE.get(os.path.basename(source), []), "-c", source, "-o", obj]
     if source.endswith(".cpp"):
         command[1:1] = ["-x", "hip"]
     result = subprocess.run(command, capture_output=True, text=True)

@@ -112,7 +112,7 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
       asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
                    :
                    : "v"(x_src[c] + k0), "s"(lds_address)
-                   : "memory", "m0");
+                   : "memory");
     }
   };
 
