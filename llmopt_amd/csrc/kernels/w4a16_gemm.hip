@@ -130,6 +130,10 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
   constexpr int W_LOADS = 2 * NW;  // vector memory loads of one fetch_w
   const uint32_t w_col = min(n0 + w_row, p.n - 1);  // columns past n are never stored
 
+  // The compiler takes the destination of these loads as written when the statement ends, while
+  // the data lands later: between a fetch_w and the wait_w of the same set, control flow must
+  // give it no reason to copy the set (a second loop with its own register allocation did, and
+  // read registers whose loads were still in flight).
   auto fetch_w = [&](Fetched &f, uint32_t k0) __attribute__((always_inline)) {
 #pragma unroll
     for (int v = 0; v < NW; ++v) {
