@@ -13,6 +13,7 @@
 // (lib/metal_w4a16_source.ml:8-966) for m <= 8.
 #include <algorithm>
 #include <cstdlib>
+#include <utility>
 
 #include "kernels.h"
 #include "kernels_internal.h"
@@ -20,6 +21,16 @@
 
 namespace llmopt {
 namespace {
+
+template <typename F, int... I>
+__device__ __forceinline__ void static_for_each(F &&f, std::integer_sequence<int, I...>) {
+  (f(std::integral_constant<int, I>{}), ...);
+}
+// f(integral_constant<0>) ... f(integral_constant<N-1>): a loop whose index is a constant in every pass
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+  static_for_each(f, std::make_integer_sequence<int, (N > 0 ? N : 0)>{});
+}
 
 constexpr int kThreads = 256;
 constexpr int kWaves = kThreads / 64;
@@ -51,8 +62,18 @@ struct GemvParams {
 // (gw = global wave index) and, inside a tile, items of U chunks.  The weight
 // segments and scales of the next item are loaded into registers before the
 // current item is decoded, so HBM latency overlaps the VALU work.
-template <int M, int R, int U, bool XLDS, bool DUAL>
+//
+// D > 0 (with XLDS): a ring of D items in flight per wave instead of one.  The
+// loads are then issued as assembly and waited for by count (vector loads
+// return in issue order, so "at most n younger loads outstanding" names the
+// ones that have landed); left to the compiler, the wait at the loop head is
+// for everything in flight and the ring degenerates to one item.  ADD (ring
+// only): the residual addend of a tile travels with its items, so that the
+// store path has no load of its own to wait for.
+template <int M, int R, int U, bool XLDS, bool DUAL, int D = 0, bool ADD = false>
 __global__ __launch_bounds__(kThreads) void w4a16_gemv_kernel(GemvParams p) {
+  static_assert(D == 0 || XLDS, "the ring of loads needs the activation in LDS");
+  static_assert(!ADD || (D > 0 && !DUAL), "the addend travels with the ring only");
   extern __shared__ uint4 x_lds[];
   const int lane = threadIdx.x & 63;
   // wave-uniform values are forced into scalar registers: tile indices, row
@@ -73,7 +94,8 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemv_kernel(GemvParams p) {
   // consumed, or the compiler has to wait for the loads right after issuing them.
   struct Item {
     u32x4_t w[R][U];
-    uint16_t s[R][U];
+    uint32_t s[R][U];  // fp16 bits in the low half
+    uint32_t addend[ADD ? C : 1][ADD ? M : 1];
   };
 
   auto tile_rows = [&](uint32_t tile, const u32x4_t *(&wrow)[R], const uint16_t *(&srow)[R]) {
@@ -105,25 +127,144 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemv_kernel(GemvParams p) {
     }
   };
 
+  // The same loads for the ring: assembly, so that nothing waits for them but wait_item.
+  // Between an issue and its wait_item the set must not be copied (its registers are
+  // written when the data lands, not when the statement ends).
+  constexpr int LOADS = 2 * R * U + (ADD ? C * M : 0);  // vector loads of one issue_item
+  auto issue_item = [&](uint32_t tile, uint32_t item, bool real, Item &out) __attribute__((always_inline)) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    const u32x4_t *wrow[R];
+    const uint16_t *srow[R];
+    tile_rows(tile, wrow, srow);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const uint32_t seg = (item * U + u) * 64 + lane;
+      const uint32_t safe = (real && seg < segs) ? seg : 0;
+      const uint32_t w_offset = safe * 16, s_offset = (safe >> 1) * 2;
+#pragma unroll
+      for (int r = 0; r < R; ++r) {
+        asm volatile("global_load_dwordx4 %0, %1, %2 nt" : "=&v"(out.w[r][u]) : "v"(w_offset), "s"(wrow[r]) : "memory");
+        asm volatile("global_load_ushort %0, %1, %2" : "=&v"(out.s[r][u]) : "v"(s_offset), "s"(srow[r]) : "memory");
+      }
+    }
+    if (ADD) {
+      const uint32_t zero = 0;
+#pragma unroll
+      for (int c = 0; c < C; ++c) {
+        const uint32_t col = min(tile * C + (uint32_t)c, sg.n - 1);
+#pragma unroll
+        for (int m = 0; m < M; ++m) {
+          const uint16_t *src = p.addend + (size_t)((uint32_t)m < p.m ? m : 0) * p.addend_stride + col;
+          asm volatile("global_load_ushort %0, %1, %2" : "=&v"(out.addend[ADD ? c : 0][ADD ? m : 0]) : "v"(zero), "s"(src) : "memory");
+        }
+      }
+    }
+#endif
+  };
+  auto wait_item = [&](Item &f, auto younger) __attribute__((always_inline)) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    constexpr int n = decltype(younger)::value;
+    static_assert(n < 64, "vmcnt is a six-bit counter");
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+        asm volatile("s_waitcnt vmcnt(%2)" : "+v"(f.w[r][u]), "+v"(f.s[r][u]) : "n"(n) : "memory");
+    if (ADD) {
+#pragma unroll
+      for (int c = 0; c < C; ++c)
+#pragma unroll
+        for (int m = 0; m < M; ++m)
+          asm volatile("" : "+v"(f.addend[ADD ? c : 0][ADD ? m : 0]));
+    }
+#endif
+  };
+
   // first weights are in flight while the activation is staged
   Item item_a, item_b;
+  Item ring[D > 0 ? D : 1];
+  uint32_t ring_tile[D > 0 ? D : 1], ring_item[D > 0 ? D : 1];
   const bool has_work = first_tile < tiles;
-  if (has_work) load_item(first_tile, 0, true, item_a);
+  uint32_t ahead_tile = first_tile, ahead_item = 0;  // the next item to request
+  auto request = [&](int d) __attribute__((always_inline)) {
+    ring_tile[d] = ahead_tile;
+    ring_item[d] = ahead_item;
+    const bool real = ahead_tile < tiles;
+    issue_item(real ? ahead_tile : first_tile, ahead_item, real, ring[d]);
+    if (++ahead_item == items_per_tile) {
+      ahead_item = 0;
+      ahead_tile += wave_count;
+    }
+  };
+  // Ring: the activation is requested first (loads return in order, so it lands before the
+  // ring and the staging below does not wait for weights), up to kXAhead vectors per thread.
+  constexpr int kXAhead = 8;
+  static_assert(kXAhead == 8, "the wait below names eight registers");
+  const uint32_t vectors_per_row = chunks * 256;  // includes zero padding
+  const uint32_t x_vectors = (uint32_t)M * vectors_per_row;  // a multiple of kThreads
+  constexpr int XA = D > 0 ? kXAhead : 1;
+  u32x4_t x_ahead[XA];
+  auto x_source = [&](uint32_t i, bool &valid) {
+    const uint32_t m = i / vectors_per_row;
+    const uint32_t kk = i - m * vectors_per_row;  // index of an 8-K block
+    valid = m < p.m && kk < (K >> 3);
+    return reinterpret_cast<const uint4 *>(p.x + (size_t)(valid ? m : 0) * K) + (valid ? kk : 0);
+  };
+  auto x_store = [&](uint32_t i, uint4 value) {
+    const uint32_t m = i / vectors_per_row;
+    const uint32_t kk = i - m * vectors_per_row;
+    const uint32_t seg = kk >> 2, j = kk & 3;
+    x_lds[((m * chunks + (seg >> 6)) * 4 + j) * 64 + (seg & 63)] = value;
+  };
+  if constexpr (D > 0) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    static_for<kXAhead>([&](auto index) __attribute__((always_inline)) {
+      constexpr int n = decltype(index)::value;
+      x_ahead[n] = u32x4_t{0, 0, 0, 0};
+      if ((uint32_t)n * kThreads < x_vectors) {  // the same for every thread
+        bool valid;
+        const uint4 *src = x_source(threadIdx.x + n * kThreads, valid);
+        asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(x_ahead[n]) : "v"(src) : "memory");
+      }
+    });
+#endif
+    // also by a wave without work (its requests read a clamped row): the wait below counts on them
+    static_for<D>([&](auto index) __attribute__((always_inline)) { request(decltype(index)::value); });
+  } else if (has_work) {
+    load_item(first_tile, 0, true, item_a);
+  }
 
   // Bias correction of w4_decode_biased per (m, chunk, lane), after the vectors.
   float *corr_lds = reinterpret_cast<float *>(x_lds + (size_t)M * chunks * 256);
   if (XLDS) {
     // LDS layout [m][chunk][j][lane] of uint4: the j-th 8-K block of every
     // lane's segment is contiguous across lanes (conflict-free b128 reads).
-    const uint32_t vectors_per_row = chunks * 256;  // includes zero padding
-    for (uint32_t i = threadIdx.x; i < (uint32_t)M * vectors_per_row; i += kThreads) {
-      const uint32_t m = i / vectors_per_row;
-      const uint32_t kk = i - m * vectors_per_row;  // index of an 8-K block
-      uint4 value = make_uint4(0, 0, 0, 0);
-      if (m < p.m && kk < (K >> 3))
-        value = pair_order(reinterpret_cast<const uint4 *>(p.x + (size_t)m * K)[kk]);
-      const uint32_t seg = kk >> 2, j = kk & 3;
-      x_lds[((m * chunks + (seg >> 6)) * 4 + j) * 64 + (seg & 63)] = value;
+    uint32_t first_vector = threadIdx.x;
+    if constexpr (D > 0) {
+#if defined(__HIP_DEVICE_COMPILE__)
+      // only the ring's requests may still be outstanding
+      asm volatile("s_waitcnt vmcnt(%8)"
+                   : "+v"(x_ahead[0]), "+v"(x_ahead[1 % XA]), "+v"(x_ahead[2 % XA]), "+v"(x_ahead[3 % XA]),
+                     "+v"(x_ahead[4 % XA]), "+v"(x_ahead[5 % XA]), "+v"(x_ahead[6 % XA]), "+v"(x_ahead[7 % XA])
+                   : "n"(D * LOADS)
+                   : "memory");
+#endif
+      static_for<kXAhead>([&](auto index) __attribute__((always_inline)) {
+        constexpr int n = decltype(index)::value;
+        if ((uint32_t)n * kThreads < x_vectors) {
+          bool valid;
+          const uint32_t i = threadIdx.x + n * kThreads;
+          (void)x_source(i, valid);
+          const uint4 loaded = pair_order(__builtin_bit_cast(uint4, x_ahead[n]));
+          x_store(i, valid ? loaded : make_uint4(0, 0, 0, 0));
+        }
+      });
+      first_vector += kXAhead * kThreads;  // anything beyond waits for the ring as well
+    }
+    for (uint32_t i = first_vector; i < x_vectors; i += kThreads) {
+      bool valid;
+      const uint4 *src = x_source(i, valid);
+      x_store(i, valid ? pair_order(*src) : make_uint4(0, 0, 0, 0));
     }
     __syncthreads();
     for (uint32_t i = threadIdx.x; i < (uint32_t)M * chunks * 64; i += kThreads) {
@@ -195,7 +336,7 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemv_kernel(GemvParams p) {
         const float correction = XLDS ? corr_lds[(m * chunks + c_safe) * 64 + lane] : 0.0f;
 #pragma unroll
         for (int r = 0; r < R; ++r)
-          acc[r][m] = fmaf(part[r][m] - correction, ok ? half_bits_to_float(cur.s[r][u]) : 0.0f,
+          acc[r][m] = fmaf(part[r][m] - correction, ok ? half_bits_to_float((uint16_t)cur.s[r][u]) : 0.0f,
                            acc[r][m]);
       }
     }
@@ -226,7 +367,9 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemv_kernel(GemvParams p) {
               value = gate / (1.0f + __expf(-gate)) * up;
             } else {
               value = total[cidx][m];
-              if (p.has_addend)
+              if (ADD)
+                value += half_bits_to_float((uint16_t)cur.addend[ADD ? cidx : 0][ADD ? m : 0]);
+              else if (D == 0 && p.has_addend)
                 value += half_bits_to_float(p.addend[(size_t)m * p.addend_stride + col]);
             }
             if (sg.y != nullptr) sg.y[(size_t)m * n + col] = float_to_half_bits(value);
@@ -249,6 +392,27 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemv_kernel(GemvParams p) {
   // the end it reads one line per row) so that no branch skips the loads:
   // with a skipped path the compiler must assume the shorter load queue and
   // waits for the fresh loads before decoding the old ones.
+  if (D > 0) {
+    // ring[d] is consumed while the D - 1 younger requests are in flight, then requested again
+    // D items ahead; requests past the last tile are still issued (one line per row, unused)
+    // so that the number of loads in flight stays what wait_item assumes.
+    bool done = false;
+    while (!done) {
+      static_for<D>([&](auto index) __attribute__((always_inline)) {
+        constexpr int d = decltype(index)::value;
+        if (done) return;
+        if (ring_tile[d] >= tiles) {
+          done = true;
+          return;
+        }
+        wait_item(ring[d], std::integral_constant<int, (D - 1) * LOADS>{});
+        consume(ring_tile[d], ring_item[d], ring[d]);
+        request(d);
+      });
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // requests in flight still target live registers
+    return;
+  }
   uint32_t tile = first_tile, item = 0;
   while (true) {
     uint32_t next_tile = tile, next_item = item;
@@ -286,7 +450,7 @@ int device_compute_units() {
 
 namespace {
 
-template <int M, int R, int U, bool DUAL>
+template <int M, int R, int U, bool DUAL, int D = 0>
 hipError_t launch_variant(const GemvParams &p, uint32_t matrices, uint32_t max_n, hipStream_t stream) {
   // a tile is R weight rows (DUAL: R/2 gate rows + the matching R/2 up rows)
   constexpr int C = DUAL ? R / 2 : R;
@@ -298,11 +462,24 @@ hipError_t launch_variant(const GemvParams &p, uint32_t matrices, uint32_t max_n
   const size_t lds_bytes = (size_t)M * chunks * 256 * sizeof(uint4) + (size_t)M * chunks * 64 * sizeof(float);
   const bool use_lds = lds_bytes <= 64 * 1024;
   const int cus = device_compute_units();
-  int per_cu = 2;  // 8 waves per CU, each with two work items of weights in flight
-  if (use_lds && lds_bytes > 80 * 1024) per_cu = 1;
+  // workgroups per CU: 12 waves with two items in flight each for the ring (measured against 8
+  // and 16), 8 waves otherwise; fewer when the activation fills the LDS
+  int per_cu = D > 0 && use_lds ? 3 : 2;
+  while (per_cu > 1 && lds_bytes * per_cu > 150 * 1024) --per_cu;
   const uint32_t wanted = (tiles + kWaves - 1) / kWaves;
   const uint32_t blocks = std::max<uint32_t>(1, std::min<uint32_t>(wanted, (uint32_t)(cus * per_cu)));
-  if (use_lds) {
+  if (use_lds && D > 0) {
+    if constexpr (!DUAL && D > 0) {
+      if (p.has_addend) {
+        hipLaunchKernelGGL((w4a16_gemv_kernel<M, R, U, true, DUAL, D, true>), dim3(blocks, matrices),
+                           dim3(kThreads), lds_bytes, stream, p);
+        return hipGetLastError();
+      }
+    }
+    if constexpr (D > 0)
+      hipLaunchKernelGGL((w4a16_gemv_kernel<M, R, U, true, DUAL, D, false>), dim3(blocks, matrices),
+                         dim3(kThreads), lds_bytes, stream, p);
+  } else if (use_lds) {
     hipLaunchKernelGGL((w4a16_gemv_kernel<M, R, U, true, DUAL>), dim3(blocks, matrices), dim3(kThreads),
                        lds_bytes, stream, p);
   } else {
@@ -316,8 +493,9 @@ template <bool DUAL>
 hipError_t launch_by_rows(const GemvParams &p, uint32_t matrices, uint32_t max_n, hipStream_t stream) {
   // small work items (2 rows x one 2048-wide K chunk) measured fastest: finer
   // interleaving of waves over the row tiles and a shorter drain at the end
-  if (p.m <= 1) return launch_variant<1, 2, 1, DUAL>(p, matrices, max_n, stream);
-  if (p.m <= 2) return launch_variant<2, 2, 1, DUAL>(p, matrices, max_n, stream);
+  // one and two rows: two items in flight per wave (deeper rings measured slower)
+  if (p.m <= 1) return launch_variant<1, 2, 1, DUAL, 2>(p, matrices, max_n, stream);
+  if (p.m <= 2) return launch_variant<2, 2, 1, DUAL, 2>(p, matrices, max_n, stream);
   if (p.m <= 4) return launch_variant<4, 2, 1, DUAL>(p, matrices, max_n, stream);
   return launch_variant<8, 2, 1, DUAL>(p, matrices, max_n, stream);
 }
