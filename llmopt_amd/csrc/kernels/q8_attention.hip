@@ -34,6 +34,7 @@ namespace {
 constexpr int kSplitMaxWaves = 4;   // KV heads per workgroup (one wave each)
 constexpr int kMaxChunkTokens = 128;  // context tokens per workgroup: 128, or 64 / 32 when that leaves CUs idle
 constexpr int kTileTokens = 16;    // tokens per MFMA tile
+constexpr int kMaxSplitChunks = 1024;  // chunks per sequence: the merge kernel keeps one weight per chunk in LDS
 
 __device__ __forceinline__ float q8_scale_at(const uint8_t *token, uint32_t token_elements,
                                              uint32_t index) {
@@ -70,21 +71,103 @@ __device__ __forceinline__ size_t partial_floats(uint32_t heads_per_kv) {
   return 32 + (size_t)heads_per_kv * D;
 }
 
+// ---- balanced split --------------------------------------------------------------------
+// With chunks of a fixed size the number of workgroups is whatever the contexts give, and the
+// device runs them in rounds: 1028 chunks on 768 resident workgroups take two rounds, the
+// second a third full.  Here the launch has a fixed number of chunk slots (what the device
+// holds at once) and every sequence gets a share of them in proportion to its context, i.e.
+// its own chunk size: one round, every workgroup with about the same number of tokens.
+// The shares depend on the context lengths, which live in device memory, so every wave works
+// them out for itself, one sequence per lane: share = 1 + floor(past * (slots - batches) / total)
+// chunks of ceil(past / share) tokens rounded up to whole tiles.  The split and
+// the merge kernel run the same instructions on the same inputs and so agree on the layout.
+struct SplitPlan {
+  uint32_t batch, first, chunks, tokens, past, slot_offset;
+  bool found;
+};
+
+// Inclusive prefix sum over the 64 lanes with DPP: shifts inside the 16-lane rows, then the
+// last lane of a row broadcast into the rows above it.  Lanes a shift has nothing for add 0.
+__device__ __forceinline__ uint32_t wave_inclusive_sum(uint32_t value) {
+  int v = (int)value;
+  v += __builtin_amdgcn_update_dpp(0, v, 0x111, 0xF, 0xF, false);  // row_shr:1
+  v += __builtin_amdgcn_update_dpp(0, v, 0x112, 0xF, 0xF, false);  // row_shr:2
+  v += __builtin_amdgcn_update_dpp(0, v, 0x114, 0xF, 0xF, false);  // row_shr:4
+  v += __builtin_amdgcn_update_dpp(0, v, 0x118, 0xF, 0xF, false);  // row_shr:8
+  v += __builtin_amdgcn_update_dpp(0, v, 0x142, 0xA, 0xF, false);  // row_bcast:15 into rows 1 and 3
+  v += __builtin_amdgcn_update_dpp(0, v, 0x143, 0xC, 0xF, false);  // row_bcast:31 into rows 2 and 3
+  return (uint32_t)v;
+}
+
+// BY_INDEX: the sequence that owns chunk slot `key`; else sequence `key` itself.
+constexpr int kPlanBlocks = 4;  // 64 sequences each: the balanced split serves batches up to 256
+
+template <bool BY_INDEX>
+__device__ __forceinline__ SplitPlan split_plan(const Q8AttentionArgs &a, uint32_t slots, uint32_t key) {
+  const uint32_t lane = __lane_id();
+  // every request goes out before the first result is used: one trip to memory
+  uint32_t past[kPlanBlocks], slot_offset[kPlanBlocks];
+#pragma unroll
+  for (int k = 0; k < kPlanBlocks; ++k) {
+    const uint32_t b = k * 64 + lane;
+    past[k] = b < a.batches ? (a.past_lengths ? a.past_lengths[b] : a.past_length) : 0;
+    slot_offset[k] = BY_INDEX && a.slot_offsets != nullptr && b < a.batches ? a.slot_offsets[b] : 0;
+  }
+  uint32_t total = 0;
+#pragma unroll
+  for (int k = 0; k < kPlanBlocks; ++k) total += past[k];
+  total = (uint32_t)__builtin_amdgcn_readlane((int)wave_inclusive_sum(total), 63);
+  // a hair below (slots - batches) / total: the shares then add up to slots at most whatever the
+  // float roundings do (a chunk beyond the last slot would have no workgroup)
+  const float ratio =
+      total != 0 ? __fmul_rn(__fdiv_rn((float)(slots - a.batches), (float)total), 0.999999f) : 0.0f;
+  // a wave is bound by the latency of its tiles, one after the other, and every chunk costs a
+  // partial result: 128-token chunks at least, shorter ones only when those leave the device idle
+  const uint32_t waves = ((total + 127) >> 7) * a.kv_heads;
+  const uint32_t least = waves >= 1024 ? 128 : waves >= 512 ? 64 : 32;
+  SplitPlan plan = {0, 0, 0, 32, 0, 0, false};
+  uint32_t carry = 0;
+#pragma unroll
+  for (int k = 0; k < kPlanBlocks; ++k) {
+    if ((uint32_t)k * 64 >= a.batches) break;
+    const uint32_t b = k * 64 + lane;
+    const uint32_t share = min(1 + (uint32_t)__fmul_rn((float)past[k], ratio), (uint32_t)kMaxSplitChunks);
+    const uint32_t tokens =
+        max(least, ((past[k] + share - 1) / share + kTileTokens - 1) & ~(uint32_t)(kTileTokens - 1));
+    const uint32_t chunks = (past[k] + tokens - 1) / tokens;
+    const uint32_t inclusive = wave_inclusive_sum(chunks);
+    const uint32_t first = carry + inclusive - chunks;
+    const bool hit = b < a.batches && (BY_INDEX ? (key >= first && key < first + chunks) : b == key);
+    const uint64_t hits = __builtin_amdgcn_ballot_w64(hit);
+    if (hits != 0 && !plan.found) {
+      const int source = __builtin_ctzll(hits);
+      plan.batch = k * 64 + source;
+      plan.first = (uint32_t)__builtin_amdgcn_readlane((int)first, source);
+      plan.chunks = (uint32_t)__builtin_amdgcn_readlane((int)chunks, source);
+      plan.tokens = (uint32_t)__builtin_amdgcn_readlane((int)tokens, source);
+      plan.past = (uint32_t)__builtin_amdgcn_readlane((int)past[k], source);
+      plan.slot_offset = (uint32_t)__builtin_amdgcn_readlane((int)slot_offset[k], source);
+      plan.found = true;
+    }
+    carry += (uint32_t)__builtin_amdgcn_readlane((int)inclusive, 63);
+  }
+  return plan;
+}
+
 // OFF32: the pool is smaller than 4 GiB, so slot byte offsets fit 32 bits and the
 // loads can use a scalar base plus a 32-bit vector offset.
 // Three waves per SIMD: left alone the register allocator takes 209 registers
 // (two waves), and the kernel is bound by the latency of each wave's requests.
 template <int D, bool OFF32, bool A16>
 __global__ __launch_bounds__(kSplitMaxWaves * 64) __attribute__((amdgpu_waves_per_eu(3, 3))) void
-q8_attention_split_kernel(Q8AttentionArgs a, uint32_t chunks_max, uint32_t chunk_tokens) {
+q8_attention_split_kernel(Q8AttentionArgs a, uint32_t chunks_max, uint32_t fixed_chunk_tokens,
+                          uint32_t balanced_slots) {
   constexpr int GROUPS = D / 64;      // scale groups per head
   constexpr int KLOADS = GROUPS;      // 16-byte K loads per lane per tile
   constexpr int VBLOCKS = D / 16;     // PV MFMAs (16 head_dim rows each)
   // One wave per KV head; the waves of a workgroup walk the same tokens, so the
   // cache lines of a token (its heads are adjacent in the pool slot, and all
   // its scales share one line) are fetched into one CU instead of eight XCDs.
-  const uint32_t chunk = blockIdx.x;
-  const uint32_t batch = blockIdx.z;
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t kv_head =
       blockIdx.y * kSplitMaxWaves + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -93,10 +176,27 @@ q8_attention_split_kernel(Q8AttentionArgs a, uint32_t chunks_max, uint32_t chunk
   const uint32_t quad = lane >> 4;
   const uint32_t heads_per_kv = a.query_heads / a.kv_heads;
 
-  const uint32_t past = a.past_lengths ? a.past_lengths[batch] : a.past_length;
+  // balanced_slots != 0: blockIdx.x is a chunk slot of the balanced split; else chunks of a
+  // fixed size, blockIdx.x the chunk and blockIdx.z the sequence
+  uint32_t chunk = blockIdx.x, batch = blockIdx.z, chunk_tokens = fixed_chunk_tokens, past, slot_offset;
+  size_t partial_index;
+  if (balanced_slots != 0) {
+    const SplitPlan plan = split_plan<true>(a, balanced_slots, blockIdx.x);
+    if (!plan.found) return;
+    batch = plan.batch;
+    chunk = blockIdx.x - plan.first;
+    chunk_tokens = plan.tokens;
+    past = plan.past;
+    slot_offset = plan.slot_offset;
+    partial_index = (size_t)kv_head * balanced_slots + blockIdx.x;
+  } else {
+    past = a.past_lengths ? a.past_lengths[batch] : a.past_length;
+    slot_offset = a.slot_offsets ? a.slot_offsets[batch] : 0;
+    partial_index = ((size_t)batch * a.kv_heads + kv_head) * chunks_max + chunk;
+  }
   const uint32_t chunk_begin = chunk * chunk_tokens;
   if (chunk_begin >= past) return;
-  const uint32_t *slots = a.slot_offsets ? a.slots + a.slot_offsets[batch] : a.slots;
+  const uint32_t *slots = a.slots + slot_offset;
   // requests that run ahead of the arithmetic stop at the chunk's last token:
   // what lies beyond belongs to another workgroup and would be fetched twice
   const uint32_t last_token = min(chunk_begin + chunk_tokens, past) - 1;
@@ -145,76 +245,108 @@ q8_attention_split_kernel(Q8AttentionArgs a, uint32_t chunks_max, uint32_t chunk
 #pragma unroll
   for (int v = 0; v < VBLOCKS; ++v) out_acc[v] = f4_t{0.0f, 0.0f, 0.0f, 0.0f};
 
-  // Loaded-but-untouched registers of one 16-token tile.  Nothing in here may be
-  // used before the tile is processed, or the loads are waited for at once.
+  // ---- requests: whole lines ------------------------------------------------------------
+  // A (token, head) row of K or V is D contiguous bytes.  D / 16 neighbouring lanes read one
+  // row with 16 bytes each, so a load instruction covers 64 / (D / 16) tokens with whole
+  // lines and a 16-token tile takes kTileTokens * D / 1024 instructions per operand - in MFMA
+  // operand order the same bytes took 2 + 8 instructions whose lane quads each touched other
+  // lines, and the kernel was bound by the number of requests, not by their bytes.  The
+  // (key, value) scales of token lane % 16 ride in one more dword per lane (lanes 0..15 key,
+  // 16..31 value).  The tile then passes through a wave-private LDS patch to reach operand
+  // order (the LDS unit serves one wave's accesses in order: no barrier).
+  constexpr int LPT = D / 16;            // lanes per (token, head) row
+  constexpr int TPI = 64 / LPT;          // tokens per load instruction
+  constexpr int KL = kTileTokens / TPI;  // load instructions per tile and operand
+  constexpr int ROW = D + 32;            // LDS row stride: conflict-free 16-byte reads down the tokens
+  const uint32_t line_token = lane / LPT, line_piece = lane % LPT;
+  __shared__ __attribute__((aligned(16))) uint8_t turn_lds[kSplitMaxWaves][2 * kTileTokens * ROW + 128];
+  uint8_t *key_patch = turn_lds[threadIdx.x >> 6];
+  uint8_t *value_patch = key_patch + kTileTokens * ROW;
+  uint32_t *scale_patch = reinterpret_cast<uint32_t *>(key_patch + 2 * kTileTokens * ROW);
+
   struct TileSlots {
-    uint32_t key;       // slot of token (tile0 + col)
-    uint32_t value[4];  // slots of tokens (tile0 + quad*4 + i)
+    uint32_t line[KL];  // slot of token (tile0 + n * TPI + line_token)
+    uint32_t scale;     // slot of token (tile0 + lane % 16)
   };
-  struct TileRaw {
-    u32x4_t k[KLOADS];          // lane (token = col, quad): 16 head_dim values per group
-    uint32_t v[4][GROUPS];      // lane (d-row = col, quad): tokens quad*4 + i
-    uint32_t k_scale[4];        // D = 128: both group scales of the token in one dword
-    uint32_t v_scale[4];        // D = 64: the single scale in the low half
-  };
-  // D = 128 reads the two adjacent fp16 scales of a (token, head) as one dword;
-  // the scale index is even because every segment offset is a multiple of 128.
-  auto load_slots = [&](uint32_t tile, TileSlots &out) __attribute__((always_inline)) {
-    const uint32_t token0 = chunk_begin + tile * kTileTokens;
-    out.key = slots[min(token0 + col, last_token)];
-#pragma unroll
-    for (int i = 0; i < 4; ++i) out.value[i] = slots[min(token0 + quad * 4 + i, last_token)];
-  };
-  // With OFF32 every address is the scalar pool base plus one 32-bit lane offset
-  // and a compile-time displacement, so a load needs no 64-bit vector add.
   // A16 = false: pool slots are only 4-byte aligned (a token stride that is not a
-  // multiple of 16, e.g. 11880 bytes); the key loads then carry that alignment.
+  // multiple of 16, e.g. 11880 bytes); the vector loads then carry that alignment.
   typedef uint32_t unaligned_u32x4_t __attribute__((ext_vector_type(4), aligned(4)));
   using KeyVector = typename std::conditional<A16, u32x4_t, unaligned_u32x4_t>::type;
-  auto load_raw = [&](const TileSlots &where, TileRaw &out) __attribute__((always_inline)) {
+  // Loaded-but-untouched registers of one 16-token tile.  Nothing in here may be
+  // used before the tile is processed, or the loads are waited for at once.
+  struct TileLine {
+    u32x4_t k[KL], v[KL];
+    uint32_t scale;  // D = 128: both group scales of the token in one dword; D = 64: one scale in the low half
+  };
+  struct TileRaw {              // the same tile in operand order
+    u32x4_t k[KLOADS];          // lane (token = col, quad): 16 head_dim values per group
+    uint32_t v[4][GROUPS];      // lane (d-row = col, quad): tokens quad*4 + i
+    uint32_t k_scale[4];        // tokens quad*4 + i
+    uint32_t v_scale[4];
+  };
+  auto load_slots = [&](uint32_t tile, TileSlots &out) __attribute__((always_inline)) {
+    const uint32_t token0 = chunk_begin + tile * kTileTokens;
+#pragma unroll
+    for (int n = 0; n < KL; ++n) out.line[n] = slots[min(token0 + n * TPI + line_token, last_token)];
+    out.scale = slots[min(token0 + col, last_token)];
+  };
+  // With OFF32 every address is the scalar pool base plus one 32-bit lane offset.
+  // D = 128 reads the two adjacent fp16 scales of a (token, head) as one dword;
+  // the scale index is even because every segment offset is a multiple of 128.
+  const uint32_t scale_byte = a.token_elements + 2 * ((quad & 1) ? value_scale_index : key_scale_index);
+  auto load_line = [&](const TileSlots &where, TileLine &out) __attribute__((always_inline)) {
     if (OFF32) {
-      const uint32_t key_offset = where.key * a.token_stride + key_base + quad * 16;
 #pragma unroll
-      for (int g = 0; g < KLOADS; ++g)
-        out.k[g] = *reinterpret_cast<const KeyVector *>(a.pool + key_offset + g * 64);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const uint32_t slot_offset = where.value[i] * a.token_stride;
-        const uint32_t value_offset = slot_offset + value_base + col * 4;
-#pragma unroll
-        for (int g = 0; g < GROUPS; ++g)
-          out.v[i][g] = *reinterpret_cast<const uint32_t *>(a.pool + value_offset + g * 64);
-        const uint32_t key_scale_offset = slot_offset + a.token_elements + 2 * key_scale_index;
-        const uint32_t value_scale_offset = slot_offset + a.token_elements + 2 * value_scale_index;
-        if (GROUPS == 2) {
-          out.k_scale[i] = *reinterpret_cast<const uint32_t *>(a.pool + key_scale_offset);
-          out.v_scale[i] = *reinterpret_cast<const uint32_t *>(a.pool + value_scale_offset);
-        } else {
-          out.k_scale[i] = *reinterpret_cast<const uint16_t *>(a.pool + key_scale_offset);
-          out.v_scale[i] = *reinterpret_cast<const uint16_t *>(a.pool + value_scale_offset);
-        }
+      for (int n = 0; n < KL; ++n) {
+        const uint32_t row = where.line[n] * a.token_stride + line_piece * 16;
+        out.k[n] = *reinterpret_cast<const KeyVector *>(a.pool + row + key_base);
+        out.v[n] = *reinterpret_cast<const KeyVector *>(a.pool + row + value_base);
       }
+      const uint32_t scale_offset = where.scale * a.token_stride + scale_byte;
+      if (GROUPS == 2)
+        out.scale = *reinterpret_cast<const uint32_t *>(a.pool + scale_offset);
+      else
+        out.scale = *reinterpret_cast<const uint16_t *>(a.pool + scale_offset);
       return;
     }
-    const uint8_t *key_slot = a.pool + (size_t)where.key * a.token_stride;
 #pragma unroll
-    for (int g = 0; g < KLOADS; ++g)
-      out.k[g] = *reinterpret_cast<const KeyVector *>(key_slot + key_base + g * 64 + quad * 16);
+    for (int n = 0; n < KL; ++n) {
+      const uint8_t *row = a.pool + (size_t)where.line[n] * a.token_stride + line_piece * 16;
+      out.k[n] = *reinterpret_cast<const KeyVector *>(row + key_base);
+      out.v[n] = *reinterpret_cast<const KeyVector *>(row + value_base);
+    }
+    const uint8_t *scale_at = a.pool + (size_t)where.scale * a.token_stride + scale_byte;
+    if (GROUPS == 2)
+      out.scale = *reinterpret_cast<const uint32_t *>(scale_at);
+    else
+      out.scale = *reinterpret_cast<const uint16_t *>(scale_at);
+  };
+  auto turn = [&](const TileLine &line, TileRaw &raw) __attribute__((always_inline)) {
+    __builtin_amdgcn_wave_barrier();
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const uint8_t *slot = a.pool + (size_t)where.value[i] * a.token_stride;
+    for (int n = 0; n < KL; ++n) {
+      const uint32_t at = (n * TPI + line_token) * ROW + line_piece * 16;
+      *reinterpret_cast<u32x4_t *>(key_patch + at) = line.k[n];
+      *reinterpret_cast<u32x4_t *>(value_patch + at) = line.v[n];
+    }
+    if (lane < 32) scale_patch[lane] = line.scale;
+    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+    for (int g = 0; g < GROUPS; ++g)
+      raw.k[g] = *reinterpret_cast<const u32x4_t *>(key_patch + col * ROW + g * 64 + quad * 16);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
 #pragma unroll
       for (int g = 0; g < GROUPS; ++g)
-        out.v[i][g] = *reinterpret_cast<const uint32_t *>(slot + value_base + g * 64 + col * 4);
-      const uint8_t *scales = slot + a.token_elements;
-      if (GROUPS == 2) {
-        out.k_scale[i] = *reinterpret_cast<const uint32_t *>(scales + 2 * key_scale_index);
-        out.v_scale[i] = *reinterpret_cast<const uint32_t *>(scales + 2 * value_scale_index);
-      } else {
-        out.k_scale[i] = *reinterpret_cast<const uint16_t *>(scales + 2 * key_scale_index);
-        out.v_scale[i] = *reinterpret_cast<const uint16_t *>(scales + 2 * value_scale_index);
-      }
+        raw.v[i][g] = *reinterpret_cast<const uint32_t *>(value_patch + (quad * 4 + i) * ROW + g * 64 + col * 4);
+    const u32x4_t key_scales = *reinterpret_cast<const u32x4_t *>(scale_patch + quad * 4);
+    const u32x4_t value_scales = *reinterpret_cast<const u32x4_t *>(scale_patch + 16 + quad * 4);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      raw.k_scale[i] = key_scales[i];
+      raw.v_scale[i] = value_scales[i];
     }
+    __builtin_amdgcn_wave_barrier();
   };
 
   auto process = [&](uint32_t tile, const TileRaw &raw) __attribute__((always_inline)) {
@@ -302,21 +434,24 @@ q8_attention_split_kernel(Q8AttentionArgs a, uint32_t chunks_max, uint32_t chunk
   const uint32_t chunk_tiles = (min(past - chunk_begin, chunk_tokens) + kTileTokens - 1) / kTileTokens;
   {
     TileSlots slots_a, slots_b;
-    TileRaw raw_a, raw_b;
+    TileLine line_a, line_b;
+    TileRaw raw;
     load_slots(0, slots_a);
     load_slots(1, slots_b);
-    load_raw(slots_a, raw_a);
+    load_line(slots_a, line_a);
     // Loads return in issue order, so the small slot loads go out before the
     // K/V loads of the same step: waiting for a slot then never waits for a
     // younger K/V request.
     for (uint32_t tile = 0; tile < chunk_tiles; tile += 2) {
       load_slots(tile + 2, slots_a);
-      load_raw(slots_b, raw_b);
-      process(tile, raw_a);
+      load_line(slots_b, line_b);
+      turn(line_a, raw);
+      process(tile, raw);
       if (tile + 1 >= chunk_tiles) break;
       load_slots(tile + 3, slots_b);
-      load_raw(slots_a, raw_a);
-      process(tile + 1, raw_b);
+      load_line(slots_a, line_a);
+      turn(line_b, raw);
+      process(tile + 1, raw);
     }
   }
 
@@ -324,9 +459,7 @@ q8_attention_split_kernel(Q8AttentionArgs a, uint32_t chunks_max, uint32_t chunk
   // out_acc[g*4+jj][i] is O[head = col][d = g*64 + 4*(quad*4 + i) + jj].
   running_sum += shfl_xor_f32(running_sum, 16);
   running_sum += shfl_xor_f32(running_sum, 32);
-  float *partial = reinterpret_cast<float *>(a.workspace) +
-                   (((size_t)batch * a.kv_heads + kv_head) * chunks_max + chunk) *
-                       partial_floats<D>(heads_per_kv);
+  float *partial = reinterpret_cast<float *>(a.workspace) + partial_index * partial_floats<D>(heads_per_kv);
   if (col < heads_per_kv) {
     if (quad == 0) {
       partial[col] = running_max;
@@ -342,8 +475,6 @@ q8_attention_split_kernel(Q8AttentionArgs a, uint32_t chunks_max, uint32_t chunk
   }
 }
 
-constexpr int kMaxSplitChunks = 1024;  // merge kernel keeps one weight per chunk in LDS
-
 constexpr int kMergeSlices = 4;  // chunk slices summed in parallel per output row
 
 // One workgroup of kMergeSlices * D threads per (batch, query head): folds the
@@ -354,7 +485,8 @@ constexpr int kMergeSlices = 4;  // chunk slices summed in parallel per output r
 template <int D>
 __global__ __launch_bounds__(kMergeSlices *D) void q8_attention_merge_kernel(Q8AttentionArgs a,
                                                                              uint32_t chunks_max,
-                                                                             uint32_t chunk_tokens) {
+                                                                             uint32_t chunk_tokens,
+                                                                             uint32_t balanced_slots) {
   constexpr int THREADS = kMergeSlices * D;
   constexpr int WAVES = THREADS / 64;
   __shared__ float reduce_lds[3][WAVES];
@@ -368,11 +500,18 @@ __global__ __launch_bounds__(kMergeSlices *D) void q8_attention_merge_kernel(Q8A
   const uint32_t heads_per_kv = a.query_heads / a.kv_heads;
   const uint32_t kv_head = head / heads_per_kv;
   const uint32_t local_head = head - kv_head * heads_per_kv;
-  const uint32_t past = a.past_lengths ? a.past_lengths[batch] : a.past_length;
-  const uint32_t chunks = (past + chunk_tokens - 1) / chunk_tokens;
   const size_t stride = partial_floats<D>(heads_per_kv);
-  const float *partial = reinterpret_cast<const float *>(a.workspace) +
-                         ((size_t)batch * a.kv_heads + kv_head) * chunks_max * stride;
+  uint32_t chunks;
+  const float *partial = reinterpret_cast<const float *>(a.workspace);
+  if (balanced_slots != 0) {
+    const SplitPlan plan = split_plan<false>(a, balanced_slots, batch);
+    chunks = plan.chunks;
+    partial += ((size_t)kv_head * balanced_slots + plan.first) * stride;
+  } else {
+    const uint32_t past = a.past_lengths ? a.past_lengths[batch] : a.past_length;
+    chunks = (past + chunk_tokens - 1) / chunk_tokens;
+    partial += ((size_t)batch * a.kv_heads + kv_head) * chunks_max * stride;
+  }
 
   // score of the current token (slice 0 holds the dot product) and the largest chunk maximum
   const size_t current = ((size_t)batch * a.kv_heads + kv_head) * D + d;
@@ -554,11 +693,45 @@ uint32_t split_chunks(const Q8AttentionArgs &a) {
   return (a.max_past_length + tokens - 1) / tokens;
 }
 
+// Waves of the split kernel a SIMD holds at once, from the registers the compiler gave it
+// (512 vector registers per SIMD lane, allocated in blocks of 8).
+template <int D>
+uint32_t split_waves_per_simd() {
+  static uint32_t cached = 0;
+  if (cached == 0) {
+    hipFuncAttributes attributes;
+    uint32_t waves = 3;
+    if (hipFuncGetAttributes(&attributes, reinterpret_cast<const void *>(&q8_attention_split_kernel<D, true, true>)) ==
+            hipSuccess &&
+        attributes.numRegs > 0)
+      waves = std::max(1, std::min(8, 512 / ((attributes.numRegs + 7) / 8 * 8)));
+    else
+      (void)hipGetLastError();
+    cached = waves;
+  }
+  return cached;
+}
+
+// Chunk slots of the balanced split (0 = fixed chunks): the chunks the device holds at once
+// (one wave per KV head and chunk), times the number of rounds that gives a sequence about
+// eight chunks - with fewer, rounding the shares down leaves slots unused.  One sequence has
+// nothing to balance, and every wave scans the context lengths, so this is for batches a wave
+// covers in a few passes.
+uint32_t balanced_split_slots(const Q8AttentionArgs &a) {
+  if (a.batches < 2 || a.batches > 64 * kPlanBlocks) return 0;
+  const uint32_t per_simd = a.head_dim == 128 ? split_waves_per_simd<128>() : split_waves_per_simd<64>();
+  const uint32_t resident = std::max<uint32_t>(1, (uint32_t)device_compute_units() * 4 * per_simd / a.kv_heads);
+  const uint32_t rounds = std::max<uint32_t>(1, (8 * a.batches + resident - 1) / resident);
+  return resident * rounds;
+}
+
 }  // namespace
 
 size_t q8_attention_workspace_bytes(const Q8AttentionArgs &a) {
   if (!use_split_path(a)) return 0;
   const size_t per_partial = 32 + (size_t)(a.query_heads / a.kv_heads) * a.head_dim;
+  const uint32_t slots = balanced_split_slots(a);
+  if (slots != 0) return (size_t)a.kv_heads * slots * per_partial * sizeof(float);
   return (size_t)a.batches * a.kv_heads * split_chunks(a) * per_partial * sizeof(float);
 }
 
@@ -569,7 +742,9 @@ hipError_t launch_q8_attention(const Q8AttentionArgs &a, hipStream_t stream) {
     if (a.workspace == nullptr || a.workspace_bytes < q8_attention_workspace_bytes(a))
       return hipErrorInvalidValue;
     const uint32_t waves = std::min<uint32_t>(a.kv_heads, kSplitMaxWaves);
-    const dim3 grid(chunks, (a.kv_heads + kSplitMaxWaves - 1) / kSplitMaxWaves, a.batches);
+    const uint32_t slots = balanced_split_slots(a);
+    const uint32_t head_groups = (a.kv_heads + kSplitMaxWaves - 1) / kSplitMaxWaves;
+    const dim3 grid(slots != 0 ? slots : chunks, head_groups, slots != 0 ? 1 : a.batches);
     const dim3 block(waves * 64);
     const dim3 merge_grid(a.query_heads, a.batches);
     const bool small_pool = a.pool_bytes > 0 && a.pool_bytes <= 0xffffffffull;
@@ -578,15 +753,15 @@ hipError_t launch_q8_attention(const Q8AttentionArgs &a, hipStream_t stream) {
     const auto launch_split = [&](auto dim_tag) {
       constexpr int D = decltype(dim_tag)::value;
       if (small_pool && aligned16)
-        hipLaunchKernelGGL((q8_attention_split_kernel<D, true, true>), grid, block, 0, stream, a, chunks, chunk_tokens);
+        hipLaunchKernelGGL((q8_attention_split_kernel<D, true, true>), grid, block, 0, stream, a, chunks, chunk_tokens, slots);
       else if (small_pool)
-        hipLaunchKernelGGL((q8_attention_split_kernel<D, true, false>), grid, block, 0, stream, a, chunks, chunk_tokens);
+        hipLaunchKernelGGL((q8_attention_split_kernel<D, true, false>), grid, block, 0, stream, a, chunks, chunk_tokens, slots);
       else if (aligned16)
-        hipLaunchKernelGGL((q8_attention_split_kernel<D, false, true>), grid, block, 0, stream, a, chunks, chunk_tokens);
+        hipLaunchKernelGGL((q8_attention_split_kernel<D, false, true>), grid, block, 0, stream, a, chunks, chunk_tokens, slots);
       else
-        hipLaunchKernelGGL((q8_attention_split_kernel<D, false, false>), grid, block, 0, stream, a, chunks, chunk_tokens);
+        hipLaunchKernelGGL((q8_attention_split_kernel<D, false, false>), grid, block, 0, stream, a, chunks, chunk_tokens, slots);
       hipLaunchKernelGGL(q8_attention_merge_kernel<D>, merge_grid, dim3(kMergeSlices * D), 0, stream, a, chunks,
-                         chunk_tokens);
+                         chunk_tokens, slots);
     };
     if (a.head_dim == 128)
       launch_split(std::integral_constant<int, 128>{});

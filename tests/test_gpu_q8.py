@@ -250,6 +250,33 @@ def test_decode_attention_per_sequence_lengths(runtime):
     assert np.all(np.isfinite(out[3]))
 
 
+@pytest.mark.parametrize("b,kvh,group,dim,seed", [(70, 2, 2, 64, 5), (130, 1, 4, 128, 6), (3, 8, 4, 128, 7)])
+def test_decode_attention_balanced_split_over_many_sequences(runtime, b, kvh, group, dim, seed):
+    """Ragged batches, also wider than the 64 sequences one planning pass of a wave covers: every
+    sequence gets its own chunk size from the device-side lengths; empty, one-token and
+    tile-boundary contexts among them, and one long context that takes most of the chunk slots."""
+    rng = np.random.default_rng(seed)
+    lengths = [int(v) for v in rng.integers(64, 400, size=b)]
+    for index, value in zip(range(0, b, max(1, b // 9)), [0, 1, 15, 16, 17, 63, 65, 127, 129]):
+        lengths[index] = value
+    lengths[b // 2] = 3000
+    h = kvh * group
+    pool, slots, offsets, te, stride, ko, vo = build_pool(rng, kvh, dim, lengths)
+    query = rng.standard_normal((b, h, 1, dim)).astype(np.float16)
+    ck = rng.standard_normal((b, kvh, 1, dim)).astype(np.float16)
+    cv = rng.standard_normal((b, kvh, 1, dim)).astype(np.float16)
+    params = PagedParams(batches=b, query_heads=h, kv_heads=kvh, past_length=0, head_dim=dim,
+                         mask_batches=0, mask_heads=0, token_elements=te, key_offset=ko,
+                         value_offset=vo, group_size=64, token_stride=stride,
+                         scale=1.0 / math.sqrt(dim), query_length=1, mask_dtype=0, window=0)
+    out = run_paged(runtime, "llmopt_attention_q8_paged_batched", query, ck, cv, pool, slots, None,
+                    params, lengths=lengths, offsets=offsets)
+    expected = oracle.paged_attention_q8(query, ck, cv, pool, slots, None, params,
+                                         past_lengths=np.array(lengths), slot_offsets=offsets)
+    assert np.all(np.isfinite(out))
+    assert_close_to_oracle(out, expected, f"balanced split b{b} kv{kvh} d{dim}")
+
+
 ROW_CASES = [
     # (b, h, kvh, dim, past, q_len, window, mask_dtype)
     (1, 2, 1, 64, 10, 1, 0, 0), (2, 4, 2, 128, 33, 1, 8, 0), (1, 3, 1, 64, 20, 3, 0, 1),
