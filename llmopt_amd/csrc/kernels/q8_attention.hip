@@ -513,16 +513,37 @@ __global__ __launch_bounds__(kMergeSlices *D) void q8_attention_merge_kernel(Q8A
     partial += ((size_t)batch * a.kv_heads + kv_head) * chunks_max * stride;
   }
 
+  // Every request goes out before the first result is used - the chunk maxima and denominators
+  // (chunk tid, tid + THREADS, ...), the first kAhead chunks of this thread's slice of the
+  // weighted sum, the current token - so the kernel waits for memory once, not once per phase.
+  constexpr int PER = kMaxSplitChunks / THREADS;  // chunks of phase 1 per thread
+  constexpr int kAhead = 8;
+  static_assert(PER * THREADS == kMaxSplitChunks, "phase 1 covers every chunk once");
+  float chunk_max[PER], chunk_denominator[PER];
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const uint32_t c = tid + i * THREADS;
+    chunk_max[i] = c < chunks ? partial[c * stride + local_head] : -INFINITY;
+    chunk_denominator[i] = c < chunks ? partial[c * stride + 16 + local_head] : 0.0f;
+  }
+  const float *column = partial + 32 + local_head * D + d;
+  float ahead[kAhead];
+#pragma unroll
+  for (int i = 0; i < kAhead; ++i) {
+    const uint32_t c = slice + i * kMergeSlices;
+    ahead[i] = c < chunks ? column[c * stride] : 0.0f;
+  }
   // score of the current token (slice 0 holds the dot product) and the largest chunk maximum
   const size_t current = ((size_t)batch * a.kv_heads + kv_head) * D + d;
+  const float current_value = slice == 0 ? half_bits_to_float(a.current_value[current]) : 0.0f;
   float dot = 0.0f;
   if (slice == 0)
     dot = half_bits_to_float(a.query[((size_t)batch * a.query_heads + head) * D + d]) *
           half_bits_to_float(a.current_key[current]);
   dot = wave_sum(dot);
   float chunk_best = -INFINITY;
-  for (uint32_t c = tid; c < chunks; c += THREADS)
-    chunk_best = fmaxf(chunk_best, partial[c * stride + local_head]);
+#pragma unroll
+  for (int i = 0; i < PER; ++i) chunk_best = fmaxf(chunk_best, chunk_max[i]);
   chunk_best = wave_max(chunk_best);
   if ((tid & 63) == 0) {
     reduce_lds[0][tid >> 6] = dot;
@@ -540,10 +561,14 @@ __global__ __launch_bounds__(kMergeSlices *D) void q8_attention_merge_kernel(Q8A
 
   // weights and denominator
   float denominator_part = 0.0f;
-  for (uint32_t c = tid; c < chunks; c += THREADS) {
-    const float weight = __builtin_amdgcn_exp2f(partial[c * stride + local_head] - best);
-    weight_lds[c] = weight;
-    denominator_part += weight * partial[c * stride + 16 + local_head];
+#pragma unroll
+  for (int i = 0; i < PER; ++i) {
+    const uint32_t c = tid + i * THREADS;
+    if (c < chunks) {
+      const float weight = __builtin_amdgcn_exp2f(chunk_max[i] - best);
+      weight_lds[c] = weight;
+      denominator_part += weight * chunk_denominator[i];
+    }
   }
   denominator_part = wave_sum(denominator_part);
   if ((tid & 63) == 0) reduce_lds[2][tid >> 6] = denominator_part;
@@ -553,9 +578,13 @@ __global__ __launch_bounds__(kMergeSlices *D) void q8_attention_merge_kernel(Q8A
 #pragma unroll
   for (int w = 0; w < WAVES; ++w) denominator += reduce_lds[2][w];
 
-  float value = slice == 0 ? current_weight * half_bits_to_float(a.current_value[current]) : 0.0f;
-  const float *column = partial + 32 + local_head * D + d;
-  uint32_t c = slice;
+  float value = current_weight * current_value;
+#pragma unroll
+  for (int i = 0; i < kAhead; ++i) {
+    const uint32_t c = slice + i * kMergeSlices;
+    if (c < chunks) value += weight_lds[c] * ahead[i];
+  }
+  uint32_t c = slice + kAhead * kMergeSlices;
   for (; c + 3 * kMergeSlices < chunks; c += 4 * kMergeSlices) {
     const float v0 = column[(c + 0 * kMergeSlices) * stride], v1 = column[(c + 1 * kMergeSlices) * stride];
     const float v2 = column[(c + 2 * kMergeSlices) * stride], v3 = column[(c + 3 * kMergeSlices) * stride];
