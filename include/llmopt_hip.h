@@ -144,6 +144,20 @@ int llmopt_hip_buffer_set_u32_array(llmopt_hip_buffer *buffer, int64_t offset,
  * `vocabulary` fp16 logits; ties go to the lowest index. */
 int llmopt_hip_buffer_argmax_f16(llmopt_hip_buffer *buffer, int64_t vocabulary, int64_t *out);
 
+/* ---- host-side token selection --------------------------------------------- */
+
+/* caml_llmopt_f16_argmax (native/ocaml_metal_stubs.m:2565-2579): index of the
+ * first maximum of `count` fp16 logits in host memory (0 for an empty row). */
+int llmopt_hip_f16_argmax(const uint16_t *logits, int64_t count, int64_t *out_index);
+/* caml_llmopt_sample_f16_native (native/ocaml_metal_stubs.m:2629-2765; called by
+ * Sampling.sample, lib/sampling.ml:193-207, on the last logits row in host memory):
+ * greedy when temperature <= 1e-4 or top_k == 1; else top-k (0 -> 64, at most 256)
+ * by a bounded min-heap, float32 softmax with temperature, min-p, top-p, and one
+ * draw from xoroshiro128+ seeded with `seed` (0 = from the clock).  Same float32
+ * operation order and tie handling as the reference: a seed gives the same token. */
+int llmopt_hip_sample_f16(const uint16_t *logits, int64_t count, double temperature, int64_t top_k,
+                          double top_p, double min_p, int64_t seed, int64_t *out_token);
+
 /* ---- dispatch ------------------------------------------------------------ */
 
 /* caml_llmopt_metal_dispatch (:1384-1454): launches one kernel and waits. */

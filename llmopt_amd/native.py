@@ -84,6 +84,9 @@ def lib() -> ctypes.CDLL:
         "llmopt_hip_buffer_set_int64": (ctypes.c_int, [vp, i64, i64]),
         "llmopt_hip_buffer_set_u32_array": (ctypes.c_int, [vp, i64, ctypes.POINTER(i64), sz]),
         "llmopt_hip_buffer_argmax_f16": (ctypes.c_int, [vp, i64, ctypes.POINTER(i64)]),
+        "llmopt_hip_f16_argmax": (ctypes.c_int, [vp, i64, ctypes.POINTER(i64)]),
+        "llmopt_hip_sample_f16": (ctypes.c_int, [vp, i64, ctypes.c_double, i64, ctypes.c_double, ctypes.c_double,
+                                                 i64, ctypes.POINTER(i64)]),
         "llmopt_hip_dispatch": (ctypes.c_int, [vp, item_p]),
         "llmopt_hip_begin_batch": (ctypes.c_int, [vp, pp]),
         "llmopt_hip_release_batch": (None, [vp]),
@@ -118,7 +121,8 @@ EXPORTED_SYMBOLS = (
     "llmopt_hip_buffer_view", "llmopt_hip_buffer_wrap", "llmopt_hip_release_buffer",
     "llmopt_hip_buffer_contents", "llmopt_hip_buffer_length", "llmopt_hip_buffer_device_pointer",
     "llmopt_hip_buffer_copy", "llmopt_hip_buffer_write", "llmopt_hip_buffer_set_int64",
-    "llmopt_hip_buffer_set_u32_array", "llmopt_hip_buffer_argmax_f16", "llmopt_hip_dispatch",
+    "llmopt_hip_buffer_set_u32_array", "llmopt_hip_buffer_argmax_f16", "llmopt_hip_f16_argmax",
+    "llmopt_hip_sample_f16", "llmopt_hip_dispatch",
     "llmopt_hip_begin_batch", "llmopt_hip_release_batch", "llmopt_hip_batch_dispatch",
     "llmopt_hip_batch_dispatch_all", "llmopt_hip_batch_copy", "llmopt_hip_batch_barrier",
     "llmopt_hip_commit_batch", "llmopt_hip_commit_batch_async",
