@@ -70,12 +70,13 @@ struct GemvParams {
 // for everything in flight and the ring degenerates to one item.  ADD (ring
 // only): the residual addend of a tile travels with its items, so that the
 // store path has no load of its own to wait for.
-// XREG (ring only, K <= 2048): a lane meets the same 32 K values in every item, so it keeps its
-// piece of the activation in registers - no LDS copy, no workgroup barrier before the first row.
+// XREG (ring only, K <= 2048 U): an item covers a whole row, so a lane meets the same U x 32 K
+// values in every item and keeps its pieces of the activation in registers - no LDS copy, no
+// workgroup barrier before the first row.
 template <int M, int R, int U, bool XLDS, bool DUAL, int D = 0, bool ADD = false, bool XREG = false>
 __global__ __launch_bounds__(kThreads) void w4a16_gemv_kernel(GemvParams p) {
   static_assert(D == 0 || XLDS, "the ring of loads needs the activation in LDS");
-  static_assert(!XREG || (D > 0 && U == 1), "the register activation belongs to the ring");
+  static_assert(!XREG || D > 0, "the register activation belongs to the ring");
   static_assert(!ADD || (D > 0 && !DUAL), "the addend travels with the ring only");
   extern __shared__ uint4 x_lds[];
   const int lane = threadIdx.x & 63;
@@ -219,45 +220,51 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemv_kernel(GemvParams p) {
     const uint32_t seg = kk >> 2, j = kk & 3;
     x_lds[((m * chunks + (seg >> 6)) * 4 + j) * 64 + (seg & 63)] = value;
   };
-  // XREG: the lane's own four vectors of every row; pair order and bias correction as in LDS
-  u32x4_t x_own[XREG ? M : 1][4];
-  uint4 x_held[XREG ? M : 1][4];
-  float correction_held[XREG ? M : 1];
+  // XREG: the lane's own four vectors per chunk of every row; pair order and bias correction as in LDS
+  u32x4_t x_own[XREG ? M : 1][XREG ? U : 1][4];
+  uint4 x_held[XREG ? M : 1][XREG ? U : 1][4];
+  float correction_held[XREG ? M : 1][XREG ? U : 1];
   if constexpr (XREG) {
 #if defined(__HIP_DEVICE_COMPILE__)
-    const uint32_t own_segment = min((uint32_t)lane, segs - 1);
 #pragma unroll
-    for (int m = 0; m < M; ++m) {
-      const uint16_t *row = p.x + (size_t)min((uint32_t)m, p.m - 1) * K + own_segment * 32;
+    for (int m = 0; m < M; ++m)
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-        asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(x_own[m][j]) : "v"(row + j * 8) : "memory");
-    }
+      for (int u = 0; u < U; ++u) {
+        const uint32_t own_segment = min((uint32_t)(u * 64 + lane), segs - 1);
+        const uint16_t *row = p.x + (size_t)min((uint32_t)m, p.m - 1) * K + own_segment * 32;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(x_own[m][u][j]) : "v"(row + j * 8) : "memory");
+      }
 #endif
     static_for<D>([&](auto index) __attribute__((always_inline)) { request(decltype(index)::value); });
 #if defined(__HIP_DEVICE_COMPILE__)
     // only the ring's requests may still be outstanding
-    asm volatile("s_waitcnt vmcnt(%1)" : "+v"(x_own[0][0]) : "n"(D * LOADS) : "memory");
+    asm volatile("s_waitcnt vmcnt(%1)" : "+v"(x_own[0][0][0]) : "n"(D * LOADS) : "memory");
 #pragma unroll
     for (int m = 0; m < M; ++m)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) asm volatile("" : "+v"(x_own[m][j]));
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) asm volatile("" : "+v"(x_own[m][u][j]));
 #endif
 #pragma unroll
-    for (int m = 0; m < M; ++m) {
-      const bool present = (uint32_t)lane < segs && (uint32_t)m < p.m;
-      float sum_a = 0.0f, sum_b = 0.0f;
+    for (int m = 0; m < M; ++m)
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const uint4 v = pair_order(__builtin_bit_cast(uint4, x_own[m][j]));
-        x_held[m][j] = present ? v : make_uint4(0, 0, 0, 0);
-        const h2_t a0 = as_h2(x_held[m][j].x), b0 = as_h2(x_held[m][j].y);
-        const h2_t a1 = as_h2(x_held[m][j].z), b1 = as_h2(x_held[m][j].w);
-        sum_a += ((float)a0[0] + (float)a0[1]) + ((float)a1[0] + (float)a1[1]);
-        sum_b += ((float)b0[0] + (float)b0[1]) + ((float)b1[0] + (float)b1[1]);
+      for (int u = 0; u < U; ++u) {
+        const bool present = (uint32_t)(u * 64 + lane) < segs && (uint32_t)m < p.m;
+        float sum_a = 0.0f, sum_b = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const uint4 v = pair_order(__builtin_bit_cast(uint4, x_own[m][u][j]));
+          x_held[m][u][j] = present ? v : make_uint4(0, 0, 0, 0);
+          const h2_t a0 = as_h2(x_held[m][u][j].x), b0 = as_h2(x_held[m][u][j].y);
+          const h2_t a1 = as_h2(x_held[m][u][j].z), b1 = as_h2(x_held[m][u][j].w);
+          sum_a += ((float)a0[0] + (float)a0[1]) + ((float)a1[0] + (float)a1[1]);
+          sum_b += ((float)b0[0] + (float)b0[1]) + ((float)b1[0] + (float)b1[1]);
+        }
+        correction_held[m][u] = 1032.0f * sum_a + 72.0f * sum_b;
       }
-      correction_held[m] = 1032.0f * sum_a + 72.0f * sum_b;
-    }
   } else if constexpr (D > 0) {
 #if defined(__HIP_DEVICE_COMPILE__)
     static_for<kXAhead>([&](auto index) __attribute__((always_inline)) {
@@ -352,7 +359,7 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemv_kernel(GemvParams p) {
 #pragma unroll
         for (int m = 0; m < M; ++m) {
           if (XREG) {
-            xp[m] = x_held[XREG ? m : 0][j];
+            xp[m] = x_held[XREG ? m : 0][XREG ? u : 0][j];
           } else if (XLDS) {
             xp[m] = x_lds[((m * chunks + c_safe) * 4 + j) * 64 + lane];
           } else {
@@ -377,7 +384,7 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemv_kernel(GemvParams p) {
       }
 #pragma unroll
       for (int m = 0; m < M; ++m) {
-        const float correction = XREG   ? correction_held[XREG ? m : 0]
+        const float correction = XREG   ? correction_held[XREG ? m : 0][XREG ? u : 0]
                                  : XLDS ? corr_lds[(m * chunks + c_safe) * 64 + lane]
                                         : 0.0f;
 #pragma unroll
@@ -514,8 +521,8 @@ hipError_t launch_variant(const GemvParams &p, uint32_t matrices, uint32_t max_n
   while (per_cu > 1 && lds_bytes * per_cu > 150 * 1024) --per_cu;
   const uint32_t wanted = (tiles + kWaves - 1) / kWaves;
   const uint32_t blocks = std::max<uint32_t>(1, std::min<uint32_t>(wanted, (uint32_t)(cus * per_cu)));
-  if constexpr (D > 0 && U == 1) {
-    if (chunks == 1) {  // K <= 2048: the activation stays in registers, no LDS
+  if constexpr (D > 0) {
+    if (chunks == (uint32_t)U) {  // an item covers the row: the activation stays in registers, no LDS
       if constexpr (!DUAL) {
         if (p.has_addend) {
           hipLaunchKernelGGL((w4a16_gemv_kernel<M, R, U, true, DUAL, D, true, true>), dim3(blocks, matrices),
