@@ -326,7 +326,7 @@ def pmc_probe(runtime, m=1):
         record_linear(batch, m, n, k, bx, bw, bs, out)
     batch.commit()
     return {"copy_kernel": "copy_vectors_kernel", "copy_bytes_read": copy_bytes, "copy_bytes_written": copy_bytes,
-            "copy_launches": 4, "gemv_kernel": "w4a16_gemv_kernel<1, 2, 1, true, false, 2, false>",
+            "copy_launches": 4, "gemv_kernel": "w4a16_gemv_kernel<1, 2, 1, true, false, 2, false, false>",
             "gemv_rows": m, "gemv_launches": COPIES, "gemv_algorithmic_bytes": gemv_bytes(m, k, n)}
 
 
@@ -428,7 +428,7 @@ def main():
                                "{(4096,4096),(4096,14336),(14336,4096)}, group-64 fp16 scales; "
                                "one step = the 12 launches, weights cycled over 16 HBM copies",
                    "bytes_per_step": gemv["bytes_per_step"]},
-        "roofline": {"bound": "hbm", "kernel": "w4a16_gemv_kernel<1, 2, 1, true, false, 2, false> (M=1) at K=4096 N=14336",
+        "roofline": {"bound": "hbm", "kernel": "w4a16_gemv_kernel<1, 2, 1, true, false, 2, false, false> (M=1) at K=4096 N=14336",
                      "achieved": headline["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": headline["hbm_frac"], "traffic": measured_traffic(),
                      "bytes_per_launch": headline["bytes"], "us_per_launch": headline["us_per_launch"]},
