@@ -151,14 +151,9 @@ __global__ __launch_bounds__(kRowWaves * 64) void rotary_qk_kernel(RotaryQkArgs 
   const uint32_t trig_batch = a.trig_batches == 1 ? 0 : batch;
   const size_t trig_base = (size_t)(trig_batch * a.tokens + token) * a.width;
   const size_t output_base = (size_t)local_row * a.width;
-  for (uint32_t col = lane; col < a.width; col += 64) {
-    const uint32_t rotated_col = col < a.half_dimension ? col + a.half_dimension : col - a.half_dimension;
-    _Float16 rotated = input[input_base + rotated_col];
-    if (col < a.half_dimension) rotated = -rotated;
-    const _Float16 direct = input[input_base + col] * cosine[trig_base + col];
-    const _Float16 turned = rotated * sine[trig_base + col];
-    output[output_base + col] = direct + turned;
-  }
+  for (uint32_t col = lane; col < a.width; col += 64)
+    output[output_base + col] =
+        rotate_half_element(input + input_base, cosine + trig_base, sine + trig_base, col, a.half_dimension);
 }
 
 // lib/metal_tensor_source.ml:306-320

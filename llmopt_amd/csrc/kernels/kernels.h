@@ -179,6 +179,15 @@ struct RotaryQkArgs {
 };
 hipError_t launch_rotary_qk(const RotaryQkArgs &args, hipStream_t stream);
 
+// The rotation of one token per sequence (tokens = 1) and, in the same launch, the Q8
+// quantisation of the rotated keys (pack.source[0] is rotary.k_output) and of the values
+// into their pool slots; pack.item_major is set.  Same arithmetic as the two launches.
+struct RotaryPackArgs {
+  RotaryQkArgs rotary;
+  Q8PackArgs pack;
+};
+hipError_t launch_rotary_qk_pack(const RotaryPackArgs &args, hipStream_t stream);
+
 // llmopt_embedding_f16 (lib/metal_tensor_source.ml:306-320): row gather, rows
 // outside [0, vocabulary) give zeros.
 struct EmbeddingArgs {

@@ -17,6 +17,16 @@
 namespace llmopt {
 namespace {
 
+// One 64-wide group, one element per lane: the stored scale and this lane's int8 value.
+__device__ __forceinline__ int8_t q8_quantize(float x, uint16_t *stored_scale) {
+  const float maximum = wave_max(fabsf(x));
+  const uint16_t stored = float_to_half_bits(maximum == 0.0f ? 1.0f : maximum / 127.0f);
+  const float scale = half_bits_to_float(stored);
+  const float rounded = rintf(x / scale);
+  *stored_scale = stored;
+  return (int8_t)(int)fminf(fmaxf(rounded, -127.0f), 127.0f);
+}
+
 template <bool PAIR>
 __global__ __launch_bounds__(256) void q8_pack_kernel(Q8PackArgs a) {
   const uint32_t lane = threadIdx.x & 63;
@@ -40,14 +50,52 @@ __global__ __launch_bounds__(256) void q8_pack_kernel(Q8PackArgs a) {
   for (int which = 0; which < (PAIR ? 2 : 1); ++which) {
     const uint16_t *source = which == 0 ? a.source[0] : a.source[1];
     const uint32_t segment_offset = a.segment_offset[which];
-    const float x = half_bits_to_float(source[source_index]);
-    const float maximum = wave_max(fabsf(x));
-    const uint16_t stored = float_to_half_bits(maximum == 0.0f ? 1.0f : maximum / 127.0f);
-    const float scale = half_bits_to_float(stored);
-    const float rounded = rintf(x / scale);
-    const int quantized = (int)fminf(fmaxf(rounded, -127.0f), 127.0f);
-    values[segment_offset + local_offset + lane] = (int8_t)quantized;
+    uint16_t stored;
+    values[segment_offset + local_offset + lane] = q8_quantize(half_bits_to_float(source[source_index]), &stored);
     if (lane == 0) scales[(segment_offset >> 6) + local_group] = stored;
+  }
+}
+
+// One wave per row of head_dim values, four rows per workgroup: the query rows of every
+// sequence (rotated), then the key rows (rotated, stored as fp16 for this step's attention and
+// as Q8 in the sequence's new pool slot), then the value rows (Q8 only).  A row is walked in
+// 64-wide pieces, which are the Q8 groups.
+__global__ __launch_bounds__(256) void rotary_qk_pack_kernel(RotaryPackArgs a) {
+  const RotaryQkArgs &r = a.rotary;
+  const Q8PackArgs &p = a.pack;
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const uint32_t q_rows = r.batches * r.q_heads, kv_rows = r.batches * r.k_heads;
+  if (row >= q_rows + 2 * kv_rows) return;
+  const bool is_q = row < q_rows;
+  const bool is_v = row >= q_rows + kv_rows;
+  const uint32_t local_row = is_q ? row : is_v ? row - q_rows - kv_rows : row - q_rows;  // [sequence, head]
+  const uint32_t heads = is_q ? r.q_heads : r.k_heads;
+  const uint32_t batch = local_row / heads;
+  const uint32_t head = local_row - batch * heads;
+  const size_t base = (size_t)local_row * r.width;
+  const _Float16 *input = reinterpret_cast<const _Float16 *>(is_q ? r.q_input : is_v ? p.source[1] : r.k_input) + base;
+  _Float16 *output = reinterpret_cast<_Float16 *>(is_q ? r.q_output : r.k_output) + base;
+  const size_t trig_base = (size_t)(r.trig_batches == 1 ? 0 : batch) * r.width;
+  const _Float16 *cosine = reinterpret_cast<const _Float16 *>(r.cosine) + trig_base;
+  const _Float16 *sine = reinterpret_cast<const _Float16 *>(r.sine) + trig_base;
+  size_t slot_base = 0;
+  if (!is_q) slot_base = (size_t)p.slots[batch] * p.token_stride;
+  int8_t *values = reinterpret_cast<int8_t *>(p.pool + slot_base);
+  uint16_t *scales = reinterpret_cast<uint16_t *>(p.pool + slot_base + p.token_elements);
+  const uint32_t segment_offset = p.segment_offset[is_v ? 1 : 0];
+  for (uint32_t col = lane; col < r.width; col += 64) {
+    _Float16 value;
+    if (is_v) {
+      value = input[col];
+    } else {
+      value = rotate_half_element(input, cosine, sine, col, r.half_dimension);
+      output[col] = value;
+    }
+    if (is_q) continue;
+    uint16_t stored;
+    values[segment_offset + head * r.width + col] = q8_quantize((float)value, &stored);
+    if (lane == 0) scales[(segment_offset >> 6) + head * (r.width >> 6) + (col >> 6)] = stored;
   }
 }
 
@@ -87,6 +135,17 @@ hipError_t launch_q8_pack(const Q8PackArgs &args, bool pair, hipStream_t stream)
     hipLaunchKernelGGL(q8_pack_kernel<true>, dim3(blocks), dim3(256), 0, stream, args);
   else
     hipLaunchKernelGGL(q8_pack_kernel<false>, dim3(blocks), dim3(256), 0, stream, args);
+  return hipGetLastError();
+}
+
+hipError_t launch_rotary_qk_pack(const RotaryPackArgs &args, hipStream_t stream) {
+  const RotaryQkArgs &r = args.rotary;
+  if (r.tokens != 1 || r.width % 64 != 0 || args.pack.items != r.batches || args.pack.heads != r.k_heads ||
+      args.pack.head_dim != r.width || !args.pack.item_major)
+    return hipErrorInvalidValue;
+  const uint32_t rows = r.batches * (r.q_heads + 2 * r.k_heads);
+  if (rows == 0) return hipSuccess;
+  hipLaunchKernelGGL(rotary_qk_pack_kernel, dim3((rows + 3) / 4), dim3(256), 0, stream, args);
   return hipGetLastError();
 }
 

@@ -103,6 +103,21 @@ __device__ __forceinline__ float wave_sum(float value) {
   return (r0 + r1) + (r2 + r3);
 }
 
+// Rotate-half position encoding of one element (lib/metal_normalization_source.ml:765-802):
+// half(half(x[col] * cos[col]) + half(+-x[col -+ half_dimension] * sin[col])), every product and
+// the sum rounded to half separately.
+__device__ __forceinline__ _Float16 rotate_half_element(const _Float16 *input, const _Float16 *cosine,
+                                                        const _Float16 *sine, uint32_t col,
+                                                        uint32_t half_dimension) {
+#pragma clang fp contract(off)
+  const uint32_t rotated_col = col < half_dimension ? col + half_dimension : col - half_dimension;
+  _Float16 rotated = input[rotated_col];
+  if (col < half_dimension) rotated = -rotated;
+  const _Float16 direct = input[col] * cosine[col];
+  const _Float16 turned = rotated * sine[col];
+  return direct + turned;
+}
+
 __device__ __forceinline__ float wave_max(float value) {
   value = fmaxf(value, __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
                            0, __builtin_bit_cast(int, value), 0xB1, 0xF, 0xF, false)));

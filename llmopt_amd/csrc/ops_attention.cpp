@@ -61,20 +61,21 @@ int cache_pack(llmopt_hip_context *context, const DispatchRecord &record) {
 
 // AttentionCachePairParams, 11 x u32 (lib/metal_cache_source.ml:22-34).
 // buffers: key_source, value_source, slots, pool.
-int cache_pack_pair_layout(llmopt_hip_context *context, const DispatchRecord &record, bool item_major) {
-  if (int status = require_buffer_count(record, 4)) return status;
-  if (int status = require_parameter_bytes(record, 44)) return status;
+// `at`: byte offset of the 11 words in the record's parameters; the buffers are
+// record.buffers[key], [value], [slots], [pool].
+int parse_pack_pair(const DispatchRecord &record, size_t at, size_t key, size_t value, size_t slots, size_t pool,
+                    bool item_major, Q8PackArgs *out) {
   Q8PackArgs args = {};
-  args.items = param_u32(record, 0);
-  args.segment_offset[0] = param_u32(record, 4);
-  args.segment_offset[1] = param_u32(record, 8);
-  args.heads = param_u32(record, 12);
-  args.head_dim = param_u32(record, 16);
-  const uint32_t group_size = param_u32(record, 20);
-  args.token_elements = param_u32(record, 24);
-  args.token_stride = param_u32(record, 32);
-  args.source_items = param_u32(record, 36);
-  args.source_offset = param_u32(record, 40);
+  args.items = param_u32(record, at + 0);
+  args.segment_offset[0] = param_u32(record, at + 4);
+  args.segment_offset[1] = param_u32(record, at + 8);
+  args.heads = param_u32(record, at + 12);
+  args.head_dim = param_u32(record, at + 16);
+  const uint32_t group_size = param_u32(record, at + 20);
+  args.token_elements = param_u32(record, at + 24);
+  args.token_stride = param_u32(record, at + 32);
+  args.source_items = param_u32(record, at + 36);
+  args.source_offset = param_u32(record, at + 40);
   args.item_major = item_major ? 1 : 0;
   if (item_major) {
     args.source_items = args.items;
@@ -90,14 +91,23 @@ int cache_pack_pair_layout(llmopt_hip_context *context, const DispatchRecord &re
   if ((uint64_t)args.source_offset + args.items > args.source_items)
     return fail(LLMOPT_ERR_INVALID, "%s source window lies outside the source", record.name.c_str());
   const uint64_t source_bytes = (uint64_t)args.heads * args.source_items * args.head_dim * 2;
-  if (int status = require_buffer_size(record.buffers[0], source_bytes, "key source")) return status;
-  if (int status = require_buffer_size(record.buffers[1], source_bytes, "value source")) return status;
-  if (int status = require_buffer_size(record.buffers[2], (uint64_t)args.items * 4, "slots")) return status;
-  if (int status = require_buffer_size(record.buffers[3], args.token_stride, "pool")) return status;
-  args.source[0] = reinterpret_cast<const uint16_t *>(record.buffers[0].device);
-  args.source[1] = reinterpret_cast<const uint16_t *>(record.buffers[1].device);
-  args.slots = reinterpret_cast<const uint32_t *>(record.buffers[2].device);
-  args.pool = record.buffers[3].device;
+  if (int status = require_buffer_size(record.buffers[key], source_bytes, "key source")) return status;
+  if (int status = require_buffer_size(record.buffers[value], source_bytes, "value source")) return status;
+  if (int status = require_buffer_size(record.buffers[slots], (uint64_t)args.items * 4, "slots")) return status;
+  if (int status = require_buffer_size(record.buffers[pool], args.token_stride, "pool")) return status;
+  args.source[0] = reinterpret_cast<const uint16_t *>(record.buffers[key].device);
+  args.source[1] = reinterpret_cast<const uint16_t *>(record.buffers[value].device);
+  args.slots = reinterpret_cast<const uint32_t *>(record.buffers[slots].device);
+  args.pool = record.buffers[pool].device;
+  *out = args;
+  return LLMOPT_OK;
+}
+
+int cache_pack_pair_layout(llmopt_hip_context *context, const DispatchRecord &record, bool item_major) {
+  if (int status = require_buffer_count(record, 4)) return status;
+  if (int status = require_parameter_bytes(record, 44)) return status;
+  Q8PackArgs args = {};
+  if (int status = parse_pack_pair(record, 0, 0, 1, 2, 3, item_major, &args)) return status;
   return launched(launch_q8_pack(args, true, context->stream), record.name.c_str());
 }
 
@@ -109,6 +119,24 @@ int cache_pack_pair(llmopt_hip_context *context, const DispatchRecord &record) {
 // each of `items` sequences, sources laid out [items, heads, head_dim].
 int cache_pack_pair_batched(llmopt_hip_context *context, const DispatchRecord &record) {
   return cache_pack_pair_layout(context, record, true);
+}
+
+// Extension (no reference kernel): llmopt_rotary_qk_f16_simd_h64 followed by
+// llmopt_cache_pack_attention_q8_pair_batched on the rotated keys, as one launch - a decode
+// step is bound by its number of launches.  Parameters: RotaryQKParams (7 words, tokens = 1)
+// then AttentionCachePairParams (11 words); buffers: q_input, k_input, cosine, sine, q_output,
+// k_output (also the quantiser's key source), value source, slots, pool.
+int rotary_qk_pack_batched(llmopt_hip_context *context, const DispatchRecord &record) {
+  if (int status = require_buffer_count(record, 9)) return status;
+  if (int status = require_parameter_bytes(record, 28 + 44)) return status;
+  RotaryPackArgs args = {};
+  if (int status = parse_rotary_qk(record, &args.rotary)) return status;
+  if (int status = parse_pack_pair(record, 28, 5, 6, 7, 8, true, &args.pack)) return status;
+  if (args.rotary.tokens != 1 || args.pack.items != args.rotary.batches || args.pack.heads != args.rotary.k_heads ||
+      args.pack.head_dim != args.rotary.width)
+    return fail(LLMOPT_ERR_INVALID, "%s requires one token per sequence and the same sequences, KV heads and width "
+                "in both parameter blocks", record.name.c_str());
+  return launched(launch_rotary_qk_pack(args, context->stream), record.name.c_str());
 }
 
 // buffers: pool, slots, destination; AttentionCacheParams.
@@ -301,6 +329,7 @@ void register_cache_kernels(std::vector<KernelEntryPoint> &table) {
   table.push_back({"llmopt_cache_pack_attention_q8_simd", cache, cache_pack});
   table.push_back({"llmopt_cache_pack_attention_q8_pair_simd", cache, cache_pack_pair});
   table.push_back({"llmopt_cache_pack_attention_q8_pair_batched", cache, cache_pack_pair_batched});
+  table.push_back({"llmopt_rotary_qk_pack_q8_batched", cache, rotary_qk_pack_batched});
   table.push_back({"llmopt_cache_unpack_attention_q8", cache, cache_unpack});
   table.push_back({"llmopt_cache_unpack_attention_q8_vec4", cache, cache_unpack});
 }

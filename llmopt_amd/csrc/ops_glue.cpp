@@ -11,6 +11,43 @@
 #include "runtime.h"
 
 namespace llmopt {
+
+// The first 28 parameter bytes and the first 6 buffers of a rotary record, checked.
+int parse_rotary_qk(const DispatchRecord &record, RotaryQkArgs *out) {
+  RotaryQkArgs args = {};
+  args.batches = param_u32(record, 0);
+  args.tokens = param_u32(record, 4);
+  args.q_heads = param_u32(record, 8);
+  args.k_heads = param_u32(record, 12);
+  args.width = param_u32(record, 16);
+  args.half_dimension = param_u32(record, 20);
+  args.trig_batches = param_u32(record, 24);
+  if (args.batches == 0 || args.tokens == 0 || args.width == 0 || args.q_heads + args.k_heads == 0)
+    return fail(LLMOPT_ERR_INVALID, "%s requires positive batches, tokens, heads and width", record.name.c_str());
+  if (args.half_dimension * 2 != args.width)
+    return fail(LLMOPT_ERR_INVALID, "%s requires half_dimension = width / 2", record.name.c_str());
+  if (args.trig_batches != 1 && args.trig_batches != args.batches)
+    return fail(LLMOPT_ERR_INVALID, "%s requires trig_batches to be 1 or batches", record.name.c_str());
+  const uint64_t token_rows = (uint64_t)args.batches * args.tokens;
+  const uint64_t q_bytes = token_rows * args.q_heads * args.width * 2;
+  const uint64_t k_bytes = token_rows * args.k_heads * args.width * 2;
+  const uint64_t trig_bytes = (uint64_t)args.trig_batches * args.tokens * args.width * 2;
+  if (int status = require_buffer_size(record.buffers[0], q_bytes, "q input")) return status;
+  if (int status = require_buffer_size(record.buffers[1], k_bytes, "k input")) return status;
+  if (int status = require_buffer_size(record.buffers[2], trig_bytes, "cosine")) return status;
+  if (int status = require_buffer_size(record.buffers[3], trig_bytes, "sine")) return status;
+  if (int status = require_buffer_size(record.buffers[4], q_bytes, "q output")) return status;
+  if (int status = require_buffer_size(record.buffers[5], k_bytes, "k output")) return status;
+  args.q_input = reinterpret_cast<const uint16_t *>(record.buffers[0].device);
+  args.k_input = reinterpret_cast<const uint16_t *>(record.buffers[1].device);
+  args.cosine = reinterpret_cast<const uint16_t *>(record.buffers[2].device);
+  args.sine = reinterpret_cast<const uint16_t *>(record.buffers[3].device);
+  args.q_output = reinterpret_cast<uint16_t *>(record.buffers[4].device);
+  args.k_output = reinterpret_cast<uint16_t *>(record.buffers[5].device);
+  *out = args;
+  return LLMOPT_OK;
+}
+
 namespace {
 
 const uint16_t *as_f16(const BoundBuffer &buffer) {
@@ -76,35 +113,7 @@ int rotary_qk(llmopt_hip_context *context, const DispatchRecord &record) {
   if (int status = require_buffer_count(record, 6)) return status;
   if (int status = require_parameter_bytes(record, 28)) return status;
   RotaryQkArgs args = {};
-  args.batches = param_u32(record, 0);
-  args.tokens = param_u32(record, 4);
-  args.q_heads = param_u32(record, 8);
-  args.k_heads = param_u32(record, 12);
-  args.width = param_u32(record, 16);
-  args.half_dimension = param_u32(record, 20);
-  args.trig_batches = param_u32(record, 24);
-  if (args.batches == 0 || args.tokens == 0 || args.width == 0 || args.q_heads + args.k_heads == 0)
-    return fail(LLMOPT_ERR_INVALID, "%s requires positive batches, tokens, heads and width", record.name.c_str());
-  if (args.half_dimension * 2 != args.width)
-    return fail(LLMOPT_ERR_INVALID, "%s requires half_dimension = width / 2", record.name.c_str());
-  if (args.trig_batches != 1 && args.trig_batches != args.batches)
-    return fail(LLMOPT_ERR_INVALID, "%s requires trig_batches to be 1 or batches", record.name.c_str());
-  const uint64_t token_rows = (uint64_t)args.batches * args.tokens;
-  const uint64_t q_bytes = token_rows * args.q_heads * args.width * 2;
-  const uint64_t k_bytes = token_rows * args.k_heads * args.width * 2;
-  const uint64_t trig_bytes = (uint64_t)args.trig_batches * args.tokens * args.width * 2;
-  if (int status = require_buffer_size(record.buffers[0], q_bytes, "q input")) return status;
-  if (int status = require_buffer_size(record.buffers[1], k_bytes, "k input")) return status;
-  if (int status = require_buffer_size(record.buffers[2], trig_bytes, "cosine")) return status;
-  if (int status = require_buffer_size(record.buffers[3], trig_bytes, "sine")) return status;
-  if (int status = require_buffer_size(record.buffers[4], q_bytes, "q output")) return status;
-  if (int status = require_buffer_size(record.buffers[5], k_bytes, "k output")) return status;
-  args.q_input = as_f16(record.buffers[0]);
-  args.k_input = as_f16(record.buffers[1]);
-  args.cosine = as_f16(record.buffers[2]);
-  args.sine = as_f16(record.buffers[3]);
-  args.q_output = as_f16_out(record.buffers[4]);
-  args.k_output = as_f16_out(record.buffers[5]);
+  if (int status = parse_rotary_qk(record, &args)) return status;
   return launched(launch_rotary_qk(args, context->stream), record.name.c_str());
 }
 

@@ -110,6 +110,10 @@ void *context_workspace(llmopt_hip_context *context, size_t bytes);
 // Returns the context's zero-initialised arrival counters (allocated on first
 // use) or nullptr with the error set.
 uint32_t *context_counters(llmopt_hip_context *context, uint32_t *count);
+struct RotaryQkArgs;
+// RotaryQKParams (the first 28 parameter bytes) and the six rotary buffers (the first six of
+// the record), checked as llmopt_rotary_qk_f16_simd_h64 checks them.
+int parse_rotary_qk(const DispatchRecord &record, RotaryQkArgs *out);
 
 void retain(RefCounted *object);
 // Returns true when the caller dropped the last reference.

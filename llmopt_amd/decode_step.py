@@ -154,7 +154,6 @@ class DecodeStep:
         out.append(("llmopt_embedding_f16", [self.tokens, self.device["embedding"], w["x"][0]],
                     u32s(m, c.vocabulary, h), (((count + 255) // 256) * 256, 1, 1), group))
         rows_grid = (((m + 7) // 8) * 256, 1, 1)
-        rope_rows_total = m * (c.q_heads + c.kv_heads)
         for index, layer in enumerate(self.device["layers"]):
             x_in, x_mid = w["x"][0], w["x"][1]
             key_offset = index * c.layer_elements
@@ -165,15 +164,14 @@ class DecodeStep:
             out.append(("llmopt_w4a16_qkv_linear_f16_g64" + suffix,
                         [w["normed"], *layer["q"], *layer["k"], *layer["v"], w["q"], w["k"], w["v"]],
                         u32s(m, h, qd, kvd, kvd), grid, group))
-            out.append(("llmopt_rotary_qk_f16_simd_h64",
-                        [w["q"], w["k"], self.cos, self.sin, w["q_rot"], w["k_rot"]],
-                        u32s(m, 1, c.q_heads, c.kv_heads, c.head_dim, c.head_dim // 2, m),
-                        (((rope_rows_total + 7) // 8) * 256, 1, 1), group))
-            out.append(("llmopt_cache_pack_attention_q8_pair_batched",
-                        [w["k_rot"], w["v"], self.new_slots, self.pool],
+            # rotation and the new token's Q8 slot in one launch (the step is bound by its launches)
+            out.append(("llmopt_rotary_qk_pack_q8_batched",
+                        [w["q"], w["k"], self.cos, self.sin, w["q_rot"], w["k_rot"], w["v"], self.new_slots,
+                         self.pool],
+                        u32s(m, 1, c.q_heads, c.kv_heads, c.head_dim, c.head_dim // 2, m) +
                         u32s(m, key_offset, value_offset, c.kv_heads, c.head_dim, 64, c.token_elements,
                              c.token_elements // 64, c.token_stride, m, 0),
-                        (m * c.kv_heads * 32, 1, 1), group))
+                        (((m * (c.q_heads + 2 * c.kv_heads) + 3) // 4) * 256, 1, 1), group))
             attention_params = struct.pack(
                 "<12IfIII", m, c.q_heads, c.kv_heads, 0, c.head_dim, 0, 0, c.token_elements, key_offset,
                 value_offset, 64, c.token_stride, 1.0 / math.sqrt(c.head_dim), 1, 0, 0)

@@ -106,6 +106,84 @@ def test_rotary_qk_h64(runtime, batches, tokens, q_heads, k_heads):
             assert float(error.max()) <= 3 * 2.0 ** -11 * max(1.0, float(np.abs(expected).max()))
 
 
+@pytest.mark.parametrize("batches,q_heads,k_heads,d,trig_batches", [(1, 9, 3, 64, 1), (5, 9, 3, 64, 5),
+                                                                     (33, 32, 8, 128, 33), (2, 4, 4, 128, 1)])
+def test_rotary_pack_in_one_launch_equals_the_two_launches(runtime, batches, q_heads, k_heads, d, trig_batches):
+    """The decode step's fused extension against the kernels it stands for, bit for bit: rotated
+    queries and keys, and the Q8 bytes and scales of the new token's keys and values in the pool."""
+    rng = np.random.default_rng(batches * 1000 + d)
+    layers = 2
+    elements = layers * 2 * k_heads * d
+    stride = elements + 2 * (elements // 64)
+    key_offset, value_offset = 2 * k_heads * d, 3 * k_heads * d  # the second layer's segments
+    capacity = batches + 3
+    q = rng.standard_normal((batches, 1, q_heads, d)).astype(np.float16)
+    k = rng.standard_normal((batches, 1, k_heads, d)).astype(np.float16)
+    v = rng.standard_normal((batches, k_heads, d)).astype(np.float16)
+    v[0, 0, :64] = 0  # an all-zero group stores scale 1.0
+    cos = np.concatenate([rope_tables(1, d, rng)[0] for _ in range(trig_batches)])
+    sin = np.concatenate([rope_tables(1, d, rng)[1] for _ in range(trig_batches)])
+    slots = rng.permutation(capacity)[:batches].astype(np.uint32)
+    start = rng.integers(0, 256, size=capacity * stride, dtype=np.uint8)
+    rotary_params = u32s(batches, 1, q_heads, k_heads, d, d // 2, trig_batches)
+    pack_params = u32s(batches, key_offset, value_offset, k_heads, d, 64, elements, elements // 64, stride,
+                       batches, 0)
+    inputs = [runtime.buffer_of_bytes(x) for x in (q, k, cos, sin)]
+    v_buffer, slot_buffer = runtime.buffer_of_bytes(v), runtime.buffer_of_bytes(slots)
+
+    def outputs():
+        return (runtime.buffer_of_bytes(np.full(q.size, np.nan, dtype=np.float16)),
+                runtime.buffer_of_bytes(np.full(k.size, np.nan, dtype=np.float16)),
+                runtime.buffer_of_bytes(start))
+
+    q_two, k_two, pool_two = outputs()
+    rows = batches * (q_heads + k_heads)
+    runtime.dispatch("llmopt_rotary_qk_f16_simd_h64", [*inputs, q_two, k_two], rotary_params,
+                     grid=(((rows + 7) // 8) * 256, 1, 1), group=(256, 1, 1))
+    runtime.dispatch("llmopt_cache_pack_attention_q8_pair_batched", [k_two, v_buffer, slot_buffer, pool_two],
+                     pack_params, grid=(batches * k_heads * (d // 64) * 64, 1, 1), group=(256, 1, 1))
+    q_one, k_one, pool_one = outputs()
+    runtime.dispatch("llmopt_rotary_qk_pack_q8_batched",
+                     [*inputs, q_one, k_one, v_buffer, slot_buffer, pool_one], rotary_params + pack_params,
+                     grid=(((batches * (q_heads + 2 * k_heads) + 3) // 4) * 256, 1, 1), group=(256, 1, 1))
+    np.testing.assert_array_equal(q_one.numpy(np.uint16, (q.size,)), q_two.numpy(np.uint16, (q.size,)))
+    np.testing.assert_array_equal(k_one.numpy(np.uint16, (k.size,)), k_two.numpy(np.uint16, (k.size,)))
+    got = pool_one.numpy(np.uint8, (capacity, stride))
+    np.testing.assert_array_equal(got, pool_two.numpy(np.uint8, (capacity, stride)))
+    # and the two launches did write: the new slots differ from the starting bytes, the others do not
+    before = start.reshape(capacity, stride)
+    untouched = np.setdiff1d(np.arange(capacity), slots)
+    np.testing.assert_array_equal(got[untouched], before[untouched])
+    assert all((got[slot] != before[slot]).any() for slot in slots)
+    # the values of the first sequence against the quantiser's definition
+    first = got[slots[0]]
+    scales = first[elements:].view(np.float16)
+    assert scales[value_offset // 64] == np.float16(1.0) and not first[value_offset:value_offset + 64].any()
+    group = v[0, 0, 64:128] if d == 128 else v[0, 1, :64]
+    scale = np.float16(np.float32(np.abs(group).max()) / np.float32(127.0))
+    assert scales[value_offset // 64 + 1] == scale
+    expected = np.clip(np.rint(group.astype(np.float32) / np.float32(scale)), -127, 127).astype(np.int8)
+    np.testing.assert_array_equal(first[value_offset + 64:value_offset + 128].view(np.int8), expected)
+
+
+def test_rotary_pack_rejects_blocks_that_disagree(runtime):
+    d, batches, heads = 64, 2, 3
+    elements = 2 * heads * d
+    stride = elements + 2 * (elements // 64)
+    half = lambda count: runtime.buffer_of_bytes(np.zeros(count, dtype=np.float16))
+    buffers = [half(batches * 9 * d), half(batches * heads * d), half(2 * d), half(2 * d), half(batches * 9 * d),
+               half(batches * heads * d), half(batches * heads * d),
+               runtime.buffer_of_bytes(np.arange(batches, dtype=np.uint32)),
+               runtime.buffer_of_bytes(np.zeros(batches * stride, dtype=np.uint8))]
+    pack = lambda items, kv: u32s(items, 0, heads * d, kv, d, 64, elements, elements // 64, stride, items, 0)
+    for rotary, cache in ((u32s(batches, 1, 9, heads, d, d // 2, 1), pack(batches, 2)),
+                          (u32s(batches, 1, 9, heads, d, d // 2, 1), pack(1, heads)),
+                          (u32s(1, 2, 9, heads, d, d // 2, 1), pack(batches, heads))):
+        with pytest.raises(Exception, match="requires one token per sequence"):
+            runtime.dispatch("llmopt_rotary_qk_pack_q8_batched", buffers, rotary + cache,
+                             grid=(256, 1, 1), group=(256, 1, 1))
+
+
 def test_embedding_gather_and_out_of_range(runtime):
     rng = np.random.default_rng(5)
     vocabulary, width = 1000, 576
