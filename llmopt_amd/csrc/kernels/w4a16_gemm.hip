@@ -54,17 +54,26 @@ __device__ __forceinline__ f16x_t zero_tile() {
 // Each wave owns WM x WN MFMA tiles of 32 x 32 outputs; the workgroup tile is
 // (4 * WM * 32) x (2 * WN * 32).  DUAL computes gate and up tiles of the same
 // outputs and stores silu(gate) * up.
-template <int WM, int WN, bool DUAL>
+// XS: LDS stages of the activation tile = steps a K loop iteration is unrolled by = weight
+// register sets.  2 for the large tiles, whose steps are long enough to cover a load; 4 (K a
+// multiple of 4 steps) for the small ones, whose steps are shorter than the trip to memory:
+// the activation copy then runs three steps ahead of its use and the weights four.
+template <int WM, int WN, bool DUAL, int XS>
 __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
+  static_assert(XS == 2 || XS == 4, "the weight stage alternates with the step: an even unroll");
+  constexpr int WS = XS;            // weight register sets
   constexpr int NW = DUAL ? 2 : 1;  // weight matrices per tile
   constexpr int BM = 4 * WM * 32;
   constexpr int BN = 2 * WN * 32;
   constexpr int W_VECTORS = (BN * BK / 32 + kThreads - 1) / kThreads;  // 32-nibble vectors per thread
   extern __shared__ __attribute__((aligned(16))) unsigned char gemm_lds[];
-  // two stages of {x[BM] rows of BK halfs, vector index swizzled; w[NW][BN] rows
-  // of LDS_STRIDE halfs}
+  // x[BM] rows of BK halfs, vector index swizzled, in XS stages; w[NW][BN] rows of LDS_STRIDE
+  // halfs in two.  XS = 2: {x, w} {x, w}; XS = 4: the four x stages, then the two of w.
   constexpr int X_HALFS = BM * BK;
-  constexpr int STAGE_HALFS = X_HALFS + NW * BN * LDS_STRIDE;
+  constexpr int W_HALFS = NW * BN * LDS_STRIDE;
+  constexpr int X_STAGE_HALFS = XS == 2 ? X_HALFS + W_HALFS : X_HALFS;  // from one x stage to the next
+  constexpr int W_STAGE_HALFS = XS == 2 ? X_HALFS + W_HALFS : W_HALFS;
+  constexpr int W_BASE_HALFS = XS == 2 ? X_HALFS : XS * X_HALFS;
   constexpr int X_CHUNKS = BM / 8 / (kThreads / 64);  // 8-row direct loads per wave and K step
   static_assert(BM / 8 % (kThreads / 64) == 0, "activation tile must divide over the waves");
   _Float16 *stage_lds = reinterpret_cast<_Float16 *>(gemm_lds);
@@ -108,7 +117,7 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
 #pragma unroll
     for (int c = 0; c < X_CHUNKS; ++c) {
       const uint32_t lds_address =
-          lds_base + (uint32_t)((stage * STAGE_HALFS + (wave * X_CHUNKS + c) * 8 * BK) * sizeof(_Float16));
+          lds_base + (uint32_t)((stage * X_STAGE_HALFS + (wave * X_CHUNKS + c) * 8 * BK) * sizeof(_Float16));
       asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off"
                    :
                    : "v"(x_src[c] + k0), "s"(lds_address)
@@ -117,8 +126,8 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
   };
 
   // Weights go global -> registers (w row tid/2, half tid%2) -> decode -> LDS.
-  // Two register sets: a set is decoded one step after it was requested and
-  // requested again right after, so every load has a whole K step to arrive.
+  // WS register sets: set s % WS holds the weights of step s; it is decoded during step
+  // s - 1 and requested again right after, for step s - 1 + WS.
   static_assert(W_VECTORS == 1, "one 32-nibble vector per thread and matrix");
   const uint32_t w_row = tid >> 1;
   const uint32_t w_half = tid & 1;
@@ -126,7 +135,7 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
     u32x4_t w[NW];
     uint32_t s[NW];  // fp16 bits in the low half
   };
-  Fetched fetched[2];
+  Fetched fetched[WS];
   constexpr int W_LOADS = 2 * NW;  // vector memory loads of one fetch_w
   const uint32_t w_col = min(n0 + w_row, p.n - 1);  // columns past n are never stored
 
@@ -163,7 +172,7 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
   // most), in natural K order.
   constexpr int ITEMS = NW * 4;
   auto store_item = [&](const Fetched &f, int stage, int item) __attribute__((always_inline)) {
-    _Float16 *w_lds = stage_lds + stage * STAGE_HALFS + X_HALFS;
+    _Float16 *w_lds = stage_lds + W_BASE_HALFS + stage * W_STAGE_HALFS;
     const int v = item / 4;
     const int j = item % 4;
     if (BN % 256 != 0 && w_row >= (uint32_t)BN) return;
@@ -194,21 +203,27 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
   const int row_base = wave_m * WM * 32;
   const int col_base = wave_n * WN * 32;
 
-  // One barrier per K step.  Step i runs its MFMAs from stage i%2 while the set
-  // fetched for step i+1 is decoded into the other stage; that set is then
-  // requested again for step i+3 (requests past the end fetch the last K block
-  // again, which nothing reads).  The issue order is fixed by hand: groups of
+  // One barrier per K step.  Step i runs its MFMAs from weight stage i % 2 and activation
+  // stage i % XS while the set fetched for step i + 1 is decoded into the other weight stage;
+  // that set is then requested again for step i + 1 + WS, and the activation copy of step
+  // i + XS - 1 goes into the stage step i - 1 read (requests past the end fetch the last K
+  // block again, which nothing reads).  Loads return in order, so the two waits count the
+  // loads issued after the one they need: every step issues X_CHUNKS copies, then W_LOADS
+  // weight loads.  The issue order is fixed by hand: groups of
   // four chained MFMAs alternate with one or two decode items, and the weight
   // operands of the next column block are read while the current one computes,
   // so the matrix pipe does not wait for the vector work, LDS or HBM.
   constexpr int BLOCKS = NW * WN;      // column blocks of a step
   constexpr int GROUPS = BLOCKS * WM;  // MFMA groups of a step
   constexpr int ITEMS_PER_GROUP = (ITEMS + GROUPS - 1) / GROUPS;
-  auto step = [&](uint32_t k0, auto parity) __attribute__((always_inline)) {
-    constexpr int stage = decltype(parity)::value;
+  constexpr int STEP_LOADS = X_CHUNKS + W_LOADS;
+  auto step = [&](uint32_t k0, auto index) __attribute__((always_inline)) {
+    constexpr int j = decltype(index)::value;  // step number modulo XS
+    constexpr int stage = j & 1;
+    constexpr int next_set = (j + 1) % WS;
     __syncthreads();  // this stage is written; the other stage's readers are done
-    const _Float16 *x_lds = stage_lds + stage * STAGE_HALFS;
-    const _Float16 *w_lds = x_lds + X_HALFS;
+    const _Float16 *x_lds = stage_lds + j * X_STAGE_HALFS;
+    const _Float16 *w_lds = stage_lds + W_BASE_HALFS + stage * W_STAGE_HALFS;
     h8_t a_frag[WM][BK / 16];
     h8_t b_frag[2][BK / 16];
     auto read_block = [&](int block) __attribute__((always_inline)) {
@@ -241,30 +256,46 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
         __builtin_amdgcn_sched_barrier(0);
         if (a == 0 && block + 1 < BLOCKS) read_block(block + 1);
         const int group = block * WM + a;
-        if (group == 0) wait_w(fetched[stage ^ 1], std::integral_constant<int, W_LOADS>{});
+        // the set was requested at the end of step i - WS: WS - 1 steps of loads are younger
+        // (XS = 2: the wait that ended the last step left one set of weight loads)
+        if (group == 0)
+          wait_w(fetched[next_set], std::integral_constant<int, XS == 2 ? W_LOADS : (WS - 1) * STEP_LOADS>{});
 #pragma unroll
         for (int n = 0; n < ITEMS_PER_GROUP; ++n)
           if (group * ITEMS_PER_GROUP + n < ITEMS)
-            store_item(fetched[stage ^ 1], stage ^ 1, group * ITEMS_PER_GROUP + n);
-        if (group == 0) fetch_x(min(k0 + BK, K - BK), stage ^ 1);
+            store_item(fetched[next_set], stage ^ 1, group * ITEMS_PER_GROUP + n);
+        if (group == 0) fetch_x(min(k0 + (XS - 1) * BK, K - BK), (j + XS - 1) % XS);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
-    fetch_w(fetched[stage ^ 1], min(k0 + 3 * BK, K - BK));
+    fetch_w(fetched[next_set], min(k0 + (1 + WS) * BK, K - BK));
     __builtin_amdgcn_sched_barrier(0);
-    wait_all(std::integral_constant<int, W_LOADS>{});  // the activation copy has landed
+    // the activation copy of step i + 1 has landed: it went out in step i + 2 - XS, before
+    // that step's weight loads and the XS - 2 steps of loads since
+    wait_all(std::integral_constant<int, (XS - 2) * STEP_LOADS + W_LOADS>{});
   };
 
-  fetch_x(0, 0);
-  fetch_w(fetched[0], 0);
-  fetch_w(fetched[1], min((uint32_t)BK, K - BK));
-  wait_w(fetched[0], std::integral_constant<int, W_LOADS>{});
+#pragma unroll
+  for (int s = 0; s < XS - 1; ++s) fetch_x(min((uint32_t)s * BK, K - BK), s);
+#pragma unroll
+  for (int s = 0; s < WS; ++s) fetch_w(fetched[s], min((uint32_t)s * BK, K - BK));
+  wait_w(fetched[0], std::integral_constant<int, (WS - 1) * W_LOADS>{});
 #pragma unroll
   for (int item = 0; item < ITEMS; ++item) store_item(fetched[0], 0, item);
-  fetch_w(fetched[0], min(2u * BK, K - BK));
-  for (uint32_t k0 = 0; k0 < K; k0 += 2 * BK) {
-    step(k0, std::integral_constant<int, 0>{});
-    if (k0 + BK < K) step(k0 + BK, std::integral_constant<int, 1>{});
+  fetch_w(fetched[0], min((uint32_t)WS * BK, K - BK));
+  if constexpr (XS == 2) {
+    for (uint32_t k0 = 0; k0 < K; k0 += 2 * BK) {
+      step(k0, std::integral_constant<int, 0>{});
+      if (k0 + BK < K) step(k0 + BK, std::integral_constant<int, 1>{});
+    }
+  } else {  // K is a multiple of XS steps: no branch between a request and its wait
+    wait_all(std::integral_constant<int, W_LOADS>{});  // every activation copy and every other set has landed
+    for (uint32_t k0 = 0; k0 < K; k0 += XS * BK) {
+      step(k0, std::integral_constant<int, 0>{});
+      step(k0 + BK, std::integral_constant<int, 1>{});
+      step(k0 + 2 * BK, std::integral_constant<int, 2>{});
+      step(k0 + 3 * BK, std::integral_constant<int, 3>{});
+    }
   }
   wait_all(std::integral_constant<int, 0>{});  // the surplus requests still target live registers
 
@@ -295,16 +326,16 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
   }
 }
 
-template <int WM, int WN, bool DUAL>
+template <int WM, int WN, bool DUAL, int XS = 2>
 hipError_t launch_tile(GemmParams &p, hipStream_t stream) {
   constexpr int NW = DUAL ? 2 : 1;
   constexpr int BM = 4 * WM * 32;
   constexpr int BN = 2 * WN * 32;
-  constexpr size_t lds_bytes =
-      2 * ((size_t)BM * BK + (size_t)NW * BN * LDS_STRIDE) * sizeof(_Float16);
+  constexpr size_t lds_bytes = ((size_t)XS * BM * BK + 2 * (size_t)NW * BN * LDS_STRIDE) * sizeof(_Float16);
+  static_assert(lds_bytes <= 160 * 1024, "a workgroup's stages must fit the CU's LDS");
   static bool configured = false;
   if (!configured) {
-    hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(&w4a16_gemm_kernel<WM, WN, DUAL>),
+    hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(&w4a16_gemm_kernel<WM, WN, DUAL, XS>),
                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (status != hipSuccess) return status;
     configured = true;
@@ -312,7 +343,7 @@ hipError_t launch_tile(GemmParams &p, hipStream_t stream) {
   p.tiles_m = (p.m + BM - 1) / BM;
   p.tiles_n = (p.n + BN - 1) / BN;
   const uint32_t blocks = p.tiles_m * p.tiles_n;
-  hipLaunchKernelGGL((w4a16_gemm_kernel<WM, WN, DUAL>), dim3(blocks), dim3(kThreads), lds_bytes, stream, p);
+  hipLaunchKernelGGL((w4a16_gemm_kernel<WM, WN, DUAL, XS>), dim3(blocks), dim3(kThreads), lds_bytes, stream, p);
   return hipGetLastError();
 }
 
@@ -325,6 +356,12 @@ hipError_t launch_gemm(GemmParams &p, hipStream_t stream) {
   if (big >= (uint64_t)cus) return launch_tile<2, 4, false>(p, stream);
   const uint64_t mid = (uint64_t)((p.m + 127) / 128) * ((p.n + 255) / 256);
   if (mid >= (uint64_t)cus) return launch_tile<1, 4, false>(p, stream);
+  // 128 x 128 tiles have steps shorter than a trip to memory.  With two stages they fit a CU
+  // twice, which covers the loads; when there is at most one tile per CU anyway, four
+  // activation stages do (K a whole number of four steps; measured 58 -> 49 us at 512 x 4096 x 4096,
+  // and nothing for the 128 x 256 tiles, which stay with two).
+  const uint64_t small = (uint64_t)((p.m + 127) / 128) * ((p.n + 127) / 128);
+  if (p.k % (4 * BK) == 0 && small <= (uint64_t)cus) return launch_tile<1, 2, false, 4>(p, stream);
   return launch_tile<1, 2, false>(p, stream);
 }
 

@@ -102,7 +102,7 @@ def test_gemv_residual_epilogue(runtime, m):
 # up to 128 rows with small weights run the matrix-core GEMV once per group of 8 rows
 GEMM_SHAPES = [(9, 64, 64), (16, 128, 128), (24, 576, 1536), (31, 100, 576), (32, 1536, 576),
                (32, 96, 14336), (33, 64, 576), (64, 576, 1536), (100, 29, 192), (128, 192, 576), (129, 64, 576), (128, 256, 512), (130, 300, 1024),
-               (512, 128, 4096)]
+               (512, 128, 4096), (200, 130, 256), (140, 260, 768), (512, 4096, 256)]
 
 
 @pytest.mark.parametrize("m,n,k", GEMM_SHAPES)
