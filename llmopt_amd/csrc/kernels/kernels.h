@@ -41,6 +41,20 @@ struct W4LinearArgs {
 // Bytes of workspace the decode path wants for this shape (0 when it does not split K).
 size_t w4a16_gemv_workspace_bytes(uint32_t m, uint32_t n, uint32_t k);
 
+// Optional RMS normalisation of the activation rows on their way into a decode kernel
+// (weight == nullptr: none): the kernel multiplies by half(x * gain * r) (weight_first) or
+// half(x * r * gain), r = rsqrt(mean(x^2) + epsilon) in float32 - the values
+// llmopt_rms_norm_f16_simd / llmopt_w4a16_swiglu_rms_f16_g64 would have written for it to read.
+// Only where w4a16_norm_in_kernel() says so.
+struct W4Norm {
+  const uint16_t *weight;  // f16 [k]
+  float epsilon;
+  uint32_t weight_first;
+};
+// True when launch_w4a16_qkv / launch_w4a16_dual_swiglu with these sizes run a kernel that can
+// normalise its activation itself (`columns` = all outputs of the launch).
+bool w4a16_norm_in_kernel(uint32_t m, uint64_t columns, uint32_t k);
+
 // Three projections of one activation in one launch
 // (llmopt_w4a16_qkv_linear_f16_g64*, lib/metal_w4a16_source.ml:218-480).
 struct W4QkvArgs {
@@ -49,6 +63,7 @@ struct W4QkvArgs {
   uint16_t *y[3];  // f16 [m, n[i]]
   uint32_t n[3];
   uint32_t m, k;
+  W4Norm norm;
 };
 
 // product[r, c] = half(silu(gate[r,c]) * up[r,c]) with gate, up fp32
@@ -58,6 +73,7 @@ struct W4DualSwigluArgs {
   W4Matrix gate, up;  // each [n, k/2]
   uint16_t *product;  // f16 [m, n]
   uint32_t m, n, k;
+  W4Norm norm;
 };
 
 hipError_t launch_w4a16_linear(const W4LinearArgs &args, hipStream_t stream);

@@ -16,6 +16,7 @@ hipError_t launch_w4a16_gemv_dual_swiglu(const W4DualSwigluArgs &args, hipStream
 // kGemvDotRows < m <= kGemvMaxRows: matrix-core GEMV
 // true when K does not fit one workgroup (more than 16 ranges of 256): only the plain
 // linear can then run (it splits K over workgroups and needs scratch)
+bool w4a16_gemv_norm_ok(uint32_t m, uint32_t k);
 bool w4a16_gemv_mfma_needs_split(uint32_t k);
 // kGemvMaxRows < m <= 128 with small weights and a K one workgroup covers: the
 // same kernel once per group of 8 rows (the weights are re-read from L2), which

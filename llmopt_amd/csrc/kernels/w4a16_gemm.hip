@@ -409,7 +409,13 @@ hipError_t launch_w4a16_linear(const W4LinearArgs &args, hipStream_t stream) {
   return launch_w4a16_gemm_linear(args, stream);
 }
 
+bool w4a16_norm_in_kernel(uint32_t m, uint64_t columns, uint32_t k) {
+  (void)columns;
+  return w4a16_gemv_norm_ok(m, k);
+}
+
 hipError_t launch_w4a16_dual_swiglu(const W4DualSwigluArgs &args, hipStream_t stream) {
+  if (args.norm.weight != nullptr && !w4a16_norm_in_kernel(args.m, 2ull * args.n, args.k)) return hipErrorInvalidValue;
   if (args.m <= kGemvDotRows) return launch_w4a16_gemv_dual_swiglu(args, stream);
   if ((args.m <= kGemvMaxRows && !w4a16_gemv_mfma_needs_split(args.k)) ||
       w4a16_gemv_mfma_row_groups_ok(args.m, 2ull * args.n, args.k))
@@ -418,6 +424,9 @@ hipError_t launch_w4a16_dual_swiglu(const W4DualSwigluArgs &args, hipStream_t st
 }
 
 hipError_t launch_w4a16_qkv(const W4QkvArgs &args, hipStream_t stream) {
+  if (args.norm.weight != nullptr &&
+      !w4a16_norm_in_kernel(args.m, (uint64_t)args.n[0] + args.n[1] + args.n[2], args.k))
+    return hipErrorInvalidValue;
   if (args.m <= kGemvDotRows) return launch_w4a16_gemv_qkv(args, stream);
   if ((args.m <= kGemvMaxRows && !w4a16_gemv_mfma_needs_split(args.k)) ||
       w4a16_gemv_mfma_row_groups_ok(args.m, (uint64_t)args.n[0] + args.n[1] + args.n[2], args.k))

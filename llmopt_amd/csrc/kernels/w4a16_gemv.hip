@@ -51,6 +51,7 @@ struct GemvParams {
   uint32_t has_addend;
   uint32_t addend_stride;
   float *y_f32;  // optional float32 copy of seg0's output (same indexing), may be null
+  W4Norm norm;   // XREG variants only
 };
 
 // M: activation rows held per lane, R: weight rows per wave and tile, U: K
@@ -222,10 +223,21 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemv_kernel(GemvParams p) {
   };
   // XREG: the lane's own four vectors per chunk of every row; pair order and bias correction as in LDS
   u32x4_t x_own[XREG ? M : 1][XREG ? U : 1][4];
+  u32x4_t gain_own[XREG ? U : 1][4];  // the RMS norm weights of the same K values, if any
   uint4 x_held[XREG ? M : 1][XREG ? U : 1][4];
   float correction_held[XREG ? M : 1][XREG ? U : 1];
   if constexpr (XREG) {
+    const bool normalise = p.norm.weight != nullptr;  // the same for every wave
 #if defined(__HIP_DEVICE_COMPILE__)
+    if (normalise) {
+#pragma unroll
+      for (int u = 0; u < U; ++u) {
+        const uint16_t *gain = p.norm.weight + min((uint32_t)(u * 64 + lane), segs - 1) * 32;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+          asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(gain_own[u][j]) : "v"(gain + j * 8) : "memory");
+      }
+    }
 #pragma unroll
     for (int m = 0; m < M; ++m)
 #pragma unroll
@@ -247,7 +259,47 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemv_kernel(GemvParams p) {
       for (int u = 0; u < U; ++u)
 #pragma unroll
         for (int j = 0; j < 4; ++j) asm volatile("" : "+v"(x_own[m][u][j]));
+    if (normalise) {
+#pragma unroll
+      for (int u = 0; u < U; ++u)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) asm volatile("" : "+v"(gain_own[u][j]));
+    }
 #endif
+    if (normalise) {
+      // The wave holds whole rows: mean square by a wave reduction, then the half values the
+      // separate normalisation kernel would have stored (float32 products in its order).
+#pragma unroll
+      for (int m = 0; m < M; ++m) {
+        float square_sum = 0.0f;
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+          const bool present = (uint32_t)(u * 64 + lane) < segs;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const h8_t x = __builtin_bit_cast(h8_t, x_own[m][u][j]);
+#pragma unroll
+            for (int e = 0; e < 8; ++e) square_sum += present ? (float)x[e] * (float)x[e] : 0.0f;
+          }
+        }
+        square_sum = wave_sum(square_sum);
+        const float inverse = rsqrtf(square_sum / (float)K + p.norm.epsilon);
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const h8_t x = __builtin_bit_cast(h8_t, x_own[m][u][j]);
+            const h8_t g = __builtin_bit_cast(h8_t, gain_own[u][j]);
+            h8_t y;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+              const float value = (float)x[e], gain = (float)g[e];
+              y[e] = (_Float16)(p.norm.weight_first ? value * gain * inverse : value * inverse * gain);
+            }
+            x_own[m][u][j] = __builtin_bit_cast(u32x4_t, y);
+          }
+      }
+    }
 #pragma unroll
     for (int m = 0; m < M; ++m)
 #pragma unroll
@@ -501,6 +553,10 @@ int device_compute_units() {
   return cached;
 }
 
+// The register-activation variants (one or two rows, K of at most one 2048-wide chunk) hold
+// whole rows per wave and can normalise them.
+bool w4a16_gemv_norm_ok(uint32_t m, uint32_t k) { return m <= (uint32_t)kGemvDotRows && k <= 2048 && k % 64 == 0; }
+
 namespace {
 
 template <int M, int R, int U, bool DUAL, int D = 0>
@@ -610,6 +666,8 @@ hipError_t launch_w4a16_gemv_qkv(const W4QkvArgs &a, hipStream_t stream) {
   p.seg0 = {a.w[0].weight, a.w[0].scale, a.y[0], a.n[0]};
   p.seg1 = {a.w[1].weight, a.w[1].scale, a.y[1], a.n[1]};
   p.seg2 = {a.w[2].weight, a.w[2].scale, a.y[2], a.n[2]};
+  p.norm = a.norm;
+  if (p.norm.weight != nullptr && !w4a16_gemv_norm_ok(a.m, a.k)) return hipErrorInvalidValue;
   return launch_by_rows<false>(p, 3, std::max(a.n[0], std::max(a.n[1], a.n[2])), stream);
 }
 
@@ -620,6 +678,8 @@ hipError_t launch_w4a16_gemv_dual_swiglu(const W4DualSwigluArgs &a, hipStream_t 
   p.k = a.k;
   p.seg0 = {a.gate.weight, a.gate.scale, a.product, a.n};
   p.seg1 = {a.up.weight, a.up.scale, a.product, a.n};
+  p.norm = a.norm;
+  if (p.norm.weight != nullptr && !w4a16_gemv_norm_ok(a.m, a.k)) return hipErrorInvalidValue;
   return launch_by_rows<true>(p, 1, a.n, stream);
 }
 

@@ -2,6 +2,8 @@
 // layout and size checks of the reference's kernels
 // (lib/metal_w4a16_source.ml; host side lib/metal_dispatch_linear.ml:252-455,
 // 938-982), bound to the gfx950 launchers.
+#include <cmath>
+
 #include "kernels/kernels.h"
 #include "runtime.h"
 
@@ -77,51 +79,116 @@ int w4a16_linear(llmopt_hip_context *context, const DispatchRecord &record) {
   return launched(launch_w4a16_linear(args, context->stream), record.name.c_str());
 }
 
+// The activation of a normalising entry: either the kernel normalises (*norm is set and *x stays
+// the raw input) or the rows are normalised into the context's scratch here (*x moves there).
+int normalise_input(llmopt_hip_context *context, const DispatchRecord &record, const W4Norm &wanted, uint32_t m,
+                    uint32_t k, uint64_t columns, const uint16_t **x, W4Norm *norm) {
+  if (!std::isfinite(wanted.epsilon) || wanted.epsilon <= 0.0f)
+    return fail(LLMOPT_ERR_INVALID, "%s requires a positive finite epsilon", record.name.c_str());
+  if (int status = require_buffer_size(record.buffers[1], (uint64_t)k * 2, "norm weight")) return status;
+  const bool aligned = ((reinterpret_cast<uintptr_t>(*x) | reinterpret_cast<uintptr_t>(wanted.weight)) & 15) == 0;
+  if (aligned && w4a16_norm_in_kernel(m, columns, k)) {
+    *norm = wanted;
+    return LLMOPT_OK;
+  }
+  uint16_t *scratch = static_cast<uint16_t *>(context_workspace(context, (size_t)m * k * 2));
+  if (scratch == nullptr) return LLMOPT_ERR_FAILURE;
+  RmsNormArgs args = {};
+  args.input = *x;
+  args.weight = wanted.weight;
+  args.output = scratch;
+  args.rows = m;
+  args.width = k;
+  args.epsilon = wanted.epsilon;
+  args.weight_first = wanted.weight_first != 0;
+  if (int status = launched(launch_rms_norm(args, context->stream), record.name.c_str())) return status;
+  *x = scratch;
+  return LLMOPT_OK;
+}
+
 // W4A16QKVParams {u32 m, k, n_q, n_k, n_v}  (lib/metal_w4a16_source.ml:211-217)
 // buffers: input, qW, qS, kW, kS, vW, vS, qOut, kOut, vOut.
-int w4a16_qkv_linear(llmopt_hip_context *context, const DispatchRecord &record) {
-  if (int status = require_buffer_count(record, 10)) return status;
-  if (int status = require_parameter_bytes(record, 20)) return status;
+// With `normalised` the record is the extension llmopt_rms_w4a16_qkv_linear_f16_g64: the norm
+// weight follows the input in the buffer list and f32 epsilon the five words.
+int qkv_linear(llmopt_hip_context *context, const DispatchRecord &record, bool normalised) {
+  const size_t b = normalised ? 1 : 0;  // buffers after the input move up by one
+  if (int status = require_buffer_count(record, 10 + b)) return status;
+  if (int status = require_parameter_bytes(record, normalised ? 24 : 20)) return status;
   const uint32_t m = param_u32(record, 0), k = param_u32(record, 4);
   const uint32_t n[3] = {param_u32(record, 8), param_u32(record, 12), param_u32(record, 16)};
   W4QkvArgs args = {};
   static const char *const labels[3] = {"query", "key", "value"};
   for (int i = 0; i < 3; ++i) {
     if (int status = check_w4_shape(record.name.c_str(), m, n[i], k)) return status;
-    if (int status = check_w4_matrix(record.buffers[1 + 2 * i], record.buffers[2 + 2 * i], n[i], k, labels[i]))
+    if (int status =
+            check_w4_matrix(record.buffers[b + 1 + 2 * i], record.buffers[b + 2 + 2 * i], n[i], k, labels[i]))
       return status;
-    if (int status = require_buffer_size(record.buffers[7 + i], (uint64_t)m * n[i] * 2, "output")) return status;
-    args.w[i] = {record.buffers[1 + 2 * i].device, as_f16(record.buffers[2 + 2 * i])};
-    args.y[i] = reinterpret_cast<uint16_t *>(record.buffers[7 + i].device);
+    if (int status = require_buffer_size(record.buffers[b + 7 + i], (uint64_t)m * n[i] * 2, "output")) return status;
+    args.w[i] = {record.buffers[b + 1 + 2 * i].device, as_f16(record.buffers[b + 2 + 2 * i])};
+    args.y[i] = reinterpret_cast<uint16_t *>(record.buffers[b + 7 + i].device);
     args.n[i] = n[i];
   }
   if (int status = require_buffer_size(record.buffers[0], (uint64_t)m * k * 2, "input")) return status;
   args.x = as_f16(record.buffers[0]);
   args.m = m;
   args.k = k;
+  if (normalised) {
+    const W4Norm norm = {as_f16(record.buffers[1]), param_f32(record, 20), 0};  // llmopt_rms_norm_f16_simd's order
+    if (int status = normalise_input(context, record, norm, m, k, (uint64_t)n[0] + n[1] + n[2], &args.x, &args.norm))
+      return status;
+  }
   return launched(launch_w4a16_qkv(args, context->stream), record.name.c_str());
+}
+
+int w4a16_qkv_linear(llmopt_hip_context *context, const DispatchRecord &record) {
+  return qkv_linear(context, record, false);
+}
+
+// Extension (no reference kernel): llmopt_rms_norm_f16_simd followed by llmopt_w4a16_qkv_linear_f16_g64
+// without the normalised rows passing through memory where the projection kernel can normalise
+// them itself, else as those two launches.  buffers: input, norm weight, qW, qS, kW, kS, vW, vS,
+// qOut, kOut, vOut; parameters W4A16QKVParams + f32 epsilon.
+int rms_w4a16_qkv_linear(llmopt_hip_context *context, const DispatchRecord &record) {
+  return qkv_linear(context, record, true);
 }
 
 // W4A16SwiGLUFFNParams {u32 m, n, k; f32 eps}: n = intermediate width, k = hidden width
 // (lib/metal_parameters.ml:45-50).  buffers: normalized, gateW, gateS, upW, upS, product.
-int w4a16_dual_swiglu(llmopt_hip_context *context, const DispatchRecord &record) {
-  if (int status = require_buffer_count(record, 6)) return status;
+int dual_swiglu(llmopt_hip_context *context, const DispatchRecord &record, bool normalised) {
+  const size_t b = normalised ? 1 : 0;
+  if (int status = require_buffer_count(record, 6 + b)) return status;
   if (int status = require_parameter_bytes(record, 16)) return status;
   const uint32_t m = param_u32(record, 0), n = param_u32(record, 4), k = param_u32(record, 8);
   if (int status = check_w4_shape(record.name.c_str(), m, n, k)) return status;
-  if (int status = require_buffer_size(record.buffers[0], (uint64_t)m * k * 2, "normalized")) return status;
-  if (int status = check_w4_matrix(record.buffers[1], record.buffers[2], n, k, "gate")) return status;
-  if (int status = check_w4_matrix(record.buffers[3], record.buffers[4], n, k, "up")) return status;
-  if (int status = require_buffer_size(record.buffers[5], (uint64_t)m * n * 2, "product")) return status;
+  if (int status = require_buffer_size(record.buffers[0], (uint64_t)m * k * 2, normalised ? "input" : "normalized"))
+    return status;
+  if (int status = check_w4_matrix(record.buffers[b + 1], record.buffers[b + 2], n, k, "gate")) return status;
+  if (int status = check_w4_matrix(record.buffers[b + 3], record.buffers[b + 4], n, k, "up")) return status;
+  if (int status = require_buffer_size(record.buffers[b + 5], (uint64_t)m * n * 2, "product")) return status;
   W4DualSwigluArgs args = {};
   args.x = as_f16(record.buffers[0]);
-  args.gate = {record.buffers[1].device, as_f16(record.buffers[2])};
-  args.up = {record.buffers[3].device, as_f16(record.buffers[4])};
-  args.product = reinterpret_cast<uint16_t *>(record.buffers[5].device);
+  args.gate = {record.buffers[b + 1].device, as_f16(record.buffers[b + 2])};
+  args.up = {record.buffers[b + 3].device, as_f16(record.buffers[b + 4])};
+  args.product = reinterpret_cast<uint16_t *>(record.buffers[b + 5].device);
   args.m = m;
   args.n = n;
   args.k = k;
+  if (normalised) {
+    const W4Norm norm = {as_f16(record.buffers[1]), param_f32(record, 12), 1};  // llmopt_w4a16_swiglu_rms_f16_g64's order
+    if (int status = normalise_input(context, record, norm, m, k, 2ull * n, &args.x, &args.norm)) return status;
+  }
   return launched(launch_w4a16_dual_swiglu(args, context->stream), record.name.c_str());
+}
+
+int w4a16_dual_swiglu(llmopt_hip_context *context, const DispatchRecord &record) {
+  return dual_swiglu(context, record, false);
+}
+
+// Extension (no reference kernel): llmopt_w4a16_swiglu_rms_f16_g64 followed by
+// llmopt_w4a16_dual_swiglu_f16_g64, as above.  buffers: input, norm weight, gateW, gateS, upW, upS,
+// product; parameters W4A16SwiGLUFFNParams.
+int rms_w4a16_dual_swiglu(llmopt_hip_context *context, const DispatchRecord &record) {
+  return dual_swiglu(context, record, true);
 }
 
 // Same parameter block; the contraction runs over n and the output has k
@@ -177,6 +244,8 @@ void register_linear_kernels(std::vector<KernelEntryPoint> &table) {
   table.push_back({"llmopt_w4a16_qkv_linear_f16_g64", qkv, w4a16_qkv_linear});
   table.push_back({"llmopt_w4a16_qkv_linear_f16_g64_m4", qkv, w4a16_qkv_linear});
   table.push_back({"llmopt_w4a16_qkv_linear_f16_g64_m8", qkv, w4a16_qkv_linear});
+  table.push_back({"llmopt_rms_w4a16_qkv_linear_f16_g64", qkv, rms_w4a16_qkv_linear});
+  table.push_back({"llmopt_rms_w4a16_dual_swiglu_f16_g64", ffn, rms_w4a16_dual_swiglu});
   table.push_back({"llmopt_w4a16_dual_swiglu_f16_g64", ffn, w4a16_dual_swiglu});
   table.push_back({"llmopt_w4a16_dual_swiglu_f16_g64_m4", ffn, w4a16_dual_swiglu});
   table.push_back({"llmopt_w4a16_dual_swiglu_f16_g64_m8", ffn, w4a16_dual_swiglu});

@@ -129,7 +129,6 @@ class DecodeStep:
         q_bytes, kv_bytes = batch * c.q_heads * c.head_dim * 2, batch * c.kv_heads * c.head_dim * 2
         self.work = {
             "x": [create(batch * h * 2), create(batch * h * 2)],
-            "normed": create(batch * h * 2),
             "q": create(q_bytes), "k": create(kv_bytes), "v": create(kv_bytes),
             "q_rot": create(q_bytes), "k_rot": create(kv_bytes),
             "attention": create(q_bytes),
@@ -153,17 +152,15 @@ class DecodeStep:
         count = m * h
         out.append(("llmopt_embedding_f16", [self.tokens, self.device["embedding"], w["x"][0]],
                     u32s(m, c.vocabulary, h), (((count + 255) // 256) * 256, 1, 1), group))
-        rows_grid = (((m + 7) // 8) * 256, 1, 1)
         for index, layer in enumerate(self.device["layers"]):
             x_in, x_mid = w["x"][0], w["x"][1]
             key_offset = index * c.layer_elements
             value_offset = key_offset + kvd
-            out.append(("llmopt_rms_norm_f16_simd", [x_in, layer["attn_norm"], w["normed"]],
-                        struct.pack("<IIf", m, h, c.epsilon), rows_grid, group))
+            # each RMSNorm rides in the projection launch that reads it
             suffix, grid = self._linear_entry(qd + 2 * kvd)
-            out.append(("llmopt_w4a16_qkv_linear_f16_g64" + suffix,
-                        [w["normed"], *layer["q"], *layer["k"], *layer["v"], w["q"], w["k"], w["v"]],
-                        u32s(m, h, qd, kvd, kvd), grid, group))
+            out.append(("llmopt_rms_w4a16_qkv_linear_f16_g64",
+                        [x_in, layer["attn_norm"], *layer["q"], *layer["k"], *layer["v"], w["q"], w["k"], w["v"]],
+                        u32s(m, h, qd, kvd, kvd) + struct.pack("<f", c.epsilon), grid, group))
             # rotation and the new token's Q8 slot in one launch (the step is bound by its launches)
             out.append(("llmopt_rotary_qk_pack_q8_batched",
                         [w["q"], w["k"], self.cos, self.sin, w["q_rot"], w["k_rot"], w["v"], self.new_slots,
@@ -184,11 +181,10 @@ class DecodeStep:
             out.append(("llmopt_w4a16_linear_f16_g64" + suffix,
                         [w["attention"], *layer["o"], x_in, x_mid], u32s(m, h, qd, 1, h), grid, group))
             ffn_params = u32s(m, c.mlp, h) + struct.pack("<f", c.epsilon)
-            out.append(("llmopt_w4a16_swiglu_rms_f16_g64", [x_mid, layer["ffn_norm"], w["normed"]],
-                        ffn_params, (m * 256, 1, 1), group))
             suffix, grid = self._linear_entry(c.mlp)
-            out.append(("llmopt_w4a16_dual_swiglu_f16_g64" + suffix,
-                        [w["normed"], *layer["gate"], *layer["up"], w["product"]], ffn_params, grid, group))
+            out.append(("llmopt_rms_w4a16_dual_swiglu_f16_g64",
+                        [x_mid, layer["ffn_norm"], *layer["gate"], *layer["up"], w["product"]], ffn_params, grid,
+                        group))
             suffix, grid = self._linear_entry(h)
             out.append(("llmopt_w4a16_down_add_f16_g64" + suffix,
                         [w["product"], *layer["down"], x_mid, x_in], ffn_params, grid, group))

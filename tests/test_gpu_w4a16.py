@@ -154,6 +154,75 @@ def test_qkv_linear(runtime, m):
                                oracle.w4a16_linear(x, packed, scale, None), f"qkv n={n}")
 
 
+@pytest.mark.parametrize("m,k", [(1, 576), (2, 576), (1, 2048), (2, 64), (3, 576), (8, 576), (40, 576), (1, 4096),
+                                 (130, 576)])
+def test_normalising_qkv_and_swiglu_entries(runtime, m, k):
+    """The extension entries that take the raw rows and the norm weight: against the oracle's
+    RMSNorm (rounded to half, as the separate kernel stores it) followed by the projections, and
+    against the two launches they stand for - to a few half roundings where the projection kernel
+    normalises itself (one or two rows, K <= 2048: its mean square is summed in another order),
+    bit for bit where the entry runs the two kernels."""
+    import struct
+    rng = np.random.default_rng(500 + 7 * m + k)
+    sizes, n = (192, 64, 64), 256
+    epsilon = 1e-5
+    x = (rng.standard_normal((m, k)) * 3.0).astype(np.float16)
+    gain = rng.uniform(0.5, 1.5, size=k).astype(np.float16)
+    mats = [w4_case(rng, 1, width, k)[1:3] for width in sizes]
+    _, gate_w, gate_s, _ = w4_case(rng, 1, n, k)
+    _, up_w, up_s, _ = w4_case(rng, 1, n, k)
+    bx, bg = runtime.buffer_of_bytes(x), runtime.buffer_of_bytes(gain)
+    weights = []
+    for packed, scale in mats:
+        weights += [runtime.buffer_of_bytes(packed), runtime.buffer_of_bytes(scale)]
+    ffn_weights = [runtime.buffer_of_bytes(a) for a in (gate_w, gate_s, up_w, up_s)]
+    suffix = "" if m == 1 else "_m4"
+    rows_grid = (((m + 7) // 8) * 256, 1, 1)
+    blank = lambda width: runtime.buffer_of_bytes(np.full((m, width), np.nan, dtype=np.float16))
+
+    # the two launches
+    normed = blank(k)
+    runtime.dispatch("llmopt_rms_norm_f16_simd", [bx, bg, normed], struct.pack("<IIf", m, k, epsilon),
+                     grid=rows_grid, group=(256, 1, 1))
+    two = [blank(width) for width in sizes]
+    runtime.dispatch("llmopt_w4a16_qkv_linear_f16_g64" + suffix, [normed, *weights, *two], qkv_params(m, k, *sizes),
+                     grid=(linear_grid(m * sum(sizes)), 1, 1), group=(256, 1, 1))
+    ffn_params = u32s(m, n, k) + struct.pack("<f", epsilon)
+    ffn_normed = blank(k)
+    runtime.dispatch("llmopt_w4a16_swiglu_rms_f16_g64", [bx, bg, ffn_normed], ffn_params,
+                     grid=(m * 256, 1, 1), group=(256, 1, 1))
+    two_product = blank(n)
+    runtime.dispatch("llmopt_w4a16_dual_swiglu_f16_g64" + suffix, [ffn_normed, *ffn_weights, two_product], ffn_params,
+                     grid=(linear_grid(m * n), 1, 1), group=(256, 1, 1))
+
+    # one launch each
+    one = [blank(width) for width in sizes]
+    runtime.dispatch("llmopt_rms_w4a16_qkv_linear_f16_g64", [bx, bg, *weights, *one],
+                     qkv_params(m, k, *sizes) + struct.pack("<f", epsilon),
+                     grid=(linear_grid(m * sum(sizes)), 1, 1), group=(256, 1, 1))
+    one_product = blank(n)
+    runtime.dispatch("llmopt_rms_w4a16_dual_swiglu_f16_g64", [bx, bg, *ffn_weights, one_product], ffn_params,
+                     grid=(linear_grid(m * n), 1, 1), group=(256, 1, 1))
+
+    in_kernel = m <= 2 and k <= 2048
+    normalised = oracle.rms_norm(x, gain, epsilon).astype(np.float16)
+    for (packed, scale), got, reference, width in zip(mats, one, two, sizes):
+        got = got.numpy(np.float16, (m, width))
+        assert_close_to_oracle(got, oracle.w4a16_linear(normalised, packed, scale, None), f"rms+qkv n={width}")
+        if in_kernel:
+            assert_close_to_oracle(got, reference.numpy(np.float16, (m, width)).astype(np.float32), "rms+qkv vs two")
+        else:
+            np.testing.assert_array_equal(got.view(np.uint16), reference.numpy(np.uint16, (m, width)))
+    got = one_product.numpy(np.float16, (m, n))
+    expected = oracle.silu_mul(oracle.w4a16_linear(normalised, gate_w, gate_s, None),
+                               oracle.w4a16_linear(normalised, up_w, up_s, None))
+    assert_close_to_oracle(got, expected, "rms+dual swiglu")
+    if in_kernel:
+        assert_close_to_oracle(got, two_product.numpy(np.float16, (m, n)).astype(np.float32), "rms+dual vs two")
+    else:
+        np.testing.assert_array_equal(got.view(np.uint16), two_product.numpy(np.uint16, (m, n)))
+
+
 @pytest.mark.parametrize("m", [1, 2, 4, 8, 9, 32, 48, 136])
 def test_swiglu_ffn_chain(runtime, m):
     """dual-SwiGLU then down+residual, the two W4A16 stages of the reference's
