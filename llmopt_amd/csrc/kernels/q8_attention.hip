@@ -754,7 +754,13 @@ uint32_t balanced_split_slots(const Q8AttentionArgs &a) {
   // whole workgroups: one wave per KV head, at most kSplitMaxWaves of them
   const uint32_t waves = std::min<uint32_t>(a.kv_heads, kSplitMaxWaves);
   const uint32_t head_groups = (a.kv_heads + kSplitMaxWaves - 1) / kSplitMaxWaves;
-  const uint32_t per_cu = std::max<uint32_t>(1, 4 * per_simd / waves);
+  // Eight waves keep a CU as busy as twelve do (the kernel is bound by the CU's own work per byte,
+  // not by its requests), and the launch takes as long as the CU with the most workgroups: the
+  // same number on every CU, and no more than that takes - fewer, longer chunks leave fewer
+  // partial results.  Measured at 16 sequences of 512..8192 tokens, 8 KV heads of 128: 256 slots
+  // (two workgroups per CU) 37.6 us, 384 (three) 39.0, 288 or 320 (two on some CUs, three on
+  // others) 42-44, 192 (one or two) 42.3.
+  const uint32_t per_cu = std::max<uint32_t>(1, std::min(4 * per_simd / waves, (8 + waves - 1) / waves));
   const uint32_t resident = std::max<uint32_t>(1, (uint32_t)device_compute_units() * per_cu / head_groups);
   const uint32_t rounds = std::max<uint32_t>(1, (16 * a.batches + resident - 1) / resident);
   return resident * rounds;
