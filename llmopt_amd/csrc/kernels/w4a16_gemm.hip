@@ -355,7 +355,8 @@ hipError_t launch_gemm(GemmParams &p, hipStream_t stream) {
   const uint64_t big = (uint64_t)((p.m + 255) / 256) * ((p.n + 255) / 256);
   if (big >= (uint64_t)cus) return launch_tile<2, 4, false>(p, stream);
   const uint64_t mid = (uint64_t)((p.m + 127) / 128) * ((p.n + 255) / 256);
-  if (mid >= (uint64_t)cus) return launch_tile<1, 4, false>(p, stream);
+  // also when a few CUs stay without a tile: 224 tiles of 128 x 256 beat 448 of 128 x 128, two on most CUs
+  if (mid * 8 >= (uint64_t)cus * 7) return launch_tile<1, 4, false>(p, stream);
   // 128 x 128 tiles have steps shorter than a trip to memory.  With two stages they fit a CU
   // twice, which covers the loads; when there is at most one tile per CU anyway, four
   // activation stages do (K a whole number of four steps; measured 58 -> 49 us at 512 x 4096 x 4096,
