@@ -375,7 +375,10 @@ Plan make_plan(uint32_t k, uint32_t max_n, uint32_t matrices, bool dual) {
   const uint32_t waves = plan.waves_k * plan.waves_t;
   const uint32_t per_cu = waves <= 4 ? 4 : waves <= 8 ? 2 : 1;
   const uint32_t resident = std::max<uint32_t>(1, cus * per_cu / (plan.slices * matrices));
-  plan.blocks = std::min(tile_groups, resident);
+  // the same number of tiles for every workgroup: 896 tiles on 256 CUs run as 224 workgroups of
+  // four rather than 256 of three or four (10.1 against 10.6 us at 4096 x 14336)
+  const uint32_t passes = (tile_groups + resident - 1) / resident;
+  plan.blocks = (tile_groups + passes - 1) / passes;
   // tiles in flight per wave: all of a workgroup's tiles when they are few
   const uint32_t rounds = (tile_groups + plan.blocks - 1) / plan.blocks;
   plan.ring = rounds <= 1 ? 1 : (rounds <= 2 || dual) ? 2 : 4;
