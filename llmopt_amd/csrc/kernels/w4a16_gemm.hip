@@ -411,8 +411,12 @@ hipError_t launch_w4a16_linear(const W4LinearArgs &args, hipStream_t stream) {
 }
 
 bool w4a16_norm_in_kernel(uint32_t m, uint64_t columns, uint32_t k) {
-  (void)columns;
-  return w4a16_gemv_norm_ok(m, k);
+  if (m <= kGemvDotRows) return w4a16_gemv_norm_ok(m, k);
+  // the matrix-core GEMV with K inside one workgroup (same conditions as the launchers below), up to
+  // 32 rows: every workgroup normalises its eight rows again, which at 128 rows costs more than
+  // the separate launch (decode step 2.83 against 2.74 ms; 1.35 against 1.39 ms at 32 rows)
+  return m <= 32 && k % 64 == 0 && k >= 8 &&
+         ((m <= kGemvMaxRows && !w4a16_gemv_mfma_needs_split(k)) || w4a16_gemv_mfma_row_groups_ok(m, columns, k));
 }
 
 hipError_t launch_w4a16_dual_swiglu(const W4DualSwigluArgs &args, hipStream_t stream) {

@@ -79,6 +79,7 @@ struct MfmaGemvParams {
   uint32_t *counters;  // one per tile, zero between launches
   float *y_f32;        // optional float32 copy of mat0's output, may be null
   uint32_t row_groups;  // > 1: blockIdx.y is a group of 8 activation rows instead of a K slice
+  W4Norm norm;          // weight != nullptr: RMS-normalise the activation rows first (one K slice only)
 };
 
 // NB = tiles in flight per wave (= tiles between two workgroup reductions)
@@ -165,6 +166,8 @@ __global__ __launch_bounds__(kMaxWaves * 64) void w4a16_gemv_mfma_kernel(MfmaGem
   uint8_t *x_stage = reinterpret_cast<uint8_t *>(flag_lds + ((NB * p.waves_t + 3) & ~3u)) + wave * kXStageBytes;
   uint4 x_loaded[4];  // requested before the weights: loads return in order
   const uint32_t x_piece = lane & 31;
+  const bool normalise = p.norm.weight != nullptr;  // the same for every workgroup
+  uint4 gain_loaded = make_uint4(0, 0, 0, 0);
   {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -173,11 +176,54 @@ __global__ __launch_bounds__(kMaxWaves * 64) void w4a16_gemv_mfma_kernel(MfmaGem
       x_loaded[i] =
           *reinterpret_cast<const uint4 *>(p.x + (size_t)(row0 + min(row, rows - 1)) * K + min(kk, K - 8));
     }
+    if (normalise) gain_loaded = *reinterpret_cast<const uint4 *>(p.norm.weight + min(k0 + x_piece * 8, K - 8));
   }
   // all tiles of the ring go out next
   Raw ring[NB];
 #pragma unroll
   for (int b = 0; b < NB; ++b) load_tile(b, ring[b]);
+  if (normalise) {
+    // RMS normalisation of the rows: a wave holds 256 of a row's K values, so the mean squares of
+    // the workgroup's waves with the same tiles meet in LDS; then the half values the separate
+    // kernel would have stored (float32 products in its order) replace the raw ones.
+    float *norm_lds = reinterpret_cast<float *>(reinterpret_cast<uint8_t *>(flag_lds + ((NB * p.waves_t + 3) & ~3u)) +
+                                                p.waves_k * p.waves_t * kXStageBytes);
+    float square[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const bool keep = k0 + x_piece * 8 < slice_end;
+      const h8_t x = __builtin_bit_cast(h8_t, x_loaded[i]);
+      float sum = 0.0f;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) sum += (float)x[e] * (float)x[e];
+      sum = keep ? sum : 0.0f;
+#pragma unroll
+      for (int step = 1; step < 32; step *= 2)  // the 32 lanes of one row
+        sum += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((int)((lane ^ step) << 2),
+                                                                       __builtin_bit_cast(int, sum)));
+      square[i] = sum;
+    }
+    if (x_piece == 0) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) norm_lds[(wt * p.waves_k + wk) * 8 + 2 * i + (lane >> 5)] = square[i];
+    }
+    __syncthreads();
+    const h8_t gain = __builtin_bit_cast(h8_t, gain_loaded);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      float total = 0.0f;
+      for (uint32_t w = 0; w < p.waves_k; ++w) total += norm_lds[(wt * p.waves_k + w) * 8 + 2 * i + (lane >> 5)];
+      const float inverse = rsqrtf(total / (float)K + p.norm.epsilon);
+      const h8_t x = __builtin_bit_cast(h8_t, x_loaded[i]);
+      h8_t y;
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const float value = (float)x[e], g = (float)gain[e];
+        y[e] = (_Float16)(p.norm.weight_first ? value * g * inverse : value * inverse * g);
+      }
+      x_loaded[i] = __builtin_bit_cast(uint4, y);
+    }
+  }
   {
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
@@ -384,7 +430,8 @@ Plan make_plan(uint32_t k, uint32_t max_n, uint32_t matrices, bool dual) {
   plan.ring = rounds <= 1 ? 1 : (rounds <= 2 || dual) ? 2 : 4;
   const int nw = dual ? 2 : 1;
   plan.lds_bytes = (size_t)plan.ring * plan.waves_t * nw * plan.waves_k * 8 * TN * sizeof(float) +
-                   (size_t)((plan.ring * plan.waves_t + 3) & ~3u) * sizeof(uint32_t) + (size_t)waves * kXStageBytes;
+                   (size_t)((plan.ring * plan.waves_t + 3) & ~3u) * sizeof(uint32_t) + (size_t)waves * kXStageBytes +
+                   (size_t)waves * 8 * sizeof(float);  // the last: mean squares of a normalising launch
   return plan;
 }
 
@@ -465,6 +512,7 @@ hipError_t launch_w4a16_gemv_mfma_qkv(const W4QkvArgs &a, hipStream_t stream) {
   p.mat1 = {a.w[1].weight, a.w[1].scale, a.y[1], a.n[1]};
   p.mat2 = {a.w[2].weight, a.w[2].scale, a.y[2], a.n[2]};
   p.row_groups = (a.m + 7) / 8;
+  p.norm = a.norm;
   const Plan plan = make_plan(a.k, std::max(a.n[0], std::max(a.n[1], a.n[2])), 3 * p.row_groups, false);
   if (plan.slices > 1) return hipErrorInvalidValue;  // callers check w4a16_gemv_mfma_needs_split
   return launch<false>(p, 3, plan, stream);
@@ -479,6 +527,7 @@ hipError_t launch_w4a16_gemv_mfma_dual_swiglu(const W4DualSwigluArgs &a, hipStre
   p.mat1 = {a.up.weight, a.up.scale, a.product, a.n};
   p.mat2 = p.mat0;
   p.row_groups = (a.m + 7) / 8;
+  p.norm = a.norm;
   const Plan plan = make_plan(a.k, a.n, p.row_groups, true);
   if (plan.slices > 1) return hipErrorInvalidValue;
   return launch<true>(p, 1, plan, stream);

@@ -155,13 +155,13 @@ def test_qkv_linear(runtime, m):
 
 
 @pytest.mark.parametrize("m,k", [(1, 576), (2, 576), (1, 2048), (2, 64), (3, 576), (8, 576), (40, 576), (1, 4096),
-                                 (130, 576)])
+                                 (130, 576), (4, 4096), (5, 64), (8, 14336), (128, 1536), (32, 576), (17, 1536)])
 def test_normalising_qkv_and_swiglu_entries(runtime, m, k):
     """The extension entries that take the raw rows and the norm weight: against the oracle's
     RMSNorm (rounded to half, as the separate kernel stores it) followed by the projections, and
     against the two launches they stand for - to a few half roundings where the projection kernel
-    normalises itself (one or two rows, K <= 2048: its mean square is summed in another order),
-    bit for bit where the entry runs the two kernels."""
+    normalises itself (its mean square is summed in another order), bit for bit where the entry
+    runs the two kernels."""
     import struct
     rng = np.random.default_rng(500 + 7 * m + k)
     sizes, n = (192, 64, 64), 256
@@ -204,7 +204,8 @@ def test_normalising_qkv_and_swiglu_entries(runtime, m, k):
     runtime.dispatch("llmopt_rms_w4a16_dual_swiglu_f16_g64", [bx, bg, *ffn_weights, one_product], ffn_params,
                      grid=(linear_grid(m * n), 1, 1), group=(256, 1, 1))
 
-    in_kernel = m <= 2 and k <= 2048
+    # one or two rows: K of one chunk; 3..32 rows: the matrix-core GEMV when one workgroup covers K
+    in_kernel = (m <= 2 and k <= 2048) or (3 <= m <= 32 and k <= 4096)
     normalised = oracle.rms_norm(x, gain, epsilon).astype(np.float16)
     for (packed, scale), got, reference, width in zip(mats, one, two, sizes):
         got = got.numpy(np.float16, (m, width))
