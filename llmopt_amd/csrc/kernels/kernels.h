@@ -80,10 +80,16 @@ hipError_t launch_w4a16_linear(const W4LinearArgs &args, hipStream_t stream);
 hipError_t launch_w4a16_qkv(const W4QkvArgs &args, hipStream_t stream);
 hipError_t launch_w4a16_dual_swiglu(const W4DualSwigluArgs &args, hipStream_t stream);
 
-// Bit-exact dequantisation q * s to float32 [n, k] (debug / parity check of the
-// unpack arithmetic; python/llmopt_backend/quantization.py:91-121).
-hipError_t launch_w4_dequant_f32(const W4Matrix &w, float *out, uint32_t n, uint32_t k,
+// The product kernels' own nibble decoders run over a whole matrix, as float32 [n, k]:
+// decoder 0 = w4_decode_pairs and 1 = w4_decode_biased (minus its bias), each times the float32
+// scale, i.e. the exact q * s of python/llmopt_backend/quantization.py:91-121; decoder 2 = the
+// prefill GEMM's staged operand half(q * s) (one fp16 rounding).
+hipError_t launch_w4_dequant_f32(const W4Matrix &w, float *out, uint32_t n, uint32_t k, uint32_t decoder,
                                  hipStream_t stream);
+// The attention kernels' int8 decoders over `count` bytes (a multiple of 4), as float32:
+// decoder 0 = int8x4_to_h2, 1 = int8x4_to_h2_biased minus its bias.
+hipError_t launch_q8_decode_f32(const uint8_t *bytes, float *out, uint32_t count, uint32_t decoder,
+                                hipStream_t stream);
 
 // ---- grouped-Q8 KV cache -----------------------------------------------------
 

@@ -41,20 +41,6 @@ __device__ __forceinline__ float q8_scale_at(const uint8_t *token, uint32_t toke
   return half_bits_to_float(reinterpret_cast<const uint16_t *>(token + token_elements)[index]);
 }
 
-// 4 int8 (already XOR 0x80 -> q + 128) to two h2 of exact integers (b0,b1),(b2,b3).
-__device__ __forceinline__ void int8x4_to_h2(uint32_t biased, h2_t &lo, h2_t &hi) {
-  const h2_t offset = {(_Float16)1152.0f, (_Float16)1152.0f};  // 1024 + 128
-  lo = as_h2(__builtin_amdgcn_perm(0x64646464u, biased, 0x04010400u)) - offset;
-  hi = as_h2(__builtin_amdgcn_perm(0x64646464u, biased, 0x04030402u)) - offset;
-}
-
-// Same without the subtraction: exact integers q + 1152.  Used for K, where the
-// bias becomes a per-head constant 1152 * sum_d(Q[d]) subtracted from the score.
-__device__ __forceinline__ void int8x4_to_h2_biased(uint32_t biased, h2_t &lo, h2_t &hi) {
-  lo = as_h2(__builtin_amdgcn_perm(0x64646464u, biased, 0x04010400u));
-  hi = as_h2(__builtin_amdgcn_perm(0x64646464u, biased, 0x04030402u));
-}
-
 __device__ __forceinline__ float shfl_xor_f32(float value, int mask) {
   const int lane = __lane_id();
   return __builtin_bit_cast(

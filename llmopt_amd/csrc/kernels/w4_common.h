@@ -73,6 +73,35 @@ __device__ __forceinline__ W4Pairs w4_decode_biased(uint32_t word) {
   return out;
 }
 
+// The prefill GEMM's B operand of one weight dword: q * s rounded to fp16 (one rounding per
+// weight, at most 2^-11 relative), the 8 values in natural K order.
+__device__ __forceinline__ uint4 w4_scaled_natural(uint32_t word, _Float16 scale) {
+  const h2_t scale2 = {scale, scale};
+  const W4Pairs q = w4_decode_pairs(word);
+  const uint32_t p04 = as_u32(q.p04 * scale2), p15 = as_u32(q.p15 * scale2);
+  const uint32_t p26 = as_u32(q.p26 * scale2), p37 = as_u32(q.p37 * scale2);
+  uint4 packed;
+  packed.x = __builtin_amdgcn_perm(p15, p04, 0x05040100u);  // k0 k1
+  packed.y = __builtin_amdgcn_perm(p37, p26, 0x05040100u);  // k2 k3
+  packed.z = __builtin_amdgcn_perm(p15, p04, 0x07060302u);  // k4 k5
+  packed.w = __builtin_amdgcn_perm(p37, p26, 0x07060302u);  // k6 k7
+  return packed;
+}
+
+// 4 int8 (already XOR 0x80 -> q + 128) to two h2 of exact integers (b0,b1),(b2,b3).
+__device__ __forceinline__ void int8x4_to_h2(uint32_t biased, h2_t &lo, h2_t &hi) {
+  const h2_t offset = {(_Float16)1152.0f, (_Float16)1152.0f};  // 1024 + 128
+  lo = as_h2(__builtin_amdgcn_perm(0x64646464u, biased, 0x04010400u)) - offset;
+  hi = as_h2(__builtin_amdgcn_perm(0x64646464u, biased, 0x04030402u)) - offset;
+}
+
+// Same without the subtraction: exact integers q + 1152.  Used for K, where the
+// bias becomes a per-head constant 1152 * sum_d(Q[d]) subtracted from the score.
+__device__ __forceinline__ void int8x4_to_h2_biased(uint32_t biased, h2_t &lo, h2_t &hi) {
+  lo = as_h2(__builtin_amdgcn_perm(0x64646464u, biased, 0x04010400u));
+  hi = as_h2(__builtin_amdgcn_perm(0x64646464u, biased, 0x04030402u));
+}
+
 // Rearranges 8 consecutive fp16 activations (x0..x7) into the pair order of
 // w4_decode_pairs: {(x0,x4), (x1,x5), (x2,x6), (x3,x7)}.
 __device__ __forceinline__ uint4 pair_order(uint4 x) {

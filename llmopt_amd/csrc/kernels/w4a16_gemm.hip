@@ -177,15 +177,7 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
     const int j = item % 4;
     if (BN % 256 != 0 && w_row >= (uint32_t)BN) return;
     const _Float16 scale = __builtin_bit_cast(_Float16, (uint16_t)f.s[v]);
-    const h2_t scale2 = {scale, scale};
-    const W4Pairs q = w4_decode_pairs(f.w[v][j]);
-    const uint32_t p04 = as_u32(q.p04 * scale2), p15 = as_u32(q.p15 * scale2);
-    const uint32_t p26 = as_u32(q.p26 * scale2), p37 = as_u32(q.p37 * scale2);
-    uint4 packed;
-    packed.x = __builtin_amdgcn_perm(p15, p04, 0x05040100u);  // k0 k1
-    packed.y = __builtin_amdgcn_perm(p37, p26, 0x05040100u);  // k2 k3
-    packed.z = __builtin_amdgcn_perm(p15, p04, 0x07060302u);  // k4 k5
-    packed.w = __builtin_amdgcn_perm(p37, p26, 0x07060302u);  // k6 k7
+    const uint4 packed = w4_scaled_natural(f.w[v][j], scale);
     *reinterpret_cast<uint4 *>(&w_lds[(v * BN + w_row) * LDS_STRIDE + w_half * 32 + j * 8]) = packed;
   };
 

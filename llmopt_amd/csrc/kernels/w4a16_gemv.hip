@@ -627,22 +627,6 @@ hipError_t launch_by_rows(const GemvParams &p, uint32_t matrices, uint32_t max_n
   return launch_variant<8, 2, 1, DUAL>(p, matrices, max_n, stream);
 }
 
-__global__ void w4_dequant_f32_kernel(const uint8_t *weight, const uint16_t *scale, float *out,
-                                      uint32_t n, uint32_t k) {
-  // one thread per packed byte
-  const size_t index = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-  const size_t bytes_per_row = k >> 1;
-  if (index >= (size_t)n * bytes_per_row) return;
-  const size_t row = index / bytes_per_row;
-  const size_t byte_in_row = index - row * bytes_per_row;
-  const uint32_t byte = weight[index];
-  const int low = (int)(byte & 15u) - ((byte & 8u) ? 16 : 0);
-  const int high = (int)(byte >> 4) - ((byte & 128u) ? 16 : 0);
-  const float s = half_bits_to_float(scale[row * (k >> 6) + (byte_in_row >> 5)]);
-  out[row * k + 2 * byte_in_row] = (float)low * s;
-  out[row * k + 2 * byte_in_row + 1] = (float)high * s;
-}
-
 }  // namespace
 
 hipError_t launch_w4a16_gemv_linear(const W4LinearArgs &a, hipStream_t stream) {
@@ -681,15 +665,6 @@ hipError_t launch_w4a16_gemv_dual_swiglu(const W4DualSwigluArgs &a, hipStream_t 
   p.norm = a.norm;
   if (p.norm.weight != nullptr && !w4a16_gemv_norm_ok(a.m, a.k)) return hipErrorInvalidValue;
   return launch_by_rows<true>(p, 1, a.n, stream);
-}
-
-hipError_t launch_w4_dequant_f32(const W4Matrix &w, float *out, uint32_t n, uint32_t k,
-                                 hipStream_t stream) {
-  const size_t total = (size_t)n * (k >> 1);
-  const uint32_t blocks = (uint32_t)((total + 255) / 256);
-  hipLaunchKernelGGL(w4_dequant_f32_kernel, dim3(blocks), dim3(256), 0, stream, w.weight, w.scale,
-                     out, n, k);
-  return hipGetLastError();
 }
 
 }  // namespace llmopt

@@ -217,18 +217,41 @@ int w4a16_down_add(llmopt_hip_context *context, const DispatchRecord &record) {
   return launched(launch_w4a16_linear(args, context->stream), record.name.c_str());
 }
 
-// Extension (no reference kernel): float32 [n,k] = q * scale, for checking the
-// unpack arithmetic bit for bit.  Parameters {u32 n, k}; buffers: packed, scale, output.
+// Extension (no reference kernel): float32 [n,k] from the product kernels' own nibble decoders,
+// for checking the unpack arithmetic bit for bit.  Parameters {u32 n, k} or {u32 n, k, decoder}:
+// decoder 0 (default) = w4_decode_pairs x scale, 1 = w4_decode_biased minus its bias x scale, 2 = the
+// prefill GEMM's staged half(q * scale).  buffers: packed, scale, output.
 int w4_dequant_f32(llmopt_hip_context *context, const DispatchRecord &record) {
   if (int status = require_buffer_count(record, 3)) return status;
-  if (int status = require_parameter_bytes(record, 8)) return status;
+  if (record.parameters.size() != 8 && record.parameters.size() != 12)
+    return fail(LLMOPT_ERR_INVALID, "%s expects an 8- or 12-byte parameter block, got %zu", record.name.c_str(),
+                record.parameters.size());
   const uint32_t n = param_u32(record, 0), k = param_u32(record, 4);
+  const uint32_t decoder = record.parameters.size() == 12 ? param_u32(record, 8) : 0;
+  if (decoder > 2) return fail(LLMOPT_ERR_INVALID, "%s knows decoders 0, 1 and 2, got %u", record.name.c_str(), decoder);
   if (int status = check_w4_shape(record.name.c_str(), 1, n, k)) return status;
   if (int status = check_w4_matrix(record.buffers[0], record.buffers[1], n, k, "W4A16")) return status;
   if (int status = require_buffer_size(record.buffers[2], (uint64_t)n * k * 4, "output")) return status;
   W4Matrix w = {record.buffers[0].device, as_f16(record.buffers[1])};
-  return launched(launch_w4_dequant_f32(w, reinterpret_cast<float *>(record.buffers[2].device), n, k,
+  return launched(launch_w4_dequant_f32(w, reinterpret_cast<float *>(record.buffers[2].device), n, k, decoder,
                                         context->stream),
+                  record.name.c_str());
+}
+
+// Extension (no reference kernel): float32 [count] from the attention kernels' own int8
+// decoders.  Parameters {u32 count, decoder}: count a multiple of 4; decoder 0 = int8x4_to_h2,
+// 1 = int8x4_to_h2_biased minus its bias.  buffers: int8 bytes, output.
+int q8_decode_f32(llmopt_hip_context *context, const DispatchRecord &record) {
+  if (int status = require_buffer_count(record, 2)) return status;
+  if (int status = require_parameter_bytes(record, 8)) return status;
+  const uint32_t count = param_u32(record, 0), decoder = param_u32(record, 4);
+  if (count == 0 || count % 4 != 0)
+    return fail(LLMOPT_ERR_INVALID, "%s requires a positive multiple of 4 bytes, got %u", record.name.c_str(), count);
+  if (decoder > 1) return fail(LLMOPT_ERR_INVALID, "%s knows decoders 0 and 1, got %u", record.name.c_str(), decoder);
+  if (int status = require_buffer_size(record.buffers[0], count, "int8")) return status;
+  if (int status = require_buffer_size(record.buffers[1], (uint64_t)count * 4, "output")) return status;
+  return launched(launch_q8_decode_f32(record.buffers[0].device, reinterpret_cast<float *>(record.buffers[1].device),
+                                       count, decoder, context->stream),
                   record.name.c_str());
 }
 
@@ -253,6 +276,7 @@ void register_linear_kernels(std::vector<KernelEntryPoint> &table) {
   table.push_back({"llmopt_w4a16_down_add_f16_g64_m4", ffn, w4a16_down_add});
   table.push_back({"llmopt_w4a16_down_add_f16_g64_m8", ffn, w4a16_down_add});
   table.push_back({"llmopt_w4_dequant_f32", linear, w4_dequant_f32});
+  table.push_back({"llmopt_q8_decode_f32", "cache", q8_decode_f32});
 }
 
 }  // namespace llmopt

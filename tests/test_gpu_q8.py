@@ -370,3 +370,25 @@ def test_decode_attention_full_size_closed_form(runtime, batches):
             want[b, 0, h] = (w_past * value_sum[kvh] + w_cur * cv[b, kvh, 0].astype(np.float64)) / \
                 (int(lengths[b]) * w_past + w_cur)
     assert_close_to_oracle(out, want, f"full-size closed form, batch {batches}")
+
+
+@pytest.mark.parametrize("decoder,name", [(0, "int8x4_to_h2"), (1, "int8x4_to_h2_biased")])
+def test_attention_int8_decoders_are_bit_exact(runtime, decoder, name):
+    """The two int8 -> fp16 decoders of the attention kernels over every byte value in every byte
+    lane: the integers oracle_q8_unpack produces for the same bytes (scale 1.0)."""
+    values = np.arange(256, dtype=np.uint8)
+    data = np.stack([np.roll(values, shift) for shift in (0, 1, 2, 3)], axis=1).reshape(-1)  # 1024 bytes
+    out = runtime.create_buffer(data.size * 4)
+    runtime.dispatch("llmopt_q8_decode_f32", [runtime.buffer_of_bytes(data), out], u32s(data.size, decoder))
+    got = out.numpy(np.float32, (data.size,))
+    np.testing.assert_array_equal(got, data.view(np.int8).astype(np.float32), err_msg=name)
+    # the oracle's unpack of the same bytes as 16 tokens of one 64-wide head with scale 1.0
+    tokens, dim = data.size // 64, 64
+    pool = np.zeros((tokens, dim + 2), dtype=np.uint8)
+    pool[:, :dim] = data.reshape(tokens, dim)
+    pool[:, dim:] = np.array([1.0], dtype=np.float16).view(np.uint8)
+    params = oracle.CacheParams(items=tokens, segment_offset=0, heads=1, head_dim=dim, group_size=64,
+                                token_elements=dim, token_groups=1, token_stride=dim + 2,
+                                source_items=tokens, source_offset=0)
+    unpacked = oracle.q8_unpack(pool.reshape(-1), np.arange(tokens, dtype=np.uint32), params)
+    np.testing.assert_array_equal(got, unpacked.astype(np.float32).reshape(-1), err_msg=name)

@@ -35,16 +35,78 @@ def run_linear(runtime, x, packed, scale, bias=None, residual=None, name=None):
     return out.numpy(np.float16, (m, n))
 
 
-def test_dequant_is_bit_exact(runtime):
-    rng = np.random.default_rng(0)
-    packed = np.arange(256, dtype=np.uint8).repeat(32).reshape(64, 128)  # every byte value
-    rng.shuffle(packed, axis=1)
+def every_byte_matrix(rng):
+    """64 rows x 256 K values in which every byte value (both nibbles) occurs in every byte lane of
+    a weight dword."""
+    packed = np.empty((64, 128), dtype=np.uint8)
+    for row in range(64):
+        values = np.arange(256, dtype=np.uint8)
+        rng.shuffle(values)
+        # rotate so that byte lane (column % 4) sees another quarter of the values on each row
+        packed[row] = np.roll(values, row)[:128] if row % 2 == 0 else np.roll(values, row)[128:]
+    return packed
+
+
+@pytest.mark.parametrize("decoder,name", [(0, "w4_decode_pairs"), (1, "w4_decode_biased")])
+def test_product_nibble_decoders_are_bit_exact(runtime, decoder, name):
+    """The two decoders every W4A16 kernel uses, over all 256 byte values in all four byte lanes
+    of a dword and a spread of fp16 scales: float32 q * s identical to the oracle's, bit for bit."""
+    rng = np.random.default_rng(decoder)
+    packed = every_byte_matrix(rng)
+    for lane in range(4):
+        assert len(set(packed[:, lane::4].reshape(-1).tolist())) == 256
     scale = rng.uniform(0.005, 0.02, size=(64, 4)).astype(np.float16)
+    scale[0] = [1.0, 2.0 ** -14, 65504.0, 6e-8]  # unit, smallest normal, largest, subnormal
     bw, bs = runtime.buffer_of_bytes(packed), runtime.buffer_of_bytes(scale)
     out = runtime.create_buffer(64 * 256 * 4)
-    runtime.dispatch("llmopt_w4_dequant_f32", [bw, bs, out], u32s(64, 256))
+    runtime.dispatch("llmopt_w4_dequant_f32", [bw, bs, out], u32s(64, 256, decoder))
     got = out.numpy(np.float32, (64, 256))
-    np.testing.assert_array_equal(got.view(np.uint32), oracle.w4_dequant(packed, scale).view(np.uint32))
+    np.testing.assert_array_equal(got.view(np.uint32), oracle.w4_dequant(packed, scale).view(np.uint32), err_msg=name)
+    # and the integers themselves, against arithmetic written here: low nibble = even K, two's complement
+    ones = np.ones((64, 4), dtype=np.float16)
+    runtime.dispatch("llmopt_w4_dequant_f32", [bw, runtime.buffer_of_bytes(ones), out], u32s(64, 256, decoder))
+    integers = out.numpy(np.float32, (64, 256))
+    low = (packed & 15).astype(np.int32)
+    high = (packed >> 4).astype(np.int32)
+    expected = np.stack([low - 16 * (low >= 8), high - 16 * (high >= 8)], axis=-1).reshape(64, 256)
+    np.testing.assert_array_equal(integers, expected.astype(np.float32), err_msg=name)
+
+
+def test_default_dequant_entry_is_bit_exact(runtime):
+    rng = np.random.default_rng(0)
+    packed = every_byte_matrix(rng)
+    scale = rng.uniform(0.005, 0.02, size=(64, 4)).astype(np.float16)
+    out = runtime.create_buffer(64 * 256 * 4)
+    runtime.dispatch("llmopt_w4_dequant_f32", [runtime.buffer_of_bytes(packed), runtime.buffer_of_bytes(scale), out],
+                     u32s(64, 256))
+    np.testing.assert_array_equal(out.numpy(np.float32, (64, 256)).view(np.uint32),
+                                  oracle.w4_dequant(packed, scale).view(np.uint32))
+
+
+def test_gemm_staged_weight_is_one_half_rounding_from_exact(runtime):
+    """The prefill GEMM keeps half(q * s) in LDS: one rounding per weight.  Over every nibble value
+    and every finite positive fp16 scale the staged value is the correctly rounded product, i.e.
+    within 2^-11 relative of q * s wherever the product is a normal half, and exact for the
+    configurations' scales times powers of two."""
+    scales = np.arange(1, 0x7C00, dtype=np.uint16).view(np.float16)  # every positive finite half
+    rows = (scales.size + 3) // 4
+    scale = np.ones(rows * 4, dtype=np.float16)
+    scale[:scales.size] = scales
+    scale = scale.reshape(rows, 4)
+    # each 64-wide group holds the 16 nibble values four times over
+    packed = np.tile(np.array([0x10, 0x32, 0x54, 0x76, 0x98, 0xBA, 0xDC, 0xFE], dtype=np.uint8), (rows, 16))
+    out = runtime.create_buffer(rows * 256 * 4)
+    runtime.dispatch("llmopt_w4_dequant_f32", [runtime.buffer_of_bytes(packed), runtime.buffer_of_bytes(scale), out],
+                     u32s(rows, 256, 2))
+    staged = out.numpy(np.float32, (rows, 256)).astype(np.float64)
+    exact = oracle.w4_dequant(packed, scale).astype(np.float64)
+    with np.errstate(over="ignore"):
+        rounded = exact.astype(np.float16).astype(np.float64)  # IEEE round-to-nearest-even, inf on overflow
+    np.testing.assert_array_equal(staged, rounded)
+    normal = (np.abs(exact) >= 2.0 ** -14) & np.isfinite(rounded)
+    relative = np.abs(staged[normal] - exact[normal]) / np.abs(exact[normal])
+    assert relative.max() <= 2.0 ** -11
+    assert np.all(np.isfinite(staged[np.abs(exact) <= 65504.0]))
 
 
 def test_reference_fixture_golden_bits(runtime, golden):
@@ -258,3 +320,90 @@ def test_swiglu_ffn_chain(runtime, m):
     expected = oracle.add(oracle.w4a16_linear(got_product, down_w, down_s, None),
                           residual.astype(np.float32))
     assert_close_to_oracle(output.numpy(np.float16, (m, k)), expected, "down+residual")
+
+
+# ---- the benchmark's own cells, at full size ------------------------------------------------
+# Every kernel instantiation the measured configurations select: the single-row ring kernel at
+# K >= 8192, the two-row variant whose activation fills 57 KB of LDS, the persistent 768-workgroup
+# grids at N = 14336 and the K = 14336 split over workgroups.  The oracle runs the whole matrix.
+SWEEP_CELLS = [(m, n, k) for m in (1, 2, 4, 8) for k, n in ((4096, 4096), (4096, 14336), (14336, 4096))]
+
+
+@pytest.mark.parametrize("m,n,k", SWEEP_CELLS)
+def test_gemv_sweep_cell_at_full_size(runtime, m, n, k):
+    rng = np.random.default_rng(31 * m + n + 7 * k)
+    x, packed, scale, bias = w4_case(rng, m, n, k, bias=True)
+    print(f"gemv sweep cell m={m} n={n} k={k}", flush=True)
+    expected = oracle.w4a16_linear(x, packed, scale, None)
+    assert_close_to_oracle(run_linear(runtime, x, packed, scale), expected, f"gemv cell {m}x{n}x{k}")
+    if m in (1, 8):  # the addend path of the same grids
+        expected_bias = oracle.add(expected, bias.astype(np.float32).reshape(1, -1))
+        assert_close_to_oracle(run_linear(runtime, x, packed, scale, bias=bias), expected_bias,
+                               f"gemv cell+bias {m}x{n}x{k}")
+
+
+def tile_covering_sample(rng, extent, block):
+    """One random index out of every `block` consecutive ones: every tile of a tiled kernel is hit."""
+    starts = np.arange(0, extent, block)
+    return np.minimum(starts + rng.integers(0, block, size=starts.size), extent - 1)
+
+
+PREFILL_CELLS = [(512, 4096, 4096), (512, 14336, 4096), (2048, 4096, 4096), (2048, 14336, 4096)]
+
+
+@pytest.mark.parametrize("m,n,k", PREFILL_CELLS)
+def test_gemm_prefill_cell_at_full_size(runtime, m, n, k):
+    """The measured prefill shapes (128x128, 128x256 and 256x256 workgroup tiles).  Three checks:
+    the oracle on a sample with one row out of every 32 and one column out of every 64 (every
+    workgroup tile and every wave tile is hit); the sum over rows of every output column against
+    the oracle applied to the summed activation (touches every output element); and linearity."""
+    rng = np.random.default_rng(3 * m + n + k)
+    x, packed, scale, _ = w4_case(rng, m, n, k)
+    print(f"gemm prefill cell m={m} n={n} k={k}", flush=True)
+    out = run_linear(runtime, x, packed, scale)
+    rows = tile_covering_sample(rng, m, 32)
+    columns = tile_covering_sample(rng, n, 64)
+    expected = oracle.w4a16_linear(x[rows], packed[columns], scale[columns], None)
+    assert_close_to_oracle(out[np.ix_(rows, columns)], expected, f"gemm cell sampled {m}x{n}x{k}")
+    # column sums: sum_r y[r, c] = (sum_r x[r]) . w[c]; fp16 rounding of the m outputs averages out
+    summed = x.astype(np.float64).sum(axis=0, keepdims=True).astype(np.float32)
+    expected_sums = oracle.w4a16_linear(summed, packed, scale, None).astype(np.float64).reshape(-1)
+    got_sums = out.astype(np.float64).sum(axis=0)
+    error = np.linalg.norm(got_sums - expected_sums) / np.linalg.norm(expected_sums)
+    assert error <= 1e-3, f"column sums differ from the oracle: rel-L2 {error:.3e}"
+    doubled = run_linear(runtime, (x.astype(np.float32) * 2).astype(np.float16), packed, scale)
+    base, twice = out.astype(np.float32), doubled.astype(np.float32)
+    normal = np.abs(base) >= 2.0 ** -13
+    np.testing.assert_array_equal(twice[normal], 2 * base[normal])
+
+
+@pytest.mark.parametrize("m", [512, 2048])
+def test_dual_swiglu_prefill_cell_at_full_size(runtime, m):
+    """silu(gate) * up at K = 4096, N = 14336: tile-covering sample against the oracle, and every
+    output element against the two plain projections of the same launch shape combined on the
+    host (their own parity is the test above)."""
+    import struct
+    n, k = 14336, 4096
+    rng = np.random.default_rng(40 + m)
+    x = rng.standard_normal((m, k)).astype(np.float16)
+    _, gate_w, gate_s, _ = w4_case(rng, 1, n, k)
+    _, up_w, up_s, _ = w4_case(rng, 1, n, k)
+    print(f"dual swiglu prefill cell m={m} n={n} k={k}", flush=True)
+    product = runtime.buffer_of_bytes(np.full((m, n), np.nan, dtype=np.float16))
+    runtime.dispatch("llmopt_w4a16_dual_swiglu_f16_g64_m4",
+                     [runtime.buffer_of_bytes(x), runtime.buffer_of_bytes(gate_w), runtime.buffer_of_bytes(gate_s),
+                      runtime.buffer_of_bytes(up_w), runtime.buffer_of_bytes(up_s), product],
+                     u32s(m, n, k) + struct.pack("<f", 1e-5),
+                     grid=(linear_grid(((m + 3) // 4) * n), 1, 1), group=(256, 1, 1))
+    got = product.numpy(np.float16, (m, n))
+    rows = tile_covering_sample(rng, m, 32)
+    columns = tile_covering_sample(rng, n, 64)
+    gate = oracle.w4a16_linear(x[rows], gate_w[columns], gate_s[columns], None)
+    up = oracle.w4a16_linear(x[rows], up_w[columns], up_s[columns], None)
+    assert_close_to_oracle(got[np.ix_(rows, columns)], oracle.silu_mul(gate, up), f"dual swiglu cell m={m}")
+    # everywhere: against silu(gate) * up of the plain projections (fp16 outputs, so a few roundings apart)
+    gate_all = run_linear(runtime, x, gate_w, gate_s).astype(np.float64)
+    up_all = run_linear(runtime, x, up_w, up_s).astype(np.float64)
+    combined = gate_all / (1.0 + np.exp(-gate_all)) * up_all
+    assert_close_to_oracle(got, combined.astype(np.float32), f"dual swiglu cell vs projections m={m}",
+                           rel_l2_tol=2e-3)
