@@ -213,6 +213,33 @@ void llmopt_hip_release_prebaked(llmopt_hip_prebaked *plan);
 int llmopt_hip_prebaked_execute(llmopt_hip_prebaked *plan, int64_t token, int64_t past_tokens,
                                 int64_t checkpoint, int64_t *out_token);
 
+/* ---- the entry point that allocates nothing ---------------------------------- */
+
+/* No counterpart in the reference.  For callers that cannot allocate device
+ * memory: code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc.  It is llmopt_attention_q8_paged_simd_* (one slot table for
+ * all sequences, no mask) with plain device pointers: `parameters` is the
+ * 64-byte Q8PagedAttentionParams block (lib/metal_cache_source.ml:352-369) in
+ * host memory, the other pointers are device memory (query f16 [b, h, q, D],
+ * current key / value f16 [b, kvh, q, D], the Q8 pool and its byte length,
+ * `slot_count` u32 slot indices, output f16 [b, q, h, D]).  The work is queued
+ * on `hip_stream` (a hipStream_t; NULL is the default stream) of the current
+ * device and not waited for.
+ * The partial results of the split-context kernels live in a fixed array of
+ * LLMOPT_NO_ALLOC_SCRATCH_BYTES in the library's code object, one copy per
+ * GPU, held until the process ends.  A call that needs more fails with
+ * LLMOPT_ERR_INVALID and launches nothing.  No hipMalloc, hipFree or other
+ * allocating routine is called.  All calls on one GPU share the array: calls
+ * ordered on one stream are safe, calls that overlap on one GPU race.
+ * llmopt_hip_create_context resolves the array's address for its device; on a
+ * device with no context the first call does (do it before a capture). */
+#define LLMOPT_NO_ALLOC_SCRATCH_BYTES (8u << 20)
+int llmopt_hip_attention_q8_paged_no_alloc(void *hip_stream, const void *parameters,
+                                           const void *query, const void *current_key,
+                                           const void *current_value, const void *pool,
+                                           size_t pool_bytes, const uint32_t *slots,
+                                           size_t slot_count, void *output);
+
 #ifdef __cplusplus
 }
 #endif

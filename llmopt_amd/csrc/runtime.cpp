@@ -265,6 +265,10 @@ int llmopt_hip_create_context(int device, llmopt_hip_context **out) {
   LLMOPT_HIP_TRY(hipStreamCreateWithFlags(&context->stream, hipStreamNonBlocking),
                  "HIP could not create a stream");
   context->owns_stream = true;
+  if (int status = no_alloc_prepare_current_device()) {
+    (void)hipStreamDestroy(context->stream);
+    return status;
+  }
   *out = context.release();
   return LLMOPT_OK;
 }

@@ -115,6 +115,10 @@ struct RotaryQkArgs;
 // the record), checked as llmopt_rotary_qk_f16_simd_h64 checks them.
 int parse_rotary_qk(const DispatchRecord &record, RotaryQkArgs *out);
 
+// Resolves, for the current device, the address of the static scratch array behind
+// llmopt_hip_attention_q8_paged_no_alloc (once per device).
+int no_alloc_prepare_current_device();
+
 void retain(RefCounted *object);
 // Returns true when the caller dropped the last reference.
 bool release(RefCounted *object);

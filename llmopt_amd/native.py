@@ -102,6 +102,7 @@ def lib() -> ctypes.CDLL:
         "llmopt_hip_prebaked_create": (ctypes.c_int, [vp, item_p, sz, vp, vp, pp]),
         "llmopt_hip_release_prebaked": (None, [vp]),
         "llmopt_hip_prebaked_execute": (ctypes.c_int, [vp, i64, i64, i64, ctypes.POINTER(i64)]),
+        "llmopt_hip_attention_q8_paged_no_alloc": (ctypes.c_int, [vp, vp, vp, vp, vp, vp, sz, vp, sz, vp]),
     }
     for name, (restype, argtypes) in signatures.items():
         function = getattr(handle, name)
@@ -128,6 +129,7 @@ EXPORTED_SYMBOLS = (
     "llmopt_hip_commit_batch", "llmopt_hip_commit_batch_async",
     "llmopt_hip_commit_batch_profiled", "llmopt_hip_abort_batch",
     "llmopt_hip_prebaked_create", "llmopt_hip_release_prebaked", "llmopt_hip_prebaked_execute",
+    "llmopt_hip_attention_q8_paged_no_alloc",
 )
 
 
@@ -222,6 +224,22 @@ def _make_item(name: str, buffers: Sequence[Buffer], parameters: bytes,
     item.group = (ctypes.c_int64 * 3)(*group)
     item.barrier_before = int(barrier_before)
     return item, (handles, raw, encoded)
+
+
+NO_ALLOC_SCRATCH_BYTES = 8 << 20  # LLMOPT_NO_ALLOC_SCRATCH_BYTES
+
+
+def attention_q8_paged_no_alloc(parameters: bytes, query: Buffer, current_key: Buffer, current_value: Buffer,
+                                pool: Buffer, slots: Buffer, output: Buffer, stream: int = 0) -> None:
+    """llmopt_hip_attention_q8_paged_no_alloc: paged Q8 decode attention that allocates nothing
+    (partial results in a fixed array of the library).  Queued on `stream`, not waited for."""
+    raw = ctypes.create_string_buffer(bytes(parameters), len(parameters))
+    if len(parameters) != 64:
+        raise LlmoptError("Q8PagedAttentionParams is a 64-byte block", -2)
+    _check(lib().llmopt_hip_attention_q8_paged_no_alloc(
+        ctypes.c_void_p(stream), raw, query.device_pointer, current_key.device_pointer,
+        current_value.device_pointer, pool.device_pointer, pool.byte_length, slots.device_pointer,
+        slots.byte_length // 4, output.device_pointer))
 
 
 class Runtime:
