@@ -8,15 +8,22 @@ Headline (`value`): W4A16 decode GEMV sweep, M in {1,2,4,8} x (K,N) in
 the 12 cases divided by the time of that pass (inputs resident in HBM): the K
 steps are captured into one HIP graph and its replay is timed with HIP events
 on the launch stream (the host-launched time of the same K steps is reported
-under `extras`).  A "step" is one such pass.  Each (K,N) keeps 16 distinct weight copies that
-steps cycle through, so a weight matrix is never re-read from the 256 MB
-Infinity Cache: every step streams its weights from HBM.
+under `extras`).  A "step" is one such pass.  Every launch of a step reads
+another copy of its weight matrix, and each (K,N) keeps enough copies (more
+than 512 MB of them) that a copy has left the 256 MB Infinity Cache long
+before its turn comes again: every launch streams its weights from HBM.
 
-Also reported in the same line: `roofline` of the dominant kernel (the M=1
-GEMV at K=4096, N=14336) from HIP events around graph-replayed launches,
-`cpu_baseline` (the C oracle on one host core over the same sweep) and, under
-`extras`, the prefill GEMM (MFMA roofline) and Q8 decode attention (HBM
-roofline, tokens/s) measurements.
+Also reported in the same line: `roofline` of the kernel with the largest
+share of the sweep's time (HIP events around graph-replayed launches of each
+of its cases), `cpu_baseline` (the C oracle on one host core over the same
+sweep) and, under `extras`, the prefill GEMM (MFMA roofline) and Q8 decode
+attention (HBM roofline, tokens/s) measurements.
+
+No number is printed unchecked: outside the timed regions the output of every
+timed GEMV, GEMM and attention case is read back and a sample of it compared
+with the CPU oracle at the path's tolerance (relative L2 1e-3, max-abs
+2e-2 x RMS); each case carries `verified`, and a failed check ends the run
+with an error instead of a JSON line.
 """
 from __future__ import annotations
 
@@ -36,7 +43,14 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 MFMA_F16_PEAK_TFLOPS = 2500.0  # MI355X dense fp16
 SEED = 20240531
-COPIES = 16
+CACHE_BYTES = 256 << 20        # Infinity Cache
+REL_L2_TOL, MAX_ABS_RMS_TOL = 1e-3, 2e-2
+
+
+def copies_for(k, n):
+    """Weight copies of one shape: at least 16, and more than twice the Infinity Cache in total."""
+    return max(16, -(-2 * CACHE_BYTES // gemv_bytes(1, k, n)) + 1)
+
 
 GEMV_SHAPES = [(4096, 4096), (4096, 14336), (14336, 4096)]
 GEMV_ROWS = [1, 2, 4, 8]
@@ -64,6 +78,37 @@ def w4_inputs(rng, m, n, k):
     return x, packed, scale
 
 
+def close_to_oracle(actual, expected):
+    """(ok, relative L2 error) at the path's tolerance."""
+    actual = np.asarray(actual, dtype=np.float64).reshape(-1)
+    expected = np.asarray(expected, dtype=np.float64).reshape(-1)
+    if actual.shape != expected.shape or not np.all(np.isfinite(actual)):
+        return False, float("inf")
+    difference = actual - expected
+    norm = float(np.sqrt(np.sum(expected ** 2)))
+    rel_l2 = float(np.sqrt(np.sum(difference ** 2))) / max(norm, 1e-30)
+    rms = norm / math.sqrt(max(1, expected.size))
+    ok = rel_l2 <= REL_L2_TOL and float(np.max(np.abs(difference))) <= MAX_ABS_RMS_TOL * rms + 1e-6
+    return bool(ok), rel_l2
+
+
+def sample_columns(rng, n, count=160):
+    """Columns of an output to check: both ends (partial tiles live there) and a random draw."""
+    edge = np.concatenate([np.arange(min(16, n)), np.arange(max(0, n - 16), n)])
+    return np.unique(np.concatenate([edge, rng.integers(0, n, size=count)]))
+
+
+def verify_linear(out_buffer, m, n, x, packed, scale, rng, rows=None):
+    """Checker (not part of any timed region): sampled columns (and rows) of a W4A16 linear
+    output against the CPU oracle."""
+    import oracle
+    columns = sample_columns(rng, n)
+    row_index = np.arange(m) if rows is None else rows
+    got = out_buffer.numpy(np.float16, (m, n))[np.ix_(row_index, columns)]
+    want = oracle.w4a16_linear(x[row_index], packed[columns], scale[columns], None)
+    return close_to_oracle(got, want)
+
+
 def record_linear(batch, m, n, k, bx, bw, bs, out):
     name = "llmopt_w4a16_linear_f16_g64" if m == 1 else "llmopt_w4a16_linear_f16_g64_m4"
     columns = m * n if m == 1 else ((m + 3) // 4) * n
@@ -71,24 +116,34 @@ def record_linear(batch, m, n, k, bx, bw, bs, out):
                    grid=(linear_grid(columns), 1, 1), group=(256, 1, 1))
 
 
+def gemv_kernel_of(m, k, n):
+    """The kernel a sweep case runs (for grouping the sweep's time by kernel)."""
+    if m <= 4:
+        return "w4a16_gemv_quad_kernel (4x4x4 matrix-core blocks, one workgroup per CU, m <= 4)"
+    return "w4a16_gemv_mfma_kernel (16x16x32 matrix-core tiles, 5 <= m <= 8)"
+
+
 def bench_gemv(runtime, steps, warmup):
     rng = np.random.default_rng(SEED)
-    weights = {}
+    weights, host = {}, {}
     for k, n in GEMV_SHAPES:
         _, packed, scale = w4_inputs(rng, 1, n, k)
+        host[(k, n)] = (packed, scale)
         weights[(k, n)] = [(runtime.buffer_of_bytes(packed), runtime.buffer_of_bytes(scale))
-                           for _ in range(COPIES)]
-    activations = {(m, k): runtime.buffer_of_bytes(rng.standard_normal((m, k)).astype(np.float16))
-                   for m in GEMV_ROWS for k in {s[0] for s in GEMV_SHAPES}}
-    outputs = {(m, n): runtime.create_buffer(m * n * 2)
-               for m in GEMV_ROWS for n in {s[1] for s in GEMV_SHAPES}}
+                           for _ in range(copies_for(k, n))]
+    host_x = {(m, k): rng.standard_normal((m, k)).astype(np.float16)
+              for m in GEMV_ROWS for k in {s[0] for s in GEMV_SHAPES}}
+    activations = {key: runtime.buffer_of_bytes(x) for key, x in host_x.items()}
+    outputs = {(m, k, n): runtime.create_buffer(m * n * 2) for m in GEMV_ROWS for k, n in GEMV_SHAPES}
 
     def record_steps(batch, count, first=0):
         for step in range(first, first + count):
-            for m in GEMV_ROWS:
+            for m_index, m in enumerate(GEMV_ROWS):
                 for k, n in GEMV_SHAPES:
-                    bw, bs = weights[(k, n)][step % COPIES]
-                    record_linear(batch, m, n, k, activations[(m, k)], bw, bs, outputs[(m, n)])
+                    # another HBM copy for every launch that reads this shape
+                    copies = weights[(k, n)]
+                    bw, bs = copies[(step * len(GEMV_ROWS) + m_index) % len(copies)]
+                    record_linear(batch, m, n, k, activations[(m, k)], bw, bs, outputs[(m, k, n)])
 
     bytes_per_step = sum(gemv_bytes(m, k, n) for m in GEMV_ROWS for k, n in GEMV_SHAPES)
 
@@ -107,47 +162,58 @@ def bench_gemv(runtime, steps, warmup):
 
     # the same K steps as ONE HIP graph (back-to-back launches, no host in the loop):
     # one untimed replay, then one replay timed by HIP events on the launch stream
+    for buffer in outputs.values():
+        buffer.write(np.full(buffer.byte_length // 2, np.nan, dtype=np.float16))
     batch = runtime.begin_batch()
     record_steps(batch, steps)
     graph_ms = batch.commit_profiled(repeats=1, use_graph=True)
     graph_ms_per_step = graph_ms / steps
+    # what the timed launches left in the outputs, against the oracle
+    check_rng = np.random.default_rng(SEED + 7)
+    verified = {}
+    for m in GEMV_ROWS:
+        for k, n in GEMV_SHAPES:
+            verified[(m, k, n)] = verify_linear(outputs[(m, k, n)], m, n, host_x[(m, k)], *host[(k, n)], check_rng)
 
-    # per-case kernel time: COPIES launches of one case per graph, HIP events
+    # per-case kernel time: one launch per HBM copy in a graph, HIP events
     cases = []
     for m in GEMV_ROWS:
         for k, n in GEMV_SHAPES:
+            copies = weights[(k, n)]
             batch = runtime.begin_batch()
-            for copy in range(COPIES):
-                bw, bs = weights[(k, n)][copy]
-                record_linear(batch, m, n, k, activations[(m, k)], bw, bs, outputs[(m, n)])
-            repeats = 8
+            for bw, bs in copies:
+                record_linear(batch, m, n, k, activations[(m, k)], bw, bs, outputs[(m, k, n)])
+            repeats = 4
             ms = batch.commit_profiled(repeats=repeats, use_graph=True)
-            us = ms * 1e3 / (repeats * COPIES)
+            us = ms * 1e3 / (repeats * len(copies))
             gbs = gemv_bytes(m, k, n) / (us * 1e-6) / 1e9
-            # warm: the same weight copy every launch (31 MB stays in the 256 MB Infinity Cache)
+            # warm: the same weight copy every launch (it stays in the 256 MB Infinity Cache)
             batch = runtime.begin_batch()
-            bw, bs = weights[(k, n)][0]
-            for _ in range(COPIES):
-                record_linear(batch, m, n, k, activations[(m, k)], bw, bs, outputs[(m, n)])
-            warm_us = batch.commit_profiled(repeats=repeats, use_graph=True) * 1e3 / (repeats * COPIES)
-            cases.append({"m": m, "k": k, "n": n, "bytes": gemv_bytes(m, k, n),
+            bw, bs = copies[0]
+            for _ in range(16):
+                record_linear(batch, m, n, k, activations[(m, k)], bw, bs, outputs[(m, k, n)])
+            warm_us = batch.commit_profiled(repeats=repeats, use_graph=True) * 1e3 / (repeats * 16)
+            ok, rel_l2 = verified[(m, k, n)]
+            cases.append({"m": m, "k": k, "n": n, "bytes": gemv_bytes(m, k, n), "kernel": gemv_kernel_of(m, k, n),
                           "us_per_launch": round(us, 3), "GBps": round(gbs, 1),
                           "hbm_frac": round(gbs / HBM_PEAK_GBS, 4),
                           "warm_us_per_launch": round(warm_us, 3),
-                          "warm_GBps": round(gemv_bytes(m, k, n) / (warm_us * 1e-6) / 1e9, 1)})
+                          "warm_GBps": round(gemv_bytes(m, k, n) / (warm_us * 1e-6) / 1e9, 1),
+                          "hbm_copies": len(copies), "verified": ok, "rel_l2": float("%.3g" % rel_l2)})
 
     # C1: the 1 x 576 -> 1536 projection of the 30-layer model (474 KB: launch/latency-bound)
     k, n = 576, 1536
-    _, packed, scale = w4_inputs(rng, 1, n, k)
-    c1_weights = [(runtime.buffer_of_bytes(packed), runtime.buffer_of_bytes(scale)) for _ in range(COPIES)]
-    c1_x = runtime.buffer_of_bytes(rng.standard_normal((1, k)).astype(np.float16))
+    c1_x, packed, scale = w4_inputs(rng, 1, n, k)
+    c1_weights = [(runtime.buffer_of_bytes(packed), runtime.buffer_of_bytes(scale)) for _ in range(16)]
     c1_out = runtime.create_buffer(n * 2)
     batch = runtime.begin_batch()
     for bw, bs in c1_weights:
-        record_linear(batch, 1, n, k, c1_x, bw, bs, c1_out)
-    c1_us = batch.commit_profiled(repeats=8, use_graph=True) * 1e3 / (8 * COPIES)
+        record_linear(batch, 1, n, k, runtime.buffer_of_bytes(c1_x), bw, bs, c1_out)
+    c1_us = batch.commit_profiled(repeats=8, use_graph=True) * 1e3 / (8 * 16)
+    ok, rel_l2 = verify_linear(c1_out, 1, n, c1_x, packed, scale, check_rng)
     c1 = {"m": 1, "k": k, "n": n, "bytes": gemv_bytes(1, k, n), "us_per_launch": round(c1_us, 3),
-          "GBps": round(gemv_bytes(1, k, n) / (c1_us * 1e-6) / 1e9, 1)}
+          "GBps": round(gemv_bytes(1, k, n) / (c1_us * 1e-6) / 1e9, 1), "verified": ok,
+          "rel_l2": float("%.3g" % rel_l2)}
     return {"bytes_per_step": bytes_per_step, "ms_per_step": ms_per_step,
             "graph_ms_per_step": graph_ms_per_step, "cases": cases, "c1": c1}
 
@@ -155,19 +221,24 @@ def bench_gemv(runtime, steps, warmup):
 def bench_gemm(runtime):
     """C3: prefill GEMM, M in {512, 2048}, K=4096, N in {4096, 14336}, plus the fused
     SwiGLU pair (two N=14336 projections combined as silu(a)*b)."""
+    import oracle
     rng = np.random.default_rng(SEED + 1)
+    check_rng = np.random.default_rng(SEED + 8)
     results = []
     k = 4096
-    packed_cache = {}
+    packed_cache, host = {}, {}
     for n in (4096, 14336):
         _, packed, scale = w4_inputs(rng, 1, n, k)
+        host[n] = (packed, scale)
         packed_cache[n] = (runtime.buffer_of_bytes(packed), runtime.buffer_of_bytes(scale),
                            runtime.buffer_of_bytes(packed[::-1].copy()), runtime.buffer_of_bytes(scale))
     for m in (512, 2048):
-        bx = runtime.buffer_of_bytes(rng.standard_normal((m, k)).astype(np.float16))
+        x = rng.standard_normal((m, k)).astype(np.float16)
+        bx = runtime.buffer_of_bytes(x)
+        rows = np.unique(np.concatenate([[0, m - 1], check_rng.integers(0, m, size=30)]))
         for n in (4096, 14336):
             bw, bs, _, _ = packed_cache[n]
-            out = runtime.create_buffer(m * n * 2)
+            out = runtime.buffer_of_bytes(np.full(m * n, np.nan, dtype=np.float16))
             batch = runtime.begin_batch()
             for _ in range(4):
                 record_linear(batch, m, n, k, bx, bw, bs, out)
@@ -175,12 +246,14 @@ def bench_gemm(runtime):
             ms = batch.commit_profiled(repeats=repeats, use_graph=True)
             us = ms * 1e3 / (repeats * 4)
             tflops = 2.0 * m * n * k / (us * 1e-6) / 1e12
+            ok, rel_l2 = verify_linear(out, m, n, x, *host[n], check_rng, rows=rows)
             results.append({"kind": "linear", "m": m, "n": n, "k": k, "us_per_launch": round(us, 2),
                             "TFLOPs": round(tflops, 1),
-                            "mfma_frac": round(tflops / MFMA_F16_PEAK_TFLOPS, 4)})
+                            "mfma_frac": round(tflops / MFMA_F16_PEAK_TFLOPS, 4),
+                            "verified": ok, "rel_l2": float("%.3g" % rel_l2)})
         n = 14336
         gate_w, gate_s, up_w, up_s = packed_cache[n]
-        product = runtime.create_buffer(m * n * 2)
+        product = runtime.buffer_of_bytes(np.full(m * n, np.nan, dtype=np.float16))
         batch = runtime.begin_batch()
         params = u32s(m, n, k) + struct.pack("<f", 1e-5)
         for _ in range(4):
@@ -190,9 +263,15 @@ def bench_gemm(runtime):
         ms = batch.commit_profiled(repeats=repeats, use_graph=True)
         us = ms * 1e3 / (repeats * 4)
         tflops = 2.0 * 2.0 * m * n * k / (us * 1e-6) / 1e12
+        columns = sample_columns(check_rng, n)
+        packed, scale = host[n]
+        want = oracle.silu_mul(oracle.w4a16_linear(x[rows], packed[columns], scale[columns], None),
+                               oracle.w4a16_linear(x[rows], packed[::-1][columns], scale[columns], None))
+        ok, rel_l2 = close_to_oracle(product.numpy(np.float16, (m, n))[np.ix_(rows, columns)], want)
         results.append({"kind": "dual_swiglu", "m": m, "n": n, "k": k, "us_per_launch": round(us, 2),
                         "TFLOPs": round(tflops, 1),
-                        "mfma_frac": round(tflops / MFMA_F16_PEAK_TFLOPS, 4)})
+                        "mfma_frac": round(tflops / MFMA_F16_PEAK_TFLOPS, 4),
+                        "verified": ok, "rel_l2": float("%.3g" % rel_l2)})
     return results
 
 
@@ -224,7 +303,7 @@ def bench_attention(runtime):
     b_slots = runtime.buffer_of_bytes(slots)
     buffers_tail = [runtime.buffer_of_bytes(lengths), runtime.buffer_of_bytes(offsets)]
     bq, bck, bcv = (runtime.buffer_of_bytes(a) for a in (query, ck, cv))
-    out = runtime.create_buffer(batches * heads * dim * 2)
+    out = runtime.buffer_of_bytes(np.full(batches * heads * dim, np.nan, dtype=np.float16))
     batch = runtime.begin_batch()
     for b_pool in pools:
         batch.dispatch("llmopt_attention_q8_paged_batched",
@@ -235,9 +314,19 @@ def bench_attention(runtime):
     us = ms * 1e3 / (repeats * len(pools))
     kv_bytes = total * stride + 2 * batches * heads * dim * 2
     gbs = kv_bytes / (us * 1e-6) / 1e9
+    # checker: the whole output against the oracle's paged attention
+    import oracle
+    want = oracle.paged_attention_q8(
+        query, ck, cv, pool.reshape(-1), slots, None,
+        oracle.PagedParams(batches=batches, query_heads=heads, kv_heads=kv_heads, past_length=0, head_dim=dim,
+                           mask_batches=0, mask_heads=0, token_elements=token_elements, key_offset=0,
+                           value_offset=kv_heads * dim, group_size=64, token_stride=stride,
+                           scale=1.0 / math.sqrt(dim), query_length=1, mask_dtype=0, window=0),
+        past_lengths=lengths, slot_offsets=offsets)
+    ok, rel_l2 = close_to_oracle(out.numpy(np.float16, (batches, 1, heads, dim)), want)
     return {"batch": batches, "sum_context": total, "bytes": kv_bytes, "us_per_call": round(us, 2),
             "GBps": round(gbs, 1), "hbm_frac": round(gbs / HBM_PEAK_GBS, 4),
-            "tokens_per_s": round(batches / (us * 1e-6), 1)}
+            "tokens_per_s": round(batches / (us * 1e-6), 1), "verified": ok, "rel_l2": float("%.3g" % rel_l2)}
 
 
 def bench_prefill_attention(runtime):
@@ -245,11 +334,13 @@ def bench_prefill_attention(runtime):
     128 at 2048 and 8192 tokens, and the 30-layer model's 9/3 heads of 64 at 2048."""
     rng = np.random.default_rng(SEED + 4)
     results = []
+    import oracle
     for heads, kv_heads, dim, length in ((32, 8, 128, 2048), (32, 8, 128, 8192), (9, 3, 64, 2048)):
-        query = runtime.buffer_of_bytes(rng.standard_normal((1, heads, length, dim)).astype(np.float16))
-        key = runtime.buffer_of_bytes(rng.standard_normal((1, kv_heads, length, dim)).astype(np.float16))
-        value = runtime.buffer_of_bytes(rng.standard_normal((1, kv_heads, length, dim)).astype(np.float16))
-        out = runtime.create_buffer(heads * length * dim * 2)
+        host_q = rng.standard_normal((1, heads, length, dim)).astype(np.float16)
+        host_k = rng.standard_normal((1, kv_heads, length, dim)).astype(np.float16)
+        host_v = rng.standard_normal((1, kv_heads, length, dim)).astype(np.float16)
+        query, key, value = (runtime.buffer_of_bytes(a) for a in (host_q, host_k, host_v))
+        out = runtime.buffer_of_bytes(np.full(heads * length * dim, np.nan, dtype=np.float16))
         params = struct.pack("<8IfIIIII", 1, heads, length, length, dim, 0, 0, 1, 1.0 / math.sqrt(dim),
                              kv_heads, 1, 0, 0, 0)
         batch = runtime.begin_batch()
@@ -259,9 +350,21 @@ def bench_prefill_attention(runtime):
         repeats = 3
         us = batch.commit_profiled(repeats=repeats, use_graph=True) * 1e3 / (repeats * 4)
         flops = 4.0 * heads * dim * (length * (length + 1) / 2)  # QK^T and PV over the causal half
+        # checker: sampled query rows of sampled heads (a causal row sees the keys up to itself)
+        got = out.numpy(np.float16, (length, heads, dim))  # token-major output
+        ok, worst = True, 0.0
+        for row in (0, 15, length // 2 + 1, length - 1):
+            for head in (0, heads // 2, heads - 1):
+                kv = head // (heads // kv_heads)
+                want = oracle.attention(host_q[:, head:head + 1, row:row + 1], host_k[:, kv:kv + 1, :row + 1],
+                                        host_v[:, kv:kv + 1, :row + 1], np.ones((1, 1, 1, row + 1), dtype=np.float32),
+                                        1.0 / math.sqrt(dim), causal=False)
+                row_ok, rel_l2 = close_to_oracle(got[row, head], want)
+                ok, worst = ok and row_ok, max(worst, rel_l2)
         results.append({"heads": heads, "kv_heads": kv_heads, "head_dim": dim, "tokens": length,
                         "us_per_launch": round(us, 2), "TFLOPs": round(flops / (us * 1e-6) / 1e12, 1),
-                        "mfma_frac": round(flops / (us * 1e-6) / 1e12 / MFMA_F16_PEAK_TFLOPS, 4)})
+                        "mfma_frac": round(flops / (us * 1e-6) / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
+                        "verified": ok, "rel_l2": float("%.3g" % worst)})
     return results
 
 
@@ -320,28 +423,41 @@ def pmc_probe(runtime, m=1):
     k, n = 4096, 14336
     x, packed, scale = w4_inputs(rng, m, n, k)
     bx, out = runtime.buffer_of_bytes(x), runtime.create_buffer(m * n * 2)
-    weights = [(runtime.buffer_of_bytes(packed), runtime.buffer_of_bytes(scale)) for _ in range(COPIES)]
+    weights = [(runtime.buffer_of_bytes(packed), runtime.buffer_of_bytes(scale)) for _ in range(copies_for(k, n))]
     batch = runtime.begin_batch()
     for bw, bs in weights:
         record_linear(batch, m, n, k, bx, bw, bs, out)
     batch.commit()
     return {"copy_kernel": "copy_vectors_kernel", "copy_bytes_read": copy_bytes, "copy_bytes_written": copy_bytes,
-            "copy_launches": 4, "gemv_kernel": "w4a16_gemv_kernel<1, 2, 1, true, false, 2, false, false>",
-            "gemv_rows": m, "gemv_launches": COPIES, "gemv_algorithmic_bytes": gemv_bytes(m, k, n)}
+            "copy_launches": 4, "gemv_kernel": gemv_kernel_of(m, k, n),
+            "gemv_rows": m, "gemv_launches": len(weights), "gemv_algorithmic_bytes": gemv_bytes(m, k, n)}
 
 
-def measured_traffic():
-    """HBM bytes per launch of the headline kernel, measured with rocprofv3 hardware counters
-    (FETCH_SIZE and WRITE_SIZE, each calibrated on a plain copy) and kept with the profile
-    summaries; None when the summary is not there."""
-    path = os.path.join(ROOT, "profiles", "w4a16_gemv_m1_k4096_n14336_hbm_traffic.txt")
+TRAFFIC_SUMMARY = "profiles/w4a16_gemv_k4096_n14336_hbm_traffic.txt"
+
+
+def measured_traffic(rows):
+    """HBM bytes per launch of the K=4096, N=14336 GEMV with `rows` activation rows, from an
+    EARLIER rocprofv3 --pmc run of `bench.py --pmc-probe` (FETCH_SIZE and WRITE_SIZE, each
+    calibrated on a plain copy) whose summary is kept with the profiles - not measured in this
+    run.  None when the summary is not there or has no line for these rows."""
     try:
-        for line in open(path):
-            if line.startswith("traffic_bytes_per_launch:"):
+        for line in open(os.path.join(ROOT, TRAFFIC_SUMMARY)):
+            if line.startswith(f"traffic_bytes_per_launch_m{rows}:"):
                 return int(line.split(":")[1])
     except OSError:
         pass
     return None
+
+
+def cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
 
 
 def cpu_baseline(passes=2):
@@ -362,7 +478,7 @@ def cpu_baseline(passes=2):
                 elapsed += time.perf_counter() - started
                 total_bytes += gemv_bytes(m, k, n)
     return {"value": round(total_bytes / elapsed / 1e9, 4), "unit": "GB/s", "cores": 1,
-            "kind": "port",
+            "kind": "port", "cpu": cpu_model(), "host_cores_visible": os.cpu_count(),
             "sample": f"{passes} passes over the whole 12-case GEMV sweep at full N and K "
                       f"({elapsed:.1f} s of single-thread oracle time)"}
 
@@ -393,10 +509,28 @@ def main():
         runtime.close()
         return
     gemv = bench_gemv(runtime, args.steps, args.warmup)
-    headline = next(c for c in gemv["cases"] if (c["m"], c["k"], c["n"]) == (1, 4096, 14336))
+    # the sweep's time by kernel; `roofline` is the kernel with the largest share
+    by_kernel = {}
+    for case in gemv["cases"]:
+        entry = by_kernel.setdefault(case["kernel"], {"kernel": case["kernel"], "launches": 0, "bytes": 0, "us": 0.0,
+                                                      "cases": []})
+        entry["launches"] += 1
+        entry["bytes"] += case["bytes"]
+        entry["us"] += case["us_per_launch"]
+        entry["cases"].append([case["m"], case["k"], case["n"]])
+    sweep_us = sum(entry["us"] for entry in by_kernel.values())
+    kernels = []
+    for entry in sorted(by_kernel.values(), key=lambda e: -e["us"]):
+        gbs = entry["bytes"] / (entry["us"] * 1e-6) / 1e9
+        kernels.append({"kernel": entry["kernel"], "share_of_sweep_time": round(entry["us"] / sweep_us, 4),
+                        "launches_per_step": entry["launches"],
+                        "bytes_per_launch": entry["bytes"] // entry["launches"],
+                        "us_per_launch": round(entry["us"] / entry["launches"], 3), "GBps": round(gbs, 1),
+                        "hbm_frac": round(gbs / HBM_PEAK_GBS, 4), "cases_m_k_n": entry["cases"]})
+    dominant = kernels[0]
     # the K steps replayed as one HIP graph, timed by HIP events on the launch stream
     value = gemv["bytes_per_step"] / (gemv["graph_ms_per_step"] * 1e-3) / 1e9
-    extras = {"gemv_cases": gemv["cases"], "gemv_c1_1x576x1536": gemv["c1"],
+    extras = {"gemv_cases": gemv["cases"], "gemv_kernels": kernels, "gemv_c1_1x576x1536": gemv["c1"],
               "gemv_eager_host_launch_GBps":
                   round(gemv["bytes_per_step"] / (gemv["ms_per_step"] * 1e-3) / 1e9, 1),
               "gemv_eager_host_launch_ms_per_step": round(gemv["ms_per_step"], 4),
@@ -411,6 +545,19 @@ def main():
     if "decode" in wanted:
         extras["decode_step"] = bench_decode_step(
             runtime, batches=tuple(int(b) for b in args.decode_batches.split(",")), use_graph=not args.decode_eager)
+    # refuse to print numbers whose outputs did not match the oracle
+    checked = [("gemv %(m)dx%(k)dx%(n)d" % c, c["verified"]) for c in gemv["cases"]]
+    checked.append(("gemv c1", gemv["c1"]["verified"]))
+    checked += [("%(kind)s %(m)dx%(n)dx%(k)d" % c, c["verified"]) for c in extras.get("prefill_gemm", [])]
+    if "q8_attention" in extras:
+        checked.append(("q8 attention", extras["q8_attention"]["verified"]))
+    checked += [("prefill attention %(heads)d/%(kv_heads)d x %(head_dim)d @ %(tokens)d" % c, c["verified"])
+                for c in extras.get("prefill_attention", [])]
+    failed = [name for name, ok in checked if not ok]
+    if failed:
+        runtime.close()
+        sys.exit("bench.py: outputs of timed cases differ from the CPU oracle beyond tolerance: " + ", ".join(failed))
+    dominant_rows = max(case[0] for case in dominant["cases_m_k_n"])
     line = {
         "metric": "W4A16 GEMV HBM GB/s (% peak); Q8 attn decode tokens/s; prefill MFMA %",
         "value": round(value, 1),
@@ -426,12 +573,18 @@ def main():
         "data": "synthetic (seeded int4 U{-8..7}, fp16 scales U[0.005,0.02], activations N(0,1))",
         "config": {"workload": "W4A16 decode GEMV sweep: M in {1,2,4,8} x (K,N) in "
                                "{(4096,4096),(4096,14336),(14336,4096)}, group-64 fp16 scales; "
-                               "one step = the 12 launches, weights cycled over 16 HBM copies",
+                               "one step = the 12 launches, every launch on another HBM copy of its weights",
                    "bytes_per_step": gemv["bytes_per_step"]},
-        "roofline": {"bound": "hbm", "kernel": "w4a16_gemv_kernel<1, 2, 1, true, false, 2, false, false> (M=1) at K=4096 N=14336",
-                     "achieved": headline["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": headline["hbm_frac"], "traffic": measured_traffic(),
-                     "bytes_per_launch": headline["bytes"], "us_per_launch": headline["us_per_launch"]},
+        "verified": True,
+        "roofline": {"bound": "hbm", "kernel": dominant["kernel"],
+                     "share_of_sweep_time": dominant["share_of_sweep_time"],
+                     "achieved": dominant["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": dominant["hbm_frac"],
+                     "traffic": measured_traffic(dominant_rows),
+                     "traffic_source": TRAFFIC_SUMMARY + " (an earlier rocprofv3 --pmc run of `bench.py --pmc-probe "
+                                       f"--pmc-rows {dominant_rows}` at K=4096 N=14336; not measured in this run)",
+                     "bytes_per_launch": dominant["bytes_per_launch"], "us_per_launch": dominant["us_per_launch"],
+                     "cases_m_k_n": dominant["cases_m_k_n"]},
         "cpu_baseline": None if args.skip_cpu else cpu_baseline(),
         "extras": extras,
     }

@@ -27,6 +27,11 @@ hipError_t launch_w4a16_gemv_mfma_linear(const W4LinearArgs &args, hipStream_t s
 hipError_t launch_w4a16_gemv_mfma_qkv(const W4QkvArgs &args, hipStream_t stream);
 hipError_t launch_w4a16_gemv_mfma_dual_swiglu(const W4DualSwigluArgs &args, hipStream_t stream);
 
+// One to four rows at the K values w4a16_gemv_quad.hip is instantiated for: whole-row-piece loads
+// on the 4x4x4 matrix-core blocks, one workgroup per CU.
+bool w4a16_gemv_quad_ok(const W4LinearArgs &args);
+hipError_t launch_w4a16_gemv_quad_linear(const W4LinearArgs &args, hipStream_t stream);
+
 hipError_t launch_w4a16_gemm_linear(const W4LinearArgs &args, hipStream_t stream);
 hipError_t launch_w4a16_gemm_dual_swiglu(const W4DualSwigluArgs &args, hipStream_t stream);
 

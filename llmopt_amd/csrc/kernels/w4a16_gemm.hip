@@ -394,6 +394,7 @@ hipError_t launch_w4a16_gemm_dual_swiglu(const W4DualSwigluArgs &a, hipStream_t 
 // ---- m-based choice between the streaming GEMV and the MFMA GEMM ------------
 
 hipError_t launch_w4a16_linear(const W4LinearArgs &args, hipStream_t stream) {
+  if (w4a16_gemv_quad_ok(args)) return launch_w4a16_gemv_quad_linear(args, stream);
   if (args.m <= kGemvDotRows) return launch_w4a16_gemv_linear(args, stream);
   if (args.m <= kGemvMaxRows && (!w4a16_gemv_mfma_needs_split(args.k) || args.workspace != nullptr))
     return launch_w4a16_gemv_mfma_linear(args, stream);

@@ -336,10 +336,37 @@ def test_gemv_sweep_cell_at_full_size(runtime, m, n, k):
     print(f"gemv sweep cell m={m} n={n} k={k}", flush=True)
     expected = oracle.w4a16_linear(x, packed, scale, None)
     assert_close_to_oracle(run_linear(runtime, x, packed, scale), expected, f"gemv cell {m}x{n}x{k}")
-    if m in (1, 8):  # the addend path of the same grids
+    if m in (1, 2, 8):  # the addend path of the same grids
         expected_bias = oracle.add(expected, bias.astype(np.float32).reshape(1, -1))
         assert_close_to_oracle(run_linear(runtime, x, packed, scale, bias=bias), expected_bias,
                                f"gemv cell+bias {m}x{n}x{k}")
+
+
+# The one-workgroup-per-CU GEMV on the 4x4x4 matrix-core blocks (1..4 rows, K = 4096 / 14336):
+# every (row quads per wave, waves, ring) choice of its launcher, a last workgroup that is only
+# partly there (N = 4100, 9004), three rows inside a four-row staging, and both addend kinds.
+QUAD_CELLS = [(3, 4096, 4096, "bias"), (2, 4100, 4096, "residual"), (4, 6144, 4096, "bias"),
+              (3, 9004, 4096, "residual"), (2, 11008, 4096, None), (4, 14336, 4096, "residual"),
+              (1, 4100, 14336, "bias"), (3, 6144, 14336, "residual"), (4, 4096, 14336, "bias"),
+              (2, 9004, 14336, None), (4, 3072, 14336, None)]
+
+
+@pytest.mark.parametrize("m,n,k,addend", QUAD_CELLS)
+def test_gemv_quad_kernel_shapes(runtime, m, n, k, addend):
+    rng = np.random.default_rng(13 * m + n + 3 * k)
+    x, packed, scale, bias = w4_case(rng, m, n, k, bias=True)
+    residual = rng.standard_normal((m, n)).astype(np.float16)
+    print(f"gemv quad cell m={m} n={n} k={k} addend={addend}", flush=True)
+    expected = oracle.w4a16_linear(x, packed, scale, None)
+    if addend == "bias":
+        expected = oracle.add(expected, bias.astype(np.float32).reshape(1, -1))
+        got = run_linear(runtime, x, packed, scale, bias=bias)
+    elif addend == "residual":
+        expected = oracle.add(expected, residual.astype(np.float32))
+        got = run_linear(runtime, x, packed, scale, residual=residual)
+    else:
+        got = run_linear(runtime, x, packed, scale)
+    assert_close_to_oracle(got, expected, f"gemv quad {m}x{n}x{k} {addend}")
 
 
 def tile_covering_sample(rng, extent, block):
