@@ -401,8 +401,25 @@ def bench_decode_step(runtime, batches=(1, 8, 32, 128), context=2048, use_graph=
         repeats = 20
         ms = graph.commit_profiled(repeats=repeats, use_graph=use_graph) / repeats
         moved = step.weight_bytes() + step.kv_bytes()
+        # the same list frozen into a retained plan: wall-clock of llmopt_hip_prebaked_execute
+        # (state launch + one graph launch + 4-byte read-back + wait), what a host stepping a
+        # sequence through the boundary pays per token
+        from llmopt_amd.native import Prebaked
+        plan = Prebaked(runtime, step.dispatches, step.tokens, step.token_ids)
+        for _ in range(3):
+            plan.execute(1, context)
+        runtime.synchronize()
+        started = time.perf_counter()
+        for _ in range(repeats):
+            plan.execute(1, context)
+        execute_ms = (time.perf_counter() - started) * 1e3 / repeats
+        single = plan.single_submission
+        del plan
         results.append({"batch": batch, "context": context, "launches": len(step.dispatches),
                         "ms_per_step": round(ms, 4), "tokens_per_s": round(batch / (ms * 1e-3), 1),
+                        "prebaked_execute_wall_ms": round(execute_ms, 4),
+                        "prebaked_execute_tokens_per_s": round(batch / (execute_ms * 1e-3), 1),
+                        "prebaked_single_submission": single,
                         "weight_bytes": step.weight_bytes(), "kv_bytes": step.kv_bytes(),
                         "GBps": round(moved / (ms * 1e-3) / 1e9, 1),
                         "hbm_frac": round(moved / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)})

@@ -47,6 +47,7 @@ typedef struct llmopt_hip_library llmopt_hip_library;
 typedef struct llmopt_hip_buffer llmopt_hip_buffer;
 typedef struct llmopt_hip_batch llmopt_hip_batch;
 typedef struct llmopt_hip_prebaked llmopt_hip_prebaked;
+typedef struct llmopt_hip_ring llmopt_hip_ring;
 
 /* One recorded dispatch: the tuple of lib/metal_native.ml:61-65 and :117-124
  * (name, buffers, parameter bytes, grid xyz, threadgroup xyz, barrier flag). */
@@ -199,19 +200,75 @@ int llmopt_hip_abort_batch(llmopt_hip_batch *batch);
 /* ---- retained decode plan ------------------------------------------------ */
 
 /* caml_llmopt_prebaked_create (:1879-2165): freezes a dispatch array; at most
- * 16 buffers and 256 parameter bytes per record. */
+ * 16 buffers and 256 parameter bytes per record.  The records are captured
+ * into one HIP graph here (nothing runs): a later execute is a single graph
+ * launch.  Paged attention records (names starting with
+ * "llmopt_attention_q8_paged_", the batched extension excepted) read their
+ * context length from a device word of the plan instead of parameter byte 12
+ * and are sized for the capacity of their slot table (buffer 4), so one graph
+ * serves every step; a plan that holds a masked one is replayed record by
+ * record from the host instead, as the reference does.  Buffers the caller
+ * rewrites between steps (rotary rows, slots, the lengths of the batched
+ * extension) are read from device memory by the kernels, replay included. */
 int llmopt_hip_prebaked_create(llmopt_hip_library *library,
                                const llmopt_hip_dispatch_item *items, size_t count,
                                llmopt_hip_buffer *token_buffer, llmopt_hip_buffer *output_buffer,
                                llmopt_hip_prebaked **out);
 void llmopt_hip_release_prebaked(llmopt_hip_prebaked *plan);
 /* caml_llmopt_prebaked_execute (:2167-2560): writes `token` (int64) at the
- * start of the token buffer, patches past_tokens into byte 12 of every record
- * whose name starts with "llmopt_attention_q8_paged_" (:2182-2195), replays
- * all records in order, waits, and returns the first int32 of the output
- * buffer in *out_token. */
+ * start of the token buffer, makes past_tokens the context length of every
+ * paged attention record (:2182-2195), replays all records in order, waits,
+ * and returns the first int32 of the output buffer in *out_token.
+ * past_tokens beyond the slot tables' capacity is LLMOPT_ERR_INVALID. */
 int llmopt_hip_prebaked_execute(llmopt_hip_prebaked *plan, int64_t token, int64_t past_tokens,
                                 int64_t checkpoint, int64_t *out_token);
+/* 1 when execute replays one HIP graph, 0 when it launches record by record
+ * (no reference counterpart; for diagnostics and tests). */
+int llmopt_hip_prebaked_is_single_submission(llmopt_hip_prebaked *plan);
+
+/* ---- ring queue ------------------------------------------------------------ */
+
+/* The submission / completion queues of lib/metal_native.ml:86-111 (256
+ * entries each, one submitting thread, one worker thread).  The worker runs
+ * one decode step of a retained plan per submission, in order, on the
+ * context's stream; while it runs it is the context's caller thread.
+ * LLMOPT_QUEUE_DEPTH (default 1, as lib/metal_native.ml:407-415) > 1 lets it
+ * queue the next step on the GPU before it waits for the previous one. */
+
+/* caml_llmopt_ring_create (native/ocaml_metal_stubs.m:1699-1710). */
+int llmopt_hip_ring_create(llmopt_hip_ring **out);
+/* caml_llmopt_ring_submit (:1712-1732): 1 when queued, 0 when 256 submissions
+ * are waiting.  token < 0 chains: the step's input is the token the previous
+ * step produced (:1546-1560).  flags == 2 stops the worker (:1538). */
+int llmopt_hip_ring_submit(llmopt_hip_ring *ring, int64_t request_id, int64_t token,
+                           int64_t past_tokens, int64_t flags);
+/* caml_llmopt_ring_wait_completion (:1734-1767): blocks for the next
+ * (request id, produced token, status 0 = ok / 1 = failed); fails with "Ring
+ * queue terminated with no completion" when the ring stops first. */
+int llmopt_hip_ring_wait_completion(llmopt_hip_ring *ring, int64_t *request_id, int64_t *token,
+                                    int64_t *status);
+/* caml_llmopt_ring_poll_completion (:1769-1797): 1 with a completion, 0 with
+ * none (the reference's None), negative on error. */
+int llmopt_hip_ring_poll_completion(llmopt_hip_ring *ring, int64_t *request_id, int64_t *token,
+                                    int64_t *status);
+/* caml_llmopt_ring_start_worker (:1799-1871): freezes the dispatch array as
+ * llmopt_hip_prebaked_create does and starts the worker thread. */
+int llmopt_hip_ring_start_worker(llmopt_hip_ring *ring, llmopt_hip_library *library,
+                                 const llmopt_hip_dispatch_item *items, size_t count,
+                                 llmopt_hip_buffer *token_buffer,
+                                 llmopt_hip_buffer *output_buffer);
+/* The same worker over a host function instead of a plan (no reference
+ * counterpart: other executors, and tests of the queue without a GPU).  The
+ * function gets the step's token (a chained step: the previous result) and
+ * context length, stores the produced token and returns LLMOPT_OK or a
+ * failure status. */
+typedef int (*llmopt_hip_ring_step)(void *user, int64_t token, int64_t past_tokens,
+                                    int32_t *out_token);
+int llmopt_hip_ring_start_worker_with(llmopt_hip_ring *ring, llmopt_hip_ring_step step,
+                                      void *user);
+/* caml_llmopt_ring_destroy (finalize_ring, :296-329): stops and joins the
+ * worker, releases the plan. */
+void llmopt_hip_ring_destroy(llmopt_hip_ring *ring);
 
 /* ---- the entry point that allocates nothing ---------------------------------- */
 

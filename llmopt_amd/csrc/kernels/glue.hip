@@ -399,6 +399,24 @@ hipError_t launch_add_f16(const PointwiseArgs &a, hipStream_t stream) {
   return hipGetLastError();
 }
 
+namespace {
+// The per-step state of a retained decode plan, written in stream order ahead of its graph:
+// the input token (given, or the previous step's output token: llmopt_chain_token_id,
+// native/ocaml_metal_stubs.m:1570-1577) and the context length every sequence attends to.
+__global__ void plan_state_kernel(int64_t *token, int64_t value, const int32_t *chain_from, uint32_t *past,
+                                  uint32_t past_value, uint32_t past_count) {
+  if (threadIdx.x == 0 && token != nullptr) *token = chain_from != nullptr ? (int64_t)*chain_from : value;
+  for (uint32_t i = threadIdx.x; i < past_count; i += blockDim.x) past[i] = past_value;
+}
+}  // namespace
+
+hipError_t launch_plan_state(int64_t *token, int64_t value, const int32_t *chain_from, uint32_t *past,
+                             uint32_t past_value, uint32_t past_count, hipStream_t stream) {
+  hipLaunchKernelGGL(plan_state_kernel, dim3(1), dim3(256), 0, stream, token, value, chain_from, past, past_value,
+                     past_count);
+  return hipGetLastError();
+}
+
 hipError_t launch_copy_bytes(void *destination, const void *source, size_t bytes, hipStream_t stream) {
   if (bytes == 0) return hipSuccess;
   const bool vector_ok = ((reinterpret_cast<uintptr_t>(destination) | reinterpret_cast<uintptr_t>(source)) & 15) == 0;

@@ -150,6 +150,8 @@ struct Q8AttentionArgs {
   size_t workspace_bytes;
 };
 
+// The longest context the split-context kernels take (longer ones run the row-serial kernel).
+constexpr uint32_t kQ8AttentionSplitTokens = 128 * 1024;
 // Bytes of workspace launch_q8_attention needs for these arguments (0 when the
 // row-serial kernel is used).
 size_t q8_attention_workspace_bytes(const Q8AttentionArgs &args);
@@ -232,6 +234,10 @@ struct PointwiseArgs {
 hipError_t launch_add_f16(const PointwiseArgs &args, hipStream_t stream);
 
 hipError_t launch_copy_bytes(void *destination, const void *source, size_t bytes, hipStream_t stream);
+// One small launch that sets a retained plan's per-step state: *token = *chain_from (when not
+// null; int32 widened) or `value` (token may be null), and past[0..past_count) = past_value.
+hipError_t launch_plan_state(int64_t *token, int64_t value, const int32_t *chain_from, uint32_t *past,
+                             uint32_t past_value, uint32_t past_count, hipStream_t stream);
 
 // Argmax over float32 logits [rows, n] in two steps with the reference's
 // candidate layout (W4A16LmHeadCandidate {f32 value, u32 index}, 256 per row,

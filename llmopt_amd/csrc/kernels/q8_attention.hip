@@ -35,6 +35,7 @@ constexpr int kSplitMaxWaves = 4;   // KV heads per workgroup (one wave each)
 constexpr int kMaxChunkTokens = 128;  // context tokens per workgroup: 128, or 64 / 32 when that leaves CUs idle
 constexpr int kTileTokens = 16;    // tokens per MFMA tile
 constexpr int kMaxSplitChunks = 1024;  // chunks per sequence: the merge kernel keeps one weight per chunk in LDS
+static_assert((uint32_t)kMaxChunkTokens * kMaxSplitChunks == kQ8AttentionSplitTokens, "kernels.h states the limit");
 
 __device__ __forceinline__ float q8_scale_at(const uint8_t *token, uint32_t token_elements,
                                              uint32_t index) {
@@ -55,6 +56,13 @@ struct SplitPartial {
 template <int D>
 __device__ __forceinline__ size_t partial_floats(uint32_t heads_per_kv) {
   return 32 + (size_t)heads_per_kv * D;
+}
+
+// Context length of sequence b.  Lengths in device memory may change between replays of a
+// captured launch; they are held to max_past_length, which sized the grid, the partial results
+// and the host's check of the slot table.
+__device__ __forceinline__ uint32_t sequence_past(const Q8AttentionArgs &a, uint32_t b) {
+  return a.past_lengths ? min(a.past_lengths[b], a.max_past_length) : a.past_length;
 }
 
 // ---- balanced split --------------------------------------------------------------------
@@ -96,7 +104,7 @@ __device__ __forceinline__ SplitPlan split_plan(const Q8AttentionArgs &a, uint32
 #pragma unroll
   for (int k = 0; k < kPlanBlocks; ++k) {
     const uint32_t b = k * 64 + lane;
-    past[k] = b < a.batches ? (a.past_lengths ? a.past_lengths[b] : a.past_length) : 0;
+    past[k] = b < a.batches ? sequence_past(a, b) : 0;
     slot_offset[k] = BY_INDEX && a.slot_offsets != nullptr && b < a.batches ? a.slot_offsets[b] : 0;
   }
   uint32_t total = 0;
@@ -176,7 +184,7 @@ q8_attention_split_kernel(Q8AttentionArgs a, uint32_t chunks_max, uint32_t fixed
     slot_offset = plan.slot_offset;
     partial_index = (size_t)kv_head * balanced_slots + blockIdx.x;
   } else {
-    past = a.past_lengths ? a.past_lengths[batch] : a.past_length;
+    past = sequence_past(a, batch);
     slot_offset = a.slot_offsets ? a.slot_offsets[batch] : 0;
     partial_index = ((size_t)batch * a.kv_heads + kv_head) * chunks_max + chunk;
   }
@@ -494,7 +502,7 @@ __global__ __launch_bounds__(kMergeSlices *D) void q8_attention_merge_kernel(Q8A
     chunks = plan.chunks;
     partial += ((size_t)kv_head * balanced_slots + plan.first) * stride;
   } else {
-    const uint32_t past = a.past_lengths ? a.past_lengths[batch] : a.past_length;
+    const uint32_t past = sequence_past(a, batch);
     chunks = (past + chunk_tokens - 1) / chunk_tokens;
     partial += ((size_t)batch * a.kv_heads + kv_head) * chunks_max * stride;
   }
@@ -605,7 +613,7 @@ __global__ __launch_bounds__(256) void q8_attention_rows_kernel(Q8AttentionArgs 
   const uint32_t kv_head = head / heads_per_kv;
   const uint32_t D = a.head_dim;
   const uint32_t groups_per_head = D >> 6;
-  const uint32_t past = a.past_lengths ? a.past_lengths[batch] : a.past_length;
+  const uint32_t past = sequence_past(a, batch);
   const uint32_t *slots = a.slot_offsets ? a.slots + a.slot_offsets[batch] : a.slots;
   const size_t query_base = (((size_t)batch * a.query_heads + head) * q_len + q_pos) * D;
   const size_t current_base = ((size_t)batch * a.kv_heads + kv_head) * q_len * D;

@@ -200,6 +200,8 @@ int paged_attention(llmopt_hip_context *context, const DispatchRecord &record, b
   args.window = param_u32(record, 60);
   args.max_past_length = batched ? param_u32(record, 64) : args.past_length;
   const char *name = record.name.c_str();
+  const bool retained = !batched && record.device_past_lengths != nullptr;
+  if (retained) args.max_past_length = record.device_past_capacity;  // see DispatchRecord
   if (int status = check_cache_geometry(name, args.kv_heads, args.head_dim, group_size,
                                         args.token_elements, args.token_stride))
     return status;
@@ -241,6 +243,10 @@ int paged_attention(llmopt_hip_context *context, const DispatchRecord &record, b
   args.slots = reinterpret_cast<const uint32_t *>(record.buffers[4].device);
   args.mask = masked ? record.buffers[5].device : nullptr;
   args.output = reinterpret_cast<uint16_t *>(record.buffers[6].device);
+  if (retained) {
+    if (masked) return fail(LLMOPT_ERR_INVALID, "%s with a mask cannot read its context length from device memory", name);
+    args.past_lengths = record.device_past_lengths;
+  }
   if (batched) {
     if (int status = require_buffer_size(record.buffers[7], (uint64_t)args.batches * 4, "past lengths")) return status;
     if (int status = require_buffer_size(record.buffers[8], (uint64_t)args.batches * 4, "slot offsets")) return status;

@@ -107,6 +107,11 @@ float param_f32(const DispatchRecord &record, size_t byte_offset) {
 
 void *context_workspace(llmopt_hip_context *context, size_t bytes) {
   if (bytes <= context->workspace_bytes) return context->workspace;
+  if (context->sizing_capture) {
+    // the launch being captured is never run: any non-null address will do
+    context->sizing_wanted = std::max(context->sizing_wanted, bytes);
+    return context->workspace ? context->workspace : static_cast<void *>(context);
+  }
   // Work already queued may still read the old block: drain before replacing.
   if (hipStreamSynchronize(context->stream) != hipSuccess) {
     fail(LLMOPT_ERR_FAILURE, "HIP stream synchronize failed while growing the workspace");
@@ -124,6 +129,7 @@ void *context_workspace(llmopt_hip_context *context, size_t bytes) {
   }
   context->workspace = block;
   context->workspace_bytes = rounded;
+  ++context->workspace_generation;
   return block;
 }
 
@@ -206,7 +212,7 @@ void drop_record(DispatchRecord *record) {
   record->buffers.clear();
 }
 
-static int use_device(llmopt_hip_context *context) {
+int use_device(llmopt_hip_context *context) {
   LLMOPT_HIP_TRY(hipSetDevice(context->device), "HIP could not select the context's device");
   return LLMOPT_OK;
 }
@@ -229,13 +235,6 @@ struct llmopt_hip_batch : llmopt::RefCounted {
   bool finished = false;
 };
 
-struct llmopt_hip_prebaked : llmopt::RefCounted {
-  llmopt_hip_library *library = nullptr;
-  std::vector<DispatchRecord> records;
-  std::vector<bool> is_paged_attention;
-  llmopt_hip_buffer *token_buffer = nullptr;
-  llmopt_hip_buffer *output_buffer = nullptr;
-};
 
 extern "C" {
 
@@ -769,86 +768,6 @@ int llmopt_hip_abort_batch(llmopt_hip_batch *batch) {
     clear_batch(batch);
     batch->finished = true;
   }
-  return LLMOPT_OK;
-}
-
-// ---- retained decode plan ----------------------------------------------------------
-int llmopt_hip_prebaked_create(llmopt_hip_library *library,
-                               const llmopt_hip_dispatch_item *items, size_t count,
-                               llmopt_hip_buffer *token_buffer, llmopt_hip_buffer *output_buffer,
-                               llmopt_hip_prebaked **out) {
-  if (out == nullptr) return fail(LLMOPT_ERR_INVALID, "plan output pointer is null");
-  *out = nullptr;
-  if (library == nullptr) return fail(LLMOPT_ERR_FAILURE, "HIP library has been finalized");
-  if (count == 0 || items == nullptr)
-    return fail(LLMOPT_ERR_INVALID, "prebaked HIP plan requires at least one dispatch");
-  for (size_t i = 0; i < count; ++i) {
-    if (items[i].buffer_count > 16)
-      return fail(LLMOPT_ERR_INVALID, "prebaked HIP dispatch exceeds 16 buffers");
-    if (items[i].parameter_bytes > 256)
-      return fail(LLMOPT_ERR_INVALID, "prebaked HIP dispatch parameters exceed 256 bytes");
-  }
-  std::unique_ptr<llmopt_hip_prebaked> plan(new llmopt_hip_prebaked());
-  plan->records.resize(count);
-  for (size_t i = 0; i < count; ++i) {
-    if (int status = build_record(library, &items[i], &plan->records[i])) {
-      for (size_t j = 0; j < i; ++j) drop_record(&plan->records[j]);
-      return status;
-    }
-    static const char prefix[] = "llmopt_attention_q8_paged_";
-    plan->is_paged_attention.push_back(strncmp(items[i].name, prefix, sizeof prefix - 1) == 0);
-  }
-  plan->library = library;
-  retain(library);
-  plan->token_buffer = token_buffer;
-  plan->output_buffer = output_buffer;
-  retain(token_buffer);
-  retain(output_buffer);
-  *out = plan.release();
-  return LLMOPT_OK;
-}
-
-void llmopt_hip_release_prebaked(llmopt_hip_prebaked *plan) {
-  if (!release(plan)) return;
-  for (DispatchRecord &record : plan->records) drop_record(&record);
-  if (plan->token_buffer) llmopt_hip_release_buffer(plan->token_buffer);
-  if (plan->output_buffer) llmopt_hip_release_buffer(plan->output_buffer);
-  llmopt_hip_release_library(plan->library);
-  delete plan;
-}
-
-int llmopt_hip_prebaked_execute(llmopt_hip_prebaked *plan, int64_t token, int64_t past_tokens,
-                                int64_t checkpoint, int64_t *out_token) {
-  (void)checkpoint;  // recurrent-state checkpoints are outside this backend's scope
-  if (plan == nullptr) return fail(LLMOPT_ERR_FAILURE, "HIP prebaked plan has been finalized");
-  llmopt_hip_context *context = plan->library->context;
-  if (int status = use_device(context)) return status;
-  if (plan->token_buffer) {
-    if (plan->token_buffer->length < 8) return fail(LLMOPT_ERR_INVALID, "buffer offset out of bounds");
-    LLMOPT_HIP_TRY(hipMemcpyAsync(plan->token_buffer->device, &token, 8, hipMemcpyHostToDevice,
-                                  context->stream),
-                   "HIP could not write the decode token");
-  }
-  for (size_t i = 0; i < plan->records.size(); ++i) {
-    DispatchRecord &record = plan->records[i];
-    if (plan->is_paged_attention[i] && record.parameters.size() >= 16) {
-      const uint32_t past = (uint32_t)past_tokens;
-      memcpy(record.parameters.data() + 12, &past, 4);
-    }
-    if (int status = launch_record(context, record)) {
-      (void)hipStreamSynchronize(context->stream);
-      return status;
-    }
-  }
-  int32_t next_token = 0;
-  if (plan->output_buffer && plan->output_buffer->length >= 4) {
-    LLMOPT_HIP_TRY(hipMemcpyAsync(&next_token, plan->output_buffer->device, 4, hipMemcpyDeviceToHost,
-                                  context->stream),
-                   "HIP could not read the decode output");
-  }
-  if (hipStreamSynchronize(context->stream) != hipSuccess)
-    return fail(LLMOPT_ERR_FAILURE, "Prebaked HIP batch failed");
-  if (out_token) *out_token = (int64_t)next_token;
   return LLMOPT_OK;
 }
 

@@ -45,6 +45,14 @@ struct llmopt_hip_context : llmopt::RefCounted {
   // on the context's single stream.
   void *workspace = nullptr;
   size_t workspace_bytes = 0;
+  // Counts replacements of the workspace block: a captured graph holds the block's address and
+  // is captured again when this has moved on.
+  uint64_t workspace_generation = 0;
+  // While a retained plan captures its records the workspace cannot be replaced (nothing may be
+  // allocated, and nodes already captured hold the old address): requests beyond the block are
+  // only recorded here, the capture is thrown away, the block grown, the capture repeated.
+  bool sizing_capture = false;
+  size_t sizing_wanted = 0;
   // Arrival counters of kernels that split one output tile over several
   // workgroups; zeroed once, every kernel leaves them zero.
   uint32_t *counters = nullptr;
@@ -80,6 +88,12 @@ struct DispatchRecord {
   int64_t grid[3];
   int64_t group[3];
   bool barrier_before = false;
+  // Set by a retained plan on llmopt_attention_q8_paged_* records: the context length is read
+  // from this device word (one per sequence, all equal) instead of parameter byte 12, and the
+  // launch is sized for `device_past_capacity` tokens, so that one captured launch serves every
+  // step of a sequence.
+  const uint32_t *device_past_lengths = nullptr;
+  uint32_t device_past_capacity = 0;
 };
 
 // A kernel handler checks buffer count, parameter length and buffer sizes
@@ -127,5 +141,7 @@ int build_record(llmopt_hip_library *library, const llmopt_hip_dispatch_item *it
                  DispatchRecord *out);
 int launch_record(llmopt_hip_context *context, const DispatchRecord &record);
 void drop_record(DispatchRecord *record);
+// Makes the context's device the calling thread's current one.
+int use_device(llmopt_hip_context *context);
 
 }  // namespace llmopt

@@ -10,6 +10,12 @@ buffer order, ready for Batch.dispatch or a Prebaked plan.
 
 Sequences of a batch have their own context lengths and slot tables, which the
 batched attention / pack entry points take as two extra buffers.
+
+A step list is built once.  What changes from token to token - the input
+tokens, each sequence's context length, the slot of the new token, the rotary
+rows of the new position - lives in device buffers the kernels read, so the
+same list (or a Prebaked plan frozen from it) serves every step: `advance`
+rewrites those buffers after a step.
 """
 from __future__ import annotations
 
@@ -104,8 +110,22 @@ class DecodeStep:
     """Device buffers and the dispatch list of one decode step for `batch` sequences."""
 
     def __init__(self, runtime: Runtime, config: DecodeConfig, weights: dict, batch: int, pool: Buffer,
-                 slots: Buffer, slot_offsets, past_lengths, new_slots, positions):
+                 slots: Buffer, slot_offsets, past_lengths, new_slots, positions, max_context=None,
+                 slots_host=None, reference_entries: bool = False):
+        """max_context: the longest context any later step will have (sizes the attention launch;
+        default: the longest now).  slots_host: the host copy of the slot table, with room behind
+        every sequence's slots for the tokens `advance` will add.  reference_entries (batch 1):
+        rotation, cache pack and attention as the reference's own three kernels
+        (llmopt_rotary_qk_f16_simd_h64, llmopt_cache_pack_attention_q8_pair_simd,
+        llmopt_attention_q8_paged_simd_h64_gqa3) instead of the batched extension entries."""
         self.runtime, self.config, self.batch = runtime, config, batch
+        self.reference_entries = reference_entries
+        if reference_entries and batch != 1:
+            raise ValueError("the reference's paged attention entries share one slot table: batch 1")
+        self.host_lengths = np.asarray(past_lengths, dtype=np.uint32).copy()
+        self.host_offsets = np.asarray(slot_offsets, dtype=np.uint32).copy()
+        self.host_positions = np.asarray(positions, dtype=np.int64).copy()
+        self.slots_host = None if slots_host is None else np.asarray(slots_host, dtype=np.uint32)
         b = runtime.buffer_of_bytes
         c = config
         h = c.hidden
@@ -117,7 +137,7 @@ class DecodeStep:
         self.new_slots = b(np.asarray(new_slots, dtype=np.uint32))
         cos, sin = rope_rows(c, positions)
         self.cos, self.sin = b(cos), b(sin)
-        self.max_past = int(max(past_lengths))
+        self.max_past = int(max(past_lengths)) if max_context is None else int(max_context)
         self.device = {
             "embedding": b(weights["embedding"]),
             "final_norm": b(weights["final_norm"]),
@@ -161,22 +181,25 @@ class DecodeStep:
             out.append(("llmopt_rms_w4a16_qkv_linear_f16_g64",
                         [x_in, layer["attn_norm"], *layer["q"], *layer["k"], *layer["v"], w["q"], w["k"], w["v"]],
                         u32s(m, h, qd, kvd, kvd) + struct.pack("<f", c.epsilon), grid, group))
-            # rotation and the new token's Q8 slot in one launch (the step is bound by its launches)
-            out.append(("llmopt_rotary_qk_pack_q8_batched",
-                        [w["q"], w["k"], self.cos, self.sin, w["q_rot"], w["k_rot"], w["v"], self.new_slots,
-                         self.pool],
-                        u32s(m, 1, c.q_heads, c.kv_heads, c.head_dim, c.head_dim // 2, m) +
-                        u32s(m, key_offset, value_offset, c.kv_heads, c.head_dim, 64, c.token_elements,
-                             c.token_elements // 64, c.token_stride, m, 0),
-                        (((m * (c.q_heads + 2 * c.kv_heads) + 3) // 4) * 256, 1, 1), group))
-            attention_params = struct.pack(
-                "<12IfIII", m, c.q_heads, c.kv_heads, 0, c.head_dim, 0, 0, c.token_elements, key_offset,
-                value_offset, 64, c.token_stride, 1.0 / math.sqrt(c.head_dim), 1, 0, 0)
-            attention_params += struct.pack("<I", self.max_past)
-            out.append(("llmopt_attention_q8_paged_batched",
-                        [w["q_rot"], w["k_rot"], w["v"], self.pool, self.slots, self.slots, w["attention"],
-                         self.past_lengths, self.slot_offsets],
-                        attention_params, (((m * c.q_heads + 7) // 8) * 256, 1, 1), group))
+            if self.reference_entries:
+                out += self._reference_attention(key_offset, value_offset)
+            else:
+                # rotation and the new token's Q8 slot in one launch (the step is bound by its launches)
+                out.append(("llmopt_rotary_qk_pack_q8_batched",
+                            [w["q"], w["k"], self.cos, self.sin, w["q_rot"], w["k_rot"], w["v"], self.new_slots,
+                             self.pool],
+                            u32s(m, 1, c.q_heads, c.kv_heads, c.head_dim, c.head_dim // 2, m) +
+                            u32s(m, key_offset, value_offset, c.kv_heads, c.head_dim, 64, c.token_elements,
+                                 c.token_elements // 64, c.token_stride, m, 0),
+                            (((m * (c.q_heads + 2 * c.kv_heads) + 3) // 4) * 256, 1, 1), group))
+                attention_params = struct.pack(
+                    "<12IfIII", m, c.q_heads, c.kv_heads, 0, c.head_dim, 0, 0, c.token_elements, key_offset,
+                    value_offset, 64, c.token_stride, 1.0 / math.sqrt(c.head_dim), 1, 0, 0)
+                attention_params += struct.pack("<I", self.max_past)
+                out.append(("llmopt_attention_q8_paged_batched",
+                            [w["q_rot"], w["k_rot"], w["v"], self.pool, self.slots, self.slots, w["attention"],
+                             self.past_lengths, self.slot_offsets],
+                            attention_params, (((m * c.q_heads + 7) // 8) * 256, 1, 1), group))
             suffix, grid = self._linear_entry(h)
             out.append(("llmopt_w4a16_linear_f16_g64" + suffix,
                         [w["attention"], *layer["o"], x_in, x_mid], u32s(m, h, qd, 1, h), grid, group))
@@ -192,6 +215,56 @@ class DecodeStep:
                     [w["x"][0], self.device["final_norm"], *self.device["lm_head"], self.token_ids],
                     u32s(m, c.vocabulary, h) + struct.pack("<f", c.epsilon), (m * 256, 1, 1), group))
         return out
+
+    def _reference_attention(self, key_offset: int, value_offset: int) -> list[tuple]:
+        """One sequence through the reference's own kernels: RotaryQKParams (lib/metal_parameters.ml),
+        AttentionCachePairParams and Q8PagedAttentionParams (lib/metal_cache_source.ml:22-34,352-369).
+        The context length at parameter byte 12 is what a Prebaked plan patches per step."""
+        c, w = self.config, self.work
+        group = (256, 1, 1)
+        rows = c.q_heads + 2 * c.kv_heads
+        attention_params = struct.pack(
+            "<12IfIII", 1, c.q_heads, c.kv_heads, int(self.host_lengths[0]), c.head_dim, 0, 0, c.token_elements,
+            key_offset, value_offset, 64, c.token_stride, 1.0 / math.sqrt(c.head_dim), 1, 0, 0)
+        name = "llmopt_attention_q8_paged_simd_h64_gqa3" if (c.head_dim, c.q_heads // c.kv_heads) == (64, 3) \
+            else "llmopt_attention_q8_paged_simd_generic"
+        return [
+            ("llmopt_rotary_qk_f16_simd_h64", [w["q"], w["k"], self.cos, self.sin, w["q_rot"], w["k_rot"]],
+             u32s(1, 1, c.q_heads, c.kv_heads, c.head_dim, c.head_dim // 2, 1), (((rows + 3) // 4) * 256, 1, 1), group),
+            ("llmopt_cache_pack_attention_q8_pair_simd", [w["k_rot"], w["v"], self.new_slots, self.pool],
+             u32s(1, key_offset, value_offset, c.kv_heads, c.head_dim, 64, c.token_elements, c.token_elements // 64,
+                  c.token_stride, 1, 0), (c.kv_heads * (c.head_dim // 64) * 64, 1, 1), (64, 1, 1)),
+            (name,
+             [w["q_rot"], w["k_rot"], w["v"], self.pool, self.slots, self.slots, w["attention"]],
+             attention_params, (((c.q_heads + 7) // 8) * 256, 1, 1), group),
+        ]
+
+    def set_reference_past(self, past_tokens: int) -> None:
+        """Host-side patch of the context length (parameter byte 12) for eager runs of a reference_entries list."""
+        patched = []
+        for name, buffers, parameters, grid, group in self.dispatches:
+            if name.startswith("llmopt_attention_q8_paged_simd"):
+                parameters = parameters[:12] + struct.pack("<I", past_tokens) + parameters[16:]
+            patched.append((name, buffers, parameters, grid, group))
+        self.dispatches = patched
+
+    def advance(self) -> None:
+        """After a step: every sequence is one token longer.  Rewrites the device buffers the next
+        step reads - context lengths, the new token's slot (the next entry of the sequence's slot
+        table) and the rotary rows of the next position."""
+        if self.slots_host is None:
+            raise ValueError("advance needs the host copy of the slot table")
+        self.host_lengths += 1
+        self.host_positions += 1
+        if int(self.host_lengths.max()) > self.max_past:
+            raise ValueError("context grew beyond max_context")
+        self.past_lengths.write(self.host_lengths)
+        self.new_slots.write(self.slots_host[self.host_offsets + self.host_lengths])
+        cos, sin = rope_rows(self.config, self.host_positions)
+        self.cos.write(cos)
+        self.sin.write(sin)
+        if self.reference_entries:
+            self.set_reference_past(int(self.host_lengths[0]))
 
     def record(self, batch) -> None:
         for name, buffers, parameters, grid, group in self.dispatches:

@@ -41,6 +41,10 @@ class DispatchItem(ctypes.Structure):
     ]
 
 
+# llmopt_hip_ring_step: int (*)(void *user, int64 token, int64 past_tokens, int32 *out_token)
+RING_STEP = ctypes.CFUNCTYPE(ctypes.c_int, ctypes.c_void_p, ctypes.c_int64, ctypes.c_int64,
+                             ctypes.POINTER(ctypes.c_int32))
+
 _lib: Optional[ctypes.CDLL] = None
 
 
@@ -102,6 +106,16 @@ def lib() -> ctypes.CDLL:
         "llmopt_hip_prebaked_create": (ctypes.c_int, [vp, item_p, sz, vp, vp, pp]),
         "llmopt_hip_release_prebaked": (None, [vp]),
         "llmopt_hip_prebaked_execute": (ctypes.c_int, [vp, i64, i64, i64, ctypes.POINTER(i64)]),
+        "llmopt_hip_prebaked_is_single_submission": (ctypes.c_int, [vp]),
+        "llmopt_hip_ring_create": (ctypes.c_int, [pp]),
+        "llmopt_hip_ring_submit": (ctypes.c_int, [vp, i64, i64, i64, i64]),
+        "llmopt_hip_ring_wait_completion": (ctypes.c_int, [vp, ctypes.POINTER(i64), ctypes.POINTER(i64),
+                                                           ctypes.POINTER(i64)]),
+        "llmopt_hip_ring_poll_completion": (ctypes.c_int, [vp, ctypes.POINTER(i64), ctypes.POINTER(i64),
+                                                           ctypes.POINTER(i64)]),
+        "llmopt_hip_ring_start_worker": (ctypes.c_int, [vp, vp, item_p, sz, vp, vp]),
+        "llmopt_hip_ring_start_worker_with": (ctypes.c_int, [vp, RING_STEP, vp]),
+        "llmopt_hip_ring_destroy": (None, [vp]),
         "llmopt_hip_attention_q8_paged_no_alloc": (ctypes.c_int, [vp, vp, vp, vp, vp, vp, sz, vp, sz, vp]),
     }
     for name, (restype, argtypes) in signatures.items():
@@ -129,6 +143,10 @@ EXPORTED_SYMBOLS = (
     "llmopt_hip_commit_batch", "llmopt_hip_commit_batch_async",
     "llmopt_hip_commit_batch_profiled", "llmopt_hip_abort_batch",
     "llmopt_hip_prebaked_create", "llmopt_hip_release_prebaked", "llmopt_hip_prebaked_execute",
+    "llmopt_hip_prebaked_is_single_submission",
+    "llmopt_hip_ring_create", "llmopt_hip_ring_submit", "llmopt_hip_ring_wait_completion",
+    "llmopt_hip_ring_poll_completion", "llmopt_hip_ring_start_worker", "llmopt_hip_ring_start_worker_with",
+    "llmopt_hip_ring_destroy",
     "llmopt_hip_attention_q8_paged_no_alloc",
 )
 
@@ -414,3 +432,78 @@ class Prebaked:
         _check(lib().llmopt_hip_prebaked_execute(self._handle, token, past_tokens, checkpoint,
                                                  ctypes.byref(out)))
         return int(out.value)
+
+    @property
+    def single_submission(self) -> bool:
+        """True when a step replays one HIP graph."""
+        status = lib().llmopt_hip_prebaked_is_single_submission(self._handle)
+        _check(status)
+        return status == 1
+
+
+def _make_items(dispatches):
+    dispatches = list(dispatches)
+    items = (DispatchItem * max(1, len(dispatches)))()
+    keep = []
+    for index, (name, buffers, parameters, grid, group) in enumerate(dispatches):
+        item, alive = _make_item(name, buffers, parameters, grid, group)
+        items[index] = item
+        keep.append(alive)
+    return items, len(dispatches), keep
+
+
+class Ring:
+    """Submission / completion queues with one worker thread (Metal_native.Ring,
+    lib/metal_native.ml:404-437)."""
+
+    def __init__(self):
+        self._handle = ctypes.c_void_p()
+        self._callback = None
+        _check(lib().llmopt_hip_ring_create(ctypes.byref(self._handle)))
+
+    def submit(self, request_id: int, token: int, past_tokens: int, flags: int = 0) -> bool:
+        status = lib().llmopt_hip_ring_submit(self._handle, request_id, token, past_tokens, flags)
+        _check(status)
+        return status == 1
+
+    def wait_completion(self) -> tuple[int, int, int]:
+        request, token, status = ctypes.c_int64(), ctypes.c_int64(), ctypes.c_int64()
+        _check(lib().llmopt_hip_ring_wait_completion(self._handle, ctypes.byref(request), ctypes.byref(token),
+                                                     ctypes.byref(status)))
+        return int(request.value), int(token.value), int(status.value)
+
+    def poll_completion(self) -> Optional[tuple[int, int, int]]:
+        request, token, status = ctypes.c_int64(), ctypes.c_int64(), ctypes.c_int64()
+        found = lib().llmopt_hip_ring_poll_completion(self._handle, ctypes.byref(request), ctypes.byref(token),
+                                                      ctypes.byref(status))
+        _check(found)
+        return (int(request.value), int(token.value), int(status.value)) if found == 1 else None
+
+    def start_worker(self, runtime: Runtime, dispatches: Iterable[tuple], token_buffer: Buffer,
+                     output_buffer: Buffer) -> None:
+        items, count, keep = _make_items(dispatches)
+        _check(lib().llmopt_hip_ring_start_worker(self._handle, runtime.library, items, count,
+                                                  token_buffer.handle, output_buffer.handle))
+        del keep
+
+    def start_worker_with(self, step) -> None:
+        """`step(token, past_tokens) -> produced token` runs on the worker thread; an exception fails the step."""
+        def trampoline(_user, token, past_tokens, out_token):
+            try:
+                out_token[0] = int(step(int(token), int(past_tokens)))
+                return 0
+            except Exception:
+                return -1
+        self._callback = RING_STEP(trampoline)
+        _check(lib().llmopt_hip_ring_start_worker_with(self._handle, self._callback, None))
+
+    def destroy(self) -> None:
+        if self._handle:
+            lib().llmopt_hip_ring_destroy(self._handle)
+            self._handle = ctypes.c_void_p()
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass

@@ -1,0 +1,185 @@
+"""Retained decode plans (llmopt_hip_prebaked_*) and the ring worker over one: several consecutive
+tokens through the frozen dispatch array against the same steps launched eagerly, and against the
+CPU oracle chain."""
+import numpy as np
+import pytest
+
+from tests.gpu_util import assert_close_to_oracle
+from tests.test_gpu_decode_step import oracle_step
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def runtime():
+    from llmopt_amd.native import Runtime
+    rt = Runtime()
+    yield rt
+    rt.close()
+
+
+def make_case(rng, config, lengths, room):
+    """A pool with every sequence's context, and a slot table with `room` free slots behind each
+    sequence's own (the slots its next tokens will take)."""
+    batch = len(lengths)
+    spans = [length + room for length in lengths]
+    capacity = sum(spans) + 3
+    order = rng.permutation(capacity).astype(np.uint32)
+    offsets = np.concatenate([[0], np.cumsum(spans)[:-1]]).astype(np.uint32)
+    slots = order[:sum(spans)]
+    stride, elements = config.token_stride, config.token_elements
+    pool = np.zeros((capacity, stride), dtype=np.uint8)
+    pool[:, :elements] = np.clip(np.rint(rng.standard_normal((capacity, elements)) * 38), -127, 127) \
+        .astype(np.int8).view(np.uint8)
+    pool[:, elements:] = rng.uniform(0.02, 0.035, (capacity, elements // 64)).astype(np.float16) \
+        .view(np.uint8).reshape(capacity, -1)
+    new_slots = slots[offsets + np.asarray(lengths, dtype=np.uint32)]
+    return pool.reshape(-1), slots, offsets, new_slots, capacity, batch
+
+
+def build_step(runtime, config, weights, case, lengths, room, **kwargs):
+    from llmopt_amd.decode_step import DecodeStep
+    pool, slots, offsets, new_slots, capacity, batch = case
+    device_pool = runtime.buffer_of_bytes(pool)
+    step = DecodeStep(runtime, config, weights, batch, device_pool, runtime.buffer_of_bytes(slots), offsets, lengths,
+                      new_slots, lengths, max_context=max(lengths) + room, slots_host=slots, **kwargs)
+    return step, device_pool
+
+
+def test_prebaked_plan_advances_a_batch_like_eager_steps(runtime):
+    """The decode step's own dispatch list (batched extension entries: lengths, slots and rotary
+    rows in device buffers) frozen into a plan: five tokens through llmopt_hip_prebaked_execute
+    leave the same tokens, hidden states and pool bytes as five eager steps - bit for bit, the
+    kernels and their launch geometry being the same."""
+    from llmopt_amd.decode_step import DecodeConfig, random_weights
+    from llmopt_amd.native import Prebaked
+    rng = np.random.default_rng(91)
+    config = DecodeConfig(layers=2, vocabulary=1000)
+    weights = random_weights(config, rng)
+    lengths, room, steps = [64, 5, 300], 8, 5
+    case = make_case(rng, config, lengths, room)
+    eager, eager_pool = build_step(runtime, config, weights, case, lengths, room)
+    frozen, frozen_pool = build_step(runtime, config, weights, case, lengths, room)
+    plan = Prebaked(runtime, frozen.dispatches, frozen.tokens, frozen.token_ids)
+    assert plan.single_submission
+    tokens = rng.integers(0, config.vocabulary, len(lengths))
+    plan_tokens = tokens.copy()
+    for index in range(steps):
+        print(f"prebaked batch step {index}", flush=True)
+        want = eager.run(tokens)
+        frozen.tokens.write(np.asarray(plan_tokens, dtype=np.int64))
+        first = plan.execute(int(plan_tokens[0]), int(frozen.host_lengths[0]))
+        got = frozen.token_ids.numpy(np.uint32, (len(lengths),))
+        assert first == int(got[0])
+        np.testing.assert_array_equal(got, want, err_msg=f"tokens of step {index}")
+        np.testing.assert_array_equal(frozen.work["x"][0].numpy(np.uint16), eager.work["x"][0].numpy(np.uint16),
+                                      err_msg=f"hidden state of step {index}")
+        np.testing.assert_array_equal(frozen_pool.numpy(np.uint8), eager_pool.numpy(np.uint8),
+                                      err_msg=f"pool after step {index}")
+        tokens, plan_tokens = want.astype(np.int64), got.astype(np.int64)
+        eager.advance()
+        frozen.advance()
+    # the new tokens did land: every step changed exactly one slot per sequence
+    changed = np.flatnonzero((frozen_pool.numpy(np.uint8).reshape(case[4], -1) !=
+                              case[0].reshape(case[4], -1)).any(axis=1))
+    assert len(changed) == steps * len(lengths)
+
+
+@pytest.mark.parametrize("first_past", [37, 0])
+def test_prebaked_plan_patches_the_reference_attention_entries(runtime, first_past):
+    """One sequence through the reference's own kernel names: the plan owns the context length
+    (llmopt_hip_prebaked_execute's past_tokens, the reference's patch of parameter byte 12).  Four
+    consecutive tokens against the CPU oracle chain and against eager launches with the byte patched
+    by the host (those size the attention launch for the context, the plan for the slot table's
+    capacity: same results up to the order of float32 sums)."""
+    from llmopt_amd.decode_step import DecodeConfig, random_weights
+    from llmopt_amd.native import Prebaked
+    rng = np.random.default_rng(17 + first_past)
+    config = DecodeConfig(layers=2, vocabulary=1000)
+    weights = random_weights(config, rng)
+    lengths, room, steps = [first_past], 70, 4
+    case = make_case(rng, config, lengths, room)
+    eager, eager_pool = build_step(runtime, config, weights, case, lengths, room, reference_entries=True)
+    frozen, frozen_pool = build_step(runtime, config, weights, case, lengths, room, reference_entries=True)
+    plan = Prebaked(runtime, frozen.dispatches, frozen.tokens, frozen.token_ids)
+    assert plan.single_submission
+    pool_host, slots, offsets, _, capacity, _ = case
+    oracle_pool = pool_host.copy()
+    token = int(rng.integers(0, config.vocabulary))
+    for index in range(steps):
+        past = first_past + index
+        print(f"prebaked reference-entry step {index} past {past}", flush=True)
+        want_token = int(eager.run([token])[0])
+        got_token = plan.execute(token, past)
+        got_hidden = frozen.work["x"][0].numpy(np.float16, (1, config.hidden))
+        hidden, logits, oracle_pool = oracle_step(config, weights, oracle_pool, slots, offsets, [past],
+                                                  [int(slots[past])], [past], [token])
+        assert_close_to_oracle(got_hidden, hidden, f"hidden state of step {index}", rel_l2_tol=4e-3)
+        assert_close_to_oracle(got_hidden, eager.work["x"][0].numpy(np.float16, (1, config.hidden)),
+                               f"plan against eager, step {index}", rel_l2_tol=2e-3)
+        rms = float(np.sqrt(np.mean(logits.astype(np.float64) ** 2)))
+        assert float(logits[0, got_token]) >= float(logits[0].max()) - 2e-2 * rms
+        assert got_token == want_token
+        stride, elements = config.token_stride, config.token_elements
+        got_slot = frozen_pool.numpy(np.uint8).reshape(capacity, stride)[int(slots[past])]
+        want_slot = oracle_pool.reshape(capacity, stride)[int(slots[past])]
+        assert np.abs(got_slot[:elements].view(np.int8).astype(np.int32) -
+                      want_slot[:elements].view(np.int8).astype(np.int32)).max() <= 1
+        # the oracle continues from the GPU's own cache contents, so that one quantum of difference
+        # in a stored key does not grow into a different continuation
+        oracle_pool = frozen_pool.numpy(np.uint8)
+        frozen_pool.copy_to(eager_pool)
+        token = got_token
+        eager.advance()
+        frozen.advance()
+    with pytest.raises(Exception) as error:
+        plan.execute(token, first_past + room + 1000)
+    assert "context tokens" in str(error.value)
+
+
+def markov_plan(runtime, rng, vocabulary=512, hidden=576):
+    """token -> embedding row -> LM-head argmax: a plan whose output token is a function of its input."""
+    from llmopt_amd.decode_step import random_w4, u32s
+    import struct
+    embedding = (rng.standard_normal((vocabulary, hidden)) * 0.5).astype(np.float16)
+    norm = rng.uniform(0.5, 1.5, hidden).astype(np.float16)
+    head_w, head_s = random_w4(rng, vocabulary, hidden)
+    b = runtime.buffer_of_bytes
+    tokens, token_ids = b(np.zeros(1, dtype=np.int64)), b(np.zeros(1, dtype=np.uint32))
+    x = runtime.create_buffer(hidden * 2)
+    dispatches = [
+        ("llmopt_embedding_f16", [tokens, b(embedding), x], u32s(1, vocabulary, hidden), (((hidden + 255) // 256) * 256, 1, 1),
+         (256, 1, 1)),
+        ("llmopt_w4a16_lm_head_argmax_f16", [x, b(norm), b(head_w), b(head_s), token_ids],
+         u32s(1, vocabulary, hidden) + struct.pack("<f", 1e-5), (256, 1, 1), (256, 1, 1)),
+    ]
+    return dispatches, tokens, token_ids
+
+
+@pytest.mark.parametrize("depth", ["1", "2"])
+def test_ring_worker_runs_chained_steps_of_a_plan(runtime, depth, monkeypatch):
+    from llmopt_amd.native import Prebaked, Ring
+    monkeypatch.setenv("LLMOPT_QUEUE_DEPTH", depth)
+    rng = np.random.default_rng(5)
+    dispatches, tokens, token_ids = markov_plan(runtime, rng)
+    # what the chain must produce: the same plan, one token at a time
+    plan = Prebaked(runtime, dispatches, tokens, token_ids)
+    expected, token = [], 5
+    for _ in range(12):
+        token = plan.execute(token, 0)
+        expected.append(token)
+    assert len(set(expected)) > 3  # not a fixed point: the chain really feeds tokens back
+    del plan
+    ring = Ring()
+    ring.start_worker(runtime, dispatches, tokens, token_ids)
+    assert ring.submit(100, 5, 0)
+    for request in range(1, 12):
+        assert ring.submit(100 + request, -1, request)  # chained: input = the previous output, on the GPU
+    done = [ring.wait_completion() for _ in range(12)]
+    assert [d[0] for d in done] == [100 + r for r in range(12)]
+    assert [d[1] for d in done] == expected
+    assert all(d[2] == 0 for d in done)
+    # an explicit token restarts the chain
+    ring.submit(7, 5, 0)
+    assert ring.wait_completion() == (7, expected[0], 0)
+    ring.destroy()
