@@ -207,6 +207,12 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemv_kernel(GemvParams p) {
   static_assert(kXAhead == 8, "the wait below names eight registers");
   const uint32_t vectors_per_row = chunks * 256;  // includes zero padding
   const uint32_t x_vectors = (uint32_t)M * vectors_per_row;  // a multiple of kThreads
+  // The staging below walks x_vectors in steps of kThreads and stores without a bound of its own:
+  // only a block size that divides the 256 vectors of a chunk keeps every index inside the LDS
+  // block (a 1024-thread block overruns it whenever rows x chunks is not a multiple of four;
+  // tests/test_gemv_index_bounds.py enumerates both).
+  static_assert(256 % kThreads == 0, "the activation staging needs a block size that divides 256");
+  static_assert(kXAhead * kThreads >= 256, "the vectors requested ahead cover at least one chunk of one row");
   constexpr int XA = D > 0 ? kXAhead : 1;
   u32x4_t x_ahead[XA];
   auto x_source = [&](uint32_t i, bool &valid) {
