@@ -40,6 +40,9 @@ struct W4LinearArgs {
 
 // Bytes of workspace the decode path wants for this shape (0 when it does not split K).
 size_t w4a16_gemv_workspace_bytes(uint32_t m, uint32_t n, uint32_t k);
+// The same for the prefill GEMM (m > kGemvMaxRows), which splits K over workgroups when its
+// tiles would leave half the CUs idle; without the workspace and the counters it does not split.
+size_t w4a16_gemm_workspace_bytes(uint32_t m, uint32_t n, uint32_t k);
 
 // Optional RMS normalisation of the activation rows on their way into a decode kernel
 // (weight == nullptr: none): the kernel multiplies by half(x * gain * r) (weight_first) or

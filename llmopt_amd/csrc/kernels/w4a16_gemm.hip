@@ -42,6 +42,12 @@ struct GemmParams {
   uint16_t *y;
   uint32_t m, n, k;
   uint32_t tiles_m, tiles_n;
+  // K split over blockIdx.y (SPLITK instantiations): every workgroup covers k_len of K, leaves
+  // its tile's float32 sums in partials[split][tile], and the last one to arrive at a tile (one
+  // counter per tile, zero between launches) adds the splits in order and stores the output.
+  uint32_t k_len;
+  float *partials;
+  uint32_t *counters;
 };
 
 __device__ __forceinline__ f16x_t zero_tile() {
@@ -58,9 +64,10 @@ __device__ __forceinline__ f16x_t zero_tile() {
 // register sets.  2 for the large tiles, whose steps are long enough to cover a load; 4 (K a
 // multiple of 4 steps) for the small ones, whose steps are shorter than the trip to memory:
 // the activation copy then runs three steps ahead of its use and the weights four.
-template <int WM, int WN, bool DUAL, int XS>
+template <int WM, int WN, bool DUAL, int XS, bool SPLITK = false>
 __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
   static_assert(XS == 2 || XS == 4, "the weight stage alternates with the step: an even unroll");
+  static_assert(!SPLITK || !DUAL, "silu(gate) * up is not linear in the K ranges");
   constexpr int WS = XS;            // weight register sets
   constexpr int NW = DUAL ? 2 : 1;  // weight matrices per tile
   constexpr int BM = 4 * WM * 32;
@@ -94,7 +101,9 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
   const uint32_t tile_n = logical / p.tiles_m;
   const uint32_t m0 = tile_m * BM;
   const uint32_t n0 = tile_n * BN;
-  const uint32_t K = p.k;
+  const uint32_t K = p.k;                                   // row stride of x and of the weights
+  const uint32_t KS = SPLITK ? p.k_len : p.k;               // this workgroup's extent of K ...
+  const uint32_t k_base = SPLITK ? blockIdx.y * p.k_len : 0;  // ... and where it begins
 
   // Activations go global -> LDS directly, 8 rows (1 KiB) per wave-wide load:
   // lane l fills physical vector l % 8 of row l / 8, i.e. fetches the logical
@@ -105,7 +114,7 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
     const uint32_t tile_row = (wave * X_CHUNKS + c) * 8 + (lane >> 3);
     const uint32_t vec = (lane & 7) ^ ((tile_row >> 1) & 7u);
     const uint32_t row = min(m0 + tile_row, p.m - 1);  // rows past m are never stored
-    x_src[c] = p.x + (size_t)row * K + vec * 8;
+    x_src[c] = p.x + (size_t)row * K + k_base + vec * 8;
   }
   // Every vector memory load of the K loop is issued as assembly and waited for
   // by hand: loads return in order, so "at most n outstanding" names exactly
@@ -146,8 +155,8 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
   auto fetch_w = [&](Fetched &f, uint32_t k0) __attribute__((always_inline)) {
 #pragma unroll
     for (int v = 0; v < NW; ++v) {
-      const void *w_src = p.w[v] + (size_t)w_col * (K >> 1) + (k0 >> 1) + w_half * 16;
-      const void *s_src = p.s[v] + (size_t)w_col * (K >> 6) + (k0 >> 6);
+      const void *w_src = p.w[v] + (size_t)w_col * (K >> 1) + ((k_base + k0) >> 1) + w_half * 16;
+      const void *s_src = p.s[v] + (size_t)w_col * (K >> 6) + ((k_base + k0) >> 6);
       asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(f.w[v]) : "v"(w_src) : "memory");
       asm volatile("global_load_ushort %0, %1, off" : "=&v"(f.s[v]) : "v"(s_src) : "memory");
     }
@@ -256,11 +265,11 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
         for (int n = 0; n < ITEMS_PER_GROUP; ++n)
           if (group * ITEMS_PER_GROUP + n < ITEMS)
             store_item(fetched[next_set], stage ^ 1, group * ITEMS_PER_GROUP + n);
-        if (group == 0) fetch_x(min(k0 + (XS - 1) * BK, K - BK), (j + XS - 1) % XS);
+        if (group == 0) fetch_x(min(k0 + (XS - 1) * BK, KS - BK), (j + XS - 1) % XS);
         __builtin_amdgcn_sched_barrier(0);
       }
     }
-    fetch_w(fetched[next_set], min(k0 + (1 + WS) * BK, K - BK));
+    fetch_w(fetched[next_set], min(k0 + (1 + WS) * BK, KS - BK));
     __builtin_amdgcn_sched_barrier(0);
     // the activation copy of step i + 1 has landed: it went out in step i + 2 - XS, before
     // that step's weight loads and the XS - 2 steps of loads since
@@ -268,21 +277,21 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
   };
 
 #pragma unroll
-  for (int s = 0; s < XS - 1; ++s) fetch_x(min((uint32_t)s * BK, K - BK), s);
+  for (int s = 0; s < XS - 1; ++s) fetch_x(min((uint32_t)s * BK, KS - BK), s);
 #pragma unroll
-  for (int s = 0; s < WS; ++s) fetch_w(fetched[s], min((uint32_t)s * BK, K - BK));
+  for (int s = 0; s < WS; ++s) fetch_w(fetched[s], min((uint32_t)s * BK, KS - BK));
   wait_w(fetched[0], std::integral_constant<int, (WS - 1) * W_LOADS>{});
 #pragma unroll
   for (int item = 0; item < ITEMS; ++item) store_item(fetched[0], 0, item);
-  fetch_w(fetched[0], min((uint32_t)WS * BK, K - BK));
+  fetch_w(fetched[0], min((uint32_t)WS * BK, KS - BK));
   if constexpr (XS == 2) {
-    for (uint32_t k0 = 0; k0 < K; k0 += 2 * BK) {
+    for (uint32_t k0 = 0; k0 < KS; k0 += 2 * BK) {
       step(k0, std::integral_constant<int, 0>{});
-      if (k0 + BK < K) step(k0 + BK, std::integral_constant<int, 1>{});
+      if (k0 + BK < KS) step(k0 + BK, std::integral_constant<int, 1>{});
     }
   } else {  // K is a multiple of XS steps: no branch between a request and its wait
     wait_all(std::integral_constant<int, W_LOADS>{});  // every activation copy and every other set has landed
-    for (uint32_t k0 = 0; k0 < K; k0 += XS * BK) {
+    for (uint32_t k0 = 0; k0 < KS; k0 += XS * BK) {
       step(k0, std::integral_constant<int, 0>{});
       step(k0 + BK, std::integral_constant<int, 1>{});
       step(k0 + 2 * BK, std::integral_constant<int, 2>{});
@@ -291,6 +300,70 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
   }
   wait_all(std::integral_constant<int, 0>{});  // the surplus requests still target live registers
 
+  if constexpr (SPLITK) {
+    // Hand-over between the workgroups of a tile through memory every CU sees: device-scope
+    // 16-byte stores and loads (no cache write-back, no per-element atomics).  A partial tile is
+    // kept in the accumulators' own layout - [wave][a][b][i / 4][lane] float4 - so a lane reads
+    // back exactly the registers its counterpart wrote, one coalesced KiB per wave instruction.
+    // One arrival per workgroup; the last to arrive adds the splits in split order, its own sums
+    // taking their place in that order: the same result whichever arrives last.
+    __shared__ uint32_t arrival_lds;
+    constexpr uint32_t kTileFloats = (uint32_t)BM * BN;
+    constexpr int QUADS = WM * WN * 4;  // float4 groups per lane
+    const size_t tile_count = (size_t)p.tiles_m * p.tiles_n;
+    auto quad_address = [&](uint32_t split, int quad) __attribute__((always_inline)) {
+      return p.partials + ((split * tile_count + logical) * kTileFloats) + ((size_t)(wave * QUADS + quad) * 64 + lane) * 4;
+    };
+#pragma unroll
+    for (int b = 0; b < WN; ++b)
+#pragma unroll
+      for (int a = 0; a < WM; ++a)
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const f4_t value = {acc[0][a][b][g * 4], acc[0][a][b][g * 4 + 1], acc[0][a][b][g * 4 + 2], acc[0][a][b][g * 4 + 3]};
+          asm volatile("global_store_dwordx4 %0, %1, off sc1" : : "v"(quad_address(blockIdx.y, (b * WM + a) * 4 + g)), "v"(value) : "memory");
+        }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();  // every wave's stores have been acknowledged
+    if (tid == 0) {
+      const uint32_t arrived = __hip_atomic_fetch_add(p.counters + logical, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      const bool last = arrived == gridDim.y - 1;
+      if (last) __hip_atomic_store(p.counters + logical, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      arrival_lds = last ? 1u : 0u;
+    }
+    __syncthreads();
+    if (arrival_lds == 0) return;
+    f4_t sum[QUADS];
+#pragma unroll
+    for (int q = 0; q < QUADS; ++q) sum[q] = f4_t{0.f, 0.f, 0.f, 0.f};
+    for (uint32_t split = 0; split < gridDim.y; ++split) {
+      if (split == blockIdx.y) {
+#pragma unroll
+        for (int b = 0; b < WN; ++b)
+#pragma unroll
+          for (int a = 0; a < WM; ++a)
+#pragma unroll
+            for (int g = 0; g < 4; ++g)
+#pragma unroll
+              for (int e = 0; e < 4; ++e) sum[(b * WM + a) * 4 + g][e] += acc[0][a][b][g * 4 + e];
+      } else {
+        f4_t other[QUADS];
+#pragma unroll
+        for (int q = 0; q < QUADS; ++q)
+          asm volatile("global_load_dwordx4 %0, %1, off sc1" : "=&v"(other[q]) : "v"(quad_address(split, q)) : "memory");
+#pragma unroll
+        for (int q = 0; q < QUADS; ++q) asm volatile("s_waitcnt vmcnt(0)" : "+v"(other[q]) : : "memory");
+#pragma unroll
+        for (int q = 0; q < QUADS; ++q) sum[q] += other[q];
+      }
+    }
+#pragma unroll
+    for (int b = 0; b < WN; ++b)
+#pragma unroll
+      for (int a = 0; a < WM; ++a)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[0][a][b][i] = sum[(b * WM + a) * 4 + i / 4][i % 4];
+  }
   // epilogue: lane owns column col, rows (i/4)*8 + (lane/32)*4 + i%4 of each tile
 #pragma unroll
   for (int b = 0; b < WN; ++b) {
@@ -318,8 +391,8 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
   }
 }
 
-template <int WM, int WN, bool DUAL, int XS = 2>
-hipError_t launch_tile(GemmParams &p, hipStream_t stream) {
+template <int WM, int WN, bool DUAL, int XS = 2, bool SPLITK = false>
+hipError_t launch_tile(GemmParams &p, hipStream_t stream, uint32_t splits = 1) {
   constexpr int NW = DUAL ? 2 : 1;
   constexpr int BM = 4 * WM * 32;
   constexpr int BN = 2 * WN * 32;
@@ -327,7 +400,7 @@ hipError_t launch_tile(GemmParams &p, hipStream_t stream) {
   static_assert(lds_bytes <= 160 * 1024, "a workgroup's stages must fit the CU's LDS");
   static bool configured = false;
   if (!configured) {
-    hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(&w4a16_gemm_kernel<WM, WN, DUAL, XS>),
+    hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(&w4a16_gemm_kernel<WM, WN, DUAL, XS, SPLITK>),
                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
     if (status != hipSuccess) return status;
     configured = true;
@@ -335,8 +408,21 @@ hipError_t launch_tile(GemmParams &p, hipStream_t stream) {
   p.tiles_m = (p.m + BM - 1) / BM;
   p.tiles_n = (p.n + BN - 1) / BN;
   const uint32_t blocks = p.tiles_m * p.tiles_n;
-  hipLaunchKernelGGL((w4a16_gemm_kernel<WM, WN, DUAL, XS>), dim3(blocks), dim3(kThreads), lds_bytes, stream, p);
+  p.k_len = p.k / splits;
+  hipLaunchKernelGGL((w4a16_gemm_kernel<WM, WN, DUAL, XS, SPLITK>), dim3(blocks, splits), dim3(kThreads), lds_bytes,
+                     stream, p);
   return hipGetLastError();
+}
+
+// K ranges per tile when 128 x 128 tiles leave at least half the CUs without one (1: no split):
+// as many as fill the device, each a whole number of four-step loop passes.
+uint32_t gemm_k_splits(uint32_t m, uint32_t n, uint32_t k) {
+  const uint64_t tiles = (uint64_t)((m + 127) / 128) * ((n + 127) / 128);
+  const uint64_t cus = (uint64_t)device_compute_units();
+  if (tiles == 0 || tiles * 2 > cus) return 1;
+  uint32_t splits = (uint32_t)std::min<uint64_t>(4, cus / tiles);
+  while (splits > 1 && (k % splits != 0 || (k / splits) % (4 * BK) != 0)) --splits;
+  return splits;
 }
 
 template <bool DUAL>
@@ -354,6 +440,11 @@ hipError_t launch_gemm(GemmParams &p, hipStream_t stream) {
   // activation stages do (K a whole number of four steps; measured 58 -> 49 us at 512 x 4096 x 4096,
   // and nothing for the 128 x 256 tiles, which stay with two).
   const uint64_t small = (uint64_t)((p.m + 127) / 128) * ((p.n + 127) / 128);
+  // Fewer tiles than half the CUs: K is split over workgroups as well, so that every CU holds a
+  // tile (128 tiles at 512 x 4096 x 4096 left half the device idle).
+  const uint32_t splits = gemm_k_splits(p.m, p.n, p.k);
+  if (splits > 1 && p.partials != nullptr && p.counters != nullptr)
+    return launch_tile<1, 2, false, 4, true>(p, stream, splits);
   if (p.k % (4 * BK) == 0 && small <= (uint64_t)cus) return launch_tile<1, 2, false, 4>(p, stream);
   return launch_tile<1, 2, false>(p, stream);
 }
@@ -374,7 +465,19 @@ hipError_t launch_w4a16_gemm_linear(const W4LinearArgs &a, hipStream_t stream) {
   p.m = a.m;
   p.n = a.n;
   p.k = a.k;
+  const uint64_t tiles = (uint64_t)((a.m + 127) / 128) * ((a.n + 127) / 128);
+  if (a.workspace != nullptr && a.counters != nullptr && tiles <= a.counter_count &&
+      a.workspace_bytes >= w4a16_gemm_workspace_bytes(a.m, a.n, a.k)) {
+    p.partials = static_cast<float *>(a.workspace);
+    p.counters = a.counters;
+  }
   return launch_gemm<false>(p, stream);
+}
+
+size_t w4a16_gemm_workspace_bytes(uint32_t m, uint32_t n, uint32_t k) {
+  const uint32_t splits = gemm_k_splits(m, n, k);
+  const size_t tiles = (size_t)((m + 127) / 128) * ((n + 127) / 128);  // whole 128 x 128 tiles of float32
+  return splits > 1 ? (size_t)splits * tiles * 128 * 128 * sizeof(float) : 0;
 }
 
 hipError_t launch_w4a16_gemm_dual_swiglu(const W4DualSwigluArgs &a, hipStream_t stream) {

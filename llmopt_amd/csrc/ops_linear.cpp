@@ -39,8 +39,8 @@ int launched(hipError_t status, const char *name) {
 // Scratch for the decode path when it splits K over workgroups (m x k beyond
 // the LDS budget); none is needed for most shapes.
 int attach_linear_scratch(llmopt_hip_context *context, W4LinearArgs *args) {
-  if (args->m > kGemvMaxRows) return LLMOPT_OK;
-  const size_t bytes = w4a16_gemv_workspace_bytes(args->m, args->n, args->k);
+  const size_t bytes = args->m > kGemvMaxRows ? w4a16_gemm_workspace_bytes(args->m, args->n, args->k)
+                                              : w4a16_gemv_workspace_bytes(args->m, args->n, args->k);
   if (bytes == 0) return LLMOPT_OK;
   args->workspace = context_workspace(context, bytes);
   if (args->workspace == nullptr) return LLMOPT_ERR_FAILURE;

@@ -106,6 +106,7 @@ float param_f32(const DispatchRecord &record, size_t byte_offset) {
 }
 
 void *context_workspace(llmopt_hip_context *context, size_t bytes) {
+  context->scratch_touched = true;
   if (bytes <= context->workspace_bytes) return context->workspace;
   if (context->sizing_capture) {
     // the launch being captured is never run: any non-null address will do
@@ -135,6 +136,7 @@ void *context_workspace(llmopt_hip_context *context, size_t bytes) {
 
 uint32_t *context_counters(llmopt_hip_context *context, uint32_t *count) {
   constexpr uint32_t kCounters = 16384;
+  context->scratch_touched = true;
   if (context->counters == nullptr) {
     void *block = nullptr;
     hipError_t status = hipMalloc(&block, kCounters * sizeof(uint32_t));
@@ -697,35 +699,70 @@ int llmopt_hip_commit_batch_profiled(llmopt_hip_batch *batch, int use_graph, int
                                      float *gpu_milliseconds) {
   if (int status = require_active_batch(batch)) return status;
   if (repeats <= 0) return fail(LLMOPT_ERR_INVALID, "profiled commit needs a positive repeat count");
+  constexpr int kMaxBranches = 4;  // hardware queues a process gets by default
+  if (use_graph < 0 || use_graph > kMaxBranches)
+    return fail(LLMOPT_ERR_INVALID, "profiled commit takes 0 (host launches), 1 (one graph) or 2..%d graph branches",
+                kMaxBranches);
   llmopt_hip_context *context = batch->library->context;
   if (int status = use_device(context)) return status;
   batch->finished = true;
   hipStream_t stream = context->stream;
-  auto launch_all = [&]() -> int {
-    for (BatchOp &op : batch->ops) {
+  const int branches = use_graph >= 2 ? use_graph : 1;
+  // Branch of every recorded operation.  One branch: the recorded order, as commit_batch runs it.
+  // Several: the caller states that the operations do not depend on each other; they are dealt
+  // round-robin onto the branches, except those that use the context's scratch memory (kernel
+  // workspace, arrival counters), which share it and stay in recorded order on branch 0.
+  std::vector<int> branch_of(batch->ops.size(), 0);
+  hipStream_t side[kMaxBranches] = {stream, nullptr, nullptr, nullptr};
+  auto launch_all = [&](bool classify, bool forked) -> int {
+    int next = 0;
+    for (size_t i = 0; i < batch->ops.size(); ++i) {
+      BatchOp &op = batch->ops[i];
+      hipStream_t target = forked ? side[branch_of[i]] : stream;
       if (op.is_copy) {
-        if (launch_copy_bytes(op.destination->device, op.source->device, op.source->length, stream) !=
-            hipSuccess)
+        if (launch_copy_bytes(op.destination->device, op.source->device, op.source->length, target) != hipSuccess)
           return fail(LLMOPT_ERR_FAILURE, "HIP batched copy failed");
-      } else if (int status = launch_record(context, op.record)) {
-        return status;
+        if (classify) branch_of[i] = branches > 1 ? next++ % branches : 0;
+        continue;
       }
+      context->scratch_touched = false;
+      context->stream = target;
+      const int status = launch_record(context, op.record);
+      context->stream = stream;
+      if (status != LLMOPT_OK) return status;
+      if (classify) branch_of[i] = (branches > 1 && !context->scratch_touched) ? next++ % branches : 0;
     }
     return LLMOPT_OK;
   };
-  // One untimed pass: first-use allocations (kernel workspace) happen here,
-  // outside any stream capture.
-  int status = launch_all();
+  // One untimed pass: first-use allocations (kernel workspace) happen here, outside any stream
+  // capture, and every operation shows whether it takes scratch memory.
+  int status = launch_all(true, false);
   if (status == LLMOPT_OK && hipStreamSynchronize(stream) != hipSuccess)
     status = fail(LLMOPT_ERR_FAILURE, "HIP batch failed");
   hipGraph_t graph = nullptr;
   hipGraphExec_t executable = nullptr;
-  hipEvent_t start = nullptr, stop = nullptr;
+  hipEvent_t start = nullptr, stop = nullptr, fork = nullptr, joined[kMaxBranches] = {};
   if (status == LLMOPT_OK && use_graph) {
-    if (hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal) != hipSuccess) {
+    for (int b = 1; b < branches && status == LLMOPT_OK; ++b)
+      if (hipStreamCreateWithFlags(&side[b], hipStreamNonBlocking) != hipSuccess ||
+          hipEventCreateWithFlags(&joined[b], hipEventDisableTiming) != hipSuccess)
+        status = fail(LLMOPT_ERR_FAILURE, "HIP could not create a graph branch");
+    if (status == LLMOPT_OK && branches > 1 && hipEventCreateWithFlags(&fork, hipEventDisableTiming) != hipSuccess)
+      status = fail(LLMOPT_ERR_FAILURE, "HIP could not create a graph branch");
+    if (status == LLMOPT_OK && hipStreamBeginCapture(stream, hipStreamCaptureModeThreadLocal) != hipSuccess) {
       status = fail(LLMOPT_ERR_FAILURE, "HIP stream capture could not begin");
-    } else {
-      status = launch_all();
+    } else if (status == LLMOPT_OK) {
+      // fork: the side streams join the capture by waiting for an event of the origin stream
+      if (branches > 1) {
+        if (hipEventRecord(fork, stream) != hipSuccess) status = fail(LLMOPT_ERR_FAILURE, "HIP graph fork failed");
+        for (int b = 1; b < branches && status == LLMOPT_OK; ++b)
+          if (hipStreamWaitEvent(side[b], fork, 0) != hipSuccess) status = fail(LLMOPT_ERR_FAILURE, "HIP graph fork failed");
+      }
+      if (status == LLMOPT_OK) status = launch_all(false, branches > 1);
+      for (int b = 1; b < branches; ++b)
+        if (hipEventRecord(joined[b], side[b]) != hipSuccess || hipStreamWaitEvent(stream, joined[b], 0) != hipSuccess) {
+          if (status == LLMOPT_OK) status = fail(LLMOPT_ERR_FAILURE, "HIP graph join failed");
+        }
       if (hipStreamEndCapture(stream, &graph) != hipSuccess && status == LLMOPT_OK)
         status = fail(LLMOPT_ERR_FAILURE, "HIP stream capture failed");
       if (status == LLMOPT_OK &&
@@ -743,7 +780,7 @@ int llmopt_hip_commit_batch_profiled(llmopt_hip_batch *batch, int use_graph, int
         if (hipGraphLaunch(executable, stream) != hipSuccess)
           status = fail(LLMOPT_ERR_FAILURE, "HIP graph launch failed");
       } else {
-        status = launch_all();
+        status = launch_all(false, false);
       }
     }
     (void)hipEventRecord(stop, stream);
@@ -759,6 +796,11 @@ int llmopt_hip_commit_batch_profiled(llmopt_hip_batch *batch, int use_graph, int
   if (executable) (void)hipGraphExecDestroy(executable);
   if (graph) (void)hipGraphDestroy(graph);
   (void)hipStreamSynchronize(stream);
+  if (fork) (void)hipEventDestroy(fork);
+  for (int b = 1; b < branches; ++b) {
+    if (joined[b]) (void)hipEventDestroy(joined[b]);
+    if (side[b]) (void)hipStreamDestroy(side[b]);
+  }
   clear_batch(batch);
   return status;
 }

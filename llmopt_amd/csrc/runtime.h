@@ -53,6 +53,9 @@ struct llmopt_hip_context : llmopt::RefCounted {
   // only recorded here, the capture is thrown away, the block grown, the capture repeated.
   bool sizing_capture = false;
   size_t sizing_wanted = 0;
+  // Set whenever a launch asks for the workspace or the counters (a profiled commit keeps such
+  // launches off its concurrent branches: they share the memory).
+  bool scratch_touched = false;
   // Arrival counters of kernels that split one output tile over several
   // workgroups; zeroed once, every kernel leaves them zero.
   uint32_t *counters = nullptr;

@@ -389,8 +389,10 @@ class Batch:
     def commit_async(self) -> None:
         _check(lib().llmopt_hip_commit_batch_async(self._handle))
 
-    def commit_profiled(self, repeats: int = 1, use_graph: bool = True) -> float:
-        """Runs the batch `repeats` times between HIP events; returns GPU milliseconds."""
+    def commit_profiled(self, repeats: int = 1, use_graph=True) -> float:
+        """Runs the batch `repeats` times between HIP events; returns GPU milliseconds.
+        use_graph: False (host launches), True (one graph, recorded order) or 2..4 (a graph of that
+        many concurrent branches, for operations that do not depend on each other)."""
         elapsed = ctypes.c_float()
         _check(lib().llmopt_hip_commit_batch_profiled(self._handle, int(use_graph), repeats,
                                                       ctypes.byref(elapsed)))
