@@ -459,12 +459,13 @@ q8_attention_split_kernel(Q8AttentionArgs a, uint32_t chunks_max, uint32_t fixed
       partial[col] = running_max;
       partial[16 + col] = running_sum;
     }
+    // a lane's sixteen values of a scale group are consecutive in d: four 16-byte stores
 #pragma unroll
-    for (int v = 0; v < VBLOCKS; ++v)
+    for (int g = 0; g < GROUPS; ++g)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const uint32_t d = (v >> 2) * 64 + 4 * (quad * 4 + i) + (v & 3);
-        partial[32 + col * D + d] = out_acc[v][i];
+        const f4_t four = {out_acc[g * 4][i], out_acc[g * 4 + 1][i], out_acc[g * 4 + 2][i], out_acc[g * 4 + 3][i]};
+        *reinterpret_cast<f4_t *>(partial + 32 + col * D + g * 64 + 4 * (quad * 4 + i)) = four;
       }
   }
 }
