@@ -18,9 +18,10 @@
 //    (max, denominator, O) go to a workspace and q8_attention_merge_kernel
 //    folds them together with the current token.
 //
-//  * q8_attention_rows_kernel: one wave per (batch, head, query position) row,
-//    serial over keys with an online softmax.  Covers everything else (mask,
-//    window, several query tokens, other head sizes).
+//  * q8_attention_general_kernel: one wave per (batch, head, query position) row,
+//    64 keys at a time, one key per lane for the scores and one value row per
+//    group of lanes for the weighted sum.  Covers everything else (mask, window,
+//    several query tokens, other head sizes, unaligned pools).
 #include <algorithm>
 #include <type_traits>
 
@@ -597,93 +598,182 @@ __global__ __launch_bounds__(kMergeSlices *D) void q8_attention_merge_kernel(Q8A
   }
 }
 
-// ---- row-serial kernel (every other configuration) ---------------------------
+// ---- general kernel (every other configuration) -------------------------------------------
+// Masks (bool / f16), sliding windows, several query tokens, head sizes up to 512, unaligned
+// pools.  One wave per output row (batch, head, query position), keys in tiles of 64 with
+// **one key per lane** for the scores: a lane walks its key's row (16-byte requests, the next
+// ones hit the line the first brought in), decodes int8 to exact halves and multiplies against
+// the query row, which every lane reads from the same LDS address (a broadcast).  No reduction
+// across lanes per key: the softmax statistics of 64 keys take one wave maximum and one wave
+// sum.  For the weighted sum of the values the lanes change roles - `lanes_per_key` lanes share
+// a value row, four (eight at D = 512) head_dim values each, 64 / lanes_per_key keys per request
+// - and take each key's probability x group scale and row address from a small LDS table the
+// score phase left; the keys that shared a lane's head_dim slice are added at the end.
+constexpr int kGeneralWaves = 4;
+constexpr int kGeneralLdsWords = 512 / 2 + 8 * 64 + 64 * 2 + 64;  // query (half2), weight[8][64], row address, kind
 
-constexpr int kMaxFragments = 8;  // head_dim <= 512
+struct GeneralRow {
+  uint32_t batch, head, q_pos, kv_head, past, key_length, first_key;
+};
 
-__global__ __launch_bounds__(256) void q8_attention_rows_kernel(Q8AttentionArgs a) {
+// ALIGNED: pool rows can be read as dwords (pool address, token stride and segment offsets are
+// multiples of four); otherwise byte by byte.
+template <bool ALIGNED>
+__global__ __launch_bounds__(kGeneralWaves * 64) void q8_attention_general_kernel(Q8AttentionArgs a) {
+  __shared__ __attribute__((aligned(16))) uint32_t general_lds[kGeneralWaves][kGeneralLdsWords];
   const uint32_t lane = threadIdx.x & 63;
-  const uint32_t row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  const uint32_t row = blockIdx.x * kGeneralWaves + (threadIdx.x >> 6);
   const uint32_t q_len = a.query_length == 0 ? 1 : a.query_length;
   const uint32_t rows = a.batches * a.query_heads * q_len;
-  if (row >= rows) return;
-  const uint32_t q_pos = row % q_len;
-  const uint32_t head = (row / q_len) % a.query_heads;
-  const uint32_t batch = row / (q_len * a.query_heads);
-  const uint32_t heads_per_kv = a.query_heads / a.kv_heads;
-  const uint32_t kv_head = head / heads_per_kv;
-  const uint32_t D = a.head_dim;
-  const uint32_t groups_per_head = D >> 6;
-  const uint32_t past = sequence_past(a, batch);
-  const uint32_t *slots = a.slot_offsets ? a.slots + a.slot_offsets[batch] : a.slots;
-  const size_t query_base = (((size_t)batch * a.query_heads + head) * q_len + q_pos) * D;
-  const size_t current_base = ((size_t)batch * a.kv_heads + kv_head) * q_len * D;
-  const uint32_t key_length = past + q_pos + 1;
-  const uint32_t first_key = a.window == 0 || key_length <= a.window ? 0 : key_length - a.window;
-  const uint32_t fragments = D >> 6;  // head_dim is a multiple of 64
+  if (row >= rows) return;  // whole wave; no workgroup barriers below
+  uint32_t *lds = general_lds[threadIdx.x >> 6];
+  uint32_t *query_lds = lds;                                      // D / 2 half pairs
+  float *weight_lds = reinterpret_cast<float *>(lds + 256);       // [group][key]: probability x value scale
+  uint64_t *address_lds = reinterpret_cast<uint64_t *>(lds + 256 + 512);  // value row of every key of the tile
+  uint32_t *kind_lds = lds + 256 + 512 + 128;                     // 1: int8 pool row, 0: fp16 current token
 
-  float q[kMaxFragments], result[kMaxFragments];
-#pragma unroll
-  for (int f = 0; f < kMaxFragments; ++f) {
-    result[f] = 0.0f;
-    q[f] = (uint32_t)f < fragments ? half_bits_to_float(a.query[query_base + f * 64 + lane]) : 0.0f;
-  }
-  float maximum = -INFINITY, denominator = 0.0f;
+  const uint32_t D = a.head_dim, groups = D >> 6;
+  GeneralRow r;
+  r.q_pos = row % q_len;
+  r.head = (row / q_len) % a.query_heads;
+  r.batch = row / (q_len * a.query_heads);
+  r.kv_head = r.head / (a.query_heads / a.kv_heads);
+  r.past = sequence_past(a, r.batch);
+  r.key_length = r.past + r.q_pos + 1;  // causal over the query tokens
+  r.first_key = a.window == 0 || r.key_length <= a.window ? 0 : r.key_length - a.window;
+  const uint32_t *slots = a.slot_offsets ? a.slots + a.slot_offsets[r.batch] : a.slots;
+  const uint16_t *query = a.query + (((size_t)r.batch * a.query_heads + r.head) * q_len + r.q_pos) * D;
+  const size_t current_base = ((size_t)r.batch * a.kv_heads + r.kv_head) * q_len * D;
   const bool masked = a.mask != nullptr && a.mask_batches > 0 && a.mask_dtype != 0;
+  const size_t mask_row =
+      masked ? (((size_t)(a.mask_batches == 1 ? 0 : r.batch) * a.mask_heads + (a.mask_heads == 1 ? 0 : r.head)) * q_len +
+                r.q_pos) * ((size_t)r.past + q_len)
+             : 0;
+  const uint32_t key_scale_index = (a.key_offset >> 6) + r.kv_head * groups;
+  const uint32_t value_scale_index = (a.value_offset >> 6) + r.kv_head * groups;
 
-  for (uint32_t key_position = first_key; key_position < key_length; ++key_position) {
-    if (masked) {
-      const uint32_t mask_batch = a.mask_batches == 1 ? 0 : batch;
-      const uint32_t mask_head = a.mask_heads == 1 ? 0 : head;
-      const size_t mask_index =
-          (((size_t)mask_batch * a.mask_heads + mask_head) * q_len + q_pos) * ((size_t)past + q_len) +
-          key_position;
-      const bool active = a.mask_dtype == 2
-                              ? half_bits_to_float(reinterpret_cast<const uint16_t *>(a.mask)[mask_index]) >= 0.0f
-                              : a.mask[mask_index] != 0;
-      if (!active) continue;
+  for (uint32_t i = lane; i < D / 2; i += 64) query_lds[i] = reinterpret_cast<const uint32_t *>(query)[i];
+  __builtin_amdgcn_wave_barrier();
+
+  // value phase geometry
+  const uint32_t per_lane = D > 256 ? 8 : 4;                 // head_dim values per lane
+  const uint32_t lanes_per_key = D / per_lane;               // 16, 32, 48 or 64
+  const uint32_t keys_per_request = 64 / lanes_per_key;      // 4, 2, 1, 1
+  const uint32_t key_sub = lane / lanes_per_key, d0 = (lane % lanes_per_key) * per_lane;
+  const bool value_lane = key_sub < keys_per_request;
+  float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
+  float maximum = -INFINITY, denominator = 0.0f;
+
+  for (uint32_t base = r.first_key; base < r.key_length; base += 64) {
+    // ---- scores: lane = key ----
+    const uint32_t key_position = base + lane;
+    const bool in_range = key_position < r.key_length;
+    const bool is_past = key_position < r.past;
+    bool active = in_range;
+    if (masked && in_range) {
+      const size_t at = mask_row + key_position;
+      active = a.mask_dtype == 2 ? half_bits_to_float(reinterpret_cast<const uint16_t *>(a.mask)[at]) >= 0.0f
+                                 : a.mask[at] != 0;
     }
-    float key[kMaxFragments], value[kMaxFragments];
-    if (key_position < past) {
-      const uint8_t *slot = a.pool + (size_t)slots[key_position] * a.token_stride;
-      const int8_t *values = reinterpret_cast<const int8_t *>(slot);
+    const uint8_t *slot = a.pool;
+    if (in_range && is_past) slot = a.pool + (size_t)slots[key_position] * a.token_stride;
+    float score = 0.0f;
+    if (in_range && is_past) {
+      const uint8_t *key_row = slot + a.key_offset + r.kv_head * D;
+      for (uint32_t g = 0; g < groups; ++g) {
+        float part = 0.0f;
 #pragma unroll
-      for (int f = 0; f < kMaxFragments; ++f) {
-        if ((uint32_t)f >= fragments) break;
-        const float ks = q8_scale_at(slot, a.token_elements, (a.key_offset >> 6) + kv_head * groups_per_head + f);
-        const float vs = q8_scale_at(slot, a.token_elements, (a.value_offset >> 6) + kv_head * groups_per_head + f);
-        key[f] = (float)values[a.key_offset + kv_head * D + f * 64 + lane] * ks;
-        value[f] = (float)values[a.value_offset + kv_head * D + f * 64 + lane] * vs;
-      }
-    } else {
-      const size_t base = current_base + (size_t)(key_position - past) * D;
+        for (int j = 0; j < 4; ++j) {
+          uint32_t words[4];
+          if (ALIGNED) {
+            const u32x4_t loaded = *reinterpret_cast<const u32x4_t __attribute__((aligned(4))) *>(key_row + g * 64 + j * 16);
+            words[0] = loaded[0], words[1] = loaded[1], words[2] = loaded[2], words[3] = loaded[3];
+          } else {
 #pragma unroll
-      for (int f = 0; f < kMaxFragments; ++f) {
-        if ((uint32_t)f >= fragments) break;
-        key[f] = half_bits_to_float(a.current_key[base + f * 64 + lane]);
-        value[f] = half_bits_to_float(a.current_value[base + f * 64 + lane]);
+            for (int w = 0; w < 4; ++w) {
+              const uint8_t *b = key_row + g * 64 + j * 16 + w * 4;
+              words[w] = (uint32_t)b[0] | ((uint32_t)b[1] << 8) | ((uint32_t)b[2] << 16) | ((uint32_t)b[3] << 24);
+            }
+          }
+          const uint4 q_lo = *reinterpret_cast<const uint4 *>(query_lds + (g * 64 + j * 16) / 2);
+          const uint4 q_hi = *reinterpret_cast<const uint4 *>(query_lds + (g * 64 + j * 16) / 2 + 4);
+          const uint32_t q_pairs[8] = {q_lo.x, q_lo.y, q_lo.z, q_lo.w, q_hi.x, q_hi.y, q_hi.z, q_hi.w};
+#pragma unroll
+          for (int w = 0; w < 4; ++w) {
+            h2_t lo, hi;
+            int8x4_to_h2(words[w] ^ 0x80808080u, lo, hi);
+            part = __builtin_amdgcn_fdot2(lo, as_h2(q_pairs[2 * w]), part, false);
+            part = __builtin_amdgcn_fdot2(hi, as_h2(q_pairs[2 * w + 1]), part, false);
+          }
+        }
+        score = fmaf(part, q8_scale_at(slot, a.token_elements, key_scale_index + g), score);
       }
+    } else if (in_range) {
+      const uint16_t *key_row = a.current_key + current_base + (size_t)(key_position - r.past) * D;
+      for (uint32_t i = 0; i < D / 2; ++i)
+        score = __builtin_amdgcn_fdot2(as_h2((uint32_t)key_row[2 * i] | ((uint32_t)key_row[2 * i + 1] << 16)),
+                                       as_h2(query_lds[i]), score, false);
     }
-    float partial_score = 0.0f;
-#pragma unroll
-    for (int f = 0; f < kMaxFragments; ++f)
-      if ((uint32_t)f < fragments) partial_score = fmaf(q[f], key[f], partial_score);
-    const float score = wave_sum(partial_score) * a.scale;
-    const float next_maximum = fmaxf(maximum, score);
-    const float previous_scale = denominator == 0.0f ? 0.0f : __expf(maximum - next_maximum);
-    const float current_scale = __expf(score - next_maximum);
-#pragma unroll
-    for (int f = 0; f < kMaxFragments; ++f)
-      if ((uint32_t)f < fragments) result[f] = result[f] * previous_scale + current_scale * value[f];
-    denominator = denominator * previous_scale + current_scale;
+    score = active ? score * a.scale : -INFINITY;
+    const float tile_maximum = wave_max(score);
+    if (tile_maximum == -INFINITY) continue;  // no key of this tile is allowed (the same for every lane)
+    const float next_maximum = fmaxf(maximum, tile_maximum);
+    const float previous_scale = __expf(maximum - next_maximum);  // 0 for the first tile with a key
+    const float probability = active ? __expf(score - next_maximum) : 0.0f;
+    denominator = denominator * previous_scale + wave_sum(probability);
     maximum = next_maximum;
-  }
-  const size_t output_base = (((size_t)batch * q_len + q_pos) * a.query_heads + head) * D;
 #pragma unroll
-  for (int f = 0; f < kMaxFragments; ++f)
-    if ((uint32_t)f < fragments)
-      a.output[output_base + f * 64 + lane] =
-          float_to_half_bits(denominator == 0.0f ? 0.0f : result[f] / denominator);
+    for (int e = 0; e < 8; ++e) acc[e] *= previous_scale;
+    // ---- hand the tile to the value phase ----
+    const uint8_t *value_row = reinterpret_cast<const uint8_t *>(a.current_value + current_base);  // a valid address for idle keys
+    if (in_range && is_past) value_row = slot + a.value_offset + r.kv_head * D;
+    else if (in_range) value_row = reinterpret_cast<const uint8_t *>(a.current_value + current_base + (size_t)(key_position - r.past) * D);
+    address_lds[lane] = reinterpret_cast<uint64_t>(value_row);
+    kind_lds[lane] = in_range && is_past ? 1u : 0u;
+    for (uint32_t g = 0; g < groups; ++g)
+      weight_lds[g * 64 + lane] =
+          in_range && is_past ? probability * q8_scale_at(slot, a.token_elements, value_scale_index + g) : probability;
+    __builtin_amdgcn_wave_barrier();
+    // ---- values: lanes_per_key lanes share a key's row ----
+    const uint32_t tile_keys = min(64u, r.key_length - base);
+    if (value_lane) {
+      for (uint32_t k0 = 0; k0 < tile_keys; k0 += keys_per_request) {
+        const uint32_t k = min(k0 + key_sub, 63u);
+        const float weight = k0 + key_sub < tile_keys ? weight_lds[(d0 >> 6) * 64 + k] : 0.0f;
+        const uint8_t *source = reinterpret_cast<const uint8_t *>(address_lds[k]);
+        if (kind_lds[k] != 0) {
+          for (uint32_t w = 0; w < per_lane / 4; ++w) {
+            const uint8_t *b = source + d0 + 4 * w;
+            uint32_t word;
+            if (ALIGNED)
+              word = *reinterpret_cast<const uint32_t *>(b);
+            else
+              word = (uint32_t)b[0] | ((uint32_t)b[1] << 8) | ((uint32_t)b[2] << 16) | ((uint32_t)b[3] << 24);
+            h2_t lo, hi;
+            int8x4_to_h2(word ^ 0x80808080u, lo, hi);
+            acc[4 * w + 0] = fmaf(weight, (float)lo[0], acc[4 * w + 0]);
+            acc[4 * w + 1] = fmaf(weight, (float)lo[1], acc[4 * w + 1]);
+            acc[4 * w + 2] = fmaf(weight, (float)hi[0], acc[4 * w + 2]);
+            acc[4 * w + 3] = fmaf(weight, (float)hi[1], acc[4 * w + 3]);
+          }
+        } else {
+          const uint16_t *halves = reinterpret_cast<const uint16_t *>(source) + d0;
+          for (uint32_t e = 0; e < per_lane; ++e) acc[e] = fmaf(weight, half_bits_to_float(halves[e]), acc[e]);
+        }
+      }
+    }
+    __builtin_amdgcn_wave_barrier();
+  }
+  // keys that shared this lane's head_dim slice (keys_per_request = 4: lanes 16 apart; 2: 32 apart)
+  if (keys_per_request >= 2)
+    for (int e = 0; e < 4; ++e) acc[e] += shfl_xor_f32(acc[e], 32);
+  if (keys_per_request == 4)
+    for (int e = 0; e < 4; ++e) acc[e] += shfl_xor_f32(acc[e], 16);
+  if (lane < lanes_per_key) {
+    uint16_t *out = a.output + (((size_t)r.batch * q_len + r.q_pos) * a.query_heads + r.head) * D + d0;
+    for (uint32_t e = 0; e < per_lane; ++e)
+      out[e] = float_to_half_bits(denominator == 0.0f ? 0.0f : acc[e] / denominator);
+  }
 }
 
 bool use_split_path(const Q8AttentionArgs &a) {
@@ -700,7 +790,7 @@ bool use_split_path(const Q8AttentionArgs &a) {
   // D = 128 reads the two group scales of a head as one aligned dword
   if (a.head_dim == 128 && (a.key_offset % 128 != 0 || a.value_offset % 128 != 0)) return false;
   if (a.max_past_length > (uint32_t)kMaxChunkTokens * kMaxSplitChunks) return false;
-  return a.max_past_length >= 64;  // short contexts: one launch of the row kernel is cheaper
+  return a.max_past_length >= 64;  // short contexts: one launch of the general kernel is cheaper
 }
 
 // A wave is bound by the latency of its tiles, one after the other: when 128-token
@@ -808,7 +898,12 @@ hipError_t launch_q8_attention(const Q8AttentionArgs &a, hipStream_t stream) {
   const uint32_t q_len = a.query_length == 0 ? 1 : a.query_length;
   const uint32_t rows = a.batches * a.query_heads * q_len;
   if (rows == 0) return hipSuccess;
-  hipLaunchKernelGGL(q8_attention_rows_kernel, dim3((rows + 3) / 4), dim3(256), 0, stream, a);
+  const dim3 grid((rows + kGeneralWaves - 1) / kGeneralWaves), block(kGeneralWaves * 64);
+  const bool aligned = ((reinterpret_cast<uintptr_t>(a.pool) | a.token_stride | a.key_offset | a.value_offset) & 3) == 0;
+  if (aligned)
+    hipLaunchKernelGGL(q8_attention_general_kernel<true>, grid, block, 0, stream, a);
+  else
+    hipLaunchKernelGGL(q8_attention_general_kernel<false>, grid, block, 0, stream, a);
   return hipGetLastError();
 }
 

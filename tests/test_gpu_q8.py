@@ -315,6 +315,43 @@ def test_row_kernel_features(runtime, b, h, kvh, dim, past, q_len, window, mask_
     assert_close_to_oracle(out, expected, "row kernel")
 
 
+GENERAL_CASES = [
+    # (b, h, kvh, dim, past, q_len, window, mask_dtype, restride): several 64-key tiles, a tile with no
+    # allowed key, a window that starts inside the context, pool rows that are not dword aligned
+    (2, 4, 2, 128, 200, 3, 0, 2, 0), (1, 8, 2, 64, 300, 1, 150, 0, 0), (1, 2, 1, 192, 130, 2, 100, 1, 0),
+    (1, 4, 4, 64, 257, 1, 0, 1, 2), (2, 2, 1, 128, 70, 2, 0, 0, 6), (1, 2, 1, 512, 65, 1, 0, 2, 0),
+]
+
+
+@pytest.mark.parametrize("b,h,kvh,dim,past,q_len,window,mask_dtype,restride", GENERAL_CASES)
+def test_general_kernel_tiles_masks_windows_alignment(runtime, b, h, kvh, dim, past, q_len, window, mask_dtype,
+                                                      restride):
+    rng = np.random.default_rng(past * 3 + dim + restride)
+    pool, slots, _, te, stride, ko, vo = build_pool(rng, kvh, dim, [past])
+    if restride:  # the same tokens at a stride that is no multiple of four
+        rows = pool.reshape(-1, stride)
+        wider = np.zeros((rows.shape[0], stride + restride), dtype=np.uint8)
+        wider[:, :stride] = rows
+        pool, stride = wider.reshape(-1), stride + restride
+    query = rng.standard_normal((b, h, q_len, dim)).astype(np.float16)
+    ck = rng.standard_normal((b, kvh, q_len, dim)).astype(np.float16)
+    cv = rng.standard_normal((b, kvh, q_len, dim)).astype(np.float16)
+    mask, mask_batches, mask_heads = None, 0, 0
+    if mask_dtype:
+        allowed = rng.random((b, h, q_len, past + q_len)) > 0.4
+        allowed[..., 64:128] = False      # a whole tile of keys without an allowed one
+        allowed[..., past:] = True        # the query tokens themselves stay visible
+        mask = allowed.astype(np.uint8) if mask_dtype == 1 else np.where(allowed, 0.0, -np.inf).astype(np.float16)
+        mask_batches, mask_heads = b, h
+    params = PagedParams(batches=b, query_heads=h, kv_heads=kvh, past_length=past, head_dim=dim,
+                         mask_batches=mask_batches, mask_heads=mask_heads, token_elements=te, key_offset=ko,
+                         value_offset=vo, group_size=64, token_stride=stride, scale=1.0 / math.sqrt(dim),
+                         query_length=q_len, mask_dtype=mask_dtype, window=window)
+    out = run_paged(runtime, "llmopt_attention_q8_paged_simd_generic", query, ck, cv, pool, slots, mask, params)
+    expected = oracle.paged_attention_q8(query, ck, cv, pool, slots, mask, params)
+    assert_close_to_oracle(out, expected, "general kernel")
+
+
 @pytest.mark.parametrize("batches", [16, 1])
 def test_decode_attention_full_size_closed_form(runtime, batches):
     """BASELINE's attention configuration (32/8 heads of 128, contexts up to 8192 tokens, scattered
