@@ -91,20 +91,45 @@ __global__ __launch_bounds__(THREADS) void w4a16_gemv_quad_kernel(QuadParams p, 
   const uint32_t row0 = blockIdx.x * rows_per_wg;
 
   // 1. activation and scale requests (clamped, never past the buffers; masked when staged)
+  // Unit e of a thread is 16-byte unit `u` of activation row `row`.  When a row is a whole
+  // number of passes of the workgroup both are known without a division: the staging runs once
+  // per unit, and every vector instruction in it costs four cycles a wave.
+  constexpr bool kWholePasses = (K / 8) % THREADS == 0;
+  constexpr uint32_t kPassesPerRow = kWholePasses ? (K / 8) / THREADS : 1;
+  auto unit_of = [&](int e, uint32_t &row, uint32_t &u, bool &inside) __attribute__((always_inline)) {
+    if constexpr (kWholePasses) {
+      row = (uint32_t)e / kPassesPerRow;
+      u = threadIdx.x + ((uint32_t)e % kPassesPerRow) * THREADS;
+      inside = true;
+    } else {
+      const uint32_t idx = threadIdx.x + e * THREADS;
+      inside = idx < kXUnits;
+      row = min(idx, kXUnits - 1) / (K / 8);
+      u = min(idx, kXUnits - 1) % (K / 8);
+    }
+  };
   uint4 xin[XPER];
 #pragma unroll
   for (int e = 0; e < XPER; ++e) {
-    const uint32_t idx = min(threadIdx.x + e * THREADS, kXUnits - 1);
-    const uint32_t row = idx / (K / 8), u = idx % (K / 8);
+    uint32_t row, u;
+    bool inside;
+    unit_of(e, row, u, inside);
     xin[e] = reinterpret_cast<const uint4 *>(p.x + (size_t)min(row, p.m - 1) * K)[u];
   }
   const uint32_t scale_units = rows_per_wg * kScaleUnitsPerRow;
   const size_t s_first = (size_t)row0 * groups * 2, s_last = (size_t)p.n * groups * 2 - 16;
-  uint4 sin[SPER];
-#pragma unroll
-  for (int e = 0; e < SPER; ++e)
-    sin[e] = *reinterpret_cast<const uint4 *>(reinterpret_cast<const unsigned char *>(p.s) +
-                                               min(s_first + (size_t)(threadIdx.x + e * THREADS) * 16, s_last));
+  // (four named registers, not an array: left as an array the compiler kept it in scratch memory
+  // and waited for these loads right here, before the first weight request, to store them there)
+  static_assert(SPER <= 4, "scale vectors per thread");
+  auto scale_request = [&](int e) __attribute__((always_inline)) {
+    return *reinterpret_cast<const uint4 *>(reinterpret_cast<const unsigned char *>(p.s) +
+                                            min(s_first + (size_t)(threadIdx.x + e * THREADS) * 16, s_last));
+  };
+  uint4 scale_in0 = make_uint4(0, 0, 0, 0), scale_in1 = scale_in0, scale_in2 = scale_in0, scale_in3 = scale_in0;
+  scale_in0 = scale_request(0);
+  if constexpr (SPER > 1) scale_in1 = scale_request(1);
+  if constexpr (SPER > 2) scale_in2 = scale_request(2);
+  if constexpr (SPER > 3) scale_in3 = scale_request(3);
   // 2. the first weights
   const uint32_t unit = __builtin_amdgcn_readfirstlane(blockIdx.x * units_per_wg + min(wave, units_per_wg - 1));
   u32x4_t wreg[DEPTH];
@@ -130,30 +155,37 @@ __global__ __launch_bounds__(THREADS) void w4a16_gemv_quad_kernel(QuadParams p, 
     __builtin_amdgcn_sched_barrier(0);
   }
   // 3. stage: pair order, the decode-bias correction of every 32-K piece, the scales
+  const h2_t bias_even = {(_Float16)1032.0f, (_Float16)1032.0f}, bias_odd = {(_Float16)72.0f, (_Float16)72.0f};
 #pragma unroll
   for (int e = 0; e < XPER; ++e) {
-    const uint32_t idx = threadIdx.x + e * THREADS;
-    const uint32_t row = min(idx, kXUnits - 1) / (K / 8), u = min(idx, kXUnits - 1) % (K / 8);
+    uint32_t row, u;
+    bool inside;
+    unit_of(e, row, u, inside);
     uint4 v = pair_order(xin[e]);
     if (row >= p.m) v = make_uint4(0, 0, 0, 0);
-    const h2_t a0 = as_h2(v.x), b0 = as_h2(v.y), a1 = as_h2(v.z), b1 = as_h2(v.w);
-    float corr = 1032.0f * (((float)a0[0] + (float)a0[1]) + ((float)a1[0] + (float)a1[1])) +
-                 72.0f * (((float)b0[0] + (float)b0[1]) + ((float)b1[0] + (float)b1[1]));
+    // 1032 * (x0 + x4 + x2 + x6) + 72 * (x1 + x5 + x3 + x7): exact products, float32 sums
+    float corr = __builtin_amdgcn_fdot2(as_h2(v.x), bias_even, 0.0f, false);
+    corr = __builtin_amdgcn_fdot2(as_h2(v.z), bias_even, corr, false);
+    corr = __builtin_amdgcn_fdot2(as_h2(v.y), bias_odd, corr, false);
+    corr = __builtin_amdgcn_fdot2(as_h2(v.w), bias_odd, corr, false);
     // the four 16-byte units of a piece sit in four neighbouring lanes (K / 8 and THREADS are multiples of 4)
     corr += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, corr), 0xB1, 0xF, 0xF, true));
     corr += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, corr), 0x4E, 0xF, 0xF, true));
-    if (idx < kXUnits) {
+    if (inside) {
       *reinterpret_cast<uint4 *>(xs + row * kRowStride + u * 16) = v;
       if ((u & 3) == 0) cin[(u >> 2) * 4 + row] = -corr;
     }
   }
   // (corrections of A rows beyond MR are never written: those rows of D are never read)
-#pragma unroll
-  for (int e = 0; e < SPER; ++e) {
+  auto scale_store = [&](int e, const uint4 &value) __attribute__((always_inline)) {
     const uint32_t idx = threadIdx.x + e * THREADS;
     if (idx < scale_units)
-      *reinterpret_cast<uint4 *>(ss + (idx / kScaleUnitsPerRow) * kScaleStride + (idx % kScaleUnitsPerRow) * 16) = sin[e];
-  }
+      *reinterpret_cast<uint4 *>(ss + (idx / kScaleUnitsPerRow) * kScaleStride + (idx % kScaleUnitsPerRow) * 16) = value;
+  };
+  scale_store(0, scale_in0);
+  if constexpr (SPER > 1) scale_store(1, scale_in1);
+  if constexpr (SPER > 2) scale_store(2, scale_in2);
+  if constexpr (SPER > 3) scale_store(3, scale_in3);
   __syncthreads();
   if (wave >= units_per_wg) {
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
