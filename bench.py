@@ -127,7 +127,7 @@ def gemv_kernel_of(m, k, n):
     return "w4a16_gemv_mfma_kernel (16x16x32 matrix-core tiles, 5 <= m <= 8)"
 
 
-def bench_gemv(runtime, steps, warmup):
+def bench_gemv(runtime, steps, warmup, serial_only=False):
     rng = np.random.default_rng(SEED)
     weights, host = {}, {}
     for k, n in GEMV_SHAPES:
@@ -175,7 +175,7 @@ def bench_gemv(runtime, steps, warmup):
     # The launches of the sweep do not depend on each other.  The same K steps as one graph of 2..4
     # concurrent branches: one launch's ramp and tail overlap its neighbours' streaming.
     concurrent = {}
-    for branches in (2, 3, 4):
+    for branches in (() if serial_only else (2, 3, 4)):
         batch = runtime.begin_batch()
         record_steps(batch, steps)
         concurrent[branches] = batch.commit_profiled(repeats=1, use_graph=branches) / steps
@@ -199,17 +199,20 @@ def bench_gemv(runtime, steps, warmup):
             us = ms * 1e3 / (repeats * len(copies))
             gbs = gemv_bytes(m, k, n) / (us * 1e-6) / 1e9
             # warm: the same weight copy every launch (it stays in the 256 MB Infinity Cache)
-            batch = runtime.begin_batch()
-            bw, bs = copies[0]
-            for _ in range(16):
-                record_linear(batch, m, n, k, activations[(m, k)], bw, bs, outputs[(m, k, n)])
-            warm_us = batch.commit_profiled(repeats=repeats, use_graph=True) * 1e3 / (repeats * 16)
+            warm_us = None
+            if not serial_only:
+                batch = runtime.begin_batch()
+                bw, bs = copies[0]
+                for _ in range(16):
+                    record_linear(batch, m, n, k, activations[(m, k)], bw, bs, outputs[(m, k, n)])
+                warm_us = batch.commit_profiled(repeats=repeats, use_graph=True) * 1e3 / (repeats * 16)
             ok, rel_l2 = verified[(m, k, n)]
             cases.append({"m": m, "k": k, "n": n, "bytes": gemv_bytes(m, k, n), "kernel": gemv_kernel_of(m, k, n),
                           "us_per_launch": round(us, 3), "GBps": round(gbs, 1),
                           "hbm_frac": round(gbs / HBM_PEAK_GBS, 4),
-                          "warm_us_per_launch": round(warm_us, 3),
-                          "warm_GBps": round(gemv_bytes(m, k, n) / (warm_us * 1e-6) / 1e9, 1),
+                          "warm_us_per_launch": None if warm_us is None else round(warm_us, 3),
+                          "warm_GBps": None if warm_us is None
+                          else round(gemv_bytes(m, k, n) / (warm_us * 1e-6) / 1e9, 1),
                           "hbm_copies": len(copies), "verified": ok, "rel_l2": float("%.3g" % rel_l2)})
 
     # C1: the 1 x 576 -> 1536 projection of the 30-layer model (474 KB: launch/latency-bound)
@@ -415,21 +418,26 @@ def bench_decode_step(runtime, batches=(1, 8, 32, 128), context=2048, use_graph=
         # the same list frozen into a retained plan: wall-clock of llmopt_hip_prebaked_execute
         # (state launch + one graph launch + 4-byte read-back + wait), what a host stepping a
         # sequence through the boundary pays per token
-        from llmopt_amd.native import Prebaked
-        plan = Prebaked(runtime, step.dispatches, step.tokens, step.token_ids)
-        for _ in range(3):
-            plan.execute(1, context)
-        runtime.synchronize()
-        started = time.perf_counter()
-        for _ in range(repeats):
-            plan.execute(1, context)
-        execute_ms = (time.perf_counter() - started) * 1e3 / repeats
-        single = plan.single_submission
-        del plan
+        # (left out of host-launched runs: those exist for the profiler, which does not survive
+        # tracing the replay of a graph of this size)
+        execute_ms, single = None, None
+        if use_graph:
+            from llmopt_amd.native import Prebaked
+            plan = Prebaked(runtime, step.dispatches, step.tokens, step.token_ids)
+            for _ in range(3):
+                plan.execute(1, context)
+            runtime.synchronize()
+            started = time.perf_counter()
+            for _ in range(repeats):
+                plan.execute(1, context)
+            execute_ms = (time.perf_counter() - started) * 1e3 / repeats
+            single = plan.single_submission
+            del plan
         results.append({"batch": batch, "context": context, "launches": len(step.dispatches),
                         "ms_per_step": round(ms, 4), "tokens_per_s": round(batch / (ms * 1e-3), 1),
-                        "prebaked_execute_wall_ms": round(execute_ms, 4),
-                        "prebaked_execute_tokens_per_s": round(batch / (execute_ms * 1e-3), 1),
+                        "prebaked_execute_wall_ms": None if execute_ms is None else round(execute_ms, 4),
+                        "prebaked_execute_tokens_per_s": None if execute_ms is None
+                        else round(batch / (execute_ms * 1e-3), 1),
                         "prebaked_single_submission": single,
                         "weight_bytes": step.weight_bytes(), "kv_bytes": step.kv_bytes(),
                         "GBps": round(moved / (ms * 1e-3) / 1e9, 1),
@@ -438,44 +446,59 @@ def bench_decode_step(runtime, batches=(1, 8, 32, 128), context=2048, use_graph=
     return results
 
 
-def pmc_probe(runtime, m=1):
+PMC_LAUNCHES_PER_CASE = 8
+
+
+def pmc_probe(runtime):
     """A short run for hardware counters (rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE): four plain
-    64 MiB device-to-device copies, whose bytes are known, then the headline GEMV (M = 1,
-    K = 4096, N = 14336) over 16 distinct weight copies.  The copy calibrates the counters."""
+    64 MiB device-to-device copies, whose bytes are known and calibrate the counters, then every
+    case of the sweep in the order the returned list gives, each PMC_LAUNCHES_PER_CASE launches
+    on distinct weight copies."""
     rng = np.random.default_rng(SEED)
     copy_bytes = 64 << 20
     source = runtime.buffer_of_bytes(rng.integers(0, 256, copy_bytes, dtype=np.uint8))
     destination = runtime.create_buffer(copy_bytes)
     for _ in range(4):
         source.copy_to(destination)
-    k, n = 4096, 14336
-    x, packed, scale = w4_inputs(rng, m, n, k)
-    bx, out = runtime.buffer_of_bytes(x), runtime.create_buffer(m * n * 2)
-    weights = [(runtime.buffer_of_bytes(packed), runtime.buffer_of_bytes(scale)) for _ in range(copies_for(k, n))]
-    batch = runtime.begin_batch()
-    for bw, bs in weights:
-        record_linear(batch, m, n, k, bx, bw, bs, out)
-    batch.commit()
+    cases = []
+    for k, n in GEMV_SHAPES:
+        x, packed, scale = w4_inputs(rng, max(GEMV_ROWS), n, k)
+        weights = [(runtime.buffer_of_bytes(packed), runtime.buffer_of_bytes(scale))
+                   for _ in range(PMC_LAUNCHES_PER_CASE)]
+        for m in GEMV_ROWS:
+            bx, out = runtime.buffer_of_bytes(x[:m]), runtime.create_buffer(m * n * 2)
+            batch = runtime.begin_batch()
+            for bw, bs in weights:
+                record_linear(batch, m, n, k, bx, bw, bs, out)
+            batch.commit()
+            cases.append({"m": m, "k": k, "n": n, "launches": PMC_LAUNCHES_PER_CASE, "kernel": gemv_kernel_of(m, k, n),
+                          "algorithmic_bytes": gemv_bytes(m, k, n)})
+        del weights
     return {"copy_kernel": "copy_vectors_kernel", "copy_bytes_read": copy_bytes, "copy_bytes_written": copy_bytes,
-            "copy_launches": 4, "gemv_kernel": gemv_kernel_of(m, k, n),
-            "gemv_rows": m, "gemv_launches": len(weights), "gemv_algorithmic_bytes": gemv_bytes(m, k, n)}
+            "copy_launches": 4, "gemv_cases_in_launch_order": cases}
 
 
-TRAFFIC_SUMMARY = "profiles/w4a16_gemv_k4096_n14336_hbm_traffic.txt"
+TRAFFIC_SUMMARY = "profiles/w4a16_gemv_sweep_hbm_traffic.txt"
 
 
-def measured_traffic(rows):
-    """HBM bytes per launch of the K=4096, N=14336 GEMV with `rows` activation rows, from an
-    EARLIER rocprofv3 --pmc run of `bench.py --pmc-probe` (FETCH_SIZE and WRITE_SIZE, each
-    calibrated on a plain copy) whose summary is kept with the profiles - not measured in this
-    run.  None when the summary is not there or has no line for these rows."""
+def measured_traffic(cases):
+    """Mean HBM bytes per launch over the given (m, k, n) cases, from an EARLIER rocprofv3 --pmc
+    run of `bench.py --pmc-probe` (FETCH_SIZE and WRITE_SIZE, each calibrated on a plain copy)
+    whose summary is kept with the profiles - not measured in this run.  None when the summary
+    is not there or lacks one of the cases."""
+    found = {}
     try:
         for line in open(os.path.join(ROOT, TRAFFIC_SUMMARY)):
-            if line.startswith(f"traffic_bytes_per_launch_m{rows}:"):
-                return int(line.split(":")[1])
+            if line.startswith("traffic_bytes_per_launch_m"):
+                key, value = line.split(":")
+                found[key.strip()] = int(value)
     except OSError:
-        pass
-    return None
+        return None
+    try:
+        values = [found["traffic_bytes_per_launch_m%d_k%d_n%d" % tuple(case)] for case in cases]
+    except KeyError:
+        return None
+    return int(round(sum(values) / len(values))) if values else None
 
 
 def cpu_model():
@@ -523,9 +546,11 @@ def main():
     parser.add_argument("--decode-eager", action="store_true",
                         help="launch the decode step from the host instead of replaying a HIP graph")
     parser.add_argument("--decode-batches", default="1,8,32,128", help="batch sizes of the decode-step extra")
-    parser.add_argument("--pmc-rows", type=int, default=1, help="activation rows of the --pmc-probe GEMV")
+    parser.add_argument("--serial-only", action="store_true",
+                        help="leave out the concurrent-branch graphs and the warm (cached) per-case loops: every "
+                             "launch of the run then is a serial, cold one (for kernel traces)")
     parser.add_argument("--pmc-probe", action="store_true",
-                        help="only the calibration copy and the headline GEMV, for rocprofv3 --pmc")
+                        help="only the calibration copies and the cases of the GEMV sweep, for rocprofv3 --pmc")
     args = parser.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py measures one GPU: this hot path has no multi-GPU part; run with --gpus 1")
@@ -533,10 +558,10 @@ def main():
     from llmopt_amd.native import Runtime
     runtime = Runtime()
     if args.pmc_probe:
-        print(json.dumps(pmc_probe(runtime, args.pmc_rows)))
+        print(json.dumps(pmc_probe(runtime)))
         runtime.close()
         return
-    gemv = bench_gemv(runtime, args.steps, args.warmup)
+    gemv = bench_gemv(runtime, args.steps, args.warmup, serial_only=args.serial_only)
     # the sweep's time by kernel; `roofline` is the kernel with the largest share
     by_kernel = {}
     for case in gemv["cases"]:
@@ -599,7 +624,6 @@ def main():
     if failed:
         runtime.close()
         sys.exit("bench.py: outputs of timed cases differ from the CPU oracle beyond tolerance: " + ", ".join(failed))
-    dominant_rows = max(case[0] for case in dominant["cases_m_k_n"])
     line = {
         "metric": "W4A16 GEMV HBM GB/s (% peak); Q8 attn decode tokens/s; prefill MFMA %",
         "value": round(value, 1),
@@ -625,9 +649,9 @@ def main():
                      "share_of_sweep_time": dominant["share_of_sweep_time"],
                      "achieved": dominant["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": dominant["hbm_frac"],
-                     "traffic": measured_traffic(dominant_rows),
-                     "traffic_source": TRAFFIC_SUMMARY + " (an earlier rocprofv3 --pmc run of `bench.py --pmc-probe "
-                                       f"--pmc-rows {dominant_rows}` at K=4096 N=14336; not measured in this run)",
+                     "traffic": measured_traffic(dominant["cases_m_k_n"]),
+                     "traffic_source": TRAFFIC_SUMMARY + " (mean over this kernel's cases, from an earlier rocprofv3 "
+                                       "--pmc run of `bench.py --pmc-probe`; not measured in this run)",
                      "bytes_per_launch": dominant["bytes_per_launch"], "us_per_launch": dominant["us_per_launch"],
                      "cases_m_k_n": dominant["cases_m_k_n"]},
         "cpu_baseline": None if args.skip_cpu else cpu_baseline(),
