@@ -223,7 +223,13 @@ void llmopt_hip_release_prebaked(llmopt_hip_prebaked *plan);
  * start of the token buffer, makes past_tokens the context length of every
  * paged attention record (:2182-2195), replays all records in order, waits,
  * and returns the first int32 of the output buffer in *out_token.
- * past_tokens beyond the slot tables' capacity is LLMOPT_ERR_INVALID. */
+ * past_tokens beyond the slot tables' capacity is LLMOPT_ERR_INVALID.
+ * Debug replays of the reference, switched on by the same environment
+ * variables (:2203-2347): LLMOPT_PROFILE_BREAKDOWN runs the records one at a
+ * time and prints GPU time by kernel name to stderr; LLMOPT_DEBUG_NAN_CHECK
+ * (steps with past_tokens > 0, or every step under LLMOPT_CHECK_PREFILL)
+ * reports the first record that leaves a NaN in a buffer that held none and
+ * returns LLMOPT_ERR_FAILURE (the reference exits the process there). */
 int llmopt_hip_prebaked_execute(llmopt_hip_prebaked *plan, int64_t token, int64_t past_tokens,
                                 int64_t checkpoint, int64_t *out_token);
 /* 1 when execute replays one HIP graph, 0 when it launches record by record

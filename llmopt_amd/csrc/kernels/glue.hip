@@ -408,7 +408,31 @@ __global__ void plan_state_kernel(int64_t *token, int64_t value, const int32_t *
   if (threadIdx.x == 0 && token != nullptr) *token = chain_from != nullptr ? (int64_t)*chain_from : value;
   for (uint32_t i = threadIdx.x; i < past_count; i += blockDim.x) past[i] = past_value;
 }
+
+// *found = 1 when the range holds a NaN (not an infinity): fp16 words, or float32 words.
+__global__ void nan_scan_kernel(const uint8_t *data, size_t words, bool f32, uint32_t *found) {
+  bool seen = false;
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < words; i += (size_t)gridDim.x * blockDim.x) {
+    if (f32) {
+      const uint32_t v = reinterpret_cast<const uint32_t *>(data)[i];
+      seen |= (v & 0x7F800000u) == 0x7F800000u && (v & 0x007FFFFFu) != 0;
+    } else {
+      const uint16_t v = reinterpret_cast<const uint16_t *>(data)[i];
+      seen |= (v & 0x7C00u) == 0x7C00u && (v & 0x03FFu) != 0;
+    }
+  }
+  if (seen) *found = 1u;  // every writer stores the same value
+}
 }  // namespace
+
+hipError_t launch_nan_scan(const void *data, size_t bytes, bool f32, uint32_t *found, hipStream_t stream) {
+  const size_t words = bytes / (f32 ? 4 : 2);
+  if (words == 0) return hipSuccess;
+  const uint32_t blocks = (uint32_t)std::min<size_t>((words + 255) / 256, 2048);
+  hipLaunchKernelGGL(nan_scan_kernel, dim3(blocks), dim3(256), 0, stream, static_cast<const uint8_t *>(data), words, f32,
+                     found);
+  return hipGetLastError();
+}
 
 hipError_t launch_plan_state(int64_t *token, int64_t value, const int32_t *chain_from, uint32_t *past,
                              uint32_t past_value, uint32_t past_count, hipStream_t stream) {

@@ -242,6 +242,10 @@ hipError_t launch_copy_bytes(void *destination, const void *source, size_t bytes
 hipError_t launch_plan_state(int64_t *token, int64_t value, const int32_t *chain_from, uint32_t *past,
                              uint32_t past_value, uint32_t past_count, hipStream_t stream);
 
+// Sets *found (device memory) to 1 when [data, data + bytes) holds a NaN, read as fp16 words or
+// (f32) as float32 words; leaves it alone otherwise.
+hipError_t launch_nan_scan(const void *data, size_t bytes, bool f32, uint32_t *found, hipStream_t stream);
+
 // Argmax over float32 logits [rows, n] in two steps with the reference's
 // candidate layout (W4A16LmHeadCandidate {f32 value, u32 index}, 256 per row,
 // lib/metal_w4a16_source.ml:1287-1319); ties go to the lowest index.

@@ -22,7 +22,9 @@
 #include <string.h>
 
 #include <algorithm>
+#include <map>
 #include <memory>
+#include <string>
 
 using namespace llmopt;
 
@@ -42,6 +44,7 @@ struct llmopt_hip_prebaked : llmopt::RefCounted {
   hipGraph_t graph = nullptr;
   hipGraphExec_t executable = nullptr;
   uint64_t workspace_generation = 0;
+  uint32_t *debug_flag = nullptr;  // device word of the NaN-check replay
 };
 
 namespace {
@@ -153,6 +156,156 @@ int enqueue_step(llmopt_hip_prebaked *plan, int64_t token, bool chain, int64_t p
   return LLMOPT_OK;
 }
 
+// ---- debug replays (native/ocaml_metal_stubs.m:2136-2347) ----------------------------------
+// LLMOPT_DEBUG_NAN_CHECK (for steps with past_tokens > 0, or every step under
+// LLMOPT_CHECK_PREFILL): the records run one at a time, and the first record that leaves a NaN
+// in one of its buffers that held none before is reported on stderr.  The reference ends the
+// process there; this library returns an error that names the record instead.
+// LLMOPT_PROFILE_BREAKDOWN: the records run one at a time between two HIP events each; GPU time
+// by kernel name goes to stderr as the reference's table.
+
+bool nan_check_applies(const std::string &name) {
+  // integer buffers and packed cache bytes are not floating point (same exclusions as the reference)
+  return name.find("_i64") == std::string::npos && name.find("cache_pack") == std::string::npos;
+}
+
+int range_has_nan(llmopt_hip_prebaked *plan, const std::string &name, const BoundBuffer &buffer, bool *bad) {
+  *bad = false;
+  if (buffer.device == nullptr || buffer.length == 0 || !nan_check_applies(name)) return LLMOPT_OK;
+  llmopt_hip_context *context = plan->library->context;
+  if (plan->debug_flag == nullptr)
+    LLMOPT_HIP_TRY(hipMalloc(reinterpret_cast<void **>(&plan->debug_flag), 4), "HIP could not allocate the NaN-check flag");
+  const bool f32 = name == "llmopt_matmul" || name.find("_f32") != std::string::npos;
+  uint32_t found = 0;
+  LLMOPT_HIP_TRY(hipMemsetAsync(plan->debug_flag, 0, 4, context->stream), "HIP could not clear the NaN-check flag");
+  LLMOPT_HIP_TRY(launch_nan_scan(buffer.device, buffer.length, f32, plan->debug_flag, context->stream),
+                 "HIP could not scan a buffer");
+  LLMOPT_HIP_TRY(hipMemcpyAsync(&found, plan->debug_flag, 4, hipMemcpyDeviceToHost, context->stream),
+                 "HIP could not read the NaN-check flag");
+  LLMOPT_HIP_TRY(hipStreamSynchronize(context->stream), "NaN-check scan failed");
+  *bad = found != 0;
+  return LLMOPT_OK;
+}
+
+int debug_step(llmopt_hip_prebaked *plan, int64_t token, int64_t past_tokens, bool nan_check, int32_t *host_token) {
+  llmopt_hip_context *context = plan->library->context;
+  if (int status = use_device(context)) return status;
+  if (past_tokens < 0 || (uint64_t)past_tokens > plan->past_capacity)
+    return fail(LLMOPT_ERR_INVALID, "prebaked HIP plan holds %u context tokens, step asks for %lld",
+                plan->past_capacity, (long long)past_tokens);
+  int64_t *token_slot = nullptr;
+  if (plan->token_buffer) {
+    if (plan->token_buffer->length < 8) return fail(LLMOPT_ERR_INVALID, "buffer offset out of bounds");
+    token_slot = reinterpret_cast<int64_t *>(plan->token_buffer->device);
+  }
+  // frozen records read the context length from the plan's device words, the others from byte 12
+  LLMOPT_HIP_TRY(launch_plan_state(token_slot, token, nullptr, plan->single_submission ? plan->device_past : nullptr,
+                                   (uint32_t)past_tokens, plan->single_submission ? plan->past_count : 0,
+                                   context->stream),
+                 "HIP could not write the decode step's state");
+  hipEvent_t before = nullptr, after = nullptr;
+  if (!nan_check) {
+    LLMOPT_HIP_TRY(hipEventCreate(&before), "HIP event creation failed");
+    LLMOPT_HIP_TRY(hipEventCreate(&after), "HIP event creation failed");
+  }
+  struct Stat { double total_ms = 0.0; size_t count = 0; };
+  std::map<std::string, Stat> stats;
+  double overall_ms = 0.0;
+  int status = LLMOPT_OK;
+  if (nan_check)
+    fprintf(stderr, "[DEBUG_NAN_CHECK] Starting check across %zu records (past_tokens=%lld)...\n", plan->records.size(),
+            (long long)past_tokens);
+  for (size_t i = 0; i < plan->records.size() && status == LLMOPT_OK; ++i) {
+    DispatchRecord &record = plan->records[i];
+    if (!plan->single_submission && plan->is_paged_attention[i] && record.parameters.size() >= 16) {
+      const uint32_t past = (uint32_t)past_tokens;
+      memcpy(record.parameters.data() + 12, &past, 4);
+    }
+    std::vector<bool> bad_before(record.buffers.size(), false);
+    if (nan_check)
+      for (size_t b = 0; b < record.buffers.size() && status == LLMOPT_OK; ++b) {
+        bool bad = false;
+        status = range_has_nan(plan, record.name, record.buffers[b], &bad);
+        bad_before[b] = bad;
+      }
+    if (status != LLMOPT_OK) break;
+    if (!nan_check && hipEventRecord(before, context->stream) != hipSuccess) status = fail(LLMOPT_ERR_FAILURE, "HIP event record failed");
+    if (status == LLMOPT_OK) status = launch_record(context, record);
+    if (status == LLMOPT_OK && !nan_check && hipEventRecord(after, context->stream) != hipSuccess)
+      status = fail(LLMOPT_ERR_FAILURE, "HIP event record failed");
+    if (hipStreamSynchronize(context->stream) != hipSuccess && status == LLMOPT_OK)
+      status = fail(LLMOPT_ERR_FAILURE, "dispatch %zu '%s' failed on the GPU", i, record.name.c_str());
+    if (status != LLMOPT_OK) break;
+    if (!nan_check) {
+      float ms = 0.0f;
+      if (hipEventElapsedTime(&ms, before, after) != hipSuccess) ms = 0.0f;
+      overall_ms += ms;
+      Stat &stat = stats[record.name];
+      stat.total_ms += ms;
+      stat.count += 1;
+      continue;
+    }
+    for (size_t b = 0; b < record.buffers.size(); ++b) {
+      bool bad = false;
+      status = range_has_nan(plan, record.name, record.buffers[b], &bad);
+      if (status != LLMOPT_OK) break;
+      if (!bad || bad_before[b]) continue;
+      uint16_t words[16] = {};
+      const size_t shown = std::min<size_t>(16, record.buffers[b].length / 2);
+      (void)hipMemcpy(words, record.buffers[b].device, shown * 2, hipMemcpyDeviceToHost);
+      fprintf(stderr, "\n==================================================\n");
+      fprintf(stderr, "[DEBUG_NAN_CHECK] FIRST NaN PRODUCED AT RECORD %zu:\n  kernel: '%s'\n", i, record.name.c_str());
+      fprintf(stderr, "  buffer: %zu (length=%zu)\n", b, record.buffers[b].length);
+      fprintf(stderr, "  grid: (%lld, %lld, %lld), group: (%lld, %lld, %lld)\n", (long long)record.grid[0],
+              (long long)record.grid[1], (long long)record.grid[2], (long long)record.group[0],
+              (long long)record.group[1], (long long)record.group[2]);
+      if (!record.parameters.empty()) {
+        fprintf(stderr, "  parameters (%zu bytes, u32):", record.parameters.size());
+        for (size_t p = 0; p + 4 <= record.parameters.size() && p < 48; p += 4) {
+          uint32_t word = 0;
+          memcpy(&word, record.parameters.data() + p, 4);
+          fprintf(stderr, " %u", word);
+        }
+        fprintf(stderr, "\n");
+      }
+      fprintf(stderr, "  first 16 half words (hex):");
+      for (size_t k = 0; k < shown; ++k) fprintf(stderr, " 0x%04x", words[k]);
+      fprintf(stderr, "\n");
+      for (size_t other = 0; other < record.buffers.size(); ++other)
+        fprintf(stderr, "  buffer[%zu]: len=%zu\n", other, record.buffers[other].length);
+      fprintf(stderr, "==================================================\n\n");
+      fflush(stderr);
+      status = fail(LLMOPT_ERR_FAILURE, "NaN check: record %zu '%s' produced the first NaN, in buffer %zu", i,
+                    record.name.c_str(), b);
+      break;
+    }
+  }
+  if (before) (void)hipEventDestroy(before);
+  if (after) (void)hipEventDestroy(after);
+  if (status != LLMOPT_OK) return status;
+  if (!nan_check) {
+    std::vector<std::pair<std::string, Stat>> order(stats.begin(), stats.end());
+    std::stable_sort(order.begin(), order.end(),
+                     [](const auto &a, const auto &b) { return a.second.total_ms > b.second.total_ms; });
+    fprintf(stderr, "\n========== DECODE KERNEL BREAKDOWN (past_tokens=%lld) ==========\n", (long long)past_tokens);
+    fprintf(stderr, "%-48s | %5s | %10s | %10s | %6s\n", "Kernel Name", "Calls", "Total (ms)", "Avg (us)", "Pct");
+    fprintf(stderr, "-------------------------------------------------+-------+------------+------------+-------\n");
+    for (const auto &entry : order)
+      fprintf(stderr, "%-48s | %5zu | %10.3f | %10.2f | %5.1f%%\n", entry.first.c_str(), entry.second.count,
+              entry.second.total_ms, entry.second.total_ms / entry.second.count * 1000.0,
+              overall_ms > 0 ? entry.second.total_ms / overall_ms * 100.0 : 0.0);
+    fprintf(stderr, "-------------------------------------------------+-------+------------+------------+-------\n");
+    fprintf(stderr, "%-48s | %5zu | %10.3f |            | 100.0%%\n", "TOTAL DISPATCHES", plan->records.size(), overall_ms);
+    fprintf(stderr, "===============================================================\n\n");
+    fflush(stderr);
+  }
+  *host_token = 0;
+  if (plan->output_buffer && plan->output_buffer->length >= 4)
+    LLMOPT_HIP_TRY(hipMemcpy(host_token, plan->output_buffer->device, 4, hipMemcpyDeviceToHost),
+                   "HIP could not read the decode output");
+  return LLMOPT_OK;
+}
+
 bool is_reference_paged_attention(const char *name) {
   static const char prefix[] = "llmopt_attention_q8_paged_";
   // the batched extension keeps its lengths in a caller-owned device buffer: nothing to patch
@@ -236,6 +389,7 @@ void llmopt_hip_release_prebaked(llmopt_hip_prebaked *plan) {
   (void)hipStreamSynchronize(context->stream);
   destroy_graph(plan);
   if (plan->device_past) (void)hipFree(plan->device_past);
+  if (plan->debug_flag) (void)hipFree(plan->debug_flag);
   for (DispatchRecord &record : plan->records) drop_record(&record);
   if (plan->token_buffer) llmopt_hip_release_buffer(plan->token_buffer);
   if (plan->output_buffer) llmopt_hip_release_buffer(plan->output_buffer);
@@ -248,6 +402,13 @@ int llmopt_hip_prebaked_execute(llmopt_hip_prebaked *plan, int64_t token, int64_
   (void)checkpoint;  // recurrent-state checkpoints (llmopt_cache_pack_checkpoint_q8_simd) are not part of this backend
   if (plan == nullptr) return fail(LLMOPT_ERR_FAILURE, "HIP prebaked plan has been finalized");
   int32_t next_token = 0;
+  const bool nan_check =
+      getenv("LLMOPT_DEBUG_NAN_CHECK") != nullptr && (past_tokens > 0 || getenv("LLMOPT_CHECK_PREFILL") != nullptr);
+  if (nan_check || getenv("LLMOPT_PROFILE_BREAKDOWN") != nullptr) {
+    if (int status = debug_step(plan, token, past_tokens, nan_check, &next_token)) return status;
+    if (out_token) *out_token = (int64_t)next_token;
+    return LLMOPT_OK;
+  }
   if (int status = enqueue_step(plan, token, false, past_tokens, &next_token)) return status;
   if (hipStreamSynchronize(plan->library->context->stream) != hipSuccess)
     return fail(LLMOPT_ERR_FAILURE, "Prebaked HIP batch failed");

@@ -183,3 +183,53 @@ def test_ring_worker_runs_chained_steps_of_a_plan(runtime, depth, monkeypatch):
     ring.submit(7, 5, 0)
     assert ring.wait_completion() == (7, expected[0], 0)
     ring.destroy()
+
+
+def test_profile_breakdown_replay_prints_gpu_time_by_kernel(runtime, monkeypatch, capfd):
+    """LLMOPT_PROFILE_BREAKDOWN (native/ocaml_metal_stubs.m:2270-2347): the records run one at a
+    time, the step's result is unchanged, and the table of GPU time by kernel name goes to stderr."""
+    from llmopt_amd.native import Prebaked
+    rng = np.random.default_rng(5)
+    dispatches, tokens, token_ids = markov_plan(runtime, rng)
+    plan = Prebaked(runtime, dispatches, tokens, token_ids)
+    want = plan.execute(5, 3)
+    capfd.readouterr()
+    monkeypatch.setenv("LLMOPT_PROFILE_BREAKDOWN", "1")
+    got = plan.execute(5, 3)
+    report = capfd.readouterr().err
+    assert got == want
+    assert "DECODE KERNEL BREAKDOWN (past_tokens=3)" in report
+    rows = {line.split("|")[0].strip(): line for line in report.splitlines() if "|" in line}
+    assert set(rows) >= {"llmopt_embedding_f16", "llmopt_w4a16_lm_head_argmax_f16", "TOTAL DISPATCHES"}
+    assert rows["llmopt_embedding_f16"].split("|")[1].strip() == "1"
+    assert float(rows["TOTAL DISPATCHES"].split("|")[2]) > 0.0
+
+
+def test_nan_check_replay_names_the_first_record_that_produces_a_nan(runtime, monkeypatch, capfd):
+    """LLMOPT_DEBUG_NAN_CHECK (native/ocaml_metal_stubs.m:2136-2268).  The embedding table holds a
+    NaN in row 7 only: token 5 passes, token 7 is reported at record 0, buffer 2 (the row it wrote;
+    the table itself held its NaN before and is not blamed).  A step with no context is only
+    checked under LLMOPT_CHECK_PREFILL, as in the reference."""
+    from llmopt_amd.native import Prebaked
+    rng = np.random.default_rng(5)
+    dispatches, tokens, token_ids = markov_plan(runtime, rng)
+    table = dispatches[0][1][1]
+    poisoned = table.numpy(np.uint16).copy().reshape(512, 576)
+    poisoned[7, 100] = 0x7E00
+    table.write(poisoned)
+    plan = Prebaked(runtime, dispatches, tokens, token_ids)
+    monkeypatch.setenv("LLMOPT_DEBUG_NAN_CHECK", "1")
+    plan.execute(5, 3)
+    assert "Starting check across 2 records (past_tokens=3)" in capfd.readouterr().err
+    with pytest.raises(Exception) as error:
+        plan.execute(7, 3)
+    assert "record 0 'llmopt_embedding_f16' produced the first NaN, in buffer 2" in str(error.value)
+    report = capfd.readouterr().err
+    assert "FIRST NaN PRODUCED AT RECORD 0" in report and "kernel: 'llmopt_embedding_f16'" in report
+    # past_tokens = 0: not checked, the step runs as usual (the NaN row flows into the argmax)
+    plan.execute(7, 0)
+    assert "DEBUG_NAN_CHECK" not in capfd.readouterr().err
+    monkeypatch.setenv("LLMOPT_CHECK_PREFILL", "1")
+    plan.execute(5, 0)  # a clean row again (a buffer that held a NaN before a record is not blamed on it)
+    with pytest.raises(Exception):
+        plan.execute(7, 0)
