@@ -140,13 +140,26 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
   static_assert(W_VECTORS == 1, "one 32-nibble vector per thread and matrix");
   const uint32_t w_row = tid >> 1;
   const uint32_t w_half = tid & 1;
+  // Two matrices of 128 columns are 256 weight rows, one per thread pair: every thread fetches and
+  // decodes one matrix (rows 0..127 gate, 128..255 up) instead of half the threads both.
+  constexpr bool kThreadPerMatrix = DUAL && NW * BN == kThreads / 2;
+  constexpr int NWF = kThreadPerMatrix ? 1 : NW;  // matrices a thread fetches
   struct Fetched {
-    u32x4_t w[NW];
-    uint32_t s[NW];  // fp16 bits in the low half
+    u32x4_t w[NWF];
+    uint32_t s[NWF];  // fp16 bits in the low half
   };
   Fetched fetched[WS];
-  constexpr int W_LOADS = 2 * NW;  // vector memory loads of one fetch_w
-  const uint32_t w_col = min(n0 + w_row, p.n - 1);  // columns past n are never stored
+  constexpr int W_LOADS = 2 * NWF;  // vector memory loads of one fetch_w
+  const uint32_t fetch_matrix = kThreadPerMatrix ? w_row / BN : 0;
+  const uint32_t fetch_row = kThreadPerMatrix ? w_row % BN : w_row;
+  const uint32_t w_col = min(n0 + fetch_row, p.n - 1);  // columns past n are never stored
+  const uint8_t *w_base[NWF];
+  const uint16_t *s_base[NWF];
+#pragma unroll
+  for (int v = 0; v < NWF; ++v) {
+    w_base[v] = kThreadPerMatrix ? (fetch_matrix ? p.w[NW - 1] : p.w[0]) : p.w[v];
+    s_base[v] = kThreadPerMatrix ? (fetch_matrix ? p.s[NW - 1] : p.s[0]) : p.s[v];
+  }
 
   // The compiler takes the destination of these loads as written when the statement ends, while
   // the data lands later: between a fetch_w and the wait_w of the same set, control flow must
@@ -154,9 +167,9 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
   // read registers whose loads were still in flight).
   auto fetch_w = [&](Fetched &f, uint32_t k0) __attribute__((always_inline)) {
 #pragma unroll
-    for (int v = 0; v < NW; ++v) {
-      const void *w_src = p.w[v] + (size_t)w_col * (K >> 1) + ((k_base + k0) >> 1) + w_half * 16;
-      const void *s_src = p.s[v] + (size_t)w_col * (K >> 6) + ((k_base + k0) >> 6);
+    for (int v = 0; v < NWF; ++v) {
+      const void *w_src = w_base[v] + (size_t)w_col * (K >> 1) + ((k_base + k0) >> 1) + w_half * 16;
+      const void *s_src = s_base[v] + (size_t)w_col * (K >> 6) + ((k_base + k0) >> 6);
       asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(f.w[v]) : "v"(w_src) : "memory");
       asm volatile("global_load_ushort %0, %1, off" : "=&v"(f.s[v]) : "v"(s_src) : "memory");
     }
@@ -164,7 +177,7 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
   // at most `younger` loads issued after those of f are still outstanding
   auto wait_w = [&](Fetched &f, auto younger) __attribute__((always_inline)) {
     constexpr int n = decltype(younger)::value;
-    if constexpr (NW == 1)
+    if constexpr (NWF == 1)
       asm volatile("s_waitcnt vmcnt(%2)" : "+v"(f.w[0]), "+v"(f.s[0]) : "n"(n) : "memory");
     else
       asm volatile("s_waitcnt vmcnt(%4)"
@@ -179,14 +192,15 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
   // The decode of one fetched set into an LDS stage, cut into items of one
   // weight dword (8 nibbles): q * s as fp16 (one rounding, 2^-11 relative at
   // most), in natural K order.
-  constexpr int ITEMS = NW * 4;
+  constexpr int ITEMS = NWF * 4;
   auto store_item = [&](const Fetched &f, int stage, int item) __attribute__((always_inline)) {
     _Float16 *w_lds = stage_lds + W_BASE_HALFS + stage * W_STAGE_HALFS;
     const int v = item / 4;
     const int j = item % 4;
-    if (BN % 256 != 0 && w_row >= (uint32_t)BN) return;
+    if (!kThreadPerMatrix && BN % 256 != 0 && w_row >= (uint32_t)BN) return;
     const _Float16 scale = __builtin_bit_cast(_Float16, (uint16_t)f.s[v]);
     const uint4 packed = w4_scaled_natural(f.w[v][j], scale);
+    // (one matrix per thread: w_row runs over the rows of both matrices, as v * BN + row does)
     *reinterpret_cast<uint4 *>(&w_lds[(v * BN + w_row) * LDS_STRIDE + w_half * 32 + j * 8]) = packed;
   };
 
