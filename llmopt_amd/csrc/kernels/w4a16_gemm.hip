@@ -134,18 +134,24 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
     }
   };
 
-  // Weights go global -> registers (w row tid/2, half tid%2) -> decode -> LDS.
+  // Weights go global -> registers (a row of 32 bytes per K step, shared by two or four threads) -> decode -> LDS.
   // WS register sets: set s % WS holds the weights of step s; it is decoded during step
   // s - 1 and requested again right after, for step s - 1 + WS.
   static_assert(W_VECTORS == 1, "one 32-nibble vector per thread and matrix");
-  const uint32_t w_row = tid >> 1;
-  const uint32_t w_half = tid & 1;
-  // Two matrices of 128 columns are 256 weight rows, one per thread pair: every thread fetches and
-  // decodes one matrix (rows 0..127 gate, 128..255 up) instead of half the threads both.
+  // Every thread takes an equal share of the decode.  Two matrices of 128 columns are 256 weight
+  // rows, one per thread pair: a thread fetches and decodes one matrix (rows 0..127 gate, 128..255
+  // up).  One matrix of 128 columns: four threads share a row, eight bytes each.  (Before, half
+  // the threads did all of it in both cases.)
   constexpr bool kThreadPerMatrix = DUAL && NW * BN == kThreads / 2;
-  constexpr int NWF = kThreadPerMatrix ? 1 : NW;  // matrices a thread fetches
+  constexpr int NWF = kThreadPerMatrix ? 1 : NW;                                   // matrices a thread fetches
+  constexpr int ROW_THREADS = (!DUAL && BN * 4 == kThreads) ? 4 : 2;             // threads sharing a row's 32 bytes
+  constexpr int DW = 8 / ROW_THREADS;                                              // dwords (of 8 nibbles) per thread
+  static_assert(DUAL || BN * ROW_THREADS == kThreads, "every thread has a row piece");
+  const uint32_t w_row = tid / ROW_THREADS;
+  const uint32_t w_half = tid % ROW_THREADS;
+  typedef uint32_t words_t __attribute__((ext_vector_type(DW)));
   struct Fetched {
-    u32x4_t w[NWF];
+    words_t w[NWF];
     uint32_t s[NWF];  // fp16 bits in the low half
   };
   Fetched fetched[WS];
@@ -168,9 +174,12 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
   auto fetch_w = [&](Fetched &f, uint32_t k0) __attribute__((always_inline)) {
 #pragma unroll
     for (int v = 0; v < NWF; ++v) {
-      const void *w_src = w_base[v] + (size_t)w_col * (K >> 1) + ((k_base + k0) >> 1) + w_half * 16;
+      const void *w_src = w_base[v] + (size_t)w_col * (K >> 1) + ((k_base + k0) >> 1) + w_half * (DW * 4);
       const void *s_src = s_base[v] + (size_t)w_col * (K >> 6) + ((k_base + k0) >> 6);
-      asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(f.w[v]) : "v"(w_src) : "memory");
+      if constexpr (DW == 4)
+        asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(f.w[v]) : "v"(w_src) : "memory");
+      else
+        asm volatile("global_load_dwordx2 %0, %1, off" : "=&v"(f.w[v]) : "v"(w_src) : "memory");
       asm volatile("global_load_ushort %0, %1, off" : "=&v"(f.s[v]) : "v"(s_src) : "memory");
     }
   };
@@ -192,16 +201,16 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
   // The decode of one fetched set into an LDS stage, cut into items of one
   // weight dword (8 nibbles): q * s as fp16 (one rounding, 2^-11 relative at
   // most), in natural K order.
-  constexpr int ITEMS = NWF * 4;
+  constexpr int ITEMS = NWF * DW;
   auto store_item = [&](const Fetched &f, int stage, int item) __attribute__((always_inline)) {
     _Float16 *w_lds = stage_lds + W_BASE_HALFS + stage * W_STAGE_HALFS;
-    const int v = item / 4;
-    const int j = item % 4;
-    if (!kThreadPerMatrix && BN % 256 != 0 && w_row >= (uint32_t)BN) return;
+    const int v = item / DW;
+    const int j = item % DW;
+    if (DUAL && !kThreadPerMatrix && w_row >= (uint32_t)BN) return;
     const _Float16 scale = __builtin_bit_cast(_Float16, (uint16_t)f.s[v]);
     const uint4 packed = w4_scaled_natural(f.w[v][j], scale);
     // (one matrix per thread: w_row runs over the rows of both matrices, as v * BN + row does)
-    *reinterpret_cast<uint4 *>(&w_lds[(v * BN + w_row) * LDS_STRIDE + w_half * 32 + j * 8]) = packed;
+    *reinterpret_cast<uint4 *>(&w_lds[(v * BN + w_row) * LDS_STRIDE + w_half * (DW * 8) + j * 8]) = packed;
   };
 
   f16x_t acc[NW][WM][WN];
