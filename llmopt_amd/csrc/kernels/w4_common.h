@@ -33,36 +33,20 @@ __device__ __forceinline__ uint16_t float_to_half_bits(float value) {
   return __builtin_bit_cast(uint16_t, (_Float16)value);  // round to nearest even
 }
 
-// Exact int4 -> fp16 decode of one dword (8 nibbles = K offsets 0..7).
+// int4 -> fp16 decode of one dword (8 nibbles = K offsets 0..7), one bit operation per pair.
 //
-// XOR with 0x88888888 turns two's complement into offset binary (q + 8).
-// OR-ing a 4-bit field into the mantissa of 1024.0 (0x6400, ulp 1) or of 64.0
-// (0x5400, ulp 1/16, field at bits 4..7) gives 1024 + (q + 8) or 64 + (q + 8)
-// exactly, so one packed subtract yields q.  The four results hold the pairs
-// (k0,k4) (k1,k5) (k2,k6) (k3,k7): the activation is arranged to match.
+// XOR with 8 turns a two's-complement nibble into offset binary (q + 8).  A 4-bit field in the
+// mantissa of 1024.0 (0x6400, ulp 1) or of 64.0 (0x5400, ulp 1/16, field at bits 4..7) reads as
+// 1024 + (q + 8) or 64 + (q + 8) exactly.  Both steps are one XOR after the mask:
+// (w & mask) ^ (magic | (0x88888888 & mask)), the magic bits lying outside the mask.  The four
+// results hold the pairs (k0,k4) (k1,k5) (k2,k6) (k3,k7): the activation is arranged to match.
 struct W4Pairs {
   h2_t p04, p15, p26, p37;
 };
 
-__device__ __forceinline__ W4Pairs w4_decode_pairs(uint32_t word) {
-  const uint32_t v = word ^ 0x88888888u;
-  const uint32_t hi = v >> 8;
-  const h2_t bias_lo = {(_Float16)1032.0f, (_Float16)1032.0f};
-  const h2_t bias_hi = {(_Float16)72.0f, (_Float16)72.0f};
-  W4Pairs out;
-  out.p04 = as_h2((v & 0x000F000Fu) | 0x64006400u) - bias_lo;
-  out.p15 = as_h2((v & 0x00F000F0u) | 0x54005400u) - bias_hi;
-  out.p26 = as_h2((hi & 0x000F000Fu) | 0x64006400u) - bias_lo;
-  out.p37 = as_h2((hi & 0x00F000F0u) | 0x54005400u) - bias_hi;
-  return out;
-}
-
-// Same decode without the subtraction: the pairs hold q + 1032 (p04, p26) and
-// q + 72 (p15, p37).  (w ^ 0x88888888) & mask | magic equals
-// (w & mask) ^ (magic | (0x88888888 & mask)) because the magic bits lie outside
-// the mask, so each pair costs one three-input bit operation.  A dot product
-// with these is corrected afterwards by 1032 * sum(x at K offsets 0,4,2,6) +
-// 72 * sum(x at K offsets 1,5,3,7), which does not depend on the weight row.
+// The pairs hold q + 1032 (p04, p26) and q + 72 (p15, p37).  A dot product with these is
+// corrected afterwards by 1032 * sum(x at K offsets 0,4,2,6) + 72 * sum(x at K offsets 1,5,3,7),
+// which does not depend on the weight row.
 __device__ __forceinline__ W4Pairs w4_decode_biased(uint32_t word) {
   const uint32_t hi = word >> 8;
   W4Pairs out;
@@ -70,6 +54,18 @@ __device__ __forceinline__ W4Pairs w4_decode_biased(uint32_t word) {
   out.p15 = as_h2((word & 0x00F000F0u) ^ 0x54805480u);
   out.p26 = as_h2((hi & 0x000F000Fu) ^ 0x64086408u);
   out.p37 = as_h2((hi & 0x00F000F0u) ^ 0x54805480u);
+  return out;
+}
+
+// Exact q: the biased decode and one packed subtract per pair.
+__device__ __forceinline__ W4Pairs w4_decode_pairs(uint32_t word) {
+  const h2_t bias_lo = {(_Float16)1032.0f, (_Float16)1032.0f};
+  const h2_t bias_hi = {(_Float16)72.0f, (_Float16)72.0f};
+  W4Pairs out = w4_decode_biased(word);
+  out.p04 -= bias_lo;
+  out.p15 -= bias_hi;
+  out.p26 -= bias_lo;
+  out.p37 -= bias_hi;
   return out;
 }
 
