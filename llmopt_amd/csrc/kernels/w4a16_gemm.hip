@@ -451,13 +451,18 @@ uint32_t gemm_k_splits(uint32_t m, uint32_t n, uint32_t k) {
 template <bool DUAL>
 hipError_t launch_gemm(GemmParams &p, hipStream_t stream) {
   if (DUAL) return launch_tile<2, 2, true>(p, stream);  // 256 x 128, two accumulator sets
-  // 256 x 256 when that still gives every CU a tile, otherwise 128 x 256 / 128 x 128
+  // 256 x 256 when that still gives every CU a tile, otherwise 256 x 128 / 128 x 256 / 128 x 128
   const int cus = device_compute_units();
   const uint64_t big = (uint64_t)((p.m + 255) / 256) * ((p.n + 255) / 256);
   if (big >= (uint64_t)cus) return launch_tile<2, 4, false>(p, stream);
-  const uint64_t mid = (uint64_t)((p.m + 127) / 128) * ((p.n + 255) / 256);
-  // also when a few CUs stay without a tile: 224 tiles of 128 x 256 beat 448 of 128 x 128, two on most CUs
-  if (mid * 8 >= (uint64_t)cus * 7) return launch_tile<1, 4, false>(p, stream);
+  // Half that size, tall (256 x 128) or wide (128 x 256), whichever pads less; the tall one when
+  // they tie (its waves read 16 operand vectors from LDS per 16 MFMAs, the wide one's 20: 76.5
+  // against 80 us at 512 x 14336, 81.7 against 86.3 at 2048 x 4096).  Also when a few CUs stay
+  // without a tile: 224 such tiles beat 448 of 128 x 128, two on most CUs.
+  const uint64_t tall = (uint64_t)((p.m + 255) / 256) * ((p.n + 127) / 128);
+  const uint64_t wide = (uint64_t)((p.m + 127) / 128) * ((p.n + 255) / 256);
+  if (std::min(tall, wide) * 8 >= (uint64_t)cus * 7)
+    return tall <= wide ? launch_tile<2, 2, false>(p, stream) : launch_tile<1, 4, false>(p, stream);
   // 128 x 128 tiles have steps shorter than a trip to memory.  With two stages they fit a CU
   // twice, which covers the loads; when there is at most one tile per CU anyway, four
   // activation stages do (K a whole number of four steps; measured 58 -> 49 us at 512 x 4096 x 4096,

@@ -375,12 +375,14 @@ def tile_covering_sample(rng, extent, block):
     return np.minimum(starts + rng.integers(0, block, size=starts.size), extent - 1)
 
 
-PREFILL_CELLS = [(512, 4096, 4096), (512, 14336, 4096), (2048, 4096, 4096), (2048, 14336, 4096)]
+# (384, 19200, 512): three row tiles of 128 pad less than two of 256, and 225 tiles fill the device: 128 x 256 tiles
+PREFILL_CELLS = [(512, 4096, 4096), (512, 14336, 4096), (2048, 4096, 4096), (2048, 14336, 4096), (384, 19200, 512)]
 
 
 @pytest.mark.parametrize("m,n,k", PREFILL_CELLS)
 def test_gemm_prefill_cell_at_full_size(runtime, m, n, k):
-    """The measured prefill shapes (128x128, 128x256 and 256x256 workgroup tiles).  Three checks:
+    """The measured prefill shapes (128x128 with split K, 256x128 and 256x256 workgroup tiles) and one
+    that takes 128x256 tiles.  Three checks:
     the oracle on a sample with one row out of every 32 and one column out of every 64 (every
     workgroup tile and every wave tile is hit); the sum over rows of every output column against
     the oracle applied to the summed activation (touches every output element); and linearity."""
