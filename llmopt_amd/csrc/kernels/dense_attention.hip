@@ -321,6 +321,244 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void dense_attention_mfma_kern
   }
 }
 
+// ---- 32 x 32 wave tiles (no mask) --------------------------------------------------------------
+//
+// The same workgroup geometry and LDS staging as the SHARED variant above (four waves = 128
+// consecutive query rows of one head; K and V rows copied global -> LDS 64 keys a stage), with
+// the arithmetic on v_mfma_f32_32x32x16_f16: a wave owns ONE tile of 32 query rows and walks the
+// keys 32 at a time.
+//
+//  * S^T = K Q^T: A = K (rows = keys), B = Q^T (columns = query rows), D / 16 chained MFMAs.  Lane
+//    (j = lane % 32, half = lane / 32) ends with the sixteen scores of query row j and keys
+//    (r / 4) * 8 + half * 4 + r % 4, r = 0..15: one row per lane, so the running maximum and sum
+//    are per-lane scalars and the two lanes of a row meet once per tile (maximum) and once at the
+//    end (sum).
+//  * O^T += V^T P^T in two steps of 16 keys: the B operand of step s is the lane's own
+//    probabilities r = 8 s .. 8 s + 7 as halves, no exchange between lanes; the A operand row i
+//    of block jj is head_dim i * (D / 32) + jj, so a lane reads D / 32 adjacent halves of each of
+//    its eight keys and regroups them in registers (one v_perm per operand dword).
+//
+// Against the 16-key tiles above: the legacy 16x16x16 MFMA of the P V product runs at half the
+// rate of the x32 shapes (16 cycles for 8192 flops), and the per-tile bookkeeping of the online
+// softmax (exchanges, rescaling, the alpha exponential) is paid once per 32 keys and 32 rows
+// instead of four times.
+template <int D>
+__global__ __launch_bounds__(kWavesPerBlock * 64) void dense_attention_tile32_kernel(DenseAttentionArgs a) {
+  constexpr int KSTEPS = D / 16;  // score MFMAs per key tile
+  constexpr int JJ = D / 32;      // adjacent head_dim values per lane and key = output blocks
+  constexpr int ROW_BYTES = D * 2;
+  constexpr int PIECES = ROW_BYTES / 16;
+  constexpr int KEYS_PER_COPY = 64 / PIECES;
+  constexpr int COPIES = kStageKeys / KEYS_PER_COPY / kWavesPerBlock;
+  constexpr int STAGE_BYTES = kStageKeys * ROW_BYTES;
+  static_assert(JJ == 2 || JJ == 4, "head_dim 64 or 128");
+  extern __shared__ __attribute__((aligned(16))) unsigned char stage_lds[];  // [2 stages][K | V]
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t wave = threadIdx.x >> 6;
+  const uint32_t row_lane = lane & 31;
+  const uint32_t half = lane >> 5;
+  const uint32_t head = blockIdx.y;
+  const uint32_t batch = blockIdx.z;
+  const uint32_t slab = a.causal ? gridDim.x - 1 - blockIdx.x : blockIdx.x;  // longest causal slabs first
+  const uint32_t q0 = (slab * kWavesPerBlock + wave) * 32;
+  const bool has_rows = q0 < a.query_length;  // a wave without rows still copies and meets the barriers
+  const uint32_t kv_heads = a.kv_heads > 0 ? a.kv_heads : a.heads;
+  const uint32_t kv_head = kv_heads < a.heads ? head / (a.heads / kv_heads) : head;
+  const uint32_t L = a.key_length;
+
+  // B operand of the score MFMAs: Q[row = row_lane][d = ks * 16 + half * 8 ..]; rows past the end repeat the last
+  h8_t q_frag[KSTEPS];
+  {
+    const uint32_t row = min(q0 + row_lane, a.query_length - 1);
+    const uint16_t *q_row = a.query + (((size_t)batch * a.heads + head) * a.query_length + row) * D;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks)
+      q_frag[ks] = __builtin_bit_cast(h8_t, *reinterpret_cast<const uint4 *>(q_row + ks * 16 + half * 8));
+  }
+  const uint16_t *key_base = a.key + ((size_t)batch * kv_heads + kv_head) * L * D;
+  const size_t value_row_stride = a.token_first_value ? (size_t)kv_heads * D : D;
+  const uint16_t *value_base = a.token_first_value
+                                   ? a.value + ((size_t)batch * L * kv_heads + kv_head) * D
+                                   : a.value + ((size_t)batch * kv_heads + kv_head) * L * D;
+
+  const float score_scale = a.scale * 1.4426950408889634f;  // softmax in base 2
+  float running_max = -INFINITY, running_sum = 0.0f;        // of this lane's row; the sum over this lane's keys
+  f16x_t out_acc[JJ];  // O^T[d = ((r / 4) * 8 + half * 4 + r % 4) * JJ + jj][row = row_lane]
+#pragma unroll
+  for (int jj = 0; jj < JJ; ++jj)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) out_acc[jj][r] = 0.0f;
+
+  uint32_t key_end = has_rows ? L : 0;
+  if (a.causal && has_rows) {
+    const uint32_t last_row = min(q0 + 32, a.query_length) - 1;
+    key_end = min((uint64_t)L, (uint64_t)a.past_length + last_row + 1);
+  }
+  uint32_t group_key_end = L;
+  if (a.causal) {
+    const uint32_t group_q0 = slab * kWavesPerBlock * 32;
+    const uint32_t last_row = min(group_q0 + kWavesPerBlock * 32, a.query_length) - 1;
+    group_key_end = min((uint64_t)L, (uint64_t)a.past_length + last_row + 1);
+  }
+  const uint32_t stages = (group_key_end + kStageKeys - 1) / kStageKeys;
+  auto copy_stage = [&](uint32_t stage) __attribute__((always_inline)) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    const uint32_t buffer_base =
+        (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char *)stage_lds + (stage & 1) * 2 * STAGE_BYTES;
+    const uint32_t row_in_copy = lane / PIECES, piece = lane % PIECES;
+#pragma unroll
+    for (int c = 0; c < COPIES; ++c) {
+      const uint32_t copy = wave * COPIES + c;
+      const uint32_t local = copy * KEYS_PER_COPY + row_in_copy;    // row within the stage
+      const uint32_t key = min(stage * kStageKeys + local, L - 1);  // rows past the end repeat the last one
+      const uint16_t *k_src = key_base + (size_t)key * D + ((piece ^ (local & (PIECES - 1))) * 8);
+      const uint16_t *v_src = value_base + (size_t)key * value_row_stride + piece * 8;
+      const uint32_t k_dst = (uint32_t)__builtin_amdgcn_readfirstlane((int)(buffer_base + copy * 1024));
+      const uint32_t v_dst = k_dst + STAGE_BYTES;
+      asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(k_src), "s"(k_dst) : "memory");
+      asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(v_src), "s"(v_dst) : "memory");
+    }
+#endif
+  };
+  auto stage_landed = [&]() __attribute__((always_inline)) {
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's copies; the barrier covers the others'
+    __syncthreads();
+  };
+  if (stages > 0) {
+    copy_stage(0);
+    stage_landed();
+  }
+
+  // scores of one tile of 32 keys: k_tile = its first row in the stage, local0 = that row's index in the stage
+  auto tile_scores = [&](const unsigned char *k_tile, uint32_t local0) __attribute__((always_inline)) {
+    f16x_t score;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) score[r] = 0.0f;
+    const uint32_t local = local0 + row_lane;
+    const unsigned char *k_row = k_tile + row_lane * ROW_BYTES;
+#pragma unroll
+    for (int ks = 0; ks < KSTEPS; ++ks) {
+      const h8_t k_frag = __builtin_bit_cast(
+          h8_t, *reinterpret_cast<const uint4 *>(k_row + (((ks * 2 + half) ^ (local & (PIECES - 1))) * 16)));
+      score = __builtin_amdgcn_mfma_f32_32x32x16_f16(k_frag, q_frag[ks], score, 0, 0, 0);
+    }
+    return score;
+  };
+  // softmax update and P V product of one tile from its scores; v_tile = its first V row in the stage
+  auto tile_update = [&](uint32_t key0, f16x_t score, const unsigned char *v_tile) __attribute__((always_inline)) {
+    // a tile of existing keys, all below the causal limit of the wave's first row, of existing
+    // rows needs no per-score test
+    const bool interior = key0 + 32 <= L && q0 + 32 <= a.query_length && (!a.causal || key0 + 31 <= a.past_length + q0);
+    float tile_max = -INFINITY;
+    if (interior) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        score[r] *= score_scale;
+        tile_max = fmaxf(tile_max, score[r]);
+      }
+    } else {
+      const uint32_t row = q0 + row_lane;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const uint32_t key = key0 + (r >> 2) * 8 + half * 4 + (r & 3);
+        bool allowed = key < L && row < a.query_length;
+        if (a.causal) allowed = allowed && key <= a.past_length + row;
+        score[r] = allowed ? score[r] * score_scale : -INFINITY;
+        tile_max = fmaxf(tile_max, score[r]);
+      }
+    }
+    tile_max = lanes_xor_max(tile_max, 32);
+    const float new_max = fmaxf(running_max, tile_max);
+    // no allowed key yet: keep every exponent finite (the probabilities are zero anyway)
+    const float reference = new_max == -INFINITY ? 0.0f : new_max;
+    const float alpha = __builtin_amdgcn_exp2f(running_max - reference);  // 0 while running_max is -inf
+    running_max = new_max;
+    h8_t p_frag[2];
+    float tile_sum = 0.0f;
+#pragma unroll
+    for (int r = 0; r < 16; ++r) {
+      const float p = __builtin_amdgcn_exp2f(score[r] - reference);
+      tile_sum += p;
+      p_frag[r >> 3][r & 7] = (_Float16)p;
+    }
+    running_sum = running_sum * alpha + tile_sum;
+    if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
+#pragma unroll
+      for (int jj = 0; jj < JJ; ++jj)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) out_acc[jj][r] *= alpha;
+    }
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      // this lane's eight keys of step s, JJ adjacent head_dim values of each
+      uint32_t raw[8][JJ / 2];
+#pragma unroll
+      for (int e = 0; e < 8; ++e) {
+        const uint32_t key_local = s * 16 + (e >> 2) * 8 + half * 4 + (e & 3);
+        const unsigned char *source = v_tile + key_local * ROW_BYTES + row_lane * (JJ * 2);
+        if constexpr (JJ == 4) {
+          const uint2 pair = *reinterpret_cast<const uint2 *>(source);
+          raw[e][0] = pair.x;
+          raw[e][1] = pair.y;
+        } else {
+          raw[e][0] = *reinterpret_cast<const uint32_t *>(source);
+        }
+      }
+#pragma unroll
+      for (int jj = 0; jj < JJ; ++jj) {
+        const uint32_t selector = (jj & 1) ? 0x07060302u : 0x05040100u;
+        uint4 operand;
+        operand.x = __builtin_amdgcn_perm(raw[1][jj >> 1], raw[0][jj >> 1], selector);
+        operand.y = __builtin_amdgcn_perm(raw[3][jj >> 1], raw[2][jj >> 1], selector);
+        operand.z = __builtin_amdgcn_perm(raw[5][jj >> 1], raw[4][jj >> 1], selector);
+        operand.w = __builtin_amdgcn_perm(raw[7][jj >> 1], raw[6][jj >> 1], selector);
+        out_acc[jj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8_t, operand), p_frag[s], out_acc[jj],
+                                                             0, 0, 0);
+      }
+    }
+  };
+
+  // The two tiles of a stage: both score chains go to the matrix pipe first, so the second runs
+  // while the vector unit works on the first tile's softmax.
+  static_assert(kStageKeys == 64, "two tiles of 32 keys per stage");
+  for (uint32_t stage = 0; stage < stages; ++stage) {
+    if (stage + 1 < stages) copy_stage(stage + 1);  // into the buffer every wave left at the last barrier
+    const unsigned char *k_stage = stage_lds + (stage & 1) * 2 * STAGE_BYTES;
+    const unsigned char *v_stage = k_stage + STAGE_BYTES;
+    const uint32_t key0 = stage * kStageKeys;
+    if (key0 < key_end) {
+      const bool second = key0 + 32 < key_end;
+      const f16x_t first_scores = tile_scores(k_stage, 0);
+      f16x_t second_scores = first_scores;
+      if (second) second_scores = tile_scores(k_stage + 32 * ROW_BYTES, 32);
+      tile_update(key0, first_scores, v_stage);
+      if (second) tile_update(key0 + 32, second_scores, v_stage + 32 * ROW_BYTES);
+    }
+    stage_landed();
+  }
+  if (!has_rows) return;
+
+  const float total = lanes_xor_sum(running_sum, 32);
+  const uint32_t row = q0 + row_lane;
+  if (row >= a.query_length) return;
+  const float inverse = total != 0.0f ? 1.0f / total : 0.0f;
+  uint16_t *out_row = a.token_first_output ? a.output + (((size_t)batch * a.query_length + row) * a.heads + head) * D
+                                           : a.output + (((size_t)batch * a.heads + head) * a.query_length + row) * D;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const uint32_t d = ((r >> 2) * 8 + half * 4 + (r & 3)) * JJ;  // the JJ blocks of one r are adjacent in head_dim
+    uint32_t packed[JJ / 2];
+#pragma unroll
+    for (int w = 0; w < JJ / 2; ++w)
+      packed[w] = (uint32_t)float_to_half_bits(out_acc[2 * w][r] * inverse) |
+                  ((uint32_t)float_to_half_bits(out_acc[2 * w + 1][r] * inverse) << 16);
+    if constexpr (JJ == 4)
+      *reinterpret_cast<uint2 *>(out_row + d) = make_uint2(packed[0], packed[1]);
+    else
+      *reinterpret_cast<uint32_t *>(out_row + d) = packed[0];
+  }
+}
+
 // ---- row-serial kernel (every other configuration) ---------------------------
 
 constexpr int kMaxFragments = 8;  // head_dim <= 512
@@ -411,24 +649,23 @@ hipError_t launch_dense_attention(const DenseAttentionArgs &a, hipStream_t strea
     const size_t lds_bytes = 2 * 2 * (size_t)kStageKeys * a.head_dim * 2;
     static bool configured = false;  // the attribute is per device function
     if (shared && !configured) {
-      hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(&dense_attention_mfma_kernel<128, true>),
+      hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(&dense_attention_tile32_kernel<128>),
                                               hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
       if (status == hipSuccess)
-        status = hipFuncSetAttribute(reinterpret_cast<const void *>(&dense_attention_mfma_kernel<64, true>),
+        status = hipFuncSetAttribute(reinterpret_cast<const void *>(&dense_attention_tile32_kernel<64>),
                                      hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
       if (status != hipSuccess) return status;
       configured = true;
     }
+    // no mask: 32 x 32 wave tiles over shared LDS stages; masks: 16-key tiles, every wave fetching its own
     if (a.head_dim == 64) {
       if (shared)
-        hipLaunchKernelGGL((dense_attention_mfma_kernel<64, true>), grid, dim3(kWavesPerBlock * 64), lds_bytes,
-                           stream, a);
+        hipLaunchKernelGGL((dense_attention_tile32_kernel<64>), grid, dim3(kWavesPerBlock * 64), lds_bytes, stream, a);
       else
         hipLaunchKernelGGL((dense_attention_mfma_kernel<64, false>), grid, dim3(kWavesPerBlock * 64), 0, stream, a);
     } else {
       if (shared)
-        hipLaunchKernelGGL((dense_attention_mfma_kernel<128, true>), grid, dim3(kWavesPerBlock * 64), lds_bytes,
-                           stream, a);
+        hipLaunchKernelGGL((dense_attention_tile32_kernel<128>), grid, dim3(kWavesPerBlock * 64), lds_bytes, stream, a);
       else
         hipLaunchKernelGGL((dense_attention_mfma_kernel<128, false>), grid, dim3(kWavesPerBlock * 64), 0, stream, a);
     }
