@@ -335,8 +335,13 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void dense_attention_mfma_kern
 //    end (sum).
 //  * O^T += V^T P^T in two steps of 16 keys: the B operand of step s is the lane's own
 //    probabilities r = 8 s .. 8 s + 7 as halves, no exchange between lanes; the A operand row i
-//    of block jj is head_dim i * (D / 32) + jj, so a lane reads D / 32 adjacent halves of each of
-//    its eight keys and regroups them in registers (one v_perm per operand dword).
+//    of block jj is head_dim 32 jj + i: eight keys at one head_dim, i.e. a column of the V tile,
+//    which ds_read_b64_tr_b16 delivers straight from the row-major stage.  In that instruction
+//    every lane names a 64-bit chunk (four halves) and lane 4 q + c of a group of sixteen receives
+//    element c of the chunks named by lanes q, 4 + q, 8 + q, 12 + q of its group: with lane 4 e + q
+//    naming (key e, head_dim chunk q) a lane gets four keys of one head_dim, and two reads make an
+//    operand.  V rows are stored with their 16-byte pieces XOR-ed by twice the key, so that the
+//    four rows a group touches lie in different banks.
 //
 // Against the 16-key tiles above: the legacy 16x16x16 MFMA of the P V product runs at half the
 // rate of the x32 shapes (16 cycles for 8192 flops), and the per-tile bookkeeping of the online
@@ -383,7 +388,7 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void dense_attention_tile32_ke
 
   const float score_scale = a.scale * 1.4426950408889634f;  // softmax in base 2
   float running_max = -INFINITY, running_sum = 0.0f;        // of this lane's row; the sum over this lane's keys
-  f16x_t out_acc[JJ];  // O^T[d = ((r / 4) * 8 + half * 4 + r % 4) * JJ + jj][row = row_lane]
+  f16x_t out_acc[JJ];  // O^T[d = 32 jj + (r / 4) * 8 + half * 4 + r % 4][row = row_lane]
 #pragma unroll
   for (int jj = 0; jj < JJ; ++jj)
 #pragma unroll
@@ -412,7 +417,7 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void dense_attention_tile32_ke
       const uint32_t local = copy * KEYS_PER_COPY + row_in_copy;    // row within the stage
       const uint32_t key = min(stage * kStageKeys + local, L - 1);  // rows past the end repeat the last one
       const uint16_t *k_src = key_base + (size_t)key * D + ((piece ^ (local & (PIECES - 1))) * 8);
-      const uint16_t *v_src = value_base + (size_t)key * value_row_stride + piece * 8;
+      const uint16_t *v_src = value_base + (size_t)key * value_row_stride + ((piece ^ ((2 * local) & (PIECES - 1))) * 8);
       const uint32_t k_dst = (uint32_t)__builtin_amdgcn_readfirstlane((int)(buffer_base + copy * 1024));
       const uint32_t v_dst = k_dst + STAGE_BYTES;
       asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(k_src), "s"(k_dst) : "memory");
@@ -424,6 +429,19 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void dense_attention_tile32_ke
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's copies; the barrier covers the others'
     __syncthreads();
   };
+  // What this lane names in a transposing read of V: key (lane / 32) * 4 + (lane % 16) / 4 of the
+  // eight keys of a read, head_dim chunk 8 jj + ((lane / 16) % 2) * 4 + lane % 4 of block jj (the
+  // multiples of 16 and 8 keys that steps and reads add leave the swizzle of a row unchanged).
+  uint32_t v_lane_offset[JJ];
+  {
+    const uint32_t group = lane >> 4, p = lane & 15;
+    const uint32_t key_in_read = (group >> 1) * 4 + (p >> 2);
+    const uint32_t chunk = (group & 1) * 4 + (p & 3);
+#pragma unroll
+    for (int jj = 0; jj < JJ; ++jj)
+      v_lane_offset[jj] = key_in_read * ROW_BYTES +
+                          (((jj * 4 + (chunk >> 1)) ^ ((2 * key_in_read) & (PIECES - 1))) * 16) + (chunk & 1) * 8;
+  }
   if (stages > 0) {
     copy_stage(0);
     stage_landed();
@@ -447,15 +465,13 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void dense_attention_tile32_ke
   // softmax update and P V product of one tile from its scores; v_tile = its first V row in the stage
   auto tile_update = [&](uint32_t key0, f16x_t score, const unsigned char *v_tile) __attribute__((always_inline)) {
     // a tile of existing keys, all below the causal limit of the wave's first row, of existing
-    // rows needs no per-score test
+    // rows needs no per-score test.  Maxima are taken over the scores as the MFMAs left them; the
+    // scale (positive) goes into the exponent's multiply-add.
     const bool interior = key0 + 32 <= L && q0 + 32 <= a.query_length && (!a.causal || key0 + 31 <= a.past_length + q0);
     float tile_max = -INFINITY;
     if (interior) {
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        score[r] *= score_scale;
-        tile_max = fmaxf(tile_max, score[r]);
-      }
+      for (int r = 0; r < 16; ++r) tile_max = fmaxf(tile_max, score[r]);
     } else {
       const uint32_t row = q0 + row_lane;
 #pragma unroll
@@ -463,7 +479,7 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void dense_attention_tile32_ke
         const uint32_t key = key0 + (r >> 2) * 8 + half * 4 + (r & 3);
         bool allowed = key < L && row < a.query_length;
         if (a.causal) allowed = allowed && key <= a.past_length + row;
-        score[r] = allowed ? score[r] * score_scale : -INFINITY;
+        score[r] = allowed ? score[r] : -INFINITY;
         tile_max = fmaxf(tile_max, score[r]);
       }
     }
@@ -471,13 +487,14 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void dense_attention_tile32_ke
     const float new_max = fmaxf(running_max, tile_max);
     // no allowed key yet: keep every exponent finite (the probabilities are zero anyway)
     const float reference = new_max == -INFINITY ? 0.0f : new_max;
-    const float alpha = __builtin_amdgcn_exp2f(running_max - reference);  // 0 while running_max is -inf
+    const float alpha = __builtin_amdgcn_exp2f((running_max - reference) * score_scale);  // 0 while running_max is -inf
     running_max = new_max;
+    const float scaled_reference = reference * score_scale;
     h8_t p_frag[2];
     float tile_sum = 0.0f;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      const float p = __builtin_amdgcn_exp2f(score[r] - reference);
+      const float p = __builtin_amdgcn_exp2f(fmaf(score[r], score_scale, -scaled_reference));
       tile_sum += p;
       p_frag[r >> 3][r & 7] = (_Float16)p;
     }
@@ -488,34 +505,20 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void dense_attention_tile32_ke
 #pragma unroll
         for (int r = 0; r < 16; ++r) out_acc[jj][r] *= alpha;
     }
+    typedef short s4_t __attribute__((ext_vector_type(4)));
+    typedef s4_t __attribute__((address_space(3))) * lds_chunk_t;
 #pragma unroll
-    for (int s = 0; s < 2; ++s) {
-      // this lane's eight keys of step s, JJ adjacent head_dim values of each
-      uint32_t raw[8][JJ / 2];
-#pragma unroll
-      for (int e = 0; e < 8; ++e) {
-        const uint32_t key_local = s * 16 + (e >> 2) * 8 + half * 4 + (e & 3);
-        const unsigned char *source = v_tile + key_local * ROW_BYTES + row_lane * (JJ * 2);
-        if constexpr (JJ == 4) {
-          const uint2 pair = *reinterpret_cast<const uint2 *>(source);
-          raw[e][0] = pair.x;
-          raw[e][1] = pair.y;
-        } else {
-          raw[e][0] = *reinterpret_cast<const uint32_t *>(source);
-        }
-      }
+    for (int s = 0; s < 2; ++s)
 #pragma unroll
       for (int jj = 0; jj < JJ; ++jj) {
-        const uint32_t selector = (jj & 1) ? 0x07060302u : 0x05040100u;
-        uint4 operand;
-        operand.x = __builtin_amdgcn_perm(raw[1][jj >> 1], raw[0][jj >> 1], selector);
-        operand.y = __builtin_amdgcn_perm(raw[3][jj >> 1], raw[2][jj >> 1], selector);
-        operand.z = __builtin_amdgcn_perm(raw[5][jj >> 1], raw[4][jj >> 1], selector);
-        operand.w = __builtin_amdgcn_perm(raw[7][jj >> 1], raw[6][jj >> 1], selector);
-        out_acc[jj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(__builtin_bit_cast(h8_t, operand), p_frag[s], out_acc[jj],
-                                                             0, 0, 0);
+        const unsigned char *source = v_tile + v_lane_offset[jj] + s * 16 * ROW_BYTES;
+        const s4_t keys_lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_chunk_t)source);
+        const s4_t keys_hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_chunk_t)(source + 8 * ROW_BYTES));
+        const h8_t operand = __builtin_bit_cast(
+            h8_t, make_uint4(__builtin_bit_cast(uint2, keys_lo).x, __builtin_bit_cast(uint2, keys_lo).y,
+                             __builtin_bit_cast(uint2, keys_hi).x, __builtin_bit_cast(uint2, keys_hi).y));
+        out_acc[jj] = __builtin_amdgcn_mfma_f32_32x32x16_f16(operand, p_frag[s], out_acc[jj], 0, 0, 0);
       }
-    }
   };
 
   // The two tiles of a stage: both score chains go to the matrix pipe first, so the second runs
@@ -545,18 +548,17 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void dense_attention_tile32_ke
   uint16_t *out_row = a.token_first_output ? a.output + (((size_t)batch * a.query_length + row) * a.heads + head) * D
                                            : a.output + (((size_t)batch * a.heads + head) * a.query_length + row) * D;
 #pragma unroll
-  for (int r = 0; r < 16; ++r) {
-    const uint32_t d = ((r >> 2) * 8 + half * 4 + (r & 3)) * JJ;  // the JJ blocks of one r are adjacent in head_dim
-    uint32_t packed[JJ / 2];
+  for (int jj = 0; jj < JJ; ++jj)
 #pragma unroll
-    for (int w = 0; w < JJ / 2; ++w)
-      packed[w] = (uint32_t)float_to_half_bits(out_acc[2 * w][r] * inverse) |
-                  ((uint32_t)float_to_half_bits(out_acc[2 * w + 1][r] * inverse) << 16);
-    if constexpr (JJ == 4)
-      *reinterpret_cast<uint2 *>(out_row + d) = make_uint2(packed[0], packed[1]);
-    else
-      *reinterpret_cast<uint32_t *>(out_row + d) = packed[0];
-  }
+    for (int g = 0; g < 4; ++g) {
+      // r = 4 g .. 4 g + 3 are adjacent in head_dim: one 8-byte store
+      uint2 packed;
+      packed.x = (uint32_t)float_to_half_bits(out_acc[jj][4 * g] * inverse) |
+                 ((uint32_t)float_to_half_bits(out_acc[jj][4 * g + 1] * inverse) << 16);
+      packed.y = (uint32_t)float_to_half_bits(out_acc[jj][4 * g + 2] * inverse) |
+                 ((uint32_t)float_to_half_bits(out_acc[jj][4 * g + 3] * inverse) << 16);
+      *reinterpret_cast<uint2 *>(out_row + 32 * jj + g * 8 + half * 4) = packed;
+    }
 }
 
 // ---- row-serial kernel (every other configuration) ---------------------------
@@ -645,7 +647,9 @@ hipError_t launch_dense_attention(const DenseAttentionArgs &a, hipStream_t strea
     // the shared variant copies 16-byte pieces of whole rows: 16-byte aligned K and V rows
     const size_t value_row_halfs = a.token_first_value ? (size_t)(a.kv_heads > 0 ? a.kv_heads : a.heads) * a.head_dim
                                                        : a.head_dim;
-    const bool shared = !masked && reinterpret_cast<uintptr_t>(a.value) % 16 == 0 && value_row_halfs % 8 == 0;
+    // (the 32 x 32 kernel takes maxima before scaling: a positive, finite scale)
+    const bool shared = !masked && reinterpret_cast<uintptr_t>(a.value) % 16 == 0 && value_row_halfs % 8 == 0 &&
+                        a.scale > 0.0f && a.scale < INFINITY;
     const size_t lds_bytes = 2 * 2 * (size_t)kStageKeys * a.head_dim * 2;
     static bool configured = false;  // the attribute is per device function
     if (shared && !configured) {
