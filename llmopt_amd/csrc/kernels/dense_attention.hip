@@ -347,25 +347,45 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void dense_attention_mfma_kern
 // rate of the x32 shapes (16 cycles for 8192 flops), and the per-tile bookkeeping of the online
 // softmax (exchanges, rescaling, the alpha exponential) is paid once per 32 keys and 32 rows
 // instead of four times.
-template <int D>
-__global__ __launch_bounds__(kWavesPerBlock * 64) void dense_attention_tile32_kernel(DenseAttentionArgs a) {
+// WAVES x 32 query rows per workgroup, STAGE_KEYS keys per LDS stage (launched as 4 x 64: 64 KB at
+// D = 128, two workgroups per CU).
+template <int D, int WAVES, int STAGE_KEYS>
+__global__ __launch_bounds__(WAVES * 64) void dense_attention_tile32_kernel(DenseAttentionArgs a) {
   constexpr int KSTEPS = D / 16;  // score MFMAs per key tile
   constexpr int JJ = D / 32;      // adjacent head_dim values per lane and key = output blocks
   constexpr int ROW_BYTES = D * 2;
   constexpr int PIECES = ROW_BYTES / 16;
   constexpr int KEYS_PER_COPY = 64 / PIECES;
-  constexpr int COPIES = kStageKeys / KEYS_PER_COPY / kWavesPerBlock;
-  constexpr int STAGE_BYTES = kStageKeys * ROW_BYTES;
+  constexpr int COPIES = STAGE_KEYS / KEYS_PER_COPY / WAVES;
+  constexpr int STAGE_BYTES = STAGE_KEYS * ROW_BYTES;
   static_assert(JJ == 2 || JJ == 4, "head_dim 64 or 128");
+  static_assert((STAGE_KEYS == 64 || STAGE_KEYS == 32) && COPIES >= 1 && COPIES * KEYS_PER_COPY * WAVES == STAGE_KEYS, "stage");
   extern __shared__ __attribute__((aligned(16))) unsigned char stage_lds[];  // [2 stages][K | V]
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t wave = threadIdx.x >> 6;
   const uint32_t row_lane = lane & 31;
   const uint32_t half = lane >> 5;
-  const uint32_t head = blockIdx.y;
-  const uint32_t batch = blockIdx.z;
-  const uint32_t slab = a.causal ? gridDim.x - 1 - blockIdx.x : blockIdx.x;  // longest causal slabs first
-  const uint32_t q0 = (slab * kWavesPerBlock + wave) * 32;
+  // Which (row slab, head, batch) this workgroup takes.  The grid is one-dimensional; rank 0.. runs over
+  // the slabs from the last (the most keys under a causal limit) to the first, heads and batches within a
+  // slab.  Workgroups go to the XCDs round-robin and, within an XCD, to its CUs in order: XCD x takes
+  // ranks x, x + 8, .. (every XCD gets every length), and of each run of two workgroups per CU the second
+  // half is taken backwards, so that the CU that got the longest of the run also gets the shortest.
+  // Without this a launch of as many workgroups as the device holds - 16 slabs x 32 heads at 2048 tokens -
+  // puts the two longest on one CU and all of one length on one XCD, and lasts as long as they do.
+  const uint32_t slabs = (a.query_length + WAVES * 32 - 1) / (WAVES * 32);
+  const uint32_t per_slab = a.heads * a.batches;
+  uint32_t rank = blockIdx.x;
+  if (a.causal && gridDim.x % 8 == 0 && a.cus_per_xcd > 0) {
+    const uint32_t xcd = blockIdx.x % 8, position = blockIdx.x / 8, run = 2 * a.cus_per_xcd;
+    const uint32_t start = position / run * run, within = position % run;
+    uint32_t taken = position;
+    if (within >= a.cus_per_xcd && start + run <= gridDim.x / 8) taken = start + a.cus_per_xcd + (run - 1 - within);
+    rank = taken * 8 + xcd;
+  }
+  const uint32_t slab = a.causal ? slabs - 1 - rank / per_slab : rank / per_slab;
+  const uint32_t head = rank % per_slab % a.heads;
+  const uint32_t batch = rank % per_slab / a.heads;
+  const uint32_t q0 = (slab * WAVES + wave) * 32;
   const bool has_rows = q0 < a.query_length;  // a wave without rows still copies and meets the barriers
   const uint32_t kv_heads = a.kv_heads > 0 ? a.kv_heads : a.heads;
   const uint32_t kv_head = kv_heads < a.heads ? head / (a.heads / kv_heads) : head;
@@ -380,9 +400,9 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void dense_attention_tile32_ke
     for (int ks = 0; ks < KSTEPS; ++ks)
       q_frag[ks] = __builtin_bit_cast(h8_t, *reinterpret_cast<const uint4 *>(q_row + ks * 16 + half * 8));
   }
-  const uint16_t *key_base = a.key + ((size_t)batch * kv_heads + kv_head) * L * D;
-  const size_t value_row_stride = a.token_first_value ? (size_t)kv_heads * D : D;
-  const uint16_t *value_base = a.token_first_value
+  [[maybe_unused]] const uint16_t *key_base = a.key + ((size_t)batch * kv_heads + kv_head) * L * D;
+  [[maybe_unused]] const size_t value_row_stride = a.token_first_value ? (size_t)kv_heads * D : D;
+  [[maybe_unused]] const uint16_t *value_base = a.token_first_value
                                    ? a.value + ((size_t)batch * L * kv_heads + kv_head) * D
                                    : a.value + ((size_t)batch * kv_heads + kv_head) * L * D;
 
@@ -401,11 +421,11 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void dense_attention_tile32_ke
   }
   uint32_t group_key_end = L;
   if (a.causal) {
-    const uint32_t group_q0 = slab * kWavesPerBlock * 32;
-    const uint32_t last_row = min(group_q0 + kWavesPerBlock * 32, a.query_length) - 1;
+    const uint32_t group_q0 = slab * WAVES * 32;
+    const uint32_t last_row = min(group_q0 + WAVES * 32, a.query_length) - 1;
     group_key_end = min((uint64_t)L, (uint64_t)a.past_length + last_row + 1);
   }
-  const uint32_t stages = (group_key_end + kStageKeys - 1) / kStageKeys;
+  const uint32_t stages = (group_key_end + STAGE_KEYS - 1) / STAGE_KEYS;
   auto copy_stage = [&](uint32_t stage) __attribute__((always_inline)) {
 #if defined(__HIP_DEVICE_COMPILE__)
     const uint32_t buffer_base =
@@ -415,7 +435,7 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void dense_attention_tile32_ke
     for (int c = 0; c < COPIES; ++c) {
       const uint32_t copy = wave * COPIES + c;
       const uint32_t local = copy * KEYS_PER_COPY + row_in_copy;    // row within the stage
-      const uint32_t key = min(stage * kStageKeys + local, L - 1);  // rows past the end repeat the last one
+      const uint32_t key = min(stage * STAGE_KEYS + local, L - 1);  // rows past the end repeat the last one
       const uint16_t *k_src = key_base + (size_t)key * D + ((piece ^ (local & (PIECES - 1))) * 8);
       const uint16_t *v_src = value_base + (size_t)key * value_row_stride + ((piece ^ ((2 * local) & (PIECES - 1))) * 8);
       const uint32_t k_dst = (uint32_t)__builtin_amdgcn_readfirstlane((int)(buffer_base + copy * 1024));
@@ -521,21 +541,24 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void dense_attention_tile32_ke
       }
   };
 
-  // The two tiles of a stage: both score chains go to the matrix pipe first, so the second runs
+  // The tiles of a stage.  Two: both score chains go to the matrix pipe first, so the second runs
   // while the vector unit works on the first tile's softmax.
-  static_assert(kStageKeys == 64, "two tiles of 32 keys per stage");
   for (uint32_t stage = 0; stage < stages; ++stage) {
     if (stage + 1 < stages) copy_stage(stage + 1);  // into the buffer every wave left at the last barrier
     const unsigned char *k_stage = stage_lds + (stage & 1) * 2 * STAGE_BYTES;
     const unsigned char *v_stage = k_stage + STAGE_BYTES;
-    const uint32_t key0 = stage * kStageKeys;
+    const uint32_t key0 = stage * STAGE_KEYS;
     if (key0 < key_end) {
-      const bool second = key0 + 32 < key_end;
       const f16x_t first_scores = tile_scores(k_stage, 0);
-      f16x_t second_scores = first_scores;
-      if (second) second_scores = tile_scores(k_stage + 32 * ROW_BYTES, 32);
-      tile_update(key0, first_scores, v_stage);
-      if (second) tile_update(key0 + 32, second_scores, v_stage + 32 * ROW_BYTES);
+      if constexpr (STAGE_KEYS == 64) {
+        const bool second = key0 + 32 < key_end;
+        f16x_t second_scores = first_scores;
+        if (second) second_scores = tile_scores(k_stage + 32 * ROW_BYTES, 32);
+        tile_update(key0, first_scores, v_stage);
+        if (second) tile_update(key0 + 32, second_scores, v_stage + 32 * ROW_BYTES);
+      } else {
+        tile_update(key0, first_scores, v_stage);
+      }
     }
     stage_landed();
   }
@@ -650,28 +673,34 @@ hipError_t launch_dense_attention(const DenseAttentionArgs &a, hipStream_t strea
     // (the 32 x 32 kernel takes maxima before scaling: a positive, finite scale)
     const bool shared = !masked && reinterpret_cast<uintptr_t>(a.value) % 16 == 0 && value_row_halfs % 8 == 0 &&
                         a.scale > 0.0f && a.scale < INFINITY;
-    const size_t lds_bytes = 2 * 2 * (size_t)kStageKeys * a.head_dim * 2;
     static bool configured = false;  // the attribute is per device function
     if (shared && !configured) {
-      hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(&dense_attention_tile32_kernel<128>),
+      hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(&dense_attention_tile32_kernel<128, 4, 64>),
                                               hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
-      if (status == hipSuccess)
-        status = hipFuncSetAttribute(reinterpret_cast<const void *>(&dense_attention_tile32_kernel<64>),
-                                     hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
       if (status != hipSuccess) return status;
       configured = true;
     }
-    // no mask: 32 x 32 wave tiles over shared LDS stages; masks: 16-key tiles, every wave fetching its own
-    if (a.head_dim == 64) {
-      if (shared)
-        hipLaunchKernelGGL((dense_attention_tile32_kernel<64>), grid, dim3(kWavesPerBlock * 64), lds_bytes, stream, a);
+    if (shared) {
+      // 32 x 32 wave tiles over shared LDS stages, four waves and 64 keys a stage.  (Workgroups of two
+      // waves with 32-key stages, twice as many and four per CU, so that short causal launches are not
+      // as long as their longest workgroup, measured slower: 105.6 against 91.2 us at 32 heads x 2048
+      // tokens - one tile per barrier, half the sharing.)
+      const size_t bytes = 2 * 2 * (size_t)64 * a.head_dim * 2;
+      const uint64_t workgroups = (uint64_t)grid.x * a.heads * a.batches;
+      if (workgroups > 0x7fffffffull) return hipErrorInvalidValue;
+      DenseAttentionArgs scheduled = a;
+      scheduled.cus_per_xcd = (uint32_t)device_compute_units() / 8;
+      if (a.head_dim == 64)
+        hipLaunchKernelGGL((dense_attention_tile32_kernel<64, 4, 64>), dim3((uint32_t)workgroups), dim3(256), bytes,
+                           stream, scheduled);
       else
-        hipLaunchKernelGGL((dense_attention_mfma_kernel<64, false>), grid, dim3(kWavesPerBlock * 64), 0, stream, a);
+        hipLaunchKernelGGL((dense_attention_tile32_kernel<128, 4, 64>), dim3((uint32_t)workgroups), dim3(256), bytes,
+                           stream, scheduled);
+    } else if (a.head_dim == 64) {
+      // masks: 16-key tiles, every wave fetching its own
+      hipLaunchKernelGGL((dense_attention_mfma_kernel<64, false>), grid, dim3(kWavesPerBlock * 64), 0, stream, a);
     } else {
-      if (shared)
-        hipLaunchKernelGGL((dense_attention_tile32_kernel<128>), grid, dim3(kWavesPerBlock * 64), lds_bytes, stream, a);
-      else
-        hipLaunchKernelGGL((dense_attention_mfma_kernel<128, false>), grid, dim3(kWavesPerBlock * 64), 0, stream, a);
+      hipLaunchKernelGGL((dense_attention_mfma_kernel<128, false>), grid, dim3(kWavesPerBlock * 64), 0, stream, a);
     }
     return hipGetLastError();
   }

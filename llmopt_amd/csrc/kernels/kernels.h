@@ -173,6 +173,7 @@ struct DenseAttentionArgs {
   uint32_t batches, heads, query_length, key_length, head_dim, mask_batches, mask_heads, causal;
   float scale;
   uint32_t kv_heads, token_first_output, past_length, token_first_value, mask_dtype;
+  uint32_t cus_per_xcd = 0;  // set by the launcher (workgroup order of the causal launch)
 };
 hipError_t launch_dense_attention(const DenseAttentionArgs &args, hipStream_t stream);
 
