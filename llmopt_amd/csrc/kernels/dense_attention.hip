@@ -8,7 +8,9 @@
 // kv_head = head / (h / kvh), output head-major [b, h, q, D] or token-major
 // [b, q, h, D]; a row with no allowed key is zero.  Scores and softmax in fp32.
 //
-//  * dense_attention_mfma_kernel<D> (D = 64, 128): a wave owns 32 query rows of
+//  * dense_attention_tile32_kernel<D> (D = 64, 128, no mask - the prefill path): 32 x 32 wave tiles
+//    on v_mfma_f32_32x32x16_f16 over K / V stages shared through LDS; described at the kernel.
+//  * dense_attention_mfma_kernel<D> (D = 64, 128, with a mask): a wave owns 32 query rows of
 //    one head and walks the keys in tiles of 16 with an online softmax in base
 //    2.  S^T = K Q^T on v_mfma_f32_16x16x32_f16, so that a lane's four scores
 //    belong to one query row (its column) and feed, converted to fp16, the B
@@ -55,27 +57,11 @@ __device__ __forceinline__ bool mask_allows(const DenseAttentionArgs &a, uint32_
 constexpr int kQueryTiles = 2;    // 16-row query tiles per wave
 constexpr int kWavesPerBlock = 4;  // consecutive 32-row slabs of one head
 
-constexpr int kStageKeys = 64;  // keys per LDS stage of the SHARED variant
-
-// SHARED: the four waves of a workgroup (128 consecutive query rows of one head) walk the same
-// keys, so K and V go global -> LDS once per workgroup, 64 keys a stage and a stage ahead of
-// the arithmetic, as direct copies that pass no registers (global_load_lds_dwordx4: 64 lanes x
-// 16 bytes land at consecutive LDS addresses, i.e. whole K / V rows side by side), and the waves
-// read their MFMA operands from LDS.  The 16-byte pieces of a K row are stored XOR-swizzled by
-// the key so that the operand reads (one piece of 8..16 different keys per cycle) hit different
-// banks.  Without SHARED every wave fetches its own tiles from global memory in operand order -
-// four times the requests, each touching 16 cache lines - which bounds the kernel by the number
-// of requests; that variant remains for masks.
-template <int D, bool SHARED>
+// Every wave fetches its own K and V tiles from global memory in operand order.
+template <int D>
 __global__ __launch_bounds__(kWavesPerBlock * 64) void dense_attention_mfma_kernel(DenseAttentionArgs a) {
   constexpr int QSTEPS = D / 32;   // score MFMAs per tile pair
   constexpr int VBLOCKS = D / 64;  // 64-wide head_dim blocks of the V transposes
-  constexpr int ROW_BYTES = D * 2;                  // a K or V row in LDS
-  constexpr int PIECES = ROW_BYTES / 16;            // 16-byte pieces per row
-  constexpr int KEYS_PER_COPY = 64 / PIECES;        // rows one copy instruction brings
-  [[maybe_unused]] constexpr int COPIES = kStageKeys / KEYS_PER_COPY / kWavesPerBlock;  // per wave, stage and operand
-  constexpr int STAGE_BYTES = kStageKeys * ROW_BYTES;
-  extern __shared__ __attribute__((aligned(16))) unsigned char stage_lds[];  // [2 stages][K | V]
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t wave = threadIdx.x >> 6;
   const uint32_t col = lane & 15;
@@ -85,9 +71,7 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void dense_attention_mfma_kern
   // with a causal limit the last rows see the most keys: hand them out first
   const uint32_t slab = a.causal ? gridDim.x - 1 - blockIdx.x : blockIdx.x;
   const uint32_t q0 = (slab * kWavesPerBlock + wave) * (kQueryTiles * 16);
-  // a wave without rows: gone (no barriers), or - SHARED - still copying and meeting the barriers
-  const bool has_rows = q0 < a.query_length;
-  if (!SHARED && !has_rows) return;
+  if (q0 >= a.query_length) return;  // a wave without rows (no barriers in this kernel)
   const uint32_t kv_heads = a.kv_heads > 0 ? a.kv_heads : a.heads;
   const uint32_t kv_head = kv_heads < a.heads ? head / (a.heads / kv_heads) : head;
   const bool masked = a.mask != nullptr && a.mask_batches > 0;
@@ -123,68 +107,18 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void dense_attention_mfma_kern
   }
 
   // keys this wave can need: all of them, or up to the causal limit of its last row
-  uint32_t key_end = has_rows ? L : 0;
-  if (a.causal && has_rows) {
+  uint32_t key_end = L;
+  if (a.causal) {
     const uint32_t last_row = min(q0 + kQueryTiles * 16, a.query_length) - 1;
     key_end = min((uint64_t)L, (uint64_t)a.past_length + last_row + 1);
   }
-  // SHARED: the keys the workgroup needs (those of its last row), in stages
-  uint32_t group_key_end = L;
-  if (SHARED && a.causal) {
-    const uint32_t group_q0 = slab * kWavesPerBlock * (kQueryTiles * 16);
-    const uint32_t last_row = min(group_q0 + kWavesPerBlock * kQueryTiles * 16, a.query_length) - 1;
-    group_key_end = min((uint64_t)L, (uint64_t)a.past_length + last_row + 1);
-  }
-  const uint32_t stages = SHARED ? (group_key_end + kStageKeys - 1) / kStageKeys : 0;
-  // copy of stage `stage` into LDS buffer stage % 2: this wave's share of the K and V rows
-  auto copy_stage = [&](uint32_t stage) __attribute__((always_inline)) {
-#if defined(__HIP_DEVICE_COMPILE__)
-    const uint32_t buffer_base =
-        (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char *)stage_lds + (stage & 1) * 2 * STAGE_BYTES;
-    const uint32_t row_in_copy = lane / PIECES, piece = lane % PIECES;
-#pragma unroll
-    for (int c = 0; c < COPIES; ++c) {
-      const uint32_t copy = wave * COPIES + c;
-      const uint32_t local = copy * KEYS_PER_COPY + row_in_copy;  // row within the stage
-      const uint32_t key = min(stage * kStageKeys + local, L - 1);  // rows past the end repeat the last one
-      const uint16_t *k_src = key_base + (size_t)key * D + ((piece ^ (local & (PIECES - 1))) * 8);
-      const uint16_t *v_src = value_base + (size_t)key * value_row_stride + piece * 8;
-      const uint32_t k_dst = (uint32_t)__builtin_amdgcn_readfirstlane((int)(buffer_base + copy * 1024));
-      const uint32_t v_dst = k_dst + STAGE_BYTES;
-      asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(k_src), "s"(k_dst) : "memory");
-      asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(v_src), "s"(v_dst) : "memory");
-    }
-#endif
-  };
-  auto stage_landed = [&]() __attribute__((always_inline)) {
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // this wave's copies; the barrier covers the others'
-    __syncthreads();
-  };
-  if (SHARED && stages > 0) {
-    copy_stage(0);
-    stage_landed();
-  }
 
-  // one 16-key tile: operands from LDS (SHARED: `tile_lds` = the tile's first row of the stage) or global
-  auto process_tile = [&](uint32_t key0, const unsigned char *k_tile, const unsigned char *v_tile, uint32_t local0)
-      __attribute__((always_inline)) {
+  // one 16-key tile
+  auto process_tile = [&](uint32_t key0) __attribute__((always_inline)) {
     // A operand: K[key = col][d = j*32 + quad*8 ..]; keys past the end repeat the last one (masked below)
     h8_t k_frag[QSTEPS];
     uint2 v_raw[VBLOCKS][4];
-    if (SHARED) {
-      const uint32_t local = local0 + col;
-      const unsigned char *k_row = k_tile + col * ROW_BYTES;
-#pragma unroll
-      for (int j = 0; j < QSTEPS; ++j)
-        k_frag[j] = __builtin_bit_cast(
-            h8_t, *reinterpret_cast<const uint4 *>(k_row + (((j * 4 + quad) ^ (local & (PIECES - 1))) * 16)));
-#pragma unroll
-      for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int blk = 0; blk < VBLOCKS; ++blk)
-          v_raw[blk][i] =
-              *reinterpret_cast<const uint2 *>(v_tile + (quad * 4 + i) * ROW_BYTES + (blk * 64 + col * 4) * 2);
-    } else {
+    {
       const uint16_t *k_row = key_base + (size_t)min(key0 + col, L - 1) * D;
 #pragma unroll
       for (int j = 0; j < QSTEPS; ++j)
@@ -278,22 +212,7 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void dense_attention_mfma_kern
     }
   };
 
-  if (SHARED) {
-    for (uint32_t stage = 0; stage < stages; ++stage) {
-      if (stage + 1 < stages) copy_stage(stage + 1);  // into the buffer every wave left at the last barrier
-      const unsigned char *k_stage = stage_lds + (stage & 1) * 2 * STAGE_BYTES;
-#pragma unroll
-      for (int sub = 0; sub < kStageKeys / 16; ++sub) {
-        const uint32_t key0 = stage * kStageKeys + sub * 16;
-        if (key0 < key_end)
-          process_tile(key0, k_stage + sub * 16 * ROW_BYTES, k_stage + STAGE_BYTES + sub * 16 * ROW_BYTES, sub * 16);
-      }
-      stage_landed();
-    }
-    if (!has_rows) return;
-  } else {
-    for (uint32_t key0 = 0; key0 < key_end; key0 += 16) process_tile(key0, nullptr, nullptr, 0);
-  }
+  for (uint32_t key0 = 0; key0 < key_end; key0 += 16) process_tile(key0);
 
   // out_acc[t][blk*4 + jj][i] is O[row = q0 + t*16 + col][d = blk*64 + 4*(quad*4 + i) + jj]
 #pragma unroll
@@ -323,10 +242,13 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void dense_attention_mfma_kern
 
 // ---- 32 x 32 wave tiles (no mask) --------------------------------------------------------------
 //
-// The same workgroup geometry and LDS staging as the SHARED variant above (four waves = 128
-// consecutive query rows of one head; K and V rows copied global -> LDS 64 keys a stage), with
-// the arithmetic on v_mfma_f32_32x32x16_f16: a wave owns ONE tile of 32 query rows and walks the
-// keys 32 at a time.
+// The four waves of a workgroup - 128 consecutive query rows of one head - walk the same keys, so
+// K and V go global -> LDS once per workgroup, 64 keys a stage and a stage ahead of the
+// arithmetic, as direct copies that pass no registers (global_load_lds_dwordx4: 64 lanes x 16
+// bytes land at consecutive LDS addresses, i.e. whole K / V rows side by side), one barrier per
+// stage.  The 16-byte pieces of a row are stored XOR-swizzled by the key so that operand reads
+// (one piece of many different keys per cycle) hit different banks.  The arithmetic runs on
+// v_mfma_f32_32x32x16_f16: a wave owns ONE tile of 32 query rows and walks the keys 32 at a time.
 //
 //  * S^T = K Q^T: A = K (rows = keys), B = Q^T (columns = query rows), D / 16 chained MFMAs.  Lane
 //    (j = lane % 32, half = lane / 32) ends with the sixteen scores of query row j and keys
@@ -698,9 +620,9 @@ hipError_t launch_dense_attention(const DenseAttentionArgs &a, hipStream_t strea
                            stream, scheduled);
     } else if (a.head_dim == 64) {
       // masks: 16-key tiles, every wave fetching its own
-      hipLaunchKernelGGL((dense_attention_mfma_kernel<64, false>), grid, dim3(kWavesPerBlock * 64), 0, stream, a);
+      hipLaunchKernelGGL((dense_attention_mfma_kernel<64>), grid, dim3(kWavesPerBlock * 64), 0, stream, a);
     } else {
-      hipLaunchKernelGGL((dense_attention_mfma_kernel<128, false>), grid, dim3(kWavesPerBlock * 64), 0, stream, a);
+      hipLaunchKernelGGL((dense_attention_mfma_kernel<128>), grid, dim3(kWavesPerBlock * 64), 0, stream, a);
     }
     return hipGetLastError();
   }
