@@ -156,6 +156,31 @@ def test_single_query_row_and_tiny_shapes(runtime):
         assert_close_to_oracle(got, want, f"tiny D={dim} q={q_len} L={length}")
 
 
+@pytest.mark.parametrize("causal", [True, False])
+def test_device_filling_launch_against_sampled_rows(runtime, causal):
+    """32 heads x 2048 rows: 512 workgroups, as many as the device holds at once.  The kernel maps
+    its one-dimensional grid to (row slab, head) itself - every XCD every slab length, the second
+    half of each run of workgroups backwards - and every output row must still be the right one:
+    all heads, one row out of every 29 (every 128-row slab is hit) against the oracle."""
+    rng = np.random.default_rng(123 + causal)
+    heads, kv_heads, length, dim = 32, 8, 2048, 64
+    query = rng.standard_normal((1, heads, length, dim)).astype(np.float16)
+    key = rng.standard_normal((1, kv_heads, length, dim)).astype(np.float16)
+    value = rng.standard_normal((1, kv_heads, length, dim)).astype(np.float16)
+    scale = 1.0 / math.sqrt(dim)
+    params = attention_params(1, heads, length, length, dim, 0, 0, causal, scale, kv_heads)
+    print(f"dense attention 32 heads x 2048 rows causal={causal}", flush=True)
+    got = run(runtime, "llmopt_attention_f16_simd_h64", query, key, value, None, params, (1, heads, length, dim))
+    rows = np.unique(np.concatenate([[0, 31, 32, length - 1], np.arange(5, length, 29)]))
+    allowed = np.ones((len(rows), length), dtype=bool)
+    if causal:
+        allowed = np.arange(length)[None, :] <= rows[:, None]
+    want = expected(query[:, :, rows], key, value, np.broadcast_to(allowed[None, None], (1, heads, len(rows), length)),
+                    scale)
+    assert_close_to_oracle(got[:, :, rows], want, f"sampled rows, causal={causal}")
+    assert not np.any(got.view(np.uint16) == 0x7e00)  # every row was written
+
+
 def test_softmax_shift_invariance_at_full_size(runtime):
     """Prefill 2048 x 2048, D = 128: a property the oracle is too slow for.  With every key equal
     the output is the running mean of V (closed form), whatever the scores are."""
