@@ -308,7 +308,12 @@ hipError_t launch_rows(const QuadParams &p, hipStream_t stream) {
     }
   }
   if (plan.waves <= 4) return launch_instance<MR, KL, 2, 8, 2, 256>(p, plan.grid, plan.waves, stream);
-  return launch_instance<MR, KL, 2, 8, 2, 448>(p, plan.grid, plan.waves, stream);
+  // (four rows of K = 14336 on more than four waves of two quads spill registers: w4a16_gemv_quad_ok
+  // sends that shape - N above 8192 at K = 14336 - to the other kernels)
+  if constexpr (MR == 4 && KL > 8)
+    return hipErrorInvalidValue;
+  else
+    return launch_instance<MR, KL, 2, 8, 2, 448>(p, plan.grid, plan.waves, stream);
 }
 
 template <int KL>
@@ -323,7 +328,10 @@ hipError_t launch_k(const QuadParams &p, hipStream_t stream) {
 bool w4a16_gemv_quad_ok(const W4LinearArgs &a) {
   if (a.m == 0 || a.m > 4 || a.y == nullptr || a.y_f32 != nullptr) return false;
   if (a.k != 4096 && a.k != 14336) return false;
-  if (a.n % 4 != 0 || quad_plan(a.n).rq == 0) return false;
+  if (a.n % 4 != 0) return false;
+  const QuadPlan plan = quad_plan(a.n);
+  if (plan.rq == 0) return false;
+  if (a.k == 14336 && a.m > 2 && plan.rq == 2 && plan.waves > 4) return false;  // no instantiation without spills
   // 16-byte loads of activation rows, weight row pieces and scale rows
   if (((reinterpret_cast<uintptr_t>(a.x) | reinterpret_cast<uintptr_t>(a.w.weight) |
         reinterpret_cast<uintptr_t>(a.w.scale)) & 15) != 0)
