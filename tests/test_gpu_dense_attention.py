@@ -144,6 +144,23 @@ def test_masks_and_rows_without_keys(runtime, mask_dtype, dim):
     assert_close_to_oracle(got, want, f"masked attention dtype={mask_dtype} D={dim}")
 
 
+@pytest.mark.parametrize("dim,q_len,length", [(128, 45, 77), (64, 33, 130), (128, 16, 64), (64, 100, 31)])
+def test_ragged_shapes_without_mask_or_causal_limit(runtime, dim, q_len, length):
+    """The 32 x 32-tile kernel with a last key tile and a last row tile that are only partly there
+    (keys past the end are staged as copies of the last row and must weigh nothing)."""
+    rng = np.random.default_rng(dim + q_len + length)
+    batches, heads, kv_heads = 2, 4, 2
+    query = rng.standard_normal((batches, heads, q_len, dim)).astype(np.float16)
+    key = rng.standard_normal((batches, kv_heads, length, dim)).astype(np.float16)
+    value = rng.standard_normal((batches, kv_heads, length, dim)).astype(np.float16)
+    scale = 1.0 / math.sqrt(dim)
+    params = attention_params(batches, heads, q_len, length, dim, 0, 0, False, scale, kv_heads)
+    got = run(runtime, f"llmopt_attention_f16_simd_h{dim}", query, key, value, None, params,
+              (batches, heads, q_len, dim))
+    want = expected(query, key, value, np.ones((batches, heads, q_len, length), dtype=bool), scale)
+    assert_close_to_oracle(got, want, f"ragged D={dim} q={q_len} L={length}")
+
+
 def test_single_query_row_and_tiny_shapes(runtime):
     rng = np.random.default_rng(21)
     for dim, q_len, length in ((64, 1, 17), (128, 3, 5), (8, 4, 9)):
