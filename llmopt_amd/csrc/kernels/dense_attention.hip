@@ -8,16 +8,8 @@
 // kv_head = head / (h / kvh), output head-major [b, h, q, D] or token-major
 // [b, q, h, D]; a row with no allowed key is zero.  Scores and softmax in fp32.
 //
-//  * dense_attention_tile32_kernel<D> (D = 64, 128, no mask - the prefill path): 32 x 32 wave tiles
-//    on v_mfma_f32_32x32x16_f16 over K / V stages shared through LDS; described at the kernel.
-//  * dense_attention_mfma_kernel<D> (D = 64, 128, with a mask): a wave owns 32 query rows of
-//    one head and walks the keys in tiles of 16 with an online softmax in base
-//    2.  S^T = K Q^T on v_mfma_f32_16x16x32_f16, so that a lane's four scores
-//    belong to one query row (its column) and feed, converted to fp16, the B
-//    operand of O^T = V^T P^T on v_mfma_f32_16x16x16f16 without any exchange
-//    between lanes; V tiles are transposed in registers (4 keys x 4 head_dim
-//    halfs per lane).  Key tiles past the causal limit of the wave's rows are
-//    skipped.
+//  * dense_attention_tile32_kernel<D> (D = 64, 128): 32 x 32 wave tiles on
+//    v_mfma_f32_32x32x16_f16 over K / V stages shared through LDS; described at the kernel.
 //  * dense_attention_rows_kernel: one wave per output row, serial over the keys
 //    (any D up to 512, every option); the direct restatement.
 #include <algorithm>
@@ -54,193 +46,9 @@ __device__ __forceinline__ bool mask_allows(const DenseAttentionArgs &a, uint32_
   return a.mask[index] != 0;
 }
 
-constexpr int kQueryTiles = 2;    // 16-row query tiles per wave
 constexpr int kWavesPerBlock = 4;  // consecutive 32-row slabs of one head
 
-// Every wave fetches its own K and V tiles from global memory in operand order.
-template <int D>
-__global__ __launch_bounds__(kWavesPerBlock * 64) void dense_attention_mfma_kernel(DenseAttentionArgs a) {
-  constexpr int QSTEPS = D / 32;   // score MFMAs per tile pair
-  constexpr int VBLOCKS = D / 64;  // 64-wide head_dim blocks of the V transposes
-  const uint32_t lane = threadIdx.x & 63;
-  const uint32_t wave = threadIdx.x >> 6;
-  const uint32_t col = lane & 15;
-  const uint32_t quad = lane >> 4;
-  const uint32_t head = blockIdx.y;
-  const uint32_t batch = blockIdx.z;
-  // with a causal limit the last rows see the most keys: hand them out first
-  const uint32_t slab = a.causal ? gridDim.x - 1 - blockIdx.x : blockIdx.x;
-  const uint32_t q0 = (slab * kWavesPerBlock + wave) * (kQueryTiles * 16);
-  if (q0 >= a.query_length) return;  // a wave without rows (no barriers in this kernel)
-  const uint32_t kv_heads = a.kv_heads > 0 ? a.kv_heads : a.heads;
-  const uint32_t kv_head = kv_heads < a.heads ? head / (a.heads / kv_heads) : head;
-  const bool masked = a.mask != nullptr && a.mask_batches > 0;
-  const uint32_t L = a.key_length;
-
-  // B operand of the score MFMAs: Q[row = col][d = j*32 + quad*8 ..], rows past the end repeat the last one
-  h8_t q_frag[kQueryTiles][QSTEPS];
-#pragma unroll
-  for (int t = 0; t < kQueryTiles; ++t) {
-    const uint32_t row = min(q0 + t * 16 + col, a.query_length - 1);
-    const uint16_t *q_row = a.query + (((size_t)batch * a.heads + head) * a.query_length + row) * D;
-#pragma unroll
-    for (int j = 0; j < QSTEPS; ++j)
-      q_frag[t][j] = __builtin_bit_cast(h8_t, *reinterpret_cast<const uint4 *>(q_row + j * 32 + quad * 8));
-  }
-
-  const uint16_t *key_base = a.key + ((size_t)batch * kv_heads + kv_head) * L * D;
-  const size_t value_row_stride = a.token_first_value ? (size_t)kv_heads * D : D;
-  const uint16_t *value_base = a.token_first_value
-                                   ? a.value + ((size_t)batch * L * kv_heads + kv_head) * D
-                                   : a.value + ((size_t)batch * kv_heads + kv_head) * L * D;
-
-  // softmax in base 2
-  const float score_scale = a.scale * 1.4426950408889634f;
-  float running_max[kQueryTiles], running_sum[kQueryTiles];  // per lane: row col of each tile; sum over this quad's keys
-  f4_t out_acc[kQueryTiles][VBLOCKS * 4];                    // O^T[d = blk*64 + 4*(quad*4+i) + jj][row col]
-#pragma unroll
-  for (int t = 0; t < kQueryTiles; ++t) {
-    running_max[t] = -INFINITY;
-    running_sum[t] = 0.0f;
-#pragma unroll
-    for (int v = 0; v < VBLOCKS * 4; ++v) out_acc[t][v] = f4_t{0.0f, 0.0f, 0.0f, 0.0f};
-  }
-
-  // keys this wave can need: all of them, or up to the causal limit of its last row
-  uint32_t key_end = L;
-  if (a.causal) {
-    const uint32_t last_row = min(q0 + kQueryTiles * 16, a.query_length) - 1;
-    key_end = min((uint64_t)L, (uint64_t)a.past_length + last_row + 1);
-  }
-
-  // one 16-key tile
-  auto process_tile = [&](uint32_t key0) __attribute__((always_inline)) {
-    // A operand: K[key = col][d = j*32 + quad*8 ..]; keys past the end repeat the last one (masked below)
-    h8_t k_frag[QSTEPS];
-    uint2 v_raw[VBLOCKS][4];
-    {
-      const uint16_t *k_row = key_base + (size_t)min(key0 + col, L - 1) * D;
-#pragma unroll
-      for (int j = 0; j < QSTEPS; ++j)
-        k_frag[j] = __builtin_bit_cast(h8_t, *reinterpret_cast<const uint4 *>(k_row + j * 32 + quad * 8));
-      // V: lane (c = col, quad) reads head_dim c*4 .. c*4+3 of keys quad*4 + i
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const uint16_t *v_row = value_base + (size_t)min(key0 + quad * 4 + i, L - 1) * value_row_stride;
-#pragma unroll
-        for (int blk = 0; blk < VBLOCKS; ++blk)
-          v_raw[blk][i] = *reinterpret_cast<const uint2 *>(v_row + blk * 64 + col * 4);
-      }
-    }
-    // 4 x 4 transposes: v_t[blk][jj] = V[keys quad*4 + 0..3][blk*64 + col*4 + jj], the A operand of PV
-    h4_t v_t[VBLOCKS][4];
-#pragma unroll
-    for (int blk = 0; blk < VBLOCKS; ++blk) {
-      const uint32_t lo01_a = __builtin_amdgcn_perm(v_raw[blk][1].x, v_raw[blk][0].x, 0x05040100u);
-      const uint32_t lo01_b = __builtin_amdgcn_perm(v_raw[blk][1].x, v_raw[blk][0].x, 0x07060302u);
-      const uint32_t lo23_a = __builtin_amdgcn_perm(v_raw[blk][3].x, v_raw[blk][2].x, 0x05040100u);
-      const uint32_t lo23_b = __builtin_amdgcn_perm(v_raw[blk][3].x, v_raw[blk][2].x, 0x07060302u);
-      const uint32_t hi01_a = __builtin_amdgcn_perm(v_raw[blk][1].y, v_raw[blk][0].y, 0x05040100u);
-      const uint32_t hi01_b = __builtin_amdgcn_perm(v_raw[blk][1].y, v_raw[blk][0].y, 0x07060302u);
-      const uint32_t hi23_a = __builtin_amdgcn_perm(v_raw[blk][3].y, v_raw[blk][2].y, 0x05040100u);
-      const uint32_t hi23_b = __builtin_amdgcn_perm(v_raw[blk][3].y, v_raw[blk][2].y, 0x07060302u);
-      v_t[blk][0] = __builtin_bit_cast(h4_t, make_uint2(lo01_a, lo23_a));
-      v_t[blk][1] = __builtin_bit_cast(h4_t, make_uint2(lo01_b, lo23_b));
-      v_t[blk][2] = __builtin_bit_cast(h4_t, make_uint2(hi01_a, hi23_a));
-      v_t[blk][3] = __builtin_bit_cast(h4_t, make_uint2(hi01_b, hi23_b));
-    }
-
-#pragma unroll
-    for (int t = 0; t < kQueryTiles; ++t) {
-      const uint32_t row = q0 + t * 16 + col;  // this lane's query row in tile t
-      // tiles that lie wholly past this tile's causal limit contribute nothing
-      if (a.causal && key0 > a.past_length + q0 + t * 16 + 15) continue;
-      f4_t score = f4_t{0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-      for (int j = 0; j < QSTEPS; ++j)
-        score = __builtin_amdgcn_mfma_f32_16x16x32_f16(k_frag[j], q_frag[t][j], score, 0, 0, 0);
-      float tile_max = -INFINITY;
-      // a tile of existing keys, all below the causal limit of the tile's first row, of
-      // existing rows and without a mask needs no per-score test
-      const bool interior = !masked && key0 + 16 <= L && q0 + t * 16 + 16 <= a.query_length &&
-                            (!a.causal || key0 + 15 <= a.past_length + q0 + t * 16);
-      if (interior) {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          score[i] *= score_scale;
-          tile_max = fmaxf(tile_max, score[i]);
-        }
-      } else {
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const uint32_t key = key0 + quad * 4 + i;
-          bool allowed = key < L && row < a.query_length;
-          if (a.causal) allowed = allowed && key <= a.past_length + row;
-          if (masked && allowed) allowed = mask_allows(a, batch, head, row, key);
-          score[i] = allowed ? score[i] * score_scale : -INFINITY;
-          tile_max = fmaxf(tile_max, score[i]);
-        }
-      }
-      tile_max = lanes_xor_max(tile_max, 16);
-      tile_max = lanes_xor_max(tile_max, 32);
-      const float new_max = fmaxf(running_max[t], tile_max);
-      // no allowed key yet: keep every exponent finite (the probabilities are zero anyway)
-      const float reference = new_max == -INFINITY ? 0.0f : new_max;
-      const float alpha = __builtin_amdgcn_exp2f(running_max[t] - reference);  // 0 while running_max is -inf
-      running_max[t] = new_max;
-      h4_t p_frag;
-      float tile_sum = 0.0f;
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const float p = __builtin_amdgcn_exp2f(score[i] - reference);
-        tile_sum += p;
-        p_frag[i] = (_Float16)p;
-      }
-      running_sum[t] = running_sum[t] * alpha + tile_sum;
-      if (__builtin_amdgcn_ballot_w64(alpha != 1.0f) != 0) {
-#pragma unroll
-        for (int v = 0; v < VBLOCKS * 4; ++v)
-#pragma unroll
-          for (int i = 0; i < 4; ++i) out_acc[t][v][i] *= alpha;
-      }
-#pragma unroll
-      for (int blk = 0; blk < VBLOCKS; ++blk)
-#pragma unroll
-        for (int jj = 0; jj < 4; ++jj)
-          out_acc[t][blk * 4 + jj] =
-              __builtin_amdgcn_mfma_f32_16x16x16f16(v_t[blk][jj], p_frag, out_acc[t][blk * 4 + jj], 0, 0, 0);
-    }
-  };
-
-  for (uint32_t key0 = 0; key0 < key_end; key0 += 16) process_tile(key0);
-
-  // out_acc[t][blk*4 + jj][i] is O[row = q0 + t*16 + col][d = blk*64 + 4*(quad*4 + i) + jj]
-#pragma unroll
-  for (int t = 0; t < kQueryTiles; ++t) {
-    float total = lanes_xor_sum(running_sum[t], 16);
-    total = lanes_xor_sum(total, 32);
-    const uint32_t row = q0 + t * 16 + col;
-    if (row >= a.query_length) continue;
-    const float inverse = total != 0.0f ? 1.0f / total : 0.0f;
-    uint16_t *out_row = a.token_first_output
-                            ? a.output + (((size_t)batch * a.query_length + row) * a.heads + head) * D
-                            : a.output + (((size_t)batch * a.heads + head) * a.query_length + row) * D;
-#pragma unroll
-    for (int blk = 0; blk < VBLOCKS; ++blk)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        // the four jj of one (blk, i) are adjacent in head_dim: one 8-byte store
-        uint2 packed;
-        packed.x = (uint32_t)float_to_half_bits(out_acc[t][blk * 4 + 0][i] * inverse) |
-                   ((uint32_t)float_to_half_bits(out_acc[t][blk * 4 + 1][i] * inverse) << 16);
-        packed.y = (uint32_t)float_to_half_bits(out_acc[t][blk * 4 + 2][i] * inverse) |
-                   ((uint32_t)float_to_half_bits(out_acc[t][blk * 4 + 3][i] * inverse) << 16);
-        *reinterpret_cast<uint2 *>(out_row + blk * 64 + 4 * (quad * 4 + i)) = packed;
-      }
-  }
-}
-
-// ---- 32 x 32 wave tiles (no mask) --------------------------------------------------------------
+// ---- 32 x 32 wave tiles ---------------------------------------------------------------------------
 //
 // The four waves of a workgroup - 128 consecutive query rows of one head - walk the same keys, so
 // K and V go global -> LDS once per workgroup, 64 keys a stage and a stage ahead of the
@@ -271,7 +79,9 @@ __global__ __launch_bounds__(kWavesPerBlock * 64) void dense_attention_mfma_kern
 // instead of four times.
 // WAVES x 32 query rows per workgroup, STAGE_KEYS keys per LDS stage (launched as 4 x 64: 64 KB at
 // D = 128, two workgroups per CU).
-template <int D, int WAVES, int STAGE_KEYS>
+// MASKED: the launch has a mask (every score is then tested; without one the instantiation carries
+// nothing of it).
+template <int D, int WAVES, int STAGE_KEYS, bool MASKED>
 __global__ __launch_bounds__(WAVES * 64) void dense_attention_tile32_kernel(DenseAttentionArgs a) {
   constexpr int KSTEPS = D / 16;  // score MFMAs per key tile
   constexpr int JJ = D / 32;      // adjacent head_dim values per lane and key = output blocks
@@ -311,6 +121,7 @@ __global__ __launch_bounds__(WAVES * 64) void dense_attention_tile32_kernel(Dens
   const bool has_rows = q0 < a.query_length;  // a wave without rows still copies and meets the barriers
   const uint32_t kv_heads = a.kv_heads > 0 ? a.kv_heads : a.heads;
   const uint32_t kv_head = kv_heads < a.heads ? head / (a.heads / kv_heads) : head;
+  constexpr bool masked = MASKED;
   const uint32_t L = a.key_length;
 
   // B operand of the score MFMAs: Q[row = row_lane][d = ks * 16 + half * 8 ..]; rows past the end repeat the last
@@ -407,9 +218,10 @@ __global__ __launch_bounds__(WAVES * 64) void dense_attention_tile32_kernel(Dens
   // softmax update and P V product of one tile from its scores; v_tile = its first V row in the stage
   auto tile_update = [&](uint32_t key0, f16x_t score, const unsigned char *v_tile) __attribute__((always_inline)) {
     // a tile of existing keys, all below the causal limit of the wave's first row, of existing
-    // rows needs no per-score test.  Maxima are taken over the scores as the MFMAs left them; the
+    // rows and without a mask needs no per-score test.  Maxima are taken over the scores as the MFMAs left them; the
     // scale (positive) goes into the exponent's multiply-add.
-    const bool interior = key0 + 32 <= L && q0 + 32 <= a.query_length && (!a.causal || key0 + 31 <= a.past_length + q0);
+    const bool interior =
+        !masked && key0 + 32 <= L && q0 + 32 <= a.query_length && (!a.causal || key0 + 31 <= a.past_length + q0);
     float tile_max = -INFINITY;
     if (interior) {
 #pragma unroll
@@ -421,6 +233,9 @@ __global__ __launch_bounds__(WAVES * 64) void dense_attention_tile32_kernel(Dens
         const uint32_t key = key0 + (r >> 2) * 8 + half * 4 + (r & 3);
         bool allowed = key < L && row < a.query_length;
         if (a.causal) allowed = allowed && key <= a.past_length + row;
+        if constexpr (masked) {
+          if (allowed) allowed = mask_allows(a, batch, head, row, key);
+        }
         score[r] = allowed ? score[r] : -INFINITY;
         tile_max = fmaxf(tile_max, score[r]);
       }
@@ -584,47 +399,46 @@ hipError_t launch_dense_attention(const DenseAttentionArgs &a, hipStream_t strea
   if (a.key_length == 0 || a.head_dim == 0 || a.head_dim > 64 * kMaxFragments) return hipErrorInvalidValue;
   const bool aligned = reinterpret_cast<uintptr_t>(a.query) % 16 == 0 && reinterpret_cast<uintptr_t>(a.key) % 16 == 0 &&
                        reinterpret_cast<uintptr_t>(a.value) % 8 == 0 && reinterpret_cast<uintptr_t>(a.output) % 8 == 0;
-  if ((a.head_dim == 64 || a.head_dim == 128) && aligned && a.query_length >= 16 && a.heads <= 65535 &&
-      a.batches <= 65535) {
-    const uint32_t slab = kWavesPerBlock * kQueryTiles * 16;
-    const dim3 grid((a.query_length + slab - 1) / slab, a.heads, a.batches);
-    const bool masked = a.mask != nullptr && a.mask_batches > 0;
-    // the shared variant copies 16-byte pieces of whole rows: 16-byte aligned K and V rows
+  if ((a.head_dim == 64 || a.head_dim == 128) && aligned && a.query_length >= 16) {
+    // K and V stages are copied as 16-byte pieces of whole rows (16-byte aligned K and V rows), and the
+    // maxima are taken before scaling (a positive, finite scale); anything else takes the row kernel
     const size_t value_row_halfs = a.token_first_value ? (size_t)(a.kv_heads > 0 ? a.kv_heads : a.heads) * a.head_dim
                                                        : a.head_dim;
-    // (the 32 x 32 kernel takes maxima before scaling: a positive, finite scale)
-    const bool shared = !masked && reinterpret_cast<uintptr_t>(a.value) % 16 == 0 && value_row_halfs % 8 == 0 &&
+    const bool staged = reinterpret_cast<uintptr_t>(a.value) % 16 == 0 && value_row_halfs % 8 == 0 &&
                         a.scale > 0.0f && a.scale < INFINITY;
-    static bool configured = false;  // the attribute is per device function
-    if (shared && !configured) {
-      hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(&dense_attention_tile32_kernel<128, 4, 64>),
-                                              hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
-      if (status != hipSuccess) return status;
-      configured = true;
-    }
-    if (shared) {
+    const uint64_t workgroups = (uint64_t)((a.query_length + kWavesPerBlock * 32 - 1) / (kWavesPerBlock * 32)) *
+                                a.heads * a.batches;
+    if (staged && workgroups <= 0x7fffffffull) {
+      const bool masked = a.mask != nullptr && a.mask_batches > 0;
+      static bool configured = false;  // the attribute is per device function
+      if (!configured) {
+        hipError_t status =
+            hipFuncSetAttribute(reinterpret_cast<const void *>(&dense_attention_tile32_kernel<128, 4, 64, false>),
+                                hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+        if (status == hipSuccess)
+          status = hipFuncSetAttribute(reinterpret_cast<const void *>(&dense_attention_tile32_kernel<128, 4, 64, true>),
+                                       hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
+        if (status != hipSuccess) return status;
+        configured = true;
+      }
       // 32 x 32 wave tiles over shared LDS stages, four waves and 64 keys a stage.  (Workgroups of two
       // waves with 32-key stages, twice as many and four per CU, so that short causal launches are not
       // as long as their longest workgroup, measured slower: 105.6 against 91.2 us at 32 heads x 2048
       // tokens - one tile per barrier, half the sharing.)
       const size_t bytes = 2 * 2 * (size_t)64 * a.head_dim * 2;
-      const uint64_t workgroups = (uint64_t)grid.x * a.heads * a.batches;
-      if (workgroups > 0x7fffffffull) return hipErrorInvalidValue;
       DenseAttentionArgs scheduled = a;
       scheduled.cus_per_xcd = (uint32_t)device_compute_units() / 8;
-      if (a.head_dim == 64)
-        hipLaunchKernelGGL((dense_attention_tile32_kernel<64, 4, 64>), dim3((uint32_t)workgroups), dim3(256), bytes,
-                           stream, scheduled);
+      const dim3 grid((uint32_t)workgroups), block(256);
+      if (a.head_dim == 64 && masked)
+        hipLaunchKernelGGL((dense_attention_tile32_kernel<64, 4, 64, true>), grid, block, bytes, stream, scheduled);
+      else if (a.head_dim == 64)
+        hipLaunchKernelGGL((dense_attention_tile32_kernel<64, 4, 64, false>), grid, block, bytes, stream, scheduled);
+      else if (masked)
+        hipLaunchKernelGGL((dense_attention_tile32_kernel<128, 4, 64, true>), grid, block, bytes, stream, scheduled);
       else
-        hipLaunchKernelGGL((dense_attention_tile32_kernel<128, 4, 64>), dim3((uint32_t)workgroups), dim3(256), bytes,
-                           stream, scheduled);
-    } else if (a.head_dim == 64) {
-      // masks: 16-key tiles, every wave fetching its own
-      hipLaunchKernelGGL((dense_attention_mfma_kernel<64>), grid, dim3(kWavesPerBlock * 64), 0, stream, a);
-    } else {
-      hipLaunchKernelGGL((dense_attention_mfma_kernel<128>), grid, dim3(kWavesPerBlock * 64), 0, stream, a);
+        hipLaunchKernelGGL((dense_attention_tile32_kernel<128, 4, 64, false>), grid, block, bytes, stream, scheduled);
+      return hipGetLastError();
     }
-    return hipGetLastError();
   }
   const uint64_t blocks = (rows + 3) / 4;
   if (blocks > 0x7fffffffull) return hipErrorInvalidValue;
