@@ -194,8 +194,9 @@ int llmopt_hip_commit_batch_async(llmopt_hip_batch *batch);
  * back to back) and returns the elapsed GPU milliseconds of the timed part.
  * use_graph = 2..4: the caller states that the recorded operations do not
  * depend on each other; the graph then has that many branches the GPU may
- * run side by side, the operations dealt onto them round-robin (those that
- * use the context's scratch memory stay on the first, in recorded order). */
+ * run side by side; every operation goes to the branch with the fewest bytes
+ * of bound buffers so far (those that use the context's scratch memory stay
+ * on the first, in recorded order). */
 int llmopt_hip_commit_batch_profiled(llmopt_hip_batch *batch, int use_graph, int repeats,
                                      float *gpu_milliseconds);
 /* caml_llmopt_metal_abort_batch (:1372-1382). */

@@ -438,3 +438,42 @@ def test_dual_swiglu_prefill_cell_at_full_size(runtime, m):
     combined = gate_all / (1.0 + np.exp(-gate_all)) * up_all
     assert_close_to_oracle(got, combined.astype(np.float32), f"dual swiglu cell vs projections m={m}",
                            rel_l2_tol=2e-3)
+
+
+@pytest.mark.parametrize("use_graph", [False, True, 2, 4])
+def test_profiled_commit_of_independent_linears(runtime, use_graph):
+    """The measuring commit (host launches, one graph, a graph of concurrent branches the launches
+    are dealt onto by their bytes) leaves what a plain commit leaves.  Among the launches: two
+    that split K over workgroups and share the context's workspace and arrival counters (8 rows,
+    K = 14336), which stay in recorded order on one branch."""
+    rng = np.random.default_rng(77)
+    shapes = [(1, 512, 4096), (8, 256, 14336), (4, 1024, 576), (2, 4096, 4096), (8, 320, 14336), (3, 64, 1536),
+              (8, 1536, 576), (1, 2048, 4096)]
+    cases = []
+    for m, n, k in shapes:
+        x, packed, scale, _ = w4_case(rng, m, n, k)
+        cases.append((m, n, k, x, packed, scale, runtime.buffer_of_bytes(x), runtime.buffer_of_bytes(packed),
+                      runtime.buffer_of_bytes(scale)))
+
+    def record(batch, outputs):
+        for (m, n, k, _, _, _, bx, bw, bs), out in zip(cases, outputs):
+            name = "llmopt_w4a16_linear_f16_g64" if m == 1 else "llmopt_w4a16_linear_f16_g64_m4"
+            columns = m * n if m == 1 else ((m + 3) // 4) * n
+            batch.dispatch(name, [bx, bw, bs, bs, out], u32s(m, n, k, 0, 0),
+                           grid=(linear_grid(columns), 1, 1), group=(256, 1, 1))
+
+    def fresh_outputs():
+        return [runtime.buffer_of_bytes(np.full((m, n), np.nan, dtype=np.float16)) for m, n, *_ in cases]
+
+    plain = fresh_outputs()
+    batch = runtime.begin_batch()
+    record(batch, plain)
+    batch.commit()
+    measured = fresh_outputs()
+    batch = runtime.begin_batch()
+    record(batch, measured)
+    assert batch.commit_profiled(repeats=2, use_graph=use_graph) > 0.0
+    for (m, n, k, x, packed, scale, *_), first, second in zip(cases, plain, measured):
+        expected = first.numpy(np.float16, (m, n))
+        assert np.array_equal(second.numpy(np.float16, (m, n)).view(np.uint16), expected.view(np.uint16)), (m, n, k)
+        assert_close_to_oracle(expected, oracle.w4a16_linear(x, packed, scale, None), f"linear {m}x{n}x{k}")
