@@ -72,6 +72,37 @@ def test_pack_is_bit_exact(runtime, name):
     np.testing.assert_array_equal(got[mask], expected[mask])
 
 
+@pytest.mark.parametrize("name", ["llmopt_cache_pack_attention_q8", "llmopt_cache_pack_attention_q8_simd"])
+def test_pack_rounds_ties_to_even(runtime, name):
+    """Every quotient x / scale lands exactly halfway between two integers: a group's largest
+    magnitude is 127 * 2^e (scale 2^e exactly) and the others are (n + 0.5) * 2^e, all exact in
+    fp16.  rint rounds them to the even neighbour, both signs (lib/metal_cache_source.ml:67-75)."""
+    rng = np.random.default_rng(17)
+    heads, dim, items = 2, 128, 24
+    token_elements, stride = layout(heads, dim)
+    source = np.empty((heads, items, dim), dtype=np.float16)
+    for head in range(heads):
+        for item in range(items):
+            for group in range(dim // 64):
+                step = np.float32(2.0) ** int(rng.integers(-6, 3))
+                n = rng.integers(0, 127, size=64).astype(np.float32)
+                sign = rng.choice([-1.0, 1.0], size=64).astype(np.float32)
+                values = sign * (n + np.float32(0.5)) * step
+                values[int(rng.integers(0, 64))] = np.float32(127.0) * step * rng.choice([-1.0, 1.0])
+                source[head, item, group * 64:(group + 1) * 64] = values.astype(np.float16)
+    assert np.array_equal(source.astype(np.float32).astype(np.float16), source)
+    slots = rng.permutation(items + 3)[:items].astype(np.uint32)
+    expected = np.zeros((items + 3) * stride, dtype=np.uint8)
+    oracle.q8_pack(source, slots, expected, oracle_cache_params(items, 0, heads, dim, token_elements, stride, items, 0))
+    quantised = expected.reshape(items + 3, stride)[slots][:, :heads * dim].view(np.int8)
+    assert np.all((quantised % 2 == 0) | (np.abs(quantised) == 127))  # every tie went to the even neighbour
+    pool = runtime.create_buffer((items + 3) * stride)
+    runtime.dispatch(name, [runtime.buffer_of_bytes(source), runtime.buffer_of_bytes(slots), pool],
+                     cache_params_bytes(items, 0, heads, dim, token_elements, stride, items, 0),
+                     grid=(items * heads * dim // 64 * 32, 1, 1), group=(256, 1, 1))
+    np.testing.assert_array_equal(pool.numpy(np.uint8), expected)
+
+
 def test_pair_pack_and_unpack_round_trip(runtime, golden):
     cycle = golden["q8_round_trip"]["value_bits_cycle"]
     heads, dim, items = 2, 64, 5
