@@ -17,7 +17,8 @@ from typing import Iterable, Optional, Sequence
 import numpy as np
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIBRARY_PATH = os.path.join(_HERE, "libllmopt_hip.so")
+# LLMOPT_HIP_LIBRARY names another build of the same library (python -m llmopt_amd.build --host-ubsan)
+LIBRARY_PATH = os.environ.get("LLMOPT_HIP_LIBRARY") or os.path.join(_HERE, "libllmopt_hip.so")
 
 
 class LlmoptError(RuntimeError):
