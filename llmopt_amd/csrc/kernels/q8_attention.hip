@@ -196,36 +196,13 @@ q8_attention_split_kernel(Q8AttentionArgs a, uint32_t chunks_max, uint32_t fixed
   // what lies beyond belongs to another workgroup and would be fetched twice
   const uint32_t last_token = min(chunk_begin + chunk_tokens, past) - 1;
 
-  // B operand of the score MFMAs: Q[head = col][d], zero for columns >= G.
-  h8_t q_frag[GROUPS][2];
-  {
-    const uint16_t *q_row =
-        a.query + ((size_t)batch * a.query_heads + kv_head * heads_per_kv + col) * D;
-#pragma unroll
-    for (int g = 0; g < GROUPS; ++g)
-#pragma unroll
-      for (int j = 0; j < 2; ++j) {
-        uint4 raw = make_uint4(0, 0, 0, 0);
-        if (col < heads_per_kv)
-          raw = *reinterpret_cast<const uint4 *>(q_row + g * 64 + quad * 16 + j * 8);
-        q_frag[g][j] = __builtin_bit_cast(h8_t, raw);
-      }
-  }
-
+  // B operand of the score MFMAs: Q[head = col][d], zero for columns >= G, and
   // 1152 * sum_d Q[head][d] per scale group: the constant the biased K decode
-  // adds to every score of this head
+  // adds to every score of this head.  Both are filled in below, behind the first requests for
+  // the context: a wave's start is a chain of trips to memory (context lengths, slot table, K/V
+  // rows), and the query rows must not add theirs to it.
+  h8_t q_frag[GROUPS][2];
   float key_bias[GROUPS];
-#pragma unroll
-  for (int g = 0; g < GROUPS; ++g) {
-    float sum = 0.0f;
-#pragma unroll
-    for (int j = 0; j < 2; ++j)
-#pragma unroll
-      for (int e = 0; e < 8; ++e) sum += (float)q_frag[g][j][e];
-    sum += shfl_xor_f32(sum, 16);
-    sum += shfl_xor_f32(sum, 32);
-    key_bias[g] = 1152.0f * sum;
-  }
   // softmax runs in base 2: exp(x) = exp2(x * log2(e))
   const float score_scale = a.scale * 1.4426950408889634f;
 
@@ -433,7 +410,36 @@ q8_attention_split_kernel(Q8AttentionArgs a, uint32_t chunks_max, uint32_t fixed
     TileRaw raw;
     load_slots(0, slots_a);
     load_slots(1, slots_b);
+    __builtin_amdgcn_sched_barrier(0);
+    // the query rows go out behind the slot requests and ahead of the first K/V rows: loads return
+    // in issue order, so waiting for the slots does not wait for them, and they have landed when
+    // the first tile has.  Every lane reads (lanes of columns >= G read the group's last head and
+    // drop it): a load under a branch is waited for where it stands.
+    uint4 q_raw[GROUPS][2];
+    {
+      const uint16_t *q_row =
+          a.query + ((size_t)batch * a.query_heads + kv_head * heads_per_kv + min(col, heads_per_kv - 1)) * D;
+#pragma unroll
+      for (int g = 0; g < GROUPS; ++g)
+#pragma unroll
+        for (int j = 0; j < 2; ++j) q_raw[g][j] = *reinterpret_cast<const uint4 *>(q_row + g * 64 + quad * 16 + j * 8);
+    }
+    __builtin_amdgcn_sched_barrier(0);
     load_line(slots_a, line_a);
+    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+    for (int g = 0; g < GROUPS; ++g) {
+      float sum = 0.0f;
+#pragma unroll
+      for (int j = 0; j < 2; ++j) {
+        q_frag[g][j] = __builtin_bit_cast(h8_t, col < heads_per_kv ? q_raw[g][j] : make_uint4(0, 0, 0, 0));
+#pragma unroll
+        for (int e = 0; e < 8; ++e) sum += (float)q_frag[g][j][e];
+      }
+      sum += shfl_xor_f32(sum, 16);
+      sum += shfl_xor_f32(sum, 32);
+      key_bias[g] = 1152.0f * sum;
+    }
     // Loads return in issue order, so the small slot loads go out before the
     // K/V loads of the same step: waiting for a slot then never waits for a
     // younger K/V request.
@@ -497,6 +503,13 @@ __global__ __launch_bounds__(kMergeSlices *D) void q8_attention_merge_kernel(Q8A
   const uint32_t kv_head = head / heads_per_kv;
   const uint32_t local_head = head - kv_head * heads_per_kv;
   const size_t stride = partial_floats<D>(heads_per_kv);
+  // The current token's operands depend on the workgroup's indices only: they are requested before
+  // the context lengths, by every thread (a load under a branch is waited for where it stands, which
+  // made them a trip to memory of their own, after the partial results had landed).
+  const size_t current = ((size_t)batch * a.kv_heads + kv_head) * D + d;
+  const uint16_t current_value_bits = a.current_value[current];
+  const uint16_t current_key_bits = a.current_key[current];
+  const uint16_t query_bits = a.query[((size_t)batch * a.query_heads + head) * D + d];
   uint32_t chunks;
   const float *partial = reinterpret_cast<const float *>(a.workspace);
   if (balanced_slots != 0) {
@@ -530,12 +543,8 @@ __global__ __launch_bounds__(kMergeSlices *D) void q8_attention_merge_kernel(Q8A
     ahead[i] = c < chunks ? column[c * stride] : 0.0f;
   }
   // score of the current token (slice 0 holds the dot product) and the largest chunk maximum
-  const size_t current = ((size_t)batch * a.kv_heads + kv_head) * D + d;
-  const float current_value = slice == 0 ? half_bits_to_float(a.current_value[current]) : 0.0f;
-  float dot = 0.0f;
-  if (slice == 0)
-    dot = half_bits_to_float(a.query[((size_t)batch * a.query_heads + head) * D + d]) *
-          half_bits_to_float(a.current_key[current]);
+  const float current_value = slice == 0 ? half_bits_to_float(current_value_bits) : 0.0f;
+  float dot = slice == 0 ? half_bits_to_float(query_bits) * half_bits_to_float(current_key_bits) : 0.0f;
   dot = wave_sum(dot);
   float chunk_best = -INFINITY;
 #pragma unroll

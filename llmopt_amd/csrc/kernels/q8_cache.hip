@@ -64,7 +64,11 @@ __global__ __launch_bounds__(256) void rotary_qk_pack_kernel(RotaryPackArgs a) {
   const RotaryQkArgs &r = a.rotary;
   const Q8PackArgs &p = a.pack;
   const uint32_t lane = threadIdx.x & 63;
-  const uint32_t row = blockIdx.x * 4 + (threadIdx.x >> 6);
+  // the row is the same for the whole wave, and said to be: which input, which output and which
+  // segment the wave takes are then scalar selects among the arguments, and its pool slot a scalar
+  // load - left to per-lane values they were vector loads from the argument block and the slot
+  // table, each a trip to memory the row's own loads had to wait for
+  const uint32_t row = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const uint32_t q_rows = r.batches * r.q_heads, kv_rows = r.batches * r.k_heads;
   if (row >= q_rows + 2 * kv_rows) return;
   const bool is_q = row < q_rows;
