@@ -20,8 +20,9 @@ before its turn comes again: every launch streams its weights from HBM.
 Also reported in the same line: `roofline` of the kernel with the largest
 share of the sweep's time (HIP events around graph-replayed launches of each
 of its cases), `cpu_baseline` (the C oracle on one host core over the same
-sweep) and, under `extras`, the prefill GEMM (MFMA roofline) and Q8 decode
-attention (HBM roofline, tokens/s) measurements.
+sweep) and, under `extras`, the prefill GEMM (MFMA roofline), Q8 decode
+attention (HBM roofline, tokens/s), dense prefill attention, the 30-layer
+model's decode step and its prompt prefill.
 
 No number is printed unchecked: outside the timed regions the output of every
 timed GEMV, GEMM and attention case is read back and a sample of it compared
@@ -446,6 +447,58 @@ def bench_decode_step(runtime, batches=(1, 8, 32, 128), context=2048, use_graph=
     return results
 
 
+def bench_prefill(runtime, lengths=(512, 2048)):
+    """Prompt prefill of the 30-layer decode model (llmopt_amd.prefill_step): all prompt tokens
+    through every layer at once - the prefill GEMMs, RoPE, the Q8 pack of every token's K/V into
+    the pool, causal dense attention - and the LM-head argmax of the last token, as one HIP graph.
+    The chain is checked against the oracle at a depth and length the CPU finishes in a second
+    (2 layers, 48 tokens; the oracle would need minutes for the timed sizes, whose kernels each
+    have their parity tests at full size)."""
+    from llmopt_amd.decode_step import DecodeConfig, random_weights
+    from llmopt_amd.prefill_step import PrefillStep
+    from tests.test_gpu_prefill_step import oracle_prefill
+    rng = np.random.default_rng(SEED + 5)
+    small = DecodeConfig(layers=2, vocabulary=1000)
+    small_weights = random_weights(small, rng)
+    count = 48
+    order = rng.permutation(count + 2).astype(np.uint32)
+    host_pool = np.zeros((count + 2) * small.token_stride, dtype=np.uint8)
+    prompt = rng.integers(0, small.vocabulary, count)
+    step = PrefillStep(runtime, small, small_weights, count, runtime.buffer_of_bytes(host_pool),
+                       runtime.buffer_of_bytes(order))
+    first = step.run(prompt)
+    hidden, logits, _ = oracle_prefill(small, small_weights, prompt, order[:count], host_pool)
+    got = step.work["x"][0].numpy(np.float16, (count, small.hidden)).astype(np.float64)
+    rel_l2 = float(np.linalg.norm(got - hidden.astype(np.float64)) / np.linalg.norm(hidden.astype(np.float64)))
+    logit_rms = float(np.sqrt(np.mean(logits.astype(np.float64) ** 2)))
+    verified = bool(np.all(np.isfinite(got)) and rel_l2 <= 4e-3 and
+                    float(logits[first]) >= float(logits.max()) - 2e-2 * logit_rms)
+    del step
+
+    config = DecodeConfig()
+    weights = random_weights(config, rng)
+    device_weights = None
+    results = []
+    for tokens in lengths:
+        pool = runtime.create_buffer((tokens + 1) * config.token_stride)
+        slots = runtime.buffer_of_bytes(np.arange(tokens + 1, dtype=np.uint32))
+        step = PrefillStep(runtime, config, weights, tokens, pool, slots, device_weights=device_weights)
+        device_weights = step.device
+        step.run(rng.integers(0, config.vocabulary, tokens))  # first-use allocations
+        graph = runtime.begin_batch()
+        step.record(graph)
+        repeats = 5
+        ms = graph.commit_profiled(repeats=repeats, use_graph=True) / repeats
+        results.append({"tokens": tokens, "layers": config.layers, "launches": len(step.dispatches),
+                        "ms_per_prefill": round(ms, 4), "tokens_per_s": round(tokens / (ms * 1e-3), 1),
+                        "TFLOPs": round(step.flops() / (ms * 1e-3) / 1e12, 1),
+                        "mfma_frac": round(step.flops() / (ms * 1e-3) / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
+                        "verified": verified, "rel_l2": round(rel_l2, 6),
+                        "verified_on": "the same chain at 2 layers x 48 tokens against the oracle"})
+        del step, pool
+    return results
+
+
 PMC_LAUNCHES_PER_CASE = 8
 
 
@@ -540,8 +593,8 @@ def main():
     parser.add_argument("--steps", type=int, default=64)
     parser.add_argument("--warmup", type=int, default=16)
     parser.add_argument("--skip-extras", action="store_true")
-    parser.add_argument("--extras", default="gemm,attention,prefill_attention,decode",
-                        help="comma-separated subset of gemm, attention, prefill_attention, decode")
+    parser.add_argument("--extras", default="gemm,attention,prefill_attention,decode,prefill",
+                        help="comma-separated subset of gemm, attention, prefill_attention, decode, prefill")
     parser.add_argument("--skip-cpu", action="store_true")
     parser.add_argument("--decode-eager", action="store_true",
                         help="launch the decode step from the host instead of replaying a HIP graph")
@@ -612,6 +665,8 @@ def main():
     if "decode" in wanted:
         extras["decode_step"] = bench_decode_step(
             runtime, batches=tuple(int(b) for b in args.decode_batches.split(",")), use_graph=not args.decode_eager)
+    if "prefill" in wanted:
+        extras["prefill_step"] = bench_prefill(runtime)
     # refuse to print numbers whose outputs did not match the oracle
     checked = [("gemv %(m)dx%(k)dx%(n)d" % c, c["verified"]) for c in gemv["cases"]]
     checked.append(("gemv c1", gemv["c1"]["verified"]))
@@ -620,6 +675,7 @@ def main():
         checked.append(("q8 attention", extras["q8_attention"]["verified"]))
     checked += [("prefill attention %(heads)d/%(kv_heads)d x %(head_dim)d @ %(tokens)d" % c, c["verified"])
                 for c in extras.get("prefill_attention", [])]
+    checked += [("prefill step @ %(tokens)d" % c, c["verified"]) for c in extras.get("prefill_step", [])]
     failed = [name for name, ok in checked if not ok]
     if failed:
         runtime.close()
