@@ -68,8 +68,23 @@ constexpr size_t quad_lds_bytes(uint32_t waves) {
 // MR: activation rows staged (m <= MR <= 4); KL: K / 512; RQ: row quads per wave; DEPTH: weight
 // loads in flight per wave; EARLY: how many of them go out before the staging waits;
 // THREADS: workgroup size (waves beyond units_per_wg only help staging).
+// Registers: a workgroup is one wave per SIMD, and told only that, the compiler spreads itself over
+// the 512 registers a lone wave may have (220 at one row of K = 14336, half of them accumulator
+// registers used as spill space) - a CU then holds nothing beside this workgroup, and launches that
+// do not depend on each other cannot run side by side on it.  Asked for three waves per SIMD (two at
+// four rows, one for the long-row instantiations with two quads per wave, which need the room) the
+// same kernels take 58-128 registers with nothing spilled and run a little faster: the serial sweep
+// 91.5 -> 90.0 us a step, 85.1 -> 82.9 on two concurrent graph branches (four branches: 70.7-72.0
+// either way, within what two runs differ by).
+template <int MR, int KL, int RQ>
+constexpr int quad_waves_per_simd() {
+  return (KL > 8 && RQ == 2) ? 1 : MR <= 2 ? 3 : 2;
+}
+
 template <int MR, int KL, int RQ, int DEPTH, int EARLY, int THREADS>
-__global__ __launch_bounds__(THREADS) void w4a16_gemv_quad_kernel(QuadParams p, uint32_t units_per_wg) {
+__global__ __launch_bounds__(THREADS)
+    __attribute__((amdgpu_waves_per_eu(quad_waves_per_simd<MR, KL, RQ>(), quad_waves_per_simd<MR, KL, RQ>()))) void
+    w4a16_gemv_quad_kernel(QuadParams p, uint32_t units_per_wg) {
   static_assert(MR >= 1 && MR <= 4 && EARLY >= 1 && EARLY <= DEPTH && DEPTH <= KL * RQ && THREADS % 64 == 0, "shape");
   constexpr uint32_t K = KL * 512, row_bytes = K / 2, groups = K / 64;
   constexpr uint32_t kRowStride = 2 * K + 16;         // bytes between activation rows in LDS
