@@ -48,6 +48,15 @@ struct GemmParams {
   uint32_t k_len;
   float *partials;
   uint32_t *counters;
+  // segments > 1: several matrices multiply the same activation in one launch (the QKV projection).
+  // Their column tiles follow each other (seg_tiles each); a workgroup's tile lies in one segment
+  // and takes its weights, scales, output and width from there.  No addend, no K split.
+  uint32_t segments;
+  const uint8_t *seg_w[3];
+  const uint16_t *seg_s[3];
+  uint16_t *seg_y[3];
+  uint32_t seg_n[3];
+  uint32_t seg_tiles[3];
 };
 
 __device__ __forceinline__ f16x_t zero_tile() {
@@ -99,8 +108,22 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
   if (total % 8 == 0) logical = (blockIdx.x % 8) * (total / 8) + blockIdx.x / 8;
   const uint32_t tile_m = logical % p.tiles_m;
   const uint32_t tile_n = logical / p.tiles_m;
+  const uint8_t *weight0 = p.w[0];
+  const uint16_t *scale0 = p.s[0];
+  uint16_t *output0 = p.y;
+  uint32_t width = p.n, tile_column = tile_n;
+  if constexpr (!DUAL && !SPLITK) {
+    if (p.segments > 1) {
+      uint32_t segment = 0;
+      while (segment + 1 < p.segments && tile_column >= p.seg_tiles[segment]) tile_column -= p.seg_tiles[segment++];
+      weight0 = p.seg_w[segment];
+      scale0 = p.seg_s[segment];
+      output0 = p.seg_y[segment];
+      width = p.seg_n[segment];
+    }
+  }
   const uint32_t m0 = tile_m * BM;
-  const uint32_t n0 = tile_n * BN;
+  const uint32_t n0 = tile_column * BN;
   const uint32_t K = p.k;                                   // row stride of x and of the weights
   const uint32_t KS = SPLITK ? p.k_len : p.k;               // this workgroup's extent of K ...
   const uint32_t k_base = SPLITK ? blockIdx.y * p.k_len : 0;  // ... and where it begins
@@ -158,13 +181,13 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
   constexpr int W_LOADS = 2 * NWF;  // vector memory loads of one fetch_w
   const uint32_t fetch_matrix = kThreadPerMatrix ? w_row / BN : 0;
   const uint32_t fetch_row = kThreadPerMatrix ? w_row % BN : w_row;
-  const uint32_t w_col = min(n0 + fetch_row, p.n - 1);  // columns past n are never stored
+  const uint32_t w_col = min(n0 + fetch_row, width - 1);  // columns past n are never stored
   const uint8_t *w_base[NWF];
   const uint16_t *s_base[NWF];
 #pragma unroll
   for (int v = 0; v < NWF; ++v) {
-    w_base[v] = kThreadPerMatrix ? (fetch_matrix ? p.w[NW - 1] : p.w[0]) : p.w[v];
-    s_base[v] = kThreadPerMatrix ? (fetch_matrix ? p.s[NW - 1] : p.s[0]) : p.s[v];
+    w_base[v] = kThreadPerMatrix ? (fetch_matrix ? p.w[NW - 1] : p.w[0]) : (v == 0 ? weight0 : p.w[v]);
+    s_base[v] = kThreadPerMatrix ? (fetch_matrix ? p.s[NW - 1] : p.s[0]) : (v == 0 ? scale0 : p.s[v]);
   }
 
   // The compiler takes the destination of these loads as written when the statement ends, while
@@ -391,7 +414,7 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
 #pragma unroll
   for (int b = 0; b < WN; ++b) {
     const uint32_t col = n0 + col_base + b * 32 + frag_row;
-    if (col >= p.n) continue;
+    if (col >= width) continue;
 #pragma unroll
     for (int a = 0; a < WM; ++a) {
 #pragma unroll
@@ -408,7 +431,7 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
           if (p.has_addend)
             value += half_bits_to_float(p.addend[(size_t)row * p.addend_stride + col]);
         }
-        p.y[(size_t)row * p.n + col] = float_to_half_bits(value);
+        output0[(size_t)row * width + col] = float_to_half_bits(value);
       }
     }
   }
@@ -430,6 +453,11 @@ hipError_t launch_tile(GemmParams &p, hipStream_t stream, uint32_t splits = 1) {
   }
   p.tiles_m = (p.m + BM - 1) / BM;
   p.tiles_n = (p.n + BN - 1) / BN;
+  if (p.segments > 1) {
+    if (DUAL || SPLITK || p.has_addend) return hipErrorInvalidValue;
+    p.tiles_n = 0;
+    for (uint32_t i = 0; i < p.segments; ++i) p.tiles_n += p.seg_tiles[i] = (p.seg_n[i] + BN - 1) / BN;
+  }
   const uint32_t blocks = p.tiles_m * p.tiles_n;
   p.k_len = p.k / splits;
   hipLaunchKernelGGL((w4a16_gemm_kernel<WM, WN, DUAL, XS, SPLITK>), dim3(blocks, splits), dim3(kThreads), lds_bytes,
@@ -560,7 +588,32 @@ hipError_t launch_w4a16_qkv(const W4QkvArgs &args, hipStream_t stream) {
   if ((args.m <= kGemvMaxRows && !w4a16_gemv_mfma_needs_split(args.k)) ||
       w4a16_gemv_mfma_row_groups_ok(args.m, (uint64_t)args.n[0] + args.n[1] + args.n[2], args.k))
     return launch_w4a16_gemv_mfma_qkv(args, stream);
-  // prefill: three GEMMs sharing the activation through L2
+  // prefill.  Small projections (at most two 128 x 128 tiles per CU over the three matrices): one
+  // launch whose column tiles run over the three matrices - each of them alone leaves most CUs
+  // without a tile and costs a launch (the 576 / 192 / 192-wide projections of the small model:
+  // 11 us each, three times a layer).
+  const uint64_t row_tiles = (args.m + 127) / 128;
+  const uint64_t tiles = row_tiles * ((args.n[0] + 127) / 128 + (args.n[1] + 127) / 128 + (args.n[2] + 127) / 128);
+  if (tiles <= 2 * (uint64_t)device_compute_units() && args.n[0] > 0 && args.n[1] > 0 && args.n[2] > 0) {
+    GemmParams p = {};
+    p.x = args.x;
+    p.m = args.m;
+    p.k = args.k;
+    p.segments = 3;
+    for (int i = 0; i < 3; ++i) {
+      p.seg_w[i] = args.w[i].weight;
+      p.seg_s[i] = args.w[i].scale;
+      p.seg_y[i] = args.y[i];
+      p.seg_n[i] = args.n[i];
+    }
+    p.w[0] = p.w[1] = p.seg_w[0];
+    p.s[0] = p.s[1] = p.seg_s[0];
+    p.y = p.seg_y[0];
+    p.n = p.seg_n[0];
+    if (p.k % (4 * BK) == 0 && tiles <= (uint64_t)device_compute_units()) return launch_tile<1, 2, false, 4>(p, stream);
+    return launch_tile<1, 2, false>(p, stream);
+  }
+  // large ones: three GEMMs sharing the activation through L2
   for (int i = 0; i < 3; ++i) {
     W4LinearArgs one = {};
     one.x = args.x;
