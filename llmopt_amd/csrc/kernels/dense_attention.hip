@@ -81,7 +81,11 @@ constexpr int kWavesPerBlock = 4;  // consecutive 32-row slabs of one head
 // D = 128, two workgroups per CU).
 // MASKED: the launch has a mask (every score is then tested; without one the instantiation carries
 // nothing of it).
-template <int D, int WAVES, int STAGE_KEYS, bool MASKED>
+// KEYSPLIT: the four waves of a workgroup share ONE slab of 32 query rows and take a quarter of every
+// 128-key stage each; their partial results meet in LDS at the end.  For launches with fewer
+// workgroups than CUs, which last as long as one wave's walk over all the keys of the last slab: the
+// walk is a quarter as long and there are four times as many workgroups.
+template <int D, int WAVES, int STAGE_KEYS, bool MASKED, bool KEYSPLIT = false>
 __global__ __launch_bounds__(WAVES * 64) void dense_attention_tile32_kernel(DenseAttentionArgs a) {
   constexpr int KSTEPS = D / 16;  // score MFMAs per key tile
   constexpr int JJ = D / 32;      // adjacent head_dim values per lane and key = output blocks
@@ -91,7 +95,11 @@ __global__ __launch_bounds__(WAVES * 64) void dense_attention_tile32_kernel(Dens
   constexpr int COPIES = STAGE_KEYS / KEYS_PER_COPY / WAVES;
   constexpr int STAGE_BYTES = STAGE_KEYS * ROW_BYTES;
   static_assert(JJ == 2 || JJ == 4, "head_dim 64 or 128");
-  static_assert((STAGE_KEYS == 64 || STAGE_KEYS == 32) && COPIES >= 1 && COPIES * KEYS_PER_COPY * WAVES == STAGE_KEYS, "stage");
+  static_assert((STAGE_KEYS == 128 || STAGE_KEYS == 64 || STAGE_KEYS == 32) && COPIES >= 1 &&
+                    COPIES * KEYS_PER_COPY * WAVES == STAGE_KEYS,
+                "stage");
+  static_assert(!KEYSPLIT || STAGE_KEYS == 32 * WAVES, "a tile of every stage per wave");
+  constexpr int ROWS = KEYSPLIT ? 32 : WAVES * 32;  // query rows per workgroup
   extern __shared__ __attribute__((aligned(16))) unsigned char stage_lds[];  // [2 stages][K | V]
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t wave = threadIdx.x >> 6;
@@ -104,7 +112,7 @@ __global__ __launch_bounds__(WAVES * 64) void dense_attention_tile32_kernel(Dens
   // half is taken backwards, so that the CU that got the longest of the run also gets the shortest.
   // Without this a launch of as many workgroups as the device holds - 16 slabs x 32 heads at 2048 tokens -
   // puts the two longest on one CU and all of one length on one XCD, and lasts as long as they do.
-  const uint32_t slabs = (a.query_length + WAVES * 32 - 1) / (WAVES * 32);
+  const uint32_t slabs = (a.query_length + ROWS - 1) / ROWS;
   const uint32_t per_slab = a.heads * a.batches;
   uint32_t rank = blockIdx.x;
   if (a.causal && gridDim.x % 8 == 0 && a.cus_per_xcd > 0) {
@@ -117,7 +125,7 @@ __global__ __launch_bounds__(WAVES * 64) void dense_attention_tile32_kernel(Dens
   const uint32_t slab = a.causal ? slabs - 1 - rank / per_slab : rank / per_slab;
   const uint32_t head = rank % per_slab % a.heads;
   const uint32_t batch = rank % per_slab / a.heads;
-  const uint32_t q0 = (slab * WAVES + wave) * 32;
+  const uint32_t q0 = KEYSPLIT ? slab * 32 : (slab * WAVES + wave) * 32;
   const bool has_rows = q0 < a.query_length;  // a wave without rows still copies and meets the barriers
   const uint32_t kv_heads = a.kv_heads > 0 ? a.kv_heads : a.heads;
   const uint32_t kv_head = kv_heads < a.heads ? head / (a.heads / kv_heads) : head;
@@ -154,8 +162,8 @@ __global__ __launch_bounds__(WAVES * 64) void dense_attention_tile32_kernel(Dens
   }
   uint32_t group_key_end = L;
   if (a.causal) {
-    const uint32_t group_q0 = slab * WAVES * 32;
-    const uint32_t last_row = min(group_q0 + WAVES * 32, a.query_length) - 1;
+    const uint32_t group_q0 = slab * ROWS;
+    const uint32_t last_row = min(group_q0 + ROWS, a.query_length) - 1;
     group_key_end = min((uint64_t)L, (uint64_t)a.past_length + last_row + 1);
   }
   const uint32_t stages = (group_key_end + STAGE_KEYS - 1) / STAGE_KEYS;
@@ -284,6 +292,13 @@ __global__ __launch_bounds__(WAVES * 64) void dense_attention_tile32_kernel(Dens
     if (stage + 1 < stages) copy_stage(stage + 1);  // into the buffer every wave left at the last barrier
     const unsigned char *k_stage = stage_lds + (stage & 1) * 2 * STAGE_BYTES;
     const unsigned char *v_stage = k_stage + STAGE_BYTES;
+    if constexpr (KEYSPLIT) {
+      const uint32_t key0 = stage * STAGE_KEYS + wave * 32;
+      if (key0 < key_end)
+        tile_update(key0, tile_scores(k_stage + wave * 32 * ROW_BYTES, wave * 32), v_stage + wave * 32 * ROW_BYTES);
+      stage_landed();
+      continue;
+    }
     const uint32_t key0 = stage * STAGE_KEYS;
     if (key0 < key_end) {
       const f16x_t first_scores = tile_scores(k_stage, 0);
@@ -298,6 +313,62 @@ __global__ __launch_bounds__(WAVES * 64) void dense_attention_tile32_kernel(Dens
       }
     }
     stage_landed();
+  }
+  if constexpr (KEYSPLIT) {
+    // The waves' shares of the slab meet in LDS (the stages are read to the end: the loop's last
+    // barrier): per wave the row maxima and denominators, and O^T as floats [d][row] - a lane's
+    // values of one register are 32 neighbouring rows.  Thread t then folds row t % 32, head_dim
+    // values (t / 32) * D / 8 .. of the four shares and stores them.
+    float *share_out = reinterpret_cast<float *>(stage_lds);                  // [WAVES][D][32]
+    float *share_max = share_out + WAVES * D * 32;                            // [WAVES][32]
+    float *share_sum = share_max + WAVES * 32;                                // [WAVES][32]
+    static_assert((WAVES * D * 32 + 2 * WAVES * 32) * sizeof(float) <= 4 * (size_t)STAGE_BYTES, "the shares fit the stages");
+    const float wave_total = lanes_xor_sum(running_sum, 32);
+    if (half == 0) {
+      share_max[wave * 32 + row_lane] = running_max;
+      share_sum[wave * 32 + row_lane] = wave_total;
+    }
+#pragma unroll
+    for (int jj = 0; jj < JJ; ++jj)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        share_out[(wave * D + 32 * jj + (r >> 2) * 8 + half * 4 + (r & 3)) * 32 + row_lane] = out_acc[jj][r];
+    __syncthreads();
+    constexpr int PER_THREAD = D / 8;  // head_dim values per thread: 32 rows x 8 threads a row
+    const uint32_t out_row_index = q0 + (threadIdx.x & 31);
+    const uint32_t d0 = (threadIdx.x >> 5) * PER_THREAD;
+    float best = -INFINITY;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) best = fmaxf(best, share_max[w * 32 + (threadIdx.x & 31)]);
+    float weight[WAVES], denominator = 0.0f;
+#pragma unroll
+    for (int w = 0; w < WAVES; ++w) {
+      const float share = share_max[w * 32 + (threadIdx.x & 31)];
+      weight[w] = share == -INFINITY ? 0.0f : __builtin_amdgcn_exp2f((share - best) * score_scale);
+      denominator += weight[w] * share_sum[w * 32 + (threadIdx.x & 31)];
+    }
+    if (out_row_index >= a.query_length) return;
+    const float inverse = denominator != 0.0f ? 1.0f / denominator : 0.0f;
+    uint16_t *out_row = a.token_first_output
+                            ? a.output + (((size_t)batch * a.query_length + out_row_index) * a.heads + head) * D
+                            : a.output + (((size_t)batch * a.heads + head) * a.query_length + out_row_index) * D;
+#pragma unroll
+    for (int e = 0; e < PER_THREAD; e += 4) {
+      float value[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float sum = 0.0f;
+#pragma unroll
+        for (int w = 0; w < WAVES; ++w)
+          if (weight[w] != 0.0f) sum += weight[w] * share_out[(w * D + d0 + e + i) * 32 + (threadIdx.x & 31)];
+        value[i] = sum * inverse;
+      }
+      uint2 packed;
+      packed.x = (uint32_t)float_to_half_bits(value[0]) | ((uint32_t)float_to_half_bits(value[1]) << 16);
+      packed.y = (uint32_t)float_to_half_bits(value[2]) | ((uint32_t)float_to_half_bits(value[3]) << 16);
+      *reinterpret_cast<uint2 *>(out_row + d0 + e) = packed;
+    }
+    return;
   }
   if (!has_rows) return;
 
@@ -412,22 +483,43 @@ hipError_t launch_dense_attention(const DenseAttentionArgs &a, hipStream_t strea
       const bool masked = a.mask != nullptr && a.mask_batches > 0;
       static bool configured = false;  // the attribute is per device function
       if (!configured) {
-        hipError_t status =
-            hipFuncSetAttribute(reinterpret_cast<const void *>(&dense_attention_tile32_kernel<128, 4, 64, false>),
-                                hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
-        if (status == hipSuccess)
-          status = hipFuncSetAttribute(reinterpret_cast<const void *>(&dense_attention_tile32_kernel<128, 4, 64, true>),
-                                       hipFuncAttributeMaxDynamicSharedMemorySize, 64 * 1024);
-        if (status != hipSuccess) return status;
+        const void *large[] = {reinterpret_cast<const void *>(&dense_attention_tile32_kernel<128, 4, 64, false>),
+                               reinterpret_cast<const void *>(&dense_attention_tile32_kernel<128, 4, 64, true>),
+                               reinterpret_cast<const void *>(&dense_attention_tile32_kernel<128, 4, 128, false, true>),
+                               reinterpret_cast<const void *>(&dense_attention_tile32_kernel<128, 4, 128, true, true>),
+                               reinterpret_cast<const void *>(&dense_attention_tile32_kernel<64, 4, 128, false, true>),
+                               reinterpret_cast<const void *>(&dense_attention_tile32_kernel<64, 4, 128, true, true>)};
+        for (const void *kernel : large) {
+          const hipError_t status = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
+          if (status != hipSuccess) return status;
+        }
         configured = true;
+      }
+      DenseAttentionArgs scheduled = a;
+      scheduled.cus_per_xcd = (uint32_t)device_compute_units() / 8;
+      // Fewer workgroups of 128 rows than CUs: the launch lasts as long as one wave's walk over the
+      // keys of its slab, so the waves of a workgroup share 32 rows and a quarter of the keys each
+      // (four times the workgroups, a quarter of the walk): 9 heads x 2048 tokens of 64, causal,
+      // 45.0 -> 22.9 us.  Larger launches keep 128 rows a workgroup: a stage of K and V then serves
+      // four times as many rows.
+      if (workgroups < (uint64_t)device_compute_units() && a.key_length >= 256) {
+        const size_t bytes = 2 * 2 * (size_t)128 * a.head_dim * 2;
+        const dim3 grid((uint32_t)((a.query_length + 31) / 32) * a.heads * a.batches), block(256);
+        if (a.head_dim == 64 && masked)
+          hipLaunchKernelGGL((dense_attention_tile32_kernel<64, 4, 128, true, true>), grid, block, bytes, stream, scheduled);
+        else if (a.head_dim == 64)
+          hipLaunchKernelGGL((dense_attention_tile32_kernel<64, 4, 128, false, true>), grid, block, bytes, stream, scheduled);
+        else if (masked)
+          hipLaunchKernelGGL((dense_attention_tile32_kernel<128, 4, 128, true, true>), grid, block, bytes, stream, scheduled);
+        else
+          hipLaunchKernelGGL((dense_attention_tile32_kernel<128, 4, 128, false, true>), grid, block, bytes, stream, scheduled);
+        return hipGetLastError();
       }
       // 32 x 32 wave tiles over shared LDS stages, four waves and 64 keys a stage.  (Workgroups of two
       // waves with 32-key stages, twice as many and four per CU, so that short causal launches are not
       // as long as their longest workgroup, measured slower: 105.6 against 91.2 us at 32 heads x 2048
       // tokens - one tile per barrier, half the sharing.)
       const size_t bytes = 2 * 2 * (size_t)64 * a.head_dim * 2;
-      DenseAttentionArgs scheduled = a;
-      scheduled.cus_per_xcd = (uint32_t)device_compute_units() / 8;
       const dim3 grid((uint32_t)workgroups), block(256);
       if (a.head_dim == 64 && masked)
         hipLaunchKernelGGL((dense_attention_tile32_kernel<64, 4, 64, true>), grid, block, bytes, stream, scheduled);

@@ -279,3 +279,46 @@ def test_rejects_bad_arguments(runtime):
     bad_heads = attention_params(1, 2, 4, 4, 64, 0, 0, False, 1.0, 3)
     with pytest.raises(Exception):
         run(runtime, "llmopt_attention_f16", query, key, key, None, bad_heads, (1, 2, 4, 64))
+
+
+@pytest.mark.parametrize("dim,heads,kv_heads,new,past,mode", [
+    (64, 9, 3, 700, 0, "causal"), (128, 4, 2, 45, 900, "causal"), (64, 2, 1, 33, 257, "none"),
+    (128, 2, 2, 130, 300, "bool"), (64, 3, 3, 64, 1000, "f16"), (128, 1, 1, 1000, 0, "causal"),
+])
+def test_small_launches_split_the_keys_of_a_slab_over_the_waves(runtime, dim, heads, kv_heads, new, past, mode):
+    """Launches with fewer 128-row workgroups than the device has CUs and at least 256 keys: the four
+    waves of a workgroup share 32 query rows and take a quarter of every 128-key stage each, and
+    their shares (maxima, denominators, weighted sums) are folded through LDS.  Causal limits with
+    cached tokens, partial last stages and tiles, rows past the end, both mask types, both layouts."""
+    rng = np.random.default_rng(dim + heads + new + past)
+    batches, length = 2, past + new
+    query = rng.standard_normal((batches, heads, new, dim)).astype(np.float16)
+    key = rng.standard_normal((batches, kv_heads, length, dim)).astype(np.float16)
+    value = rng.standard_normal((batches, kv_heads, length, dim)).astype(np.float16)
+    scale = 1.0 / math.sqrt(dim)
+    mask, mask_batches, mask_heads, mask_dtype = None, 0, 0, 0
+    if mode == "causal":
+        allowed = np.broadcast_to((np.arange(length)[None, :] <= past + np.arange(new)[:, None])[None, None],
+                                  (batches, heads, new, length))
+    elif mode == "none":
+        allowed = np.ones((batches, heads, new, length), dtype=bool)
+    else:
+        mask_batches, mask_heads = batches, heads
+        allowed = rng.random((batches, heads, new, length)) < 0.5
+        allowed[:, :, 3, :] = False      # a row without keys
+        allowed[:, :, 5, :200] = False   # a row whose first shares are empty
+        mask_dtype = 1 if mode == "bool" else 2
+        mask = allowed.astype(np.uint8) if mode == "bool" else np.where(allowed, 0.0, -np.inf).astype(np.float16)
+    token_major = (new + past) % 2 == 1
+    params = attention_params(batches, heads, new, length, dim, mask_batches, mask_heads, mode == "causal", scale,
+                              kv_heads, token_first_output=int(token_major), past_length=past if mode == "causal" else 0,
+                              token_first_value=int(token_major), mask_dtype=mask_dtype)
+    value_in = np.ascontiguousarray(value.transpose(0, 2, 1, 3)) if token_major else value
+    out_shape = (batches, new, heads, dim) if token_major else (batches, heads, new, dim)
+    got = run(runtime, f"llmopt_attention_f16_simd_h{dim}", query, key, value_in, mask, params, out_shape)
+    if token_major:
+        got = got.transpose(0, 2, 1, 3)
+    want = expected(query, key, value, allowed, scale)
+    if mode in ("bool", "f16"):
+        assert np.all(got[:, :, 3, :].view(np.uint16) == 0)
+    assert_close_to_oracle(got, want, f"key-split D={dim} {heads}/{kv_heads} {new} new after {past}, {mode}")
