@@ -66,6 +66,19 @@ __device__ __forceinline__ uint32_t sequence_past(const Q8AttentionArgs &a, uint
   return a.past_lengths ? min(a.past_lengths[b], a.max_past_length) : a.past_length;
 }
 
+// Pool tokens the split kernels read for sequence b: with a sliding window the last window - 1
+// cached tokens (the window counts the current token: first_key = key_length - window,
+// lib/metal_cache_source.ml:430-431), i.e. a shorter context that starts `first` entries into
+// the sequence's slot table.
+struct PoolSpan {
+  uint32_t first, length;
+};
+__device__ __forceinline__ PoolSpan sequence_span(const Q8AttentionArgs &a, uint32_t b) {
+  const uint32_t past = sequence_past(a, b);
+  const uint32_t first = (a.window == 0 || past < a.window) ? 0 : past + 1 - a.window;
+  return {first, past - first};
+}
+
 // ---- balanced split --------------------------------------------------------------------
 // With chunks of a fixed size the number of workgroups is whatever the contexts give, and the
 // device runs them in rounds: 1028 chunks on 768 resident workgroups take two rounds, the
@@ -105,8 +118,9 @@ __device__ __forceinline__ SplitPlan split_plan(const Q8AttentionArgs &a, uint32
 #pragma unroll
   for (int k = 0; k < kPlanBlocks; ++k) {
     const uint32_t b = k * 64 + lane;
-    past[k] = b < a.batches ? sequence_past(a, b) : 0;
-    slot_offset[k] = BY_INDEX && a.slot_offsets != nullptr && b < a.batches ? a.slot_offsets[b] : 0;
+    const PoolSpan span = b < a.batches ? sequence_span(a, b) : PoolSpan{0, 0};
+    past[k] = span.length;
+    slot_offset[k] = (BY_INDEX && a.slot_offsets != nullptr && b < a.batches ? a.slot_offsets[b] : 0) + span.first;
   }
   uint32_t total = 0;
 #pragma unroll
@@ -185,8 +199,9 @@ q8_attention_split_kernel(Q8AttentionArgs a, uint32_t chunks_max, uint32_t fixed
     slot_offset = plan.slot_offset;
     partial_index = (size_t)kv_head * balanced_slots + blockIdx.x;
   } else {
-    past = sequence_past(a, batch);
-    slot_offset = a.slot_offsets ? a.slot_offsets[batch] : 0;
+    const PoolSpan span = sequence_span(a, batch);
+    past = span.length;
+    slot_offset = (a.slot_offsets ? a.slot_offsets[batch] : 0) + span.first;
     partial_index = ((size_t)batch * a.kv_heads + kv_head) * chunks_max + chunk;
   }
   const uint32_t chunk_begin = chunk * chunk_tokens;
@@ -517,7 +532,7 @@ __global__ __launch_bounds__(kMergeSlices *D) void q8_attention_merge_kernel(Q8A
     chunks = plan.chunks;
     partial += ((size_t)kv_head * balanced_slots + plan.first) * stride;
   } else {
-    const uint32_t past = sequence_past(a, batch);
+    const uint32_t past = sequence_span(a, batch).length;
     chunks = (past + chunk_tokens - 1) / chunk_tokens;
     partial += ((size_t)batch * a.kv_heads + kv_head) * chunks_max * stride;
   }
@@ -673,6 +688,12 @@ __global__ __launch_bounds__(kGeneralWaves * 64) void q8_attention_general_kerne
   float acc[8] = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
   float maximum = -INFINITY, denominator = 0.0f;
 
+  // A wave's tile is a chain of trips to memory (slot table, key rows, value rows), one tile after
+  // the other, and a load under a branch is waited for where it stands.  So: the slot of the next
+  // tile's key is requested a tile ahead; the pool requests of a tile go out for every lane, at a
+  // clamped valid address, and what a lane has no use for is dropped afterwards.
+  const uint32_t last_past = r.past == 0 ? 0 : r.past - 1;
+  uint32_t next_slot = r.past != 0 ? slots[min(r.first_key + lane, last_past)] : 0;
   for (uint32_t base = r.first_key; base < r.key_length; base += 64) {
     // ---- scores: lane = key ----
     const uint32_t key_position = base + lane;
@@ -684,40 +705,75 @@ __global__ __launch_bounds__(kGeneralWaves * 64) void q8_attention_general_kerne
       active = a.mask_dtype == 2 ? half_bits_to_float(reinterpret_cast<const uint16_t *>(a.mask)[at]) >= 0.0f
                                  : a.mask[at] != 0;
     }
-    const uint8_t *slot = a.pool;
-    if (in_range && is_past) slot = a.pool + (size_t)slots[key_position] * a.token_stride;
+    // (lanes without a pool key read slot `next_slot` of a valid key of the sequence, or the pool's first token)
+    const uint8_t *slot = a.pool + (size_t)next_slot * a.token_stride;
+    if (r.past != 0) next_slot = slots[min(key_position + 64, last_past)];
     float score = 0.0f;
-    if (in_range && is_past) {
+    if (r.past != 0 && base < r.past) {
       const uint8_t *key_row = slot + a.key_offset + r.kv_head * D;
-      for (uint32_t g = 0; g < groups; ++g) {
-        float part = 0.0f;
+      float key_scale[8];
+#pragma unroll
+      for (int g = 0; g < 8; ++g)
+        key_scale[g] = q8_scale_at(slot, a.token_elements, key_scale_index + min((uint32_t)g, groups - 1));
+      auto load_group = [&](uint32_t g, uint32_t (&words)[16]) __attribute__((always_inline)) {
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          uint32_t words[4];
           if (ALIGNED) {
             const u32x4_t loaded = *reinterpret_cast<const u32x4_t __attribute__((aligned(4))) *>(key_row + g * 64 + j * 16);
-            words[0] = loaded[0], words[1] = loaded[1], words[2] = loaded[2], words[3] = loaded[3];
+            words[4 * j] = loaded[0], words[4 * j + 1] = loaded[1], words[4 * j + 2] = loaded[2], words[4 * j + 3] = loaded[3];
           } else {
 #pragma unroll
             for (int w = 0; w < 4; ++w) {
               const uint8_t *b = key_row + g * 64 + j * 16 + w * 4;
-              words[w] = (uint32_t)b[0] | ((uint32_t)b[1] << 8) | ((uint32_t)b[2] << 16) | ((uint32_t)b[3] << 24);
+              words[4 * j + w] = (uint32_t)b[0] | ((uint32_t)b[1] << 8) | ((uint32_t)b[2] << 16) | ((uint32_t)b[3] << 24);
             }
           }
+        }
+      };
+      auto dot_group = [&](uint32_t g, const uint32_t (&words)[16]) __attribute__((always_inline)) {
+        float part = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
           const uint4 q_lo = *reinterpret_cast<const uint4 *>(query_lds + (g * 64 + j * 16) / 2);
           const uint4 q_hi = *reinterpret_cast<const uint4 *>(query_lds + (g * 64 + j * 16) / 2 + 4);
           const uint32_t q_pairs[8] = {q_lo.x, q_lo.y, q_lo.z, q_lo.w, q_hi.x, q_hi.y, q_hi.z, q_hi.w};
 #pragma unroll
           for (int w = 0; w < 4; ++w) {
             h2_t lo, hi;
-            int8x4_to_h2(words[w] ^ 0x80808080u, lo, hi);
+            int8x4_to_h2(words[4 * j + w] ^ 0x80808080u, lo, hi);
             part = __builtin_amdgcn_fdot2(lo, as_h2(q_pairs[2 * w]), part, false);
             part = __builtin_amdgcn_fdot2(hi, as_h2(q_pairs[2 * w + 1]), part, false);
           }
         }
-        score = fmaf(part, q8_scale_at(slot, a.token_elements, key_scale_index + g), score);
+        return part;
+      };
+      auto scale_of = [&](uint32_t g) __attribute__((always_inline)) {
+        float scale = key_scale[0];
+#pragma unroll
+        for (int e = 1; e < 8; ++e) scale = g == (uint32_t)e ? key_scale[e] : scale;
+        return scale;
+      };
+      if (groups <= 2) {
+        // the whole key row (64 or 128 bytes) in one trip
+        uint32_t first[16], second[16];
+        load_group(0, first);
+        load_group(groups - 1, second);
+        score = dot_group(0, first) * key_scale[0];
+        if (groups == 2) score = fmaf(dot_group(1, second), key_scale[1], score);
+      } else {
+        // four scale groups (256 bytes of the key row) per trip
+        for (uint32_t g = 0; g < groups; g += 4) {
+          uint32_t words[4][16];
+#pragma unroll
+          for (int e = 0; e < 4; ++e) load_group(min(g + e, groups - 1), words[e]);
+#pragma unroll
+          for (int e = 0; e < 4; ++e)
+            if (g + e < groups) score = fmaf(dot_group(g + e, words[e]), scale_of(g + e), score);
+        }
       }
-    } else if (in_range) {
+    }
+    if (in_range && !is_past) {
+      score = 0.0f;
       const uint16_t *key_row = a.current_key + current_base + (size_t)(key_position - r.past) * D;
       for (uint32_t i = 0; i < D / 2; ++i)
         score = __builtin_amdgcn_fdot2(as_h2((uint32_t)key_row[2 * i] | ((uint32_t)key_row[2 * i + 1] << 16)),
@@ -745,30 +801,48 @@ __global__ __launch_bounds__(kGeneralWaves * 64) void q8_attention_general_kerne
     __builtin_amdgcn_wave_barrier();
     // ---- values: lanes_per_key lanes share a key's row ----
     const uint32_t tile_keys = min(64u, r.key_length - base);
+    const uint32_t pool_keys = base < r.past ? min(tile_keys, r.past - base) : 0;  // the tile's first keys
     if (value_lane) {
-      for (uint32_t k0 = 0; k0 < tile_keys; k0 += keys_per_request) {
+      // pool rows, sixteen requests on the way at a time: every slot of the tile's table holds a valid
+      // address, so the requests go out whether or not the key counts, and its weight decides
+      constexpr int AHEAD = 16;
+      for (uint32_t k0 = 0; k0 < pool_keys; k0 += keys_per_request * AHEAD) {
+        uint32_t word[AHEAD][2];
+        float weight[AHEAD];
+#pragma unroll
+        for (int u = 0; u < AHEAD; ++u) {
+          const uint32_t wanted = k0 + u * keys_per_request + key_sub;
+          const uint32_t k = min(wanted, 63u);
+          weight[u] = wanted < pool_keys ? weight_lds[(d0 >> 6) * 64 + k] : 0.0f;
+          const uint8_t *b = reinterpret_cast<const uint8_t *>(address_lds[k]) + d0;
+#pragma unroll
+          for (int w = 0; w < 2; ++w) {
+            const uint8_t *at = b + (per_lane == 8 ? 4 * w : 0);
+            if (ALIGNED)
+              word[u][w] = *reinterpret_cast<const uint32_t *>(at);
+            else
+              word[u][w] = (uint32_t)at[0] | ((uint32_t)at[1] << 8) | ((uint32_t)at[2] << 16) | ((uint32_t)at[3] << 24);
+          }
+        }
+#pragma unroll
+        for (int u = 0; u < AHEAD; ++u)
+#pragma unroll
+          for (int w = 0; w < 2; ++w) {
+            h2_t lo, hi;
+            int8x4_to_h2(word[u][w] ^ 0x80808080u, lo, hi);
+            const float share = (w == 0 || per_lane == 8) ? weight[u] : 0.0f;
+            acc[4 * w + 0] = fmaf(share, (float)lo[0], acc[4 * w + 0]);
+            acc[4 * w + 1] = fmaf(share, (float)lo[1], acc[4 * w + 1]);
+            acc[4 * w + 2] = fmaf(share, (float)hi[0], acc[4 * w + 2]);
+            acc[4 * w + 3] = fmaf(share, (float)hi[1], acc[4 * w + 3]);
+          }
+      }
+      // the query tokens' own fp16 rows (the last keys; at most query_length of them in all)
+      for (uint32_t k0 = pool_keys; k0 < tile_keys; k0 += keys_per_request) {
         const uint32_t k = min(k0 + key_sub, 63u);
         const float weight = k0 + key_sub < tile_keys ? weight_lds[(d0 >> 6) * 64 + k] : 0.0f;
-        const uint8_t *source = reinterpret_cast<const uint8_t *>(address_lds[k]);
-        if (kind_lds[k] != 0) {
-          for (uint32_t w = 0; w < per_lane / 4; ++w) {
-            const uint8_t *b = source + d0 + 4 * w;
-            uint32_t word;
-            if (ALIGNED)
-              word = *reinterpret_cast<const uint32_t *>(b);
-            else
-              word = (uint32_t)b[0] | ((uint32_t)b[1] << 8) | ((uint32_t)b[2] << 16) | ((uint32_t)b[3] << 24);
-            h2_t lo, hi;
-            int8x4_to_h2(word ^ 0x80808080u, lo, hi);
-            acc[4 * w + 0] = fmaf(weight, (float)lo[0], acc[4 * w + 0]);
-            acc[4 * w + 1] = fmaf(weight, (float)lo[1], acc[4 * w + 1]);
-            acc[4 * w + 2] = fmaf(weight, (float)hi[0], acc[4 * w + 2]);
-            acc[4 * w + 3] = fmaf(weight, (float)hi[1], acc[4 * w + 3]);
-          }
-        } else {
-          const uint16_t *halves = reinterpret_cast<const uint16_t *>(source) + d0;
-          for (uint32_t e = 0; e < per_lane; ++e) acc[e] = fmaf(weight, half_bits_to_float(halves[e]), acc[e]);
-        }
+        const uint16_t *halves = reinterpret_cast<const uint16_t *>(address_lds[k]) + d0;
+        for (uint32_t e = 0; e < per_lane; ++e) acc[e] = fmaf(weight, half_bits_to_float(halves[e]), acc[e]);
       }
     }
     __builtin_amdgcn_wave_barrier();
@@ -785,10 +859,15 @@ __global__ __launch_bounds__(kGeneralWaves * 64) void q8_attention_general_kerne
   }
 }
 
+// The longest span of pool tokens a sequence of the launch can have (see sequence_span).
+uint32_t longest_span(const Q8AttentionArgs &a) {
+  return a.window != 0 && a.max_past_length >= a.window ? a.window - 1 : a.max_past_length;
+}
+
 bool use_split_path(const Q8AttentionArgs &a) {
   const uint32_t q_len = a.query_length == 0 ? 1 : a.query_length;
   const bool masked = a.mask != nullptr && a.mask_batches > 0 && a.mask_dtype != 0;
-  if (q_len != 1 || masked || a.window != 0) return false;
+  if (q_len != 1 || masked) return false;
   if (a.head_dim != 64 && a.head_dim != 128) return false;
   if (a.kv_heads == 0 || a.query_heads % a.kv_heads != 0) return false;
   if (a.query_heads / a.kv_heads > 16) return false;
@@ -798,22 +877,22 @@ bool use_split_path(const Q8AttentionArgs &a) {
   if (a.token_elements % 2 != 0) return false;
   // D = 128 reads the two group scales of a head as one aligned dword
   if (a.head_dim == 128 && (a.key_offset % 128 != 0 || a.value_offset % 128 != 0)) return false;
-  if (a.max_past_length > (uint32_t)kMaxChunkTokens * kMaxSplitChunks) return false;
-  return a.max_past_length >= 64;  // short contexts: one launch of the general kernel is cheaper
+  if (longest_span(a) > (uint32_t)kMaxChunkTokens * kMaxSplitChunks) return false;
+  return longest_span(a) >= 64;  // short contexts: one launch of the general kernel is cheaper
 }
 
 // A wave is bound by the latency of its tiles, one after the other: when 128-token
 // chunks give fewer waves than the device holds, shorter chunks finish sooner.
 uint32_t split_chunk_tokens(const Q8AttentionArgs &a) {
-  const uint64_t waves = (uint64_t)a.batches * a.kv_heads * ((a.max_past_length + 127) / 128);
+  const uint64_t waves = (uint64_t)a.batches * a.kv_heads * ((longest_span(a) + 127) / 128);
   uint32_t tokens = waves >= 1024 ? 128 : waves >= 512 ? 64 : 32;
-  while ((a.max_past_length + tokens - 1) / tokens > (uint32_t)kMaxSplitChunks) tokens *= 2;
+  while ((longest_span(a) + tokens - 1) / tokens > (uint32_t)kMaxSplitChunks) tokens *= 2;
   return tokens;
 }
 
 uint32_t split_chunks(const Q8AttentionArgs &a) {
   const uint32_t tokens = split_chunk_tokens(a);
-  return (a.max_past_length + tokens - 1) / tokens;
+  return (longest_span(a) + tokens - 1) / tokens;
 }
 
 // Waves of the split kernel a SIMD holds at once, from the registers the compiler gave it

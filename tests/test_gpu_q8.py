@@ -308,6 +308,62 @@ def test_decode_attention_balanced_split_over_many_sequences(runtime, b, kvh, gr
     assert_close_to_oracle(out, expected, f"balanced split b{b} kv{kvh} d{dim}")
 
 
+@pytest.mark.parametrize("b,kvh,group,dim,window,seed", [(9, 3, 3, 64, 200, 1), (70, 2, 4, 128, 65, 2),
+                                                         (4, 8, 4, 128, 1024, 3), (3, 1, 1, 64, 4000, 4)])
+def test_decode_attention_sliding_window_over_ragged_batch(runtime, b, kvh, group, dim, window, seed):
+    """A sliding window on the split-over-context kernels: every sequence reads its last window - 1
+    cached tokens (the window counts the current token) through a slot table entered `first` entries
+    in.  Contexts below, at and above the window, empty ones, and windows that start inside a tile."""
+    rng = np.random.default_rng(100 + seed)
+    lengths = [int(v) for v in rng.integers(1, 3 * window // 2 + 200, size=b)]
+    for index, value in zip(range(b), [2 * window + 37, window - 1, window, window + 1, 0, 1, window - 2]):
+        lengths[index] = value
+    h = kvh * group
+    pool, slots, offsets, te, stride, ko, vo = build_pool(rng, kvh, dim, lengths)
+    query = rng.standard_normal((b, h, 1, dim)).astype(np.float16)
+    ck = rng.standard_normal((b, kvh, 1, dim)).astype(np.float16)
+    cv = rng.standard_normal((b, kvh, 1, dim)).astype(np.float16)
+    params = PagedParams(batches=b, query_heads=h, kv_heads=kvh, past_length=0, head_dim=dim,
+                         mask_batches=0, mask_heads=0, token_elements=te, key_offset=ko,
+                         value_offset=vo, group_size=64, token_stride=stride,
+                         scale=1.0 / math.sqrt(dim), query_length=1, mask_dtype=0, window=window)
+    out = run_paged(runtime, "llmopt_attention_q8_paged_batched", query, ck, cv, pool, slots, None,
+                    params, lengths=lengths, offsets=offsets)
+    expected = oracle.paged_attention_q8(query, ck, cv, pool, slots, None, params,
+                                         past_lengths=np.array(lengths), slot_offsets=offsets)
+    assert np.all(np.isfinite(out))
+    assert_close_to_oracle(out, expected, f"window {window} b{b} kv{kvh} d{dim}")
+    # the window moves the result: without it the same launch gives something else
+    no_window = PagedParams.from_buffer_copy(bytes(params))
+    no_window.window = 0
+    unwindowed = oracle.paged_attention_q8(query, ck, cv, pool, slots, None, no_window,
+                                           past_lengths=np.array(lengths), slot_offsets=offsets)
+    assert np.abs(unwindowed[0].astype(np.float64) - expected[0].astype(np.float64)).max() > 1e-3
+
+
+@pytest.mark.parametrize("name,h,kvh,dim,past,window", [
+    ("llmopt_attention_q8_paged_simd_h64_gqa3", 9, 3, 64, 2048, 512),
+    ("llmopt_attention_q8_paged_simd_generic", 32, 8, 128, 700, 300),
+    ("llmopt_attention_q8_paged_simd_h64", 4, 4, 64, 100, 100),
+    ("llmopt_attention_q8_paged_simd_generic", 8, 2, 128, 99, 100)])
+def test_reference_entries_with_sliding_window(runtime, name, h, kvh, dim, past, window):
+    """The reference's own entries (one context length for the whole batch) with a window: the
+    split-over-context kernels when the windowed context has 64 tokens or more."""
+    rng = np.random.default_rng(past + window)
+    b = 2
+    pool, slots, _, te, stride, ko, vo = build_pool(rng, kvh, dim, [past])
+    query = rng.standard_normal((b, h, 1, dim)).astype(np.float16)
+    ck = rng.standard_normal((b, kvh, 1, dim)).astype(np.float16)
+    cv = rng.standard_normal((b, kvh, 1, dim)).astype(np.float16)
+    params = PagedParams(batches=b, query_heads=h, kv_heads=kvh, past_length=past, head_dim=dim,
+                         mask_batches=0, mask_heads=0, token_elements=te, key_offset=ko,
+                         value_offset=vo, group_size=64, token_stride=stride,
+                         scale=1.0 / math.sqrt(dim), query_length=1, mask_dtype=0, window=window)
+    out = run_paged(runtime, name, query, ck, cv, pool, slots, None, params)
+    expected = oracle.paged_attention_q8(query, ck, cv, pool, slots, None, params)
+    assert_close_to_oracle(out, expected, f"{name} window {window} of {past}")
+
+
 ROW_CASES = [
     # (b, h, kvh, dim, past, q_len, window, mask_dtype)
     (1, 2, 1, 64, 10, 1, 0, 0), (2, 4, 2, 128, 33, 1, 8, 0), (1, 3, 1, 64, 20, 3, 0, 1),
