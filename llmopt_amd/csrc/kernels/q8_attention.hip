@@ -8,8 +8,8 @@
 //
 // Two kernels:
 //
-//  * q8_attention_split_kernel (decode fast path: one query token, no mask, no
-//    window, D in {64,128}, up to 16 query heads per KV head).  HBM-bound: the
+//  * q8_attention_split_kernel (decode fast path: one query token, no mask, with or
+//    without a sliding window, D in {64,128,256}, up to 16 query heads per KV head).  HBM-bound: the
 //    context is split into chunks across workgroups, every KV byte is read once
 //    per KV head and shared by all query heads of the group through the MFMA
 //    column dimension.  int8 -> exact fp16 integers in registers; the fp16
@@ -20,8 +20,8 @@
 //
 //  * q8_attention_general_kernel: one wave per (batch, head, query position) row,
 //    64 keys at a time, one key per lane for the scores and one value row per
-//    group of lanes for the weighted sum.  Covers everything else (mask, window,
-//    several query tokens, other head sizes, unaligned pools).
+//    group of lanes for the weighted sum.  Covers everything else (masks,
+//    several query tokens, other head sizes, unaligned pools, contexts under 64 tokens).
 #include <algorithm>
 #include <type_traits>
 
@@ -166,12 +166,20 @@ __device__ __forceinline__ SplitPlan split_plan(const Q8AttentionArgs &a, uint32
 // OFF32: the pool is smaller than 4 GiB, so slot byte offsets fit 32 bits and the
 // loads can use a scalar base plus a 32-bit vector offset.
 // Three waves per SIMD: left alone the register allocator takes 209 registers
-// (two waves), and the kernel is bound by the latency of each wave's requests.
+// (two waves), and the kernel is bound by the latency of each wave's requests.  (Heads of 256:
+// two waves; a tile's lines, operands and the 64 output registers do not fit a third.)
+template <int D>
+constexpr int split_waves_wanted() {
+  return D <= 128 ? 3 : 2;
+}
+
 template <int D, bool OFF32, bool A16>
-__global__ __launch_bounds__(kSplitMaxWaves * 64) __attribute__((amdgpu_waves_per_eu(3, 3))) void
+__global__ __launch_bounds__(kSplitMaxWaves * 64)
+    __attribute__((amdgpu_waves_per_eu(split_waves_wanted<D>(), split_waves_wanted<D>()))) void
 q8_attention_split_kernel(Q8AttentionArgs a, uint32_t chunks_max, uint32_t fixed_chunk_tokens,
                           uint32_t balanced_slots) {
   constexpr int GROUPS = D / 64;      // scale groups per head
+  constexpr int SW = (GROUPS + 1) / 2;  // dwords that hold a (token, head)'s fp16 group scales
   constexpr int KLOADS = GROUPS;      // 16-byte K loads per lane per tile
   constexpr int VBLOCKS = D / 16;     // PV MFMAs (16 head_dim rows each)
   // One wave per KV head; the waves of a workgroup walk the same tokens, so the
@@ -246,7 +254,7 @@ q8_attention_split_kernel(Q8AttentionArgs a, uint32_t chunks_max, uint32_t fixed
   constexpr int KL = kTileTokens / TPI;  // load instructions per tile and operand
   constexpr int ROW = D + 32;            // LDS row stride: conflict-free 16-byte reads down the tokens
   const uint32_t line_token = lane / LPT, line_piece = lane % LPT;
-  __shared__ __attribute__((aligned(16))) uint8_t turn_lds[kSplitMaxWaves][2 * kTileTokens * ROW + 128];
+  __shared__ __attribute__((aligned(16))) uint8_t turn_lds[kSplitMaxWaves][2 * kTileTokens * ROW + 128 * SW];
   uint8_t *key_patch = turn_lds[threadIdx.x >> 6];
   uint8_t *value_patch = key_patch + kTileTokens * ROW;
   uint32_t *scale_patch = reinterpret_cast<uint32_t *>(key_patch + 2 * kTileTokens * ROW);
@@ -263,13 +271,13 @@ q8_attention_split_kernel(Q8AttentionArgs a, uint32_t chunks_max, uint32_t fixed
   // used before the tile is processed, or the loads are waited for at once.
   struct TileLine {
     u32x4_t k[KL], v[KL];
-    uint32_t scale;  // D = 128: both group scales of the token in one dword; D = 64: one scale in the low half
+    uint32_t scale[SW];  // two group scales of the token per dword (D = 64: one scale in the low half)
   };
   struct TileRaw {              // the same tile in operand order
     u32x4_t k[KLOADS];          // lane (token = col, quad): 16 head_dim values per group
     uint32_t v[4][GROUPS];      // lane (d-row = col, quad): tokens quad*4 + i
-    uint32_t k_scale[4];        // tokens quad*4 + i
-    uint32_t v_scale[4];
+    uint32_t k_scale[4][SW];    // tokens quad*4 + i
+    uint32_t v_scale[4][SW];
   };
   auto load_slots = [&](uint32_t tile, TileSlots &out) __attribute__((always_inline)) {
     const uint32_t token0 = chunk_begin + tile * kTileTokens;
@@ -290,10 +298,12 @@ q8_attention_split_kernel(Q8AttentionArgs a, uint32_t chunks_max, uint32_t fixed
         out.v[n] = *reinterpret_cast<const KeyVector *>(a.pool + row + value_base);
       }
       const uint32_t scale_offset = where.scale * a.token_stride + scale_byte;
-      if (GROUPS == 2)
-        out.scale = *reinterpret_cast<const uint32_t *>(a.pool + scale_offset);
-      else
-        out.scale = *reinterpret_cast<const uint16_t *>(a.pool + scale_offset);
+      if (GROUPS >= 2) {
+#pragma unroll
+        for (int w = 0; w < SW; ++w) out.scale[w] = *reinterpret_cast<const uint32_t *>(a.pool + scale_offset + 4 * w);
+      } else {
+        out.scale[0] = *reinterpret_cast<const uint16_t *>(a.pool + scale_offset);
+      }
       return;
     }
 #pragma unroll
@@ -303,10 +313,12 @@ q8_attention_split_kernel(Q8AttentionArgs a, uint32_t chunks_max, uint32_t fixed
       out.v[n] = *reinterpret_cast<const KeyVector *>(row + value_base);
     }
     const uint8_t *scale_at = a.pool + (size_t)where.scale * a.token_stride + scale_byte;
-    if (GROUPS == 2)
-      out.scale = *reinterpret_cast<const uint32_t *>(scale_at);
-    else
-      out.scale = *reinterpret_cast<const uint16_t *>(scale_at);
+    if (GROUPS >= 2) {
+#pragma unroll
+      for (int w = 0; w < SW; ++w) out.scale[w] = *reinterpret_cast<const uint32_t *>(scale_at + 4 * w);
+    } else {
+      out.scale[0] = *reinterpret_cast<const uint16_t *>(scale_at);
+    }
   };
   auto turn = [&](const TileLine &line, TileRaw &raw) __attribute__((always_inline)) {
     __builtin_amdgcn_wave_barrier();
@@ -316,7 +328,10 @@ q8_attention_split_kernel(Q8AttentionArgs a, uint32_t chunks_max, uint32_t fixed
       *reinterpret_cast<u32x4_t *>(key_patch + at) = line.k[n];
       *reinterpret_cast<u32x4_t *>(value_patch + at) = line.v[n];
     }
-    if (lane < 32) scale_patch[lane] = line.scale;
+    if (lane < 32) {
+#pragma unroll
+      for (int w = 0; w < SW; ++w) scale_patch[w * 32 + lane] = line.scale[w];
+    }
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
     for (int g = 0; g < GROUPS; ++g)
@@ -326,12 +341,15 @@ q8_attention_split_kernel(Q8AttentionArgs a, uint32_t chunks_max, uint32_t fixed
 #pragma unroll
       for (int g = 0; g < GROUPS; ++g)
         raw.v[i][g] = *reinterpret_cast<const uint32_t *>(value_patch + (quad * 4 + i) * ROW + g * 64 + col * 4);
-    const u32x4_t key_scales = *reinterpret_cast<const u32x4_t *>(scale_patch + quad * 4);
-    const u32x4_t value_scales = *reinterpret_cast<const u32x4_t *>(scale_patch + 16 + quad * 4);
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      raw.k_scale[i] = key_scales[i];
-      raw.v_scale[i] = value_scales[i];
+    for (int w = 0; w < SW; ++w) {
+      const u32x4_t key_scales = *reinterpret_cast<const u32x4_t *>(scale_patch + w * 32 + quad * 4);
+      const u32x4_t value_scales = *reinterpret_cast<const u32x4_t *>(scale_patch + w * 32 + 16 + quad * 4);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        raw.k_scale[i][w] = key_scales[i];
+        raw.v_scale[i][w] = value_scales[i];
+      }
     }
     __builtin_amdgcn_wave_barrier();
   };
@@ -354,7 +372,7 @@ q8_attention_split_kernel(Q8AttentionArgs a, uint32_t chunks_max, uint32_t fixed
 #pragma unroll
       for (int i = 0; i < 4; ++i)
         score[i] = fmaf(part[i] - key_bias[g],
-                        half_bits_to_float((uint16_t)(raw.k_scale[i] >> (16 * g))), score[i]);
+                        half_bits_to_float((uint16_t)(raw.k_scale[i][g >> 1] >> (16 * (g & 1)))), score[i]);
     }
     float tile_max = -INFINITY;
 #pragma unroll
@@ -393,7 +411,7 @@ q8_attention_split_kernel(Q8AttentionArgs a, uint32_t chunks_max, uint32_t fixed
       h4_t p_frag;
 #pragma unroll
       for (int i = 0; i < 4; ++i)
-        p_frag[i] = (_Float16)(p[i] * half_bits_to_float((uint16_t)(raw.v_scale[i] >> (16 * g))));
+        p_frag[i] = (_Float16)(p[i] * half_bits_to_float((uint16_t)(raw.v_scale[i][g >> 1] >> (16 * (g & 1)))));
       const uint32_t a0 = raw.v[0][g] ^ 0x80808080u, a1 = raw.v[1][g] ^ 0x80808080u;
       const uint32_t a2 = raw.v[2][g] ^ 0x80808080u, a3 = raw.v[3][g] ^ 0x80808080u;
       const uint32_t t01_lo = __builtin_amdgcn_perm(a1, a0, 0x05010400u);
@@ -868,15 +886,15 @@ bool use_split_path(const Q8AttentionArgs &a) {
   const uint32_t q_len = a.query_length == 0 ? 1 : a.query_length;
   const bool masked = a.mask != nullptr && a.mask_batches > 0 && a.mask_dtype != 0;
   if (q_len != 1 || masked) return false;
-  if (a.head_dim != 64 && a.head_dim != 128) return false;
+  if (a.head_dim != 64 && a.head_dim != 128 && a.head_dim != 256) return false;
   if (a.kv_heads == 0 || a.query_heads % a.kv_heads != 0) return false;
   if (a.query_heads / a.kv_heads > 16) return false;
   // 4-byte aligned K and V loads from pool slots (16-byte aligned K loads when the stride allows)
   if (a.token_stride % 4 != 0 || a.key_offset % 4 != 0 || a.value_offset % 4 != 0) return false;
   if ((reinterpret_cast<uintptr_t>(a.pool) & 3) != 0) return false;
   if (a.token_elements % 2 != 0) return false;
-  // D = 128 reads the two group scales of a head as one aligned dword
-  if (a.head_dim == 128 && (a.key_offset % 128 != 0 || a.value_offset % 128 != 0)) return false;
+  // D >= 128 reads the group scales of a head two to an aligned dword
+  if (a.head_dim >= 128 && (a.key_offset % 128 != 0 || a.value_offset % 128 != 0)) return false;
   if (longest_span(a) > (uint32_t)kMaxChunkTokens * kMaxSplitChunks) return false;
   return longest_span(a) >= 64;  // short contexts: one launch of the general kernel is cheaper
 }
@@ -923,7 +941,9 @@ uint32_t split_waves_per_simd() {
 // covers in a few passes.
 uint32_t balanced_split_slots(const Q8AttentionArgs &a) {
   if (a.batches < 2 || a.batches > 64 * kPlanBlocks) return 0;
-  const uint32_t per_simd = a.head_dim == 128 ? split_waves_per_simd<128>() : split_waves_per_simd<64>();
+  const uint32_t per_simd = a.head_dim == 256   ? split_waves_per_simd<256>()
+                            : a.head_dim == 128 ? split_waves_per_simd<128>()
+                                                : split_waves_per_simd<64>();
   // whole workgroups: one wave per KV head, at most kSplitMaxWaves of them
   const uint32_t waves = std::min<uint32_t>(a.kv_heads, kSplitMaxWaves);
   const uint32_t head_groups = (a.kv_heads + kSplitMaxWaves - 1) / kSplitMaxWaves;
@@ -977,7 +997,9 @@ hipError_t launch_q8_attention(const Q8AttentionArgs &a, hipStream_t stream) {
       hipLaunchKernelGGL(q8_attention_merge_kernel<D>, merge_grid, dim3(kMergeSlices * D), 0, stream, a, chunks,
                          chunk_tokens, slots);
     };
-    if (a.head_dim == 128)
+    if (a.head_dim == 256)
+      launch_split(std::integral_constant<int, 256>{});
+    else if (a.head_dim == 128)
       launch_split(std::integral_constant<int, 128>{});
     else
       launch_split(std::integral_constant<int, 64>{});

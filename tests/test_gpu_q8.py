@@ -281,7 +281,8 @@ def test_decode_attention_per_sequence_lengths(runtime):
     assert np.all(np.isfinite(out[3]))
 
 
-@pytest.mark.parametrize("b,kvh,group,dim,seed", [(70, 2, 2, 64, 5), (130, 1, 4, 128, 6), (3, 8, 4, 128, 7)])
+@pytest.mark.parametrize("b,kvh,group,dim,seed", [(70, 2, 2, 64, 5), (130, 1, 4, 128, 6), (3, 8, 4, 128, 7),
+                                                   (5, 4, 4, 256, 8), (70, 1, 2, 256, 9), (2, 6, 1, 256, 10)])
 def test_decode_attention_balanced_split_over_many_sequences(runtime, b, kvh, group, dim, seed):
     """Ragged batches, also wider than the 64 sequences one planning pass of a wave covers: every
     sequence gets its own chunk size from the device-side lengths; empty, one-token and
@@ -309,7 +310,8 @@ def test_decode_attention_balanced_split_over_many_sequences(runtime, b, kvh, gr
 
 
 @pytest.mark.parametrize("b,kvh,group,dim,window,seed", [(9, 3, 3, 64, 200, 1), (70, 2, 4, 128, 65, 2),
-                                                         (4, 8, 4, 128, 1024, 3), (3, 1, 1, 64, 4000, 4)])
+                                                         (4, 8, 4, 128, 1024, 3), (3, 1, 1, 64, 4000, 4),
+                                                         (8, 2, 8, 256, 333, 5)])
 def test_decode_attention_sliding_window_over_ragged_batch(runtime, b, kvh, group, dim, window, seed):
     """A sliding window on the split-over-context kernels: every sequence reads its last window - 1
     cached tokens (the window counts the current token) through a slot table entered `first` entries
@@ -345,7 +347,9 @@ def test_decode_attention_sliding_window_over_ragged_batch(runtime, b, kvh, grou
     ("llmopt_attention_q8_paged_simd_h64_gqa3", 9, 3, 64, 2048, 512),
     ("llmopt_attention_q8_paged_simd_generic", 32, 8, 128, 700, 300),
     ("llmopt_attention_q8_paged_simd_h64", 4, 4, 64, 100, 100),
-    ("llmopt_attention_q8_paged_simd_generic", 8, 2, 128, 99, 100)])
+    ("llmopt_attention_q8_paged_simd_generic", 8, 2, 128, 99, 100),
+    ("llmopt_attention_q8_paged_simd_h256", 16, 4, 256, 1024, 0),
+    ("llmopt_attention_q8_paged_simd_h256", 8, 1, 256, 777, 512)])
 def test_reference_entries_with_sliding_window(runtime, name, h, kvh, dim, past, window):
     """The reference's own entries (one context length for the whole batch) with a window: the
     split-over-context kernels when the windowed context has 64 tokens or more."""
