@@ -94,7 +94,10 @@ __global__ __launch_bounds__(WAVES * 64) void dense_attention_tile32_kernel(Dens
   constexpr int KEYS_PER_COPY = 64 / PIECES;
   constexpr int COPIES = STAGE_KEYS / KEYS_PER_COPY / WAVES;
   constexpr int STAGE_BYTES = STAGE_KEYS * ROW_BYTES;
-  static_assert(JJ == 2 || JJ == 4, "head_dim 64 or 128");
+  static_assert(JJ == 2 || JJ == 4 || JJ == 8, "head_dim 64, 128 or 256");
+  // V rows are swizzled by twice the key within the row's first sixteen pieces at most: reads 8 and 16 keys
+  // further down must find the same swizzle
+  constexpr int VMASK = (PIECES < 16 ? PIECES : 16) - 1;
   static_assert((STAGE_KEYS == 128 || STAGE_KEYS == 64 || STAGE_KEYS == 32) && COPIES >= 1 &&
                     COPIES * KEYS_PER_COPY * WAVES == STAGE_KEYS,
                 "stage");
@@ -178,7 +181,7 @@ __global__ __launch_bounds__(WAVES * 64) void dense_attention_tile32_kernel(Dens
       const uint32_t local = copy * KEYS_PER_COPY + row_in_copy;    // row within the stage
       const uint32_t key = min(stage * STAGE_KEYS + local, L - 1);  // rows past the end repeat the last one
       const uint16_t *k_src = key_base + (size_t)key * D + ((piece ^ (local & (PIECES - 1))) * 8);
-      const uint16_t *v_src = value_base + (size_t)key * value_row_stride + ((piece ^ ((2 * local) & (PIECES - 1))) * 8);
+      const uint16_t *v_src = value_base + (size_t)key * value_row_stride + ((piece ^ ((2 * local) & VMASK)) * 8);
       const uint32_t k_dst = (uint32_t)__builtin_amdgcn_readfirstlane((int)(buffer_base + copy * 1024));
       const uint32_t v_dst = k_dst + STAGE_BYTES;
       asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" : : "v"(k_src), "s"(k_dst) : "memory");
@@ -201,7 +204,7 @@ __global__ __launch_bounds__(WAVES * 64) void dense_attention_tile32_kernel(Dens
 #pragma unroll
     for (int jj = 0; jj < JJ; ++jj)
       v_lane_offset[jj] = key_in_read * ROW_BYTES +
-                          (((jj * 4 + (chunk >> 1)) ^ ((2 * key_in_read) & (PIECES - 1))) * 16) + (chunk & 1) * 8;
+                          (((jj * 4 + (chunk >> 1)) ^ ((2 * key_in_read) & VMASK)) * 16) + (chunk & 1) * 8;
   }
   if (stages > 0) {
     copy_stage(0);
@@ -470,7 +473,7 @@ hipError_t launch_dense_attention(const DenseAttentionArgs &a, hipStream_t strea
   if (a.key_length == 0 || a.head_dim == 0 || a.head_dim > 64 * kMaxFragments) return hipErrorInvalidValue;
   const bool aligned = reinterpret_cast<uintptr_t>(a.query) % 16 == 0 && reinterpret_cast<uintptr_t>(a.key) % 16 == 0 &&
                        reinterpret_cast<uintptr_t>(a.value) % 8 == 0 && reinterpret_cast<uintptr_t>(a.output) % 8 == 0;
-  if ((a.head_dim == 64 || a.head_dim == 128) && aligned && a.query_length >= 16) {
+  if ((a.head_dim == 64 || a.head_dim == 128 || a.head_dim == 256) && aligned && a.query_length >= 16) {
     // K and V stages are copied as 16-byte pieces of whole rows (16-byte aligned K and V rows), and the
     // maxima are taken before scaling (a positive, finite scale); anything else takes the row kernel
     const size_t value_row_halfs = a.token_first_value ? (size_t)(a.kv_heads > 0 ? a.kv_heads : a.heads) * a.head_dim
@@ -488,7 +491,9 @@ hipError_t launch_dense_attention(const DenseAttentionArgs &a, hipStream_t strea
                                reinterpret_cast<const void *>(&dense_attention_tile32_kernel<128, 4, 128, false, true>),
                                reinterpret_cast<const void *>(&dense_attention_tile32_kernel<128, 4, 128, true, true>),
                                reinterpret_cast<const void *>(&dense_attention_tile32_kernel<64, 4, 128, false, true>),
-                               reinterpret_cast<const void *>(&dense_attention_tile32_kernel<64, 4, 128, true, true>)};
+                               reinterpret_cast<const void *>(&dense_attention_tile32_kernel<64, 4, 128, true, true>),
+                               reinterpret_cast<const void *>(&dense_attention_tile32_kernel<256, 4, 64, false>),
+                               reinterpret_cast<const void *>(&dense_attention_tile32_kernel<256, 4, 64, true>)};
         for (const void *kernel : large) {
           const hipError_t status = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
           if (status != hipSuccess) return status;
@@ -502,7 +507,7 @@ hipError_t launch_dense_attention(const DenseAttentionArgs &a, hipStream_t strea
       // (four times the workgroups, a quarter of the walk): 9 heads x 2048 tokens of 64, causal,
       // 45.0 -> 22.9 us.  Larger launches keep 128 rows a workgroup: a stage of K and V then serves
       // four times as many rows.
-      if (workgroups < (uint64_t)device_compute_units() && a.key_length >= 256) {
+      if (workgroups < (uint64_t)device_compute_units() && a.key_length >= 256 && a.head_dim <= 128) {
         const size_t bytes = 2 * 2 * (size_t)128 * a.head_dim * 2;
         const dim3 grid((uint32_t)((a.query_length + 31) / 32) * a.heads * a.batches), block(256);
         if (a.head_dim == 64 && masked)
@@ -521,7 +526,12 @@ hipError_t launch_dense_attention(const DenseAttentionArgs &a, hipStream_t strea
       // tokens - one tile per barrier, half the sharing.)
       const size_t bytes = 2 * 2 * (size_t)64 * a.head_dim * 2;
       const dim3 grid((uint32_t)workgroups), block(256);
-      if (a.head_dim == 64 && masked)
+      // (heads of 256: 128 KB of stages, one workgroup per CU with all of its registers)
+      if (a.head_dim == 256 && masked)
+        hipLaunchKernelGGL((dense_attention_tile32_kernel<256, 4, 64, true>), grid, block, bytes, stream, scheduled);
+      else if (a.head_dim == 256)
+        hipLaunchKernelGGL((dense_attention_tile32_kernel<256, 4, 64, false>), grid, block, bytes, stream, scheduled);
+      else if (a.head_dim == 64 && masked)
         hipLaunchKernelGGL((dense_attention_tile32_kernel<64, 4, 64, true>), grid, block, bytes, stream, scheduled);
       else if (a.head_dim == 64)
         hipLaunchKernelGGL((dense_attention_tile32_kernel<64, 4, 64, false>), grid, block, bytes, stream, scheduled);

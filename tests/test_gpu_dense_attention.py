@@ -281,15 +281,10 @@ def test_rejects_bad_arguments(runtime):
         run(runtime, "llmopt_attention_f16", query, key, key, None, bad_heads, (1, 2, 4, 64))
 
 
-@pytest.mark.parametrize("dim,heads,kv_heads,new,past,mode", [
-    (64, 9, 3, 700, 0, "causal"), (128, 4, 2, 45, 900, "causal"), (64, 2, 1, 33, 257, "none"),
-    (128, 2, 2, 130, 300, "bool"), (64, 3, 3, 64, 1000, "f16"), (128, 1, 1, 1000, 0, "causal"),
-])
-def test_small_launches_split_the_keys_of_a_slab_over_the_waves(runtime, dim, heads, kv_heads, new, past, mode):
-    """Launches with fewer 128-row workgroups than the device has CUs and at least 256 keys: the four
-    waves of a workgroup share 32 query rows and take a quarter of every 128-key stage each, and
-    their shares (maxima, denominators, weighted sums) are folded through LDS.  Causal limits with
-    cached tokens, partial last stages and tiles, rows past the end, both mask types, both layouts."""
+def check_attention_case(runtime, dim, heads, kv_heads, new, past, mode):
+    """Two sequences of `new` query tokens after `past` cached ones against the oracle: causal limits,
+    no limit, bool and f16 masks with a row without keys and a row whose first keys are all masked;
+    head-major or token-major V and output by the parity of the length."""
     rng = np.random.default_rng(dim + heads + new + past)
     batches, length = 2, past + new
     query = rng.standard_normal((batches, heads, new, dim)).astype(np.float16)
@@ -321,4 +316,26 @@ def test_small_launches_split_the_keys_of_a_slab_over_the_waves(runtime, dim, he
     want = expected(query, key, value, allowed, scale)
     if mode in ("bool", "f16"):
         assert np.all(got[:, :, 3, :].view(np.uint16) == 0)
-    assert_close_to_oracle(got, want, f"key-split D={dim} {heads}/{kv_heads} {new} new after {past}, {mode}")
+    assert_close_to_oracle(got, want, f"D={dim} {heads}/{kv_heads} {new} new after {past}, {mode}")
+
+
+@pytest.mark.parametrize("dim,heads,kv_heads,new,past,mode", [
+    (64, 9, 3, 700, 0, "causal"), (128, 4, 2, 45, 900, "causal"), (64, 2, 1, 33, 257, "none"),
+    (128, 2, 2, 130, 300, "bool"), (64, 3, 3, 64, 1000, "f16"), (128, 1, 1, 1000, 0, "causal"),
+])
+def test_small_launches_split_the_keys_of_a_slab_over_the_waves(runtime, dim, heads, kv_heads, new, past, mode):
+    """Launches with fewer 128-row workgroups than the device has CUs and at least 256 keys: the four
+    waves of a workgroup share 32 query rows and take a quarter of every 128-key stage each, and
+    their shares (maxima, denominators, weighted sums) are folded through LDS.  Causal limits with
+    cached tokens, partial last stages and tiles, rows past the end, both mask types, both layouts."""
+    check_attention_case(runtime, dim, heads, kv_heads, new, past, mode)
+
+
+@pytest.mark.parametrize("heads,kv_heads,new,past,mode", [
+    (4, 2, 300, 0, "causal"), (2, 1, 45, 211, "causal"), (2, 2, 33, 100, "none"), (3, 1, 130, 70, "bool"),
+    (2, 2, 64, 191, "f16"), (8, 4, 16, 0, "causal"),
+])
+def test_heads_of_256_on_the_tile_kernel(runtime, heads, kv_heads, new, past, mode):
+    """llmopt_attention_f16_simd_h256 with sixteen query rows or more: the 32 x 32 tile kernel with
+    eight output blocks per wave and 128 KB of K and V stages per workgroup."""
+    check_attention_case(runtime, 256, heads, kv_heads, new, past, mode)
