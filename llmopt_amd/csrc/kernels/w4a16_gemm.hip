@@ -70,9 +70,10 @@ __device__ __forceinline__ f16x_t zero_tile() {
 // (4 * WM * 32) x (2 * WN * 32).  DUAL computes gate and up tiles of the same
 // outputs and stores silu(gate) * up.
 // XS: LDS stages of the activation tile = steps a K loop iteration is unrolled by = weight
-// register sets.  2 for the large tiles, whose steps are long enough to cover a load; 4 (K a
-// multiple of 4 steps) for the small ones, whose steps are shorter than the trip to memory:
-// the activation copy then runs three steps ahead of its use and the weights four.
+// register sets.  2 for the large tiles, whose steps are long enough to cover a load; 4 for the
+// small ones, whose steps are shorter than the trip to memory: the activation copy then runs
+// three steps ahead of its use and the weights four (K is rounded up to whole passes of four
+// steps, the surplus steps run on zero weights).
 template <int WM, int WN, bool DUAL, int XS, bool SPLITK = false>
 __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
   static_assert(XS == 2 || XS == 4, "the weight stage alternates with the step: an even unroll");
@@ -225,12 +226,15 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
   // weight dword (8 nibbles): q * s as fp16 (one rounding, 2^-11 relative at
   // most), in natural K order.
   constexpr int ITEMS = NWF * DW;
-  auto store_item = [&](const Fetched &f, int stage, int item) __attribute__((always_inline)) {
+  // live = false: the set belongs to a step past the end of K (XS = 4 rounds the steps up to whole
+  // loop passes; the requests of such a step are clamped to the last K block): it is stored as
+  // zeros, so the step's MFMAs add nothing.
+  auto store_item = [&](const Fetched &f, int stage, int item, bool live) __attribute__((always_inline)) {
     _Float16 *w_lds = stage_lds + W_BASE_HALFS + stage * W_STAGE_HALFS;
     const int v = item / DW;
     const int j = item % DW;
     if (DUAL && !kThreadPerMatrix && w_row >= (uint32_t)BN) return;
-    const _Float16 scale = __builtin_bit_cast(_Float16, (uint16_t)f.s[v]);
+    const _Float16 scale = live ? __builtin_bit_cast(_Float16, (uint16_t)f.s[v]) : (_Float16)0.0f;
     const uint4 packed = w4_scaled_natural(f.w[v][j], scale);
     // (one matrix per thread: w_row runs over the rows of both matrices, as v * BN + row does)
     *reinterpret_cast<uint4 *>(&w_lds[(v * BN + w_row) * LDS_STRIDE + w_half * (DW * 8) + j * 8]) = packed;
@@ -310,7 +314,7 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
 #pragma unroll
         for (int n = 0; n < ITEMS_PER_GROUP; ++n)
           if (group * ITEMS_PER_GROUP + n < ITEMS)
-            store_item(fetched[next_set], stage ^ 1, group * ITEMS_PER_GROUP + n);
+            store_item(fetched[next_set], stage ^ 1, group * ITEMS_PER_GROUP + n, XS == 2 || k0 + BK < KS);
         if (group == 0) fetch_x(min(k0 + (XS - 1) * BK, KS - BK), (j + XS - 1) % XS);
         __builtin_amdgcn_sched_barrier(0);
       }
@@ -328,14 +332,14 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
   for (int s = 0; s < WS; ++s) fetch_w(fetched[s], min((uint32_t)s * BK, KS - BK));
   wait_w(fetched[0], std::integral_constant<int, (WS - 1) * W_LOADS>{});
 #pragma unroll
-  for (int item = 0; item < ITEMS; ++item) store_item(fetched[0], 0, item);
+  for (int item = 0; item < ITEMS; ++item) store_item(fetched[0], 0, item, true);
   fetch_w(fetched[0], min((uint32_t)WS * BK, KS - BK));
   if constexpr (XS == 2) {
     for (uint32_t k0 = 0; k0 < KS; k0 += 2 * BK) {
       step(k0, std::integral_constant<int, 0>{});
       if (k0 + BK < KS) step(k0 + BK, std::integral_constant<int, 1>{});
     }
-  } else {  // K is a multiple of XS steps: no branch between a request and its wait
+  } else {  // whole passes of XS steps (the surplus ones multiply by zeros): no branch between a request and its wait
     wait_all(std::integral_constant<int, W_LOADS>{});  // every activation copy and every other set has landed
     for (uint32_t k0 = 0; k0 < KS; k0 += XS * BK) {
       step(k0, std::integral_constant<int, 0>{});
@@ -417,6 +421,17 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
     if (col >= width) continue;
 #pragma unroll
     for (int a = 0; a < WM; ++a) {
+      // The sixteen addends of a 32 x 32 block are requested together, for rows past m at the last
+      // row's address: a load under a per-element test is waited for where it stands, and the
+      // epilogue of a tile with a residual was sixteen trips to memory per block, one after the other.
+      uint16_t addend_bits[16] = {};
+      if (!DUAL && p.has_addend) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+          const uint32_t row = m0 + row_base + a * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3);
+          addend_bits[i] = p.addend[(size_t)min(row, p.m - 1) * p.addend_stride + col];
+        }
+      }
 #pragma unroll
       for (int i = 0; i < 16; ++i) {
         const uint32_t row = m0 + row_base + a * 32 + (i >> 2) * 8 + (lane >> 5) * 4 + (i & 3);
@@ -428,8 +443,7 @@ __global__ __launch_bounds__(kThreads) void w4a16_gemm_kernel(GemmParams p) {
           value = gate / (1.0f + __expf(-gate)) * up;
         } else {
           value = acc[0][a][b][i];
-          if (p.has_addend)
-            value += half_bits_to_float(p.addend[(size_t)row * p.addend_stride + col]);
+          if (p.has_addend) value += half_bits_to_float(addend_bits[i]);
         }
         output0[(size_t)row * width + col] = float_to_half_bits(value);
       }
@@ -478,9 +492,16 @@ uint32_t gemm_k_splits(uint32_t m, uint32_t n, uint32_t k) {
 
 template <bool DUAL>
 hipError_t launch_gemm(GemmParams &p, hipStream_t stream) {
-  if (DUAL) return launch_tile<2, 2, true>(p, stream);  // 256 x 128, two accumulator sets
-  // 256 x 256 when that still gives every CU a tile, otherwise 256 x 128 / 128 x 256 / 128 x 128
   const int cus = device_compute_units();
+  if (DUAL) {
+    // 256 x 128, two accumulator sets; 128 x 128 with four activation stages when even those tiles
+    // leave CUs without one (the decode model's 576 -> 1536 pair at 2048 rows: 96 tiles of 256 x 128,
+    // whose nine two-stage steps each wait out a trip to memory)
+    const uint64_t small_pair = (uint64_t)((p.m + 127) / 128) * ((p.n + 127) / 128);
+    if (small_pair <= (uint64_t)cus) return launch_tile<1, 2, true, 4>(p, stream);
+    return launch_tile<2, 2, true>(p, stream);
+  }
+  // 256 x 256 when that still gives every CU a tile, otherwise 256 x 128 / 128 x 256 / 128 x 128
   const uint64_t big = (uint64_t)((p.m + 255) / 256) * ((p.n + 255) / 256);
   if (big >= (uint64_t)cus) return launch_tile<2, 4, false>(p, stream);
   // Half that size, tall (256 x 128) or wide (128 x 256), whichever pads less; the tall one when
@@ -493,15 +514,15 @@ hipError_t launch_gemm(GemmParams &p, hipStream_t stream) {
     return tall <= wide ? launch_tile<2, 2, false>(p, stream) : launch_tile<1, 4, false>(p, stream);
   // 128 x 128 tiles have steps shorter than a trip to memory.  With two stages they fit a CU
   // twice, which covers the loads; when there is at most one tile per CU anyway, four
-  // activation stages do (K a whole number of four steps; measured 58 -> 49 us at 512 x 4096 x 4096,
-  // and nothing for the 128 x 256 tiles, which stay with two).
+  // activation stages do (measured 58 -> 49 us at 512 x 4096 x 4096, and nothing for the 128 x 256
+  // tiles, which stay with two).
   const uint64_t small = (uint64_t)((p.m + 127) / 128) * ((p.n + 127) / 128);
   // Fewer tiles than half the CUs: K is split over workgroups as well, so that every CU holds a
   // tile (128 tiles at 512 x 4096 x 4096 left half the device idle).
   const uint32_t splits = gemm_k_splits(p.m, p.n, p.k);
   if (splits > 1 && p.partials != nullptr && p.counters != nullptr)
     return launch_tile<1, 2, false, 4, true>(p, stream, splits);
-  if (p.k % (4 * BK) == 0 && small <= (uint64_t)cus) return launch_tile<1, 2, false, 4>(p, stream);
+  if (small <= (uint64_t)cus) return launch_tile<1, 2, false, 4>(p, stream);
   return launch_tile<1, 2, false>(p, stream);
 }
 
@@ -610,7 +631,7 @@ hipError_t launch_w4a16_qkv(const W4QkvArgs &args, hipStream_t stream) {
     p.s[0] = p.s[1] = p.seg_s[0];
     p.y = p.seg_y[0];
     p.n = p.seg_n[0];
-    if (p.k % (4 * BK) == 0 && tiles <= (uint64_t)device_compute_units()) return launch_tile<1, 2, false, 4>(p, stream);
+    if (tiles <= (uint64_t)device_compute_units()) return launch_tile<1, 2, false, 4>(p, stream);
     return launch_tile<1, 2, false>(p, stream);
   }
   // large ones: three GEMMs sharing the activation through L2

@@ -320,6 +320,11 @@ __global__ __launch_bounds__(kMaxWaves * 64) void w4a16_gemv_mfma_kernel(MfmaGem
       const uint32_t tile = (blockIdx.x + (first_round + slot) * gridDim.x) * p.waves_t + lane_t;
       const uint32_t col = tile * TN + col_in_tile;
       const bool writer = in_range && tile < tiles && m < rows && col < mat.n;
+      // the addend is requested here, by every thread at a clamped address, and used at the store:
+      // under the writer's test it would be a trip to memory of its own after the sums are ready
+      uint16_t addend_bits = 0;
+      if (!DUAL && p.has_addend)
+        addend_bits = p.addend[(size_t)(row0 + min(m, rows - 1)) * p.addend_stride + min(col, mat.n - 1)];
       float total[NW];
 #pragma unroll
       for (int v = 0; v < NW; ++v) total[v] = 0.0f;
@@ -379,7 +384,7 @@ __global__ __launch_bounds__(kMaxWaves * 64) void w4a16_gemv_mfma_kernel(MfmaGem
           value = total[0] / (1.0f + __expf(-total[0])) * total[NW - 1];
         } else {
           value = total[0];
-          if (p.has_addend) value += half_bits_to_float(p.addend[(size_t)(row0 + m) * p.addend_stride + col]);
+          if (p.has_addend) value += half_bits_to_float(addend_bits);
         }
         if (mat.y != nullptr) mat.y[(size_t)(row0 + m) * mat.n + col] = float_to_half_bits(value);
         if (!DUAL && p.y_f32 != nullptr) p.y_f32[(size_t)(row0 + m) * mat.n + col] = value;

@@ -164,7 +164,9 @@ def test_gemv_residual_epilogue(runtime, m):
 # up to 128 rows with small weights run the matrix-core GEMV once per group of 8 rows
 GEMM_SHAPES = [(9, 64, 64), (16, 128, 128), (24, 576, 1536), (31, 100, 576), (32, 1536, 576),
                (32, 96, 14336), (33, 64, 576), (64, 576, 1536), (100, 29, 192), (128, 192, 576), (129, 64, 576), (128, 256, 512), (130, 300, 1024),
-               (512, 128, 4096), (200, 130, 256), (140, 260, 768), (512, 4096, 256)]
+               (512, 128, 4096), (200, 130, 256), (140, 260, 768), (512, 4096, 256),
+               # K that is not a whole number of four-step passes on the four-stage small tiles: 9, 1 and 5 steps
+               (300, 576, 576), (2048, 192, 64), (513, 200, 320)]
 
 
 @pytest.mark.parametrize("m,n,k", GEMM_SHAPES)
@@ -286,7 +288,7 @@ def test_normalising_qkv_and_swiglu_entries(runtime, m, k):
         np.testing.assert_array_equal(got.view(np.uint16), two_product.numpy(np.uint16, (m, n)))
 
 
-@pytest.mark.parametrize("m", [1, 2, 4, 8, 9, 32, 48, 136])
+@pytest.mark.parametrize("m", [1, 2, 4, 8, 9, 32, 48, 136, 600])
 def test_swiglu_ffn_chain(runtime, m):
     """dual-SwiGLU then down+residual, the two W4A16 stages of the reference's
     FFN macro-op; the intermediate product is rounded to f16 between stages
