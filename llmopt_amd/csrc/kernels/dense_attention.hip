@@ -79,14 +79,22 @@ constexpr int kWavesPerBlock = 4;  // consecutive 32-row slabs of one head
 // instead of four times.
 // WAVES x 32 query rows per workgroup, STAGE_KEYS keys per LDS stage (launched as 4 x 64: 64 KB at
 // D = 128, two workgroups per CU).
-// MASKED: the launch has a mask (every score is then tested; without one the instantiation carries
+// MASK: 0 no mask, 1 a mask of bytes, 2 of halves (every score is then tested; without one the instantiation carries
 // nothing of it).
 // KEYSPLIT: the four waves of a workgroup share ONE slab of 32 query rows and take a quarter of every
 // 128-key stage each; their partial results meet in LDS at the end.  For launches with fewer
 // workgroups than CUs, which last as long as one wave's walk over all the keys of the last slab: the
 // walk is a quarter as long and there are four times as many workgroups.
-template <int D, int WAVES, int STAGE_KEYS, bool MASKED, bool KEYSPLIT = false>
-__global__ __launch_bounds__(WAVES * 64) void dense_attention_tile32_kernel(DenseAttentionArgs a) {
+template <int D>
+constexpr int tile32_waves_per_simd() {
+  return D <= 128 ? 2 : 1;
+}
+
+template <int D, int WAVES, int STAGE_KEYS, int MASK, bool KEYSPLIT = false>
+__global__ __launch_bounds__(WAVES * 64)
+    __attribute__((amdgpu_waves_per_eu(tile32_waves_per_simd<D>(), tile32_waves_per_simd<D>()))) void
+    dense_attention_tile32_kernel(DenseAttentionArgs a) {
+  constexpr bool MASKED = MASK != 0;
   constexpr int KSTEPS = D / 16;  // score MFMAs per key tile
   constexpr int JJ = D / 32;      // adjacent head_dim values per lane and key = output blocks
   constexpr int ROW_BYTES = D * 2;
@@ -150,6 +158,72 @@ __global__ __launch_bounds__(WAVES * 64) void dense_attention_tile32_kernel(Dens
                                    ? a.value + ((size_t)batch * L * kv_heads + kv_head) * D
                                    : a.value + ((size_t)batch * kv_heads + kv_head) * L * D;
 
+  // ---- mask ----
+  // A lane's sixteen scores of a tile are four runs of four consecutive keys of one query row.  Their
+  // mask values are requested a stage ahead, for every lane at clamped addresses (a load under a
+  // per-score test is waited for where it stands: sixteen trips to memory per tile), as one dword
+  // (bool) or two (f16) per run when rows of the mask are a multiple of four keys, else element by
+  // element; a tile whose 32 x 32 mask values allow nothing is skipped whole.
+  constexpr int TILES = KEYSPLIT ? 1 : STAGE_KEYS / 32;  // tiles of a stage this wave works on
+  struct MaskRaw {
+    uint32_t w[MASK == 2 ? 8 : MASK == 1 ? 4 : 1];
+  };
+  [[maybe_unused]] const size_t mask_row =
+      masked ? (((size_t)(a.mask_batches == 1 ? 0 : batch) * a.mask_heads + (a.mask_heads == 1 ? 0 : head)) *
+                    a.query_length + min(q0 + row_lane, a.query_length - 1)) * L
+             : 0;
+  [[maybe_unused]] const bool mask_runs =
+      masked && L % 4 == 0 && L >= 4 && reinterpret_cast<uintptr_t>(a.mask) % 8 == 0;  // the same for every lane
+  [[maybe_unused]] auto mask_request = [&](uint32_t key0, MaskRaw &raw) __attribute__((always_inline)) {
+    if constexpr (MASK == 2) {
+      {
+        const uint16_t *row = reinterpret_cast<const uint16_t *>(a.mask) + mask_row;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const uint32_t key = key0 + g * 8 + half * 4;
+          if (mask_runs) {
+            const uint2 run = *reinterpret_cast<const uint2 *>(row + min(key, L - 4));
+            raw.w[2 * g] = run.x;
+            raw.w[2 * g + 1] = run.y;
+          } else {
+            raw.w[2 * g] = (uint32_t)row[min(key, L - 1)] | ((uint32_t)row[min(key + 1, L - 1)] << 16);
+            raw.w[2 * g + 1] = (uint32_t)row[min(key + 2, L - 1)] | ((uint32_t)row[min(key + 3, L - 1)] << 16);
+          }
+        }
+      }
+    } else if constexpr (MASK == 1) {
+      {
+        const uint8_t *row = a.mask + mask_row;
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+          const uint32_t key = key0 + g * 8 + half * 4;
+          if (mask_runs)
+            raw.w[g] = *reinterpret_cast<const uint32_t *>(row + min(key, L - 4));
+          else
+            raw.w[g] = (uint32_t)row[min(key, L - 1)] | ((uint32_t)row[min(key + 1, L - 1)] << 8) |
+                       ((uint32_t)row[min(key + 2, L - 1)] << 16) | ((uint32_t)row[min(key + 3, L - 1)] << 24);
+        }
+      }
+    }
+  };
+  // bit r: the mask allows score r (keys past the end read a clamped element; they fail the range test anyway).
+  // With whole runs a run that starts past L - 4 was read from L - 4: its keys are all past the end.
+  [[maybe_unused]] auto mask_bits = [&](const MaskRaw &raw) __attribute__((always_inline)) {
+    uint32_t bits = 0;
+    if constexpr (MASKED) {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        bool allowed;
+        if constexpr (MASK == 2)
+          allowed = half_bits_to_float((uint16_t)(raw.w[2 * (r >> 2) + ((r & 3) >> 1)] >> (16 * (r & 1)))) >= 0.0f;
+        else
+          allowed = ((raw.w[r >> 2] >> (8 * (r & 3))) & 0xffu) != 0;
+        bits |= allowed ? (1u << r) : 0u;
+      }
+    }
+    return bits;
+  };
+
   const float score_scale = a.scale * 1.4426950408889634f;  // softmax in base 2
   float running_max = -INFINITY, running_sum = 0.0f;        // of this lane's row; the sum over this lane's keys
   f16x_t out_acc[JJ];  // O^T[d = 32 jj + (r / 4) * 8 + half * 4 + r % 4][row = row_lane]
@@ -206,7 +280,16 @@ __global__ __launch_bounds__(WAVES * 64) void dense_attention_tile32_kernel(Dens
       v_lane_offset[jj] = key_in_read * ROW_BYTES +
                           (((jj * 4 + (chunk >> 1)) ^ ((2 * key_in_read) & VMASK)) * 16) + (chunk & 1) * 8;
   }
+  // first key of this wave's tile t of a stage
+  auto tile_key0 = [&](uint32_t stage, int t) __attribute__((always_inline)) {
+    return stage * STAGE_KEYS + (KEYSPLIT ? wave * 32 : (uint32_t)t * 32);
+  };
+  MaskRaw mask_raw[TILES];
   if (stages > 0) {
+    if constexpr (MASKED) {
+#pragma unroll
+      for (int t = 0; t < TILES; ++t) mask_request(tile_key0(0, t), mask_raw[t]);
+    }
     copy_stage(0);
     stage_landed();
   }
@@ -227,7 +310,8 @@ __global__ __launch_bounds__(WAVES * 64) void dense_attention_tile32_kernel(Dens
     return score;
   };
   // softmax update and P V product of one tile from its scores; v_tile = its first V row in the stage
-  auto tile_update = [&](uint32_t key0, f16x_t score, const unsigned char *v_tile) __attribute__((always_inline)) {
+  auto tile_update = [&](uint32_t key0, f16x_t score, const unsigned char *v_tile, uint32_t allowed_bits)
+                         __attribute__((always_inline)) {
     // a tile of existing keys, all below the causal limit of the wave's first row, of existing
     // rows and without a mask needs no per-score test.  Maxima are taken over the scores as the MFMAs left them; the
     // scale (positive) goes into the exponent's multiply-add.
@@ -244,9 +328,7 @@ __global__ __launch_bounds__(WAVES * 64) void dense_attention_tile32_kernel(Dens
         const uint32_t key = key0 + (r >> 2) * 8 + half * 4 + (r & 3);
         bool allowed = key < L && row < a.query_length;
         if (a.causal) allowed = allowed && key <= a.past_length + row;
-        if constexpr (masked) {
-          if (allowed) allowed = mask_allows(a, batch, head, row, key);
-        }
+        if constexpr (masked) allowed = allowed && ((allowed_bits >> r) & 1u) != 0;
         score[r] = allowed ? score[r] : -INFINITY;
         tile_max = fmaxf(tile_max, score[r]);
       }
@@ -292,28 +374,55 @@ __global__ __launch_bounds__(WAVES * 64) void dense_attention_tile32_kernel(Dens
   // The tiles of a stage.  Two: both score chains go to the matrix pipe first, so the second runs
   // while the vector unit works on the first tile's softmax.
   for (uint32_t stage = 0; stage < stages; ++stage) {
-    if (stage + 1 < stages) copy_stage(stage + 1);  // into the buffer every wave left at the last barrier
+    // The mask values of this stage were requested a stage ago and landed with that stage's copies
+    // (stage_landed waits for everything): they are turned into bits before anything new is
+    // requested, so that no wait for them stands behind the next stage's copies.
+    uint32_t allowed_bits[TILES];
+    bool live[TILES];
+#pragma unroll
+    for (int t = 0; t < TILES; ++t) {
+      allowed_bits[t] = MASKED ? mask_bits(mask_raw[t]) : 0xffffu;
+      live[t] = tile_key0(stage, t) < key_end && (!MASKED || __builtin_amdgcn_ballot_w64(allowed_bits[t] != 0) != 0);
+    }
+    if (stage + 1 < stages) {
+      copy_stage(stage + 1);  // into the buffer every wave left at the last barrier
+      if constexpr (MASKED) {
+#pragma unroll
+        for (int t = 0; t < TILES; ++t) mask_request(tile_key0(stage + 1, t), mask_raw[t]);
+      }
+    }
     const unsigned char *k_stage = stage_lds + (stage & 1) * 2 * STAGE_BYTES;
     const unsigned char *v_stage = k_stage + STAGE_BYTES;
     if constexpr (KEYSPLIT) {
-      const uint32_t key0 = stage * STAGE_KEYS + wave * 32;
-      if (key0 < key_end)
-        tile_update(key0, tile_scores(k_stage + wave * 32 * ROW_BYTES, wave * 32), v_stage + wave * 32 * ROW_BYTES);
+      if (live[0])
+        tile_update(tile_key0(stage, 0), tile_scores(k_stage + wave * 32 * ROW_BYTES, wave * 32),
+                    v_stage + wave * 32 * ROW_BYTES, allowed_bits[0]);
       stage_landed();
       continue;
     }
     const uint32_t key0 = stage * STAGE_KEYS;
-    if (key0 < key_end) {
-      const f16x_t first_scores = tile_scores(k_stage, 0);
-      if constexpr (STAGE_KEYS == 64) {
+    if constexpr (!MASKED && STAGE_KEYS == 64) {
+      // (without a mask the second tile exists whenever the first does, except at the very end)
+      if (key0 < key_end) {
+        const f16x_t first_scores = tile_scores(k_stage, 0);
         const bool second = key0 + 32 < key_end;
         f16x_t second_scores = first_scores;
         if (second) second_scores = tile_scores(k_stage + 32 * ROW_BYTES, 32);
-        tile_update(key0, first_scores, v_stage);
-        if (second) tile_update(key0 + 32, second_scores, v_stage + 32 * ROW_BYTES);
-      } else {
-        tile_update(key0, first_scores, v_stage);
+        tile_update(key0, first_scores, v_stage, 0xffffu);
+        if (second) tile_update(key0 + 32, second_scores, v_stage + 32 * ROW_BYTES, 0xffffu);
       }
+    } else if constexpr (STAGE_KEYS == 64) {
+      f16x_t first_scores, second_scores;
+      if (live[0]) first_scores = tile_scores(k_stage, 0);
+      if (live[1]) second_scores = tile_scores(k_stage + 32 * ROW_BYTES, 32);
+      if (live[0]) tile_update(key0, first_scores, v_stage, allowed_bits[0]);
+      if (live[1]) tile_update(key0 + 32, second_scores, v_stage + 32 * ROW_BYTES, allowed_bits[1]);
+    } else {
+#pragma unroll
+      for (int t = 0; t < TILES; ++t)
+        if (live[t])
+          tile_update(key0 + t * 32, tile_scores(k_stage + t * 32 * ROW_BYTES, t * 32), v_stage + t * 32 * ROW_BYTES,
+                      allowed_bits[t]);
     }
     stage_landed();
   }
@@ -465,6 +574,31 @@ __global__ __launch_bounds__(256) void dense_attention_rows_kernel(DenseAttentio
   }
 }
 
+template <int D, int WAVES, int STAGE_KEYS, int MASK, bool KEYSPLIT>
+hipError_t launch_tile32_instance(uint32_t grid, const DenseAttentionArgs &a, hipStream_t stream) {
+  constexpr size_t bytes = 2 * 2 * (size_t)STAGE_KEYS * D * 2;  // two stages of K and V
+  auto kernel = &dense_attention_tile32_kernel<D, WAVES, STAGE_KEYS, MASK, KEYSPLIT>;
+  if constexpr (bytes >= 64 * 1024) {
+    static bool configured = false;  // the attribute is per device function
+    if (!configured) {
+      const hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
+                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
+      if (status != hipSuccess) return status;
+      configured = true;
+    }
+  }
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(WAVES * 64), bytes, stream, a);
+  return hipGetLastError();
+}
+
+// mask: 0 none, 1 bytes, 2 halves
+template <int D, int WAVES, int STAGE_KEYS, bool KEYSPLIT>
+hipError_t launch_tile32(int mask, uint32_t grid, const DenseAttentionArgs &a, hipStream_t stream) {
+  if (mask == 2) return launch_tile32_instance<D, WAVES, STAGE_KEYS, 2, KEYSPLIT>(grid, a, stream);
+  if (mask == 1) return launch_tile32_instance<D, WAVES, STAGE_KEYS, 1, KEYSPLIT>(grid, a, stream);
+  return launch_tile32_instance<D, WAVES, STAGE_KEYS, 0, KEYSPLIT>(grid, a, stream);
+}
+
 }  // namespace
 
 hipError_t launch_dense_attention(const DenseAttentionArgs &a, hipStream_t stream) {
@@ -483,23 +617,7 @@ hipError_t launch_dense_attention(const DenseAttentionArgs &a, hipStream_t strea
     const uint64_t workgroups = (uint64_t)((a.query_length + kWavesPerBlock * 32 - 1) / (kWavesPerBlock * 32)) *
                                 a.heads * a.batches;
     if (staged && workgroups <= 0x7fffffffull) {
-      const bool masked = a.mask != nullptr && a.mask_batches > 0;
-      static bool configured = false;  // the attribute is per device function
-      if (!configured) {
-        const void *large[] = {reinterpret_cast<const void *>(&dense_attention_tile32_kernel<128, 4, 64, false>),
-                               reinterpret_cast<const void *>(&dense_attention_tile32_kernel<128, 4, 64, true>),
-                               reinterpret_cast<const void *>(&dense_attention_tile32_kernel<128, 4, 128, false, true>),
-                               reinterpret_cast<const void *>(&dense_attention_tile32_kernel<128, 4, 128, true, true>),
-                               reinterpret_cast<const void *>(&dense_attention_tile32_kernel<64, 4, 128, false, true>),
-                               reinterpret_cast<const void *>(&dense_attention_tile32_kernel<64, 4, 128, true, true>),
-                               reinterpret_cast<const void *>(&dense_attention_tile32_kernel<256, 4, 64, false>),
-                               reinterpret_cast<const void *>(&dense_attention_tile32_kernel<256, 4, 64, true>)};
-        for (const void *kernel : large) {
-          const hipError_t status = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024);
-          if (status != hipSuccess) return status;
-        }
-        configured = true;
-      }
+      const int mask = (a.mask != nullptr && a.mask_batches > 0) ? (a.mask_dtype == 2 ? 2 : 1) : 0;
       DenseAttentionArgs scheduled = a;
       scheduled.cus_per_xcd = (uint32_t)device_compute_units() / 8;
       // Fewer workgroups of 128 rows than CUs: the launch lasts as long as one wave's walk over the
@@ -508,38 +626,18 @@ hipError_t launch_dense_attention(const DenseAttentionArgs &a, hipStream_t strea
       // 45.0 -> 22.9 us.  Larger launches keep 128 rows a workgroup: a stage of K and V then serves
       // four times as many rows.
       if (workgroups < (uint64_t)device_compute_units() && a.key_length >= 256 && a.head_dim <= 128) {
-        const size_t bytes = 2 * 2 * (size_t)128 * a.head_dim * 2;
-        const dim3 grid((uint32_t)((a.query_length + 31) / 32) * a.heads * a.batches), block(256);
-        if (a.head_dim == 64 && masked)
-          hipLaunchKernelGGL((dense_attention_tile32_kernel<64, 4, 128, true, true>), grid, block, bytes, stream, scheduled);
-        else if (a.head_dim == 64)
-          hipLaunchKernelGGL((dense_attention_tile32_kernel<64, 4, 128, false, true>), grid, block, bytes, stream, scheduled);
-        else if (masked)
-          hipLaunchKernelGGL((dense_attention_tile32_kernel<128, 4, 128, true, true>), grid, block, bytes, stream, scheduled);
-        else
-          hipLaunchKernelGGL((dense_attention_tile32_kernel<128, 4, 128, false, true>), grid, block, bytes, stream, scheduled);
-        return hipGetLastError();
+        const uint32_t grid = (uint32_t)((a.query_length + 31) / 32) * a.heads * a.batches;
+        if (a.head_dim == 64) return launch_tile32<64, 4, 128, true>(mask, grid, scheduled, stream);
+        return launch_tile32<128, 4, 128, true>(mask, grid, scheduled, stream);
       }
       // 32 x 32 wave tiles over shared LDS stages, four waves and 64 keys a stage.  (Workgroups of two
       // waves with 32-key stages, twice as many and four per CU, so that short causal launches are not
       // as long as their longest workgroup, measured slower: 105.6 against 91.2 us at 32 heads x 2048
-      // tokens - one tile per barrier, half the sharing.)
-      const size_t bytes = 2 * 2 * (size_t)64 * a.head_dim * 2;
-      const dim3 grid((uint32_t)workgroups), block(256);
-      // (heads of 256: 128 KB of stages, one workgroup per CU with all of its registers)
-      if (a.head_dim == 256 && masked)
-        hipLaunchKernelGGL((dense_attention_tile32_kernel<256, 4, 64, true>), grid, block, bytes, stream, scheduled);
-      else if (a.head_dim == 256)
-        hipLaunchKernelGGL((dense_attention_tile32_kernel<256, 4, 64, false>), grid, block, bytes, stream, scheduled);
-      else if (a.head_dim == 64 && masked)
-        hipLaunchKernelGGL((dense_attention_tile32_kernel<64, 4, 64, true>), grid, block, bytes, stream, scheduled);
-      else if (a.head_dim == 64)
-        hipLaunchKernelGGL((dense_attention_tile32_kernel<64, 4, 64, false>), grid, block, bytes, stream, scheduled);
-      else if (masked)
-        hipLaunchKernelGGL((dense_attention_tile32_kernel<128, 4, 64, true>), grid, block, bytes, stream, scheduled);
-      else
-        hipLaunchKernelGGL((dense_attention_tile32_kernel<128, 4, 64, false>), grid, block, bytes, stream, scheduled);
-      return hipGetLastError();
+      // tokens - one tile per barrier, half the sharing.)  Heads of 256: 128 KB of stages, one
+      // workgroup per CU with all of its registers.
+      if (a.head_dim == 256) return launch_tile32<256, 4, 64, false>(mask, (uint32_t)workgroups, scheduled, stream);
+      if (a.head_dim == 64) return launch_tile32<64, 4, 64, false>(mask, (uint32_t)workgroups, scheduled, stream);
+      return launch_tile32<128, 4, 64, false>(mask, (uint32_t)workgroups, scheduled, stream);
     }
   }
   const uint64_t blocks = (rows + 3) / 4;
