@@ -126,14 +126,16 @@ __global__ __launch_bounds__(WAVES * 64)
   const uint32_t slabs = (a.query_length + ROWS - 1) / ROWS;
   const uint32_t per_slab = a.heads * a.batches;
   uint32_t rank = blockIdx.x;
-  if (a.causal && gridDim.x % 8 == 0 && a.cus_per_xcd > 0) {
+  // (a mask is taken for a causal one as far as the order goes: later rows see more keys)
+  const bool longest_first = a.causal || MASKED;
+  if (longest_first && gridDim.x % 8 == 0 && a.cus_per_xcd > 0) {
     const uint32_t xcd = blockIdx.x % 8, position = blockIdx.x / 8, run = 2 * a.cus_per_xcd;
     const uint32_t start = position / run * run, within = position % run;
     uint32_t taken = position;
     if (within >= a.cus_per_xcd && start + run <= gridDim.x / 8) taken = start + a.cus_per_xcd + (run - 1 - within);
     rank = taken * 8 + xcd;
   }
-  const uint32_t slab = a.causal ? slabs - 1 - rank / per_slab : rank / per_slab;
+  const uint32_t slab = longest_first ? slabs - 1 - rank / per_slab : rank / per_slab;
   const uint32_t head = rank % per_slab % a.heads;
   const uint32_t batch = rank % per_slab / a.heads;
   const uint32_t q0 = KEYSPLIT ? slab * 32 : (slab * WAVES + wave) * 32;
@@ -244,10 +246,10 @@ __global__ __launch_bounds__(WAVES * 64)
     group_key_end = min((uint64_t)L, (uint64_t)a.past_length + last_row + 1);
   }
   const uint32_t stages = (group_key_end + STAGE_KEYS - 1) / STAGE_KEYS;
-  auto copy_stage = [&](uint32_t stage) __attribute__((always_inline)) {
+  auto copy_stage = [&](uint32_t stage, uint32_t buffer) __attribute__((always_inline)) {
 #if defined(__HIP_DEVICE_COMPILE__)
     const uint32_t buffer_base =
-        (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char *)stage_lds + (stage & 1) * 2 * STAGE_BYTES;
+        (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char *)stage_lds + buffer * 2 * STAGE_BYTES;
     const uint32_t row_in_copy = lane / PIECES, piece = lane % PIECES;
 #pragma unroll
     for (int c = 0; c < COPIES; ++c) {
@@ -284,13 +286,49 @@ __global__ __launch_bounds__(WAVES * 64)
   auto tile_key0 = [&](uint32_t stage, int t) __attribute__((always_inline)) {
     return stage * STAGE_KEYS + (KEYSPLIT ? wave * 32 : (uint32_t)t * 32);
   };
+  // With a mask, the stages of keys that have anything for this slab of rows come from a map a pass
+  // over the mask left (one bit per mask row group, slab and stage): wave 0 turns the slab's bits
+  // into the list of its live stages, and the loop below walks that list - a stage the mask forbids
+  // costs nothing.  Without a map (no scratch given, or more stages than the list holds) every stage
+  // is walked and only its arithmetic is skipped.
+  constexpr uint32_t kMaxLive = 2048;
+  [[maybe_unused]] __shared__ uint16_t live_list[MASKED ? kMaxLive : 1];
+  [[maybe_unused]] __shared__ uint32_t live_count_lds;
+  bool listed = false;
+  uint32_t walk = stages;  // stages to walk
+  if constexpr (MASKED) {
+    listed = a.stage_map != nullptr && stages <= kMaxLive;
+    if (listed) {
+      const uint32_t total_stages = (L + STAGE_KEYS - 1) / STAGE_KEYS, map_stride = (total_stages + 7) / 8;
+      const uint32_t group = (a.mask_batches == 1 ? 0 : batch) * a.mask_heads + (a.mask_heads == 1 ? 0 : head);
+      const uint8_t *map = a.stage_map + ((size_t)group * slabs + slab) * map_stride;
+      if (wave == 0) {
+        uint32_t count = 0;
+        for (uint32_t base = 0; base < stages; base += 64) {
+          const uint32_t stage = base + lane;
+          const bool live = stage < stages && ((map[min(stage, stages - 1) >> 3] >> (stage & 7)) & 1u) != 0;
+          const uint64_t votes = __builtin_amdgcn_ballot_w64(live);
+          if (live) live_list[count + __builtin_popcountll(votes & ((1ull << lane) - 1))] = (uint16_t)stage;
+          count += (uint32_t)__builtin_popcountll(votes);
+        }
+        if (lane == 0) live_count_lds = count;
+      }
+      __syncthreads();
+      walk = live_count_lds;
+    }
+  }
+  auto stage_at = [&](uint32_t index) __attribute__((always_inline)) -> uint32_t {
+    if constexpr (MASKED) return listed ? (uint32_t)live_list[index] : index;
+    return index;
+  };
   MaskRaw mask_raw[TILES];
-  if (stages > 0) {
+  if (walk > 0) {
+    const uint32_t first = stage_at(0);
     if constexpr (MASKED) {
 #pragma unroll
-      for (int t = 0; t < TILES; ++t) mask_request(tile_key0(0, t), mask_raw[t]);
+      for (int t = 0; t < TILES; ++t) mask_request(tile_key0(first, t), mask_raw[t]);
     }
-    copy_stage(0);
+    copy_stage(first, 0);
     stage_landed();
   }
 
@@ -315,8 +353,9 @@ __global__ __launch_bounds__(WAVES * 64)
     // a tile of existing keys, all below the causal limit of the wave's first row, of existing
     // rows and without a mask needs no per-score test.  Maxima are taken over the scores as the MFMAs left them; the
     // scale (positive) goes into the exponent's multiply-add.
-    const bool interior =
-        !masked && key0 + 32 <= L && q0 + 32 <= a.query_length && (!a.causal || key0 + 31 <= a.past_length + q0);
+    // (with a mask: when it allows all 32 x 32 scores of the tile)
+    const bool interior = (!masked || __builtin_amdgcn_ballot_w64(allowed_bits != 0xffffu) == 0) && key0 + 32 <= L &&
+                          q0 + 32 <= a.query_length && (!a.causal || key0 + 31 <= a.past_length + q0);
     float tile_max = -INFINITY;
     if (interior) {
 #pragma unroll
@@ -373,7 +412,8 @@ __global__ __launch_bounds__(WAVES * 64)
 
   // The tiles of a stage.  Two: both score chains go to the matrix pipe first, so the second runs
   // while the vector unit works on the first tile's softmax.
-  for (uint32_t stage = 0; stage < stages; ++stage) {
+  for (uint32_t index = 0; index < walk; ++index) {
+    const uint32_t stage = stage_at(index);
     // The mask values of this stage were requested a stage ago and landed with that stage's copies
     // (stage_landed waits for everything): they are turned into bits before anything new is
     // requested, so that no wait for them stands behind the next stage's copies.
@@ -384,14 +424,15 @@ __global__ __launch_bounds__(WAVES * 64)
       allowed_bits[t] = MASKED ? mask_bits(mask_raw[t]) : 0xffffu;
       live[t] = tile_key0(stage, t) < key_end && (!MASKED || __builtin_amdgcn_ballot_w64(allowed_bits[t] != 0) != 0);
     }
-    if (stage + 1 < stages) {
-      copy_stage(stage + 1);  // into the buffer every wave left at the last barrier
+    if (index + 1 < walk) {
+      const uint32_t next = stage_at(index + 1);
+      copy_stage(next, (index + 1) & 1);  // into the buffer every wave left at the last barrier
       if constexpr (MASKED) {
 #pragma unroll
-        for (int t = 0; t < TILES; ++t) mask_request(tile_key0(stage + 1, t), mask_raw[t]);
+        for (int t = 0; t < TILES; ++t) mask_request(tile_key0(next, t), mask_raw[t]);
       }
     }
-    const unsigned char *k_stage = stage_lds + (stage & 1) * 2 * STAGE_BYTES;
+    const unsigned char *k_stage = stage_lds + (index & 1) * 2 * STAGE_BYTES;
     const unsigned char *v_stage = k_stage + STAGE_BYTES;
     if constexpr (KEYSPLIT) {
       if (live[0])
@@ -504,6 +545,81 @@ __global__ __launch_bounds__(WAVES * 64)
     }
 }
 
+// ---- which stages of keys a mask leaves to a slab of query rows ------------------------------
+//
+// One workgroup of 1024 threads per (eight stages of keys, slab of query rows, mask row group): a thread
+// ORs one run of four consecutive keys down its share of the slab's rows (sixteen or eight), the lanes of a stage vote, and
+// the workgroup stores the eight answers as one byte of the map the attention kernel reads.
+// rows_per_slab x stage_keys is the attention launch's geometry: 128 x 64, or 32 x 128 when the
+// keys of a slab are split over the waves.
+__global__ __launch_bounds__(1024) void mask_stage_map_kernel(DenseAttentionArgs a, uint32_t rows_per_slab,
+                                                              uint32_t stage_keys, uint32_t map_stride) {
+  __shared__ uint32_t chunk_bits;
+  const uint32_t chunk = blockIdx.x, slab = blockIdx.y, group = blockIdx.z;
+  const uint32_t L = a.key_length;
+  const uint32_t runs = 2 * stage_keys;                   // runs of four keys in eight stages: 128 or 256
+  const uint32_t row_groups = 1024 / runs;                // 8 or 4
+  const uint32_t rows_each = rows_per_slab / row_groups;  // 16 or 8
+  const uint32_t run = threadIdx.x % runs, row_group = threadIdx.x / runs;
+  const uint32_t key = chunk * 8 * stage_keys + run * 4;
+  const uint32_t row0 = slab * rows_per_slab + row_group * rows_each;
+  const bool whole_runs = L % 4 == 0 && L >= 4 && reinterpret_cast<uintptr_t>(a.mask) % 8 == 0;
+  const size_t group_base = (size_t)group * a.query_length * L;
+  if (threadIdx.x == 0) chunk_bits = 0;
+  // every request goes out before the first value is looked at (rows past the end repeat the last one,
+  // a run past the end the last whole run: what they say is dropped below)
+  constexpr int kRows = 16;
+  uint32_t any = 0;
+  const uint32_t last_row = a.query_length - 1;
+  if (whole_runs) {
+    const uint32_t at_key = min(key, L - 4);
+    if (a.mask_dtype == 2) {
+      const uint16_t *mask = reinterpret_cast<const uint16_t *>(a.mask) + group_base + at_key;
+      uint2 four[kRows];
+#pragma unroll
+      for (int r = 0; r < kRows; ++r) four[r] = *reinterpret_cast<const uint2 *>(mask + (size_t)min(row0 + r, last_row) * L);
+#pragma unroll
+      for (int r = 0; r < kRows; ++r) {
+        const bool counts = (uint32_t)r < rows_each && row0 + r <= last_row;
+        const bool allowed = half_bits_to_float((uint16_t)four[r].x) >= 0.0f || half_bits_to_float((uint16_t)(four[r].x >> 16)) >= 0.0f ||
+                             half_bits_to_float((uint16_t)four[r].y) >= 0.0f || half_bits_to_float((uint16_t)(four[r].y >> 16)) >= 0.0f;
+        any |= counts && allowed ? 1u : 0u;
+      }
+    } else {
+      const uint8_t *mask = a.mask + group_base + at_key;
+      uint32_t four[kRows];
+#pragma unroll
+      for (int r = 0; r < kRows; ++r) four[r] = *reinterpret_cast<const uint32_t *>(mask + (size_t)min(row0 + r, last_row) * L);
+#pragma unroll
+      for (int r = 0; r < kRows; ++r) any |= ((uint32_t)r < rows_each && row0 + r <= last_row && four[r] != 0) ? 1u : 0u;
+    }
+    if (key >= L) any = 0;
+  } else {
+    // rows of the mask that are not whole runs: element by element
+    for (uint32_t r = 0; r < rows_each && row0 + r <= last_row; ++r)
+      for (uint32_t e = 0; e < 4 && key + e < L; ++e) {
+        const size_t at = group_base + (size_t)(row0 + r) * L + key + e;
+        const bool allowed = a.mask_dtype == 2 ? half_bits_to_float(reinterpret_cast<const uint16_t *>(a.mask)[at]) >= 0.0f
+                                               : a.mask[at] != 0;
+        any |= allowed ? 1u : 0u;
+      }
+  }
+  __syncthreads();
+  // the lanes of one stage are stage_keys / 4 neighbours (16 or 32) of one wave
+  const uint64_t votes = __builtin_amdgcn_ballot_w64(any != 0);
+  if ((threadIdx.x & 63) == 0) {
+    const uint32_t lanes_per_stage = stage_keys / 4, stages_per_wave = 64 / lanes_per_stage;
+    const uint32_t first_stage = run / lanes_per_stage;
+    const uint64_t lanes = lanes_per_stage == 32 ? 0xffffffffull : 0xffffull;
+    uint32_t bits = 0;
+    for (uint32_t j = 0; j < stages_per_wave; ++j)
+      if ((votes >> (j * lanes_per_stage)) & lanes) bits |= 1u << (first_stage + j);
+    if (bits != 0) atomicOr(&chunk_bits, bits);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) a.stage_map[((size_t)group * gridDim.y + slab) * map_stride + chunk] = (uint8_t)chunk_bits;
+}
+
 // ---- row-serial kernel (every other configuration) ---------------------------
 
 constexpr int kMaxFragments = 8;  // head_dim <= 512
@@ -599,33 +715,76 @@ hipError_t launch_tile32(int mask, uint32_t grid, const DenseAttentionArgs &a, h
   return launch_tile32_instance<D, WAVES, STAGE_KEYS, 0, KEYSPLIT>(grid, a, stream);
 }
 
+// Which kernel a launch takes and the slabs and stages it works in.
+struct Tile32Geometry {
+  bool tiled;       // the 32 x 32 tile kernel (else the row-serial one)
+  bool key_split;   // 32-row slabs whose keys are split over the waves, 128-key stages
+  uint32_t rows_per_slab, stage_keys, slabs;
+  uint64_t workgroups;  // of 128 rows
+};
+
+Tile32Geometry tile32_geometry(const DenseAttentionArgs &a) {
+  Tile32Geometry g = {false, false, 128, 64, 0, 0};
+  const bool aligned = reinterpret_cast<uintptr_t>(a.query) % 16 == 0 && reinterpret_cast<uintptr_t>(a.key) % 16 == 0 &&
+                       reinterpret_cast<uintptr_t>(a.value) % 8 == 0 && reinterpret_cast<uintptr_t>(a.output) % 8 == 0;
+  if (!((a.head_dim == 64 || a.head_dim == 128 || a.head_dim == 256) && aligned && a.query_length >= 16)) return g;
+  // K and V stages are copied as 16-byte pieces of whole rows (16-byte aligned K and V rows), and the
+  // maxima are taken before scaling (a positive, finite scale); anything else takes the row kernel
+  const size_t value_row_halfs = a.token_first_value ? (size_t)(a.kv_heads > 0 ? a.kv_heads : a.heads) * a.head_dim
+                                                     : a.head_dim;
+  const bool staged = reinterpret_cast<uintptr_t>(a.value) % 16 == 0 && value_row_halfs % 8 == 0 &&
+                      a.scale > 0.0f && a.scale < INFINITY;
+  g.workgroups = (uint64_t)((a.query_length + kWavesPerBlock * 32 - 1) / (kWavesPerBlock * 32)) * a.heads * a.batches;
+  if (!staged || g.workgroups > 0x7fffffffull) return g;
+  g.tiled = true;
+  g.key_split = g.workgroups < (uint64_t)device_compute_units() && a.key_length >= 256 && a.head_dim <= 128;
+  if (g.key_split) g.rows_per_slab = 32, g.stage_keys = 128;
+  g.slabs = (a.query_length + g.rows_per_slab - 1) / g.rows_per_slab;
+  return g;
+}
+
+bool dense_masked(const DenseAttentionArgs &a) { return a.mask != nullptr && a.mask_batches > 0; }
+
+uint32_t stage_map_stride(const DenseAttentionArgs &a, const Tile32Geometry &g) {
+  return ((a.key_length + g.stage_keys - 1) / g.stage_keys + 7) / 8;
+}
+
 }  // namespace
+
+size_t dense_attention_workspace_bytes(const DenseAttentionArgs &a) {
+  if (!dense_masked(a) || a.batches == 0 || a.heads == 0 || a.query_length == 0 || a.key_length == 0) return 0;
+  const Tile32Geometry g = tile32_geometry(a);
+  if (!g.tiled) return 0;
+  return (size_t)a.mask_batches * a.mask_heads * g.slabs * stage_map_stride(a, g);
+}
 
 hipError_t launch_dense_attention(const DenseAttentionArgs &a, hipStream_t stream) {
   const uint64_t rows = (uint64_t)a.batches * a.heads * a.query_length;
   if (rows == 0) return hipSuccess;
   if (a.key_length == 0 || a.head_dim == 0 || a.head_dim > 64 * kMaxFragments) return hipErrorInvalidValue;
-  const bool aligned = reinterpret_cast<uintptr_t>(a.query) % 16 == 0 && reinterpret_cast<uintptr_t>(a.key) % 16 == 0 &&
-                       reinterpret_cast<uintptr_t>(a.value) % 8 == 0 && reinterpret_cast<uintptr_t>(a.output) % 8 == 0;
-  if ((a.head_dim == 64 || a.head_dim == 128 || a.head_dim == 256) && aligned && a.query_length >= 16) {
-    // K and V stages are copied as 16-byte pieces of whole rows (16-byte aligned K and V rows), and the
-    // maxima are taken before scaling (a positive, finite scale); anything else takes the row kernel
-    const size_t value_row_halfs = a.token_first_value ? (size_t)(a.kv_heads > 0 ? a.kv_heads : a.heads) * a.head_dim
-                                                       : a.head_dim;
-    const bool staged = reinterpret_cast<uintptr_t>(a.value) % 16 == 0 && value_row_halfs % 8 == 0 &&
-                        a.scale > 0.0f && a.scale < INFINITY;
-    const uint64_t workgroups = (uint64_t)((a.query_length + kWavesPerBlock * 32 - 1) / (kWavesPerBlock * 32)) *
-                                a.heads * a.batches;
-    if (staged && workgroups <= 0x7fffffffull) {
-      const int mask = (a.mask != nullptr && a.mask_batches > 0) ? (a.mask_dtype == 2 ? 2 : 1) : 0;
+  const Tile32Geometry geometry = tile32_geometry(a);
+  {
+    if (geometry.tiled) {
+      const uint64_t workgroups = geometry.workgroups;
+      const int mask = dense_masked(a) ? (a.mask_dtype == 2 ? 2 : 1) : 0;
       DenseAttentionArgs scheduled = a;
       scheduled.cus_per_xcd = (uint32_t)device_compute_units() / 8;
+      // the pass over the mask that says which stages of keys each slab of rows has to walk
+      if (mask != 0 && a.stage_map != nullptr) {
+        const uint32_t stride = stage_map_stride(a, geometry);
+        const uint64_t groups = (uint64_t)a.mask_batches * a.mask_heads;
+        if (a.stage_map_bytes < groups * geometry.slabs * stride || geometry.slabs > 65535 || groups > 65535)
+          scheduled.stage_map = nullptr;
+        else
+          hipLaunchKernelGGL(mask_stage_map_kernel, dim3(stride, geometry.slabs, (uint32_t)groups), dim3(1024), 0, stream, a,
+                             geometry.rows_per_slab, geometry.stage_keys, stride);
+      }
       // Fewer workgroups of 128 rows than CUs: the launch lasts as long as one wave's walk over the
       // keys of its slab, so the waves of a workgroup share 32 rows and a quarter of the keys each
       // (four times the workgroups, a quarter of the walk): 9 heads x 2048 tokens of 64, causal,
       // 45.0 -> 22.9 us.  Larger launches keep 128 rows a workgroup: a stage of K and V then serves
       // four times as many rows.
-      if (workgroups < (uint64_t)device_compute_units() && a.key_length >= 256 && a.head_dim <= 128) {
+      if (geometry.key_split) {
         const uint32_t grid = (uint32_t)((a.query_length + 31) / 32) * a.heads * a.batches;
         if (a.head_dim == 64) return launch_tile32<64, 4, 128, true>(mask, grid, scheduled, stream);
         return launch_tile32<128, 4, 128, true>(mask, grid, scheduled, stream);

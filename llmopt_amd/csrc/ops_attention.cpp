@@ -324,6 +324,12 @@ int dense_attention(llmopt_hip_context *context, const DispatchRecord &record) {
   args.key = reinterpret_cast<const uint16_t *>(record.buffers[1].device);
   args.value = reinterpret_cast<const uint16_t *>(record.buffers[2].device);
   args.output = reinterpret_cast<uint16_t *>(record.buffers[4].device);
+  const size_t map_bytes = dense_attention_workspace_bytes(args);
+  if (map_bytes > 0) {
+    args.stage_map = static_cast<uint8_t *>(context_workspace(context, map_bytes));
+    if (args.stage_map == nullptr) return LLMOPT_ERR_FAILURE;
+    args.stage_map_bytes = map_bytes;
+  }
   return launched(launch_dense_attention(args, context->stream), name);
 }
 
