@@ -339,3 +339,36 @@ def test_heads_of_256_on_the_tile_kernel(runtime, heads, kv_heads, new, past, mo
     """llmopt_attention_f16_simd_h256 with sixteen query rows or more: the 32 x 32 tile kernel with
     eight output blocks per wave and 128 KB of K and V stages per workgroup."""
     check_attention_case(runtime, 256, heads, kv_heads, new, past, mode)
+
+
+@pytest.mark.parametrize("dim,heads,kv_heads,batches,tokens,past,mask_dtype,window", [
+    (128, 16, 4, 3, 700, 0, 2, 0),     # 288 workgroups of 128 rows: the four-wave slabs, f16 causal mask
+    (64, 24, 8, 2, 650, 70, 1, 0),     # byte mask of a suffix over cached tokens
+    (128, 16, 16, 3, 640, 0, 2, 150),  # sliding window: the first stages of later slabs are forbidden too
+    (64, 3, 1, 1, 900, 0, 2, 0),       # few workgroups: 32-row slabs with the keys split over the waves
+    (128, 2, 2, 1, 515, 0, 1, 200),    # the same with a window and rows that are not whole runs of four keys
+    (256, 2, 1, 2, 300, 33, 2, 64),
+])
+def test_masks_that_forbid_whole_stages(runtime, dim, heads, kv_heads, batches, tokens, past, mask_dtype, window):
+    """The masks the reference's prefill builds (lib/serving_engine.ml:303-321, 1194-1201): causal over
+    the new tokens after `past` cached ones, optionally a sliding window, as halves (0 / -inf) or
+    bytes, one mask for all batches and heads.  Most stages of keys are forbidden to most slabs of
+    rows: the pass over the mask says which, and the attention kernel walks only the others."""
+    rng = np.random.default_rng(dim + heads + tokens + past + window)
+    length = past + tokens
+    query = rng.standard_normal((batches, heads, tokens, dim)).astype(np.float16)
+    key = rng.standard_normal((batches, kv_heads, length, dim)).astype(np.float16)
+    value = rng.standard_normal((batches, kv_heads, length, dim)).astype(np.float16)
+    scale = 1.0 / math.sqrt(dim)
+    position = past + np.arange(tokens)[:, None]
+    keys = np.arange(length)[None, :]
+    visible = keys <= position
+    if window:
+        visible &= keys > position - window
+    allowed = np.broadcast_to(visible[None, None], (batches, heads, tokens, length))
+    mask = np.where(visible, 0.0, -np.inf).astype(np.float16) if mask_dtype == 2 else visible.astype(np.uint8)
+    params = attention_params(batches, heads, tokens, length, dim, 1, 1, False, scale, kv_heads, mask_dtype=mask_dtype)
+    got = run(runtime, f"llmopt_attention_f16_simd_h{dim}", query, key, value, mask[None, None], params,
+              (batches, heads, tokens, dim))
+    want = expected(query, key, value, allowed, scale)
+    assert_close_to_oracle(got, want, f"mask of whole stages D={dim} {heads}/{kv_heads} x {tokens} after {past}, window {window}")
