@@ -346,21 +346,29 @@ def bench_attention(runtime):
 
 def bench_prefill_attention(runtime):
     """Dense causal fp16 attention of a prefill (the step that fills the KV cache): 32/8 heads of
-    128 at 2048 and 8192 tokens, and the 30-layer model's 9/3 heads of 64 at 2048."""
+    128 at 2048 and 8192 tokens, the 30-layer model's 9/3 heads of 64 at 2048, and the first case
+    again with the causal limit given as a mask."""
     rng = np.random.default_rng(SEED + 4)
     results = []
     import oracle
-    for heads, kv_heads, dim, length in ((32, 8, 128, 2048), (32, 8, 128, 8192), (9, 3, 64, 2048)):
+    # the last case takes the causal limit as the reference's prefill passes it: an additive f16 mask of
+    # 0 / -inf over [tokens, tokens] (attention_mask_buffer, lib/serving_engine.ml:303-321) instead of the flag
+    for heads, kv_heads, dim, length, masked in ((32, 8, 128, 2048, False), (32, 8, 128, 8192, False),
+                                                 (9, 3, 64, 2048, False), (32, 8, 128, 2048, True)):
         host_q = rng.standard_normal((1, heads, length, dim)).astype(np.float16)
         host_k = rng.standard_normal((1, kv_heads, length, dim)).astype(np.float16)
         host_v = rng.standard_normal((1, kv_heads, length, dim)).astype(np.float16)
         query, key, value = (runtime.buffer_of_bytes(a) for a in (host_q, host_k, host_v))
         out = runtime.buffer_of_bytes(np.full(heads * length * dim, np.nan, dtype=np.float16))
-        params = struct.pack("<8IfIIIII", 1, heads, length, length, dim, 0, 0, 1, 1.0 / math.sqrt(dim),
-                             kv_heads, 1, 0, 0, 0)
+        mask = query
+        if masked:
+            visible = np.arange(length)[None, :] <= np.arange(length)[:, None]
+            mask = runtime.buffer_of_bytes(np.where(visible, 0.0, -np.inf).astype(np.float16))
+        params = struct.pack("<8IfIIIII", 1, heads, length, length, dim, int(masked), int(masked), int(not masked),
+                             1.0 / math.sqrt(dim), kv_heads, 1, 0, 0, 2 if masked else 0)
         batch = runtime.begin_batch()
         for _ in range(4):
-            batch.dispatch(f"llmopt_attention_f16_simd_h{dim}", [query, key, value, query, out], params,
+            batch.dispatch(f"llmopt_attention_f16_simd_h{dim}", [query, key, value, mask, out], params,
                            grid=(heads * ((length + 31) // 32) * 128, 1, 1), group=(128, 1, 1))
         repeats = 3
         us = batch.commit_profiled(repeats=repeats, use_graph=True) * 1e3 / (repeats * 4)
@@ -377,7 +385,7 @@ def bench_prefill_attention(runtime):
                 row_ok, rel_l2 = close_to_oracle(got[row, head], want)
                 ok, worst = ok and row_ok, max(worst, rel_l2)
         results.append({"heads": heads, "kv_heads": kv_heads, "head_dim": dim, "tokens": length,
-                        "us_per_launch": round(us, 2), "TFLOPs": round(flops / (us * 1e-6) / 1e12, 1),
+                        "causal_by": "f16 mask" if masked else "flag", "us_per_launch": round(us, 2), "TFLOPs": round(flops / (us * 1e-6) / 1e12, 1),
                         "mfma_frac": round(flops / (us * 1e-6) / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
                         "verified": ok, "rel_l2": float("%.3g" % worst)})
     return results
