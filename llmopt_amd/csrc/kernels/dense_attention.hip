@@ -755,6 +755,9 @@ size_t dense_attention_workspace_bytes(const DenseAttentionArgs &a) {
   if (!dense_masked(a) || a.batches == 0 || a.heads == 0 || a.query_length == 0 || a.key_length == 0) return 0;
   const Tile32Geometry g = tile32_geometry(a);
   if (!g.tiled) return 0;
+  // a few stages only: walking them all (their arithmetic is skipped where the mask forbids it) costs
+  // less than another launch ahead of the attention kernel
+  if ((a.key_length + g.stage_keys - 1) / g.stage_keys <= 4) return 0;
   return (size_t)a.mask_batches * a.mask_heads * g.slabs * stage_map_stride(a, g);
 }
 

@@ -877,6 +877,95 @@ __global__ __launch_bounds__(kGeneralWaves * 64) void q8_attention_general_kerne
   }
 }
 
+// ---- several query tokens: a half-precision copy of the context and the dense tile kernel ----
+//
+// The reference prefills a suffix over cached tokens with this entry (query_length new tokens, a
+// byte mask that is causal over them: suffix_causal_mask, lib/serving_engine.ml:1194-1201).  A wave
+// per output row re-reads the context once per row; with sixteen query tokens or more the context
+// of the layer is instead written out once as halves - pool tokens as half(float(int8) *
+// float(scale)), the new tokens' K and V copied behind them - and the dense kernel, which shares
+// every K / V tile among 128 query rows on the matrix cores, runs over that copy with the same
+// mask, the causal limit over the new tokens and token-major output.  The copy rounds a cached
+// value once more (2^-11 relative at most), where the row kernel multiplies int8 by scale in
+// float32: within the tolerance the path's results are held to.
+__global__ __launch_bounds__(256) void q8_context_as_halves_kernel(Q8AttentionArgs a, uint16_t *key16, uint16_t *value16) {
+  const uint32_t q_len = a.query_length, L = a.past_length + q_len, D = a.head_dim, pieces = D / 8;
+  const uint64_t index = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+  if (index >= (uint64_t)a.batches * a.kv_heads * L * pieces) return;
+  const bool is_value = blockIdx.y != 0;
+  const uint32_t piece = (uint32_t)(index % pieces), token = (uint32_t)(index / pieces % L);
+  const uint32_t kv_head = (uint32_t)(index / pieces / L % a.kv_heads), batch = (uint32_t)(index / pieces / L / a.kv_heads);
+  uint16_t *destination =
+      (is_value ? value16 : key16) + (((size_t)batch * a.kv_heads + kv_head) * L + token) * D + piece * 8;
+  uint4 halves;
+  if (token < a.past_length) {
+    const uint8_t *slot = a.pool + (size_t)a.slots[token] * a.token_stride;
+    const uint32_t element = (is_value ? a.value_offset : a.key_offset) + kv_head * D + piece * 8;
+    const float scale = q8_scale_at(slot, a.token_elements, element >> 6);
+    const uint8_t *bytes = slot + element;
+    uint32_t packed[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float low = (float)(int8_t)bytes[2 * e] * scale, high = (float)(int8_t)bytes[2 * e + 1] * scale;
+      packed[e] = (uint32_t)float_to_half_bits(low) | ((uint32_t)float_to_half_bits(high) << 16);
+    }
+    halves = make_uint4(packed[0], packed[1], packed[2], packed[3]);
+  } else {
+    const uint16_t *source = (is_value ? a.current_value : a.current_key) +
+                             (((size_t)batch * a.kv_heads + kv_head) * q_len + (token - a.past_length)) * D + piece * 8;
+    halves = *reinterpret_cast<const uint4 *>(source);
+  }
+  *reinterpret_cast<uint4 *>(destination) = halves;
+}
+
+bool use_dense_copy_path(const Q8AttentionArgs &a) {
+  const uint32_t q_len = a.query_length == 0 ? 1 : a.query_length;
+  if (q_len < 16 || a.window != 0 || a.past_lengths != nullptr || a.slot_offsets != nullptr) return false;
+  if (a.head_dim != 64 && a.head_dim != 128 && a.head_dim != 256) return false;
+  if (a.kv_heads == 0 || a.query_heads % a.kv_heads != 0) return false;
+  if (!(a.scale > 0.0f && a.scale < INFINITY)) return false;
+  if ((uint64_t)a.past_length + q_len > 0x7fffffffull) return false;
+  // 16-byte copies of the new tokens' rows; what the dense tile kernel asks of its operands
+  return ((reinterpret_cast<uintptr_t>(a.query) | reinterpret_cast<uintptr_t>(a.current_key) |
+           reinterpret_cast<uintptr_t>(a.current_value)) & 15) == 0 &&
+         (reinterpret_cast<uintptr_t>(a.output) & 7) == 0;
+}
+
+// Where the copy and the dense kernel's own scratch lie in the workspace, and the dense launch.
+struct DenseCopyPlan {
+  size_t operand_bytes;  // one of K, V as halves (a multiple of 256)
+  size_t map_bytes, total_bytes;
+  DenseAttentionArgs dense;
+};
+
+DenseCopyPlan dense_copy_plan(const Q8AttentionArgs &a, void *workspace) {
+  DenseCopyPlan plan = {};
+  const uint32_t q_len = a.query_length, L = a.past_length + q_len;
+  plan.operand_bytes = ((size_t)a.batches * a.kv_heads * L * a.head_dim * 2 + 255) & ~(size_t)255;
+  // (sizing without a workspace yet: any address with the workspace's alignment gives the same answer)
+  uint8_t *base = workspace != nullptr ? static_cast<uint8_t *>(workspace) : reinterpret_cast<uint8_t *>((uintptr_t)4096);
+  const bool masked = a.mask != nullptr && a.mask_batches > 0 && a.mask_dtype != 0;
+  DenseAttentionArgs &d = plan.dense;
+  d.query = a.query;
+  d.key = reinterpret_cast<const uint16_t *>(base);
+  d.value = reinterpret_cast<const uint16_t *>(base + plan.operand_bytes);
+  d.mask = masked ? a.mask : nullptr;
+  d.output = a.output;
+  d.batches = a.batches, d.heads = a.query_heads, d.query_length = q_len, d.key_length = L, d.head_dim = a.head_dim;
+  d.mask_batches = masked ? a.mask_batches : 0, d.mask_heads = masked ? a.mask_heads : 0;
+  d.causal = 1;  // key_length of query token q is past_length + q + 1 (lib/metal_cache_source.ml:429)
+  d.scale = a.scale;
+  d.kv_heads = a.kv_heads, d.token_first_output = 1, d.past_length = a.past_length, d.token_first_value = 0;
+  d.mask_dtype = masked ? a.mask_dtype : 0;
+  plan.map_bytes = dense_attention_workspace_bytes(d);
+  plan.total_bytes = 2 * plan.operand_bytes + plan.map_bytes;
+  if (plan.map_bytes > 0) {
+    d.stage_map = base + 2 * plan.operand_bytes;
+    d.stage_map_bytes = plan.map_bytes;
+  }
+  return plan;
+}
+
 // The longest span of pool tokens a sequence of the launch can have (see sequence_span).
 uint32_t longest_span(const Q8AttentionArgs &a) {
   return a.window != 0 && a.max_past_length >= a.window ? a.window - 1 : a.max_past_length;
@@ -962,6 +1051,7 @@ uint32_t balanced_split_slots(const Q8AttentionArgs &a) {
 }  // namespace
 
 size_t q8_attention_workspace_bytes(const Q8AttentionArgs &a) {
+  if (use_dense_copy_path(a)) return dense_copy_plan(a, nullptr).total_bytes;
   if (!use_split_path(a)) return 0;
   const size_t per_partial = 32 + (size_t)(a.query_heads / a.kv_heads) * a.head_dim;
   const uint32_t slots = balanced_split_slots(a);
@@ -970,6 +1060,18 @@ size_t q8_attention_workspace_bytes(const Q8AttentionArgs &a) {
 }
 
 hipError_t launch_q8_attention(const Q8AttentionArgs &a, hipStream_t stream) {
+  if (use_dense_copy_path(a)) {
+    if (a.batches == 0 || a.query_heads == 0) return hipSuccess;
+    const DenseCopyPlan plan = dense_copy_plan(a, a.workspace);
+    // (a workspace that is not 16-byte aligned - none the runtime hands out is - sends the dense launch to its row kernel)
+    if (a.workspace == nullptr || a.workspace_bytes < plan.total_bytes) return hipErrorInvalidValue;
+    const uint64_t threads = (uint64_t)a.batches * a.kv_heads * plan.dense.key_length * (a.head_dim / 8);
+    if ((threads + 255) / 256 > 0x7fffffffull) return hipErrorInvalidValue;
+    uint8_t *base = static_cast<uint8_t *>(a.workspace);
+    hipLaunchKernelGGL(q8_context_as_halves_kernel, dim3((uint32_t)((threads + 255) / 256), 2), dim3(256), 0, stream, a,
+                       reinterpret_cast<uint16_t *>(base), reinterpret_cast<uint16_t *>(base + plan.operand_bytes));
+    return launch_dense_attention(plan.dense, stream);
+  }
   if (use_split_path(a)) {
     const uint32_t chunks = split_chunks(a);
     const uint32_t chunk_tokens = split_chunk_tokens(a);

@@ -520,3 +520,37 @@ def test_attention_int8_decoders_are_bit_exact(runtime, decoder, name):
                                 source_items=tokens, source_offset=0)
     unpacked = oracle.q8_unpack(pool.reshape(-1), np.arange(tokens, dtype=np.uint32), params)
     np.testing.assert_array_equal(got, unpacked.astype(np.float32).reshape(-1), err_msg=name)
+
+
+@pytest.mark.parametrize("name,b,h,kvh,dim,past,q_len,mask_dtype", [
+    ("llmopt_attention_q8_paged_simd_h64_gqa3", 1, 9, 3, 64, 74, 118, 1),   # the reference's suffix prefill
+    ("llmopt_attention_q8_paged_simd_generic", 2, 8, 2, 128, 300, 45, 1),
+    ("llmopt_attention_q8_paged_simd_generic", 1, 4, 4, 128, 0, 16, 2),    # nothing cached yet
+    ("llmopt_attention_q8_paged_simd_h64", 1, 4, 4, 64, 1000, 200, 2),
+    ("llmopt_attention_q8_paged_simd_h256", 1, 4, 2, 256, 130, 33, 1),
+    ("llmopt_attention_q8_paged_simd_generic", 1, 32, 8, 128, 515, 140, 1),
+])
+def test_suffix_prefill_over_cached_tokens(runtime, name, b, h, kvh, dim, past, q_len, mask_dtype):
+    """Sixteen query tokens or more over a Q8 context, with the mask the reference builds for a suffix
+    (causal over the new tokens, every cached token visible; lib/serving_engine.ml:1194-1201) as bytes
+    or halves, plus a few holes: the context is copied out as halves once and the dense tile kernel
+    runs over it.  Token-major output, GQA, a row whose mask allows nothing."""
+    rng = np.random.default_rng(past * 3 + q_len + dim)
+    pool, slots, _, te, stride, ko, vo = build_pool(rng, kvh, dim, [max(past, 1)])
+    slots = slots[:past]
+    query = rng.standard_normal((b, h, q_len, dim)).astype(np.float16)
+    ck = rng.standard_normal((b, kvh, q_len, dim)).astype(np.float16)
+    cv = rng.standard_normal((b, kvh, q_len, dim)).astype(np.float16)
+    visible = np.arange(past + q_len)[None, :] <= past + np.arange(q_len)[:, None]
+    visible = np.broadcast_to(visible, (b, 1, q_len, past + q_len)).copy()
+    visible &= rng.random(visible.shape) > 0.05
+    visible[:, :, 2, :] = False
+    mask = visible.astype(np.uint8) if mask_dtype == 1 else np.where(visible, 0.0, -np.inf).astype(np.float16)
+    params = PagedParams(batches=b, query_heads=h, kv_heads=kvh, past_length=past, head_dim=dim,
+                         mask_batches=b, mask_heads=1, token_elements=te, key_offset=ko, value_offset=vo,
+                         group_size=64, token_stride=stride, scale=1.0 / math.sqrt(dim), query_length=q_len,
+                         mask_dtype=mask_dtype, window=0)
+    out = run_paged(runtime, name, query, ck, cv, pool, slots, mask, params)
+    expected = oracle.paged_attention_q8(query, ck, cv, pool, slots, mask, params)
+    assert np.all(out[:, 2].view(np.uint16) == 0)
+    assert_close_to_oracle(out, expected, f"suffix prefill {name} {q_len} new after {past}")
