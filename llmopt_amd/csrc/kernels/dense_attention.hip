@@ -90,11 +90,16 @@ constexpr int tile32_waves_per_simd() {
   return D <= 128 ? 2 : 1;
 }
 
-template <int D, int WAVES, int STAGE_KEYS, int MASK, bool KEYSPLIT = false>
-__global__ __launch_bounds__(WAVES * 64)
+// PAIR: two groups of WAVES waves share the slab's query rows and take alternate stages of its keys (each
+// group with its own two LDS stages); group 1 hands its maxima, denominators and sums to group 0 through
+// LDS at the end.  For launches of one or two workgroups per CU: such a launch lasts as long as its
+// longest slab's walk over the keys, wave by wave, and the walk is half as long this way.
+template <int D, int WAVES, int STAGE_KEYS, int MASK, bool KEYSPLIT = false, bool PAIR = false>
+__global__ __launch_bounds__(WAVES * 64 * (PAIR ? 2 : 1))
     __attribute__((amdgpu_waves_per_eu(tile32_waves_per_simd<D>(), tile32_waves_per_simd<D>()))) void
     dense_attention_tile32_kernel(DenseAttentionArgs a) {
   constexpr bool MASKED = MASK != 0;
+  static_assert(!PAIR || !KEYSPLIT, "one way of splitting the keys at a time");
   constexpr int KSTEPS = D / 16;  // score MFMAs per key tile
   constexpr int JJ = D / 32;      // adjacent head_dim values per lane and key = output blocks
   constexpr int ROW_BYTES = D * 2;
@@ -111,9 +116,12 @@ __global__ __launch_bounds__(WAVES * 64)
                 "stage");
   static_assert(!KEYSPLIT || STAGE_KEYS == 32 * WAVES, "a tile of every stage per wave");
   constexpr int ROWS = KEYSPLIT ? 32 : WAVES * 32;  // query rows per workgroup
-  extern __shared__ __attribute__((aligned(16))) unsigned char stage_lds[];  // [2 stages][K | V]
+  extern __shared__ __attribute__((aligned(16))) unsigned char stage_lds[];  // [group][2 stages][K | V]
   const uint32_t lane = threadIdx.x & 63;
-  const uint32_t wave = threadIdx.x >> 6;
+  const uint32_t wave_of_all = threadIdx.x >> 6;
+  const uint32_t group = PAIR ? wave_of_all / WAVES : 0;  // which of the two halves of the stages
+  const uint32_t wave = PAIR ? wave_of_all % WAVES : wave_of_all;
+  unsigned char *group_lds = stage_lds + group * 4 * STAGE_BYTES;
   const uint32_t row_lane = lane & 31;
   const uint32_t half = lane >> 5;
   // Which (row slab, head, batch) this workgroup takes.  The grid is one-dimensional; rank 0.. runs over
@@ -132,7 +140,9 @@ __global__ __launch_bounds__(WAVES * 64)
     const uint32_t xcd = blockIdx.x % 8, position = blockIdx.x / 8, run = 2 * a.cus_per_xcd;
     const uint32_t start = position / run * run, within = position % run;
     uint32_t taken = position;
-    if (within >= a.cus_per_xcd && start + run <= gridDim.x / 8) taken = start + a.cus_per_xcd + (run - 1 - within);
+    // (PAIR: a CU holds one workgroup at a time and takes the next in rank order when it is done)
+    if (!PAIR && within >= a.cus_per_xcd && start + run <= gridDim.x / 8)
+      taken = start + a.cus_per_xcd + (run - 1 - within);
     rank = taken * 8 + xcd;
   }
   const uint32_t slab = longest_first ? slabs - 1 - rank / per_slab : rank / per_slab;
@@ -249,7 +259,7 @@ __global__ __launch_bounds__(WAVES * 64)
   auto copy_stage = [&](uint32_t stage, uint32_t buffer) __attribute__((always_inline)) {
 #if defined(__HIP_DEVICE_COMPILE__)
     const uint32_t buffer_base =
-        (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char *)stage_lds + buffer * 2 * STAGE_BYTES;
+        (uint32_t)(size_t)(__attribute__((address_space(3))) unsigned char *)group_lds + buffer * 2 * STAGE_BYTES;
     const uint32_t row_in_copy = lane / PIECES, piece = lane % PIECES;
 #pragma unroll
     for (int c = 0; c < COPIES; ++c) {
@@ -300,9 +310,9 @@ __global__ __launch_bounds__(WAVES * 64)
     listed = a.stage_map != nullptr && stages <= kMaxLive;
     if (listed) {
       const uint32_t total_stages = (L + STAGE_KEYS - 1) / STAGE_KEYS, map_stride = (total_stages + 7) / 8;
-      const uint32_t group = (a.mask_batches == 1 ? 0 : batch) * a.mask_heads + (a.mask_heads == 1 ? 0 : head);
-      const uint8_t *map = a.stage_map + ((size_t)group * slabs + slab) * map_stride;
-      if (wave == 0) {
+      const uint32_t mask_group = (a.mask_batches == 1 ? 0 : batch) * a.mask_heads + (a.mask_heads == 1 ? 0 : head);
+      const uint8_t *map = a.stage_map + ((size_t)mask_group * slabs + slab) * map_stride;
+      if (wave_of_all == 0) {
         uint32_t count = 0;
         for (uint32_t base = 0; base < stages; base += 64) {
           const uint32_t stage = base + lane;
@@ -321,14 +331,19 @@ __global__ __launch_bounds__(WAVES * 64)
     if constexpr (MASKED) return listed ? (uint32_t)live_list[index] : index;
     return index;
   };
+  // step s of the loop below works on entry walk_index(s) of the walk (PAIR: the groups take alternate entries)
+  const uint32_t steps = PAIR ? (walk + 1) / 2 : walk;
+  auto walk_index = [&](uint32_t step) __attribute__((always_inline)) { return PAIR ? 2 * step + group : step; };
   MaskRaw mask_raw[TILES];
   if (walk > 0) {
-    const uint32_t first = stage_at(0);
-    if constexpr (MASKED) {
+    if (walk_index(0) < walk) {
+      const uint32_t first = stage_at(walk_index(0));
+      if constexpr (MASKED) {
 #pragma unroll
-      for (int t = 0; t < TILES; ++t) mask_request(tile_key0(first, t), mask_raw[t]);
+        for (int t = 0; t < TILES; ++t) mask_request(tile_key0(first, t), mask_raw[t]);
+      }
+      copy_stage(first, 0);
     }
-    copy_stage(first, 0);
     stage_landed();
   }
 
@@ -412,8 +427,10 @@ __global__ __launch_bounds__(WAVES * 64)
 
   // The tiles of a stage.  Two: both score chains go to the matrix pipe first, so the second runs
   // while the vector unit works on the first tile's softmax.
-  for (uint32_t index = 0; index < walk; ++index) {
-    const uint32_t stage = stage_at(index);
+  for (uint32_t step = 0; step < steps; ++step) {
+    const uint32_t index = walk_index(step);
+    const bool active = index < walk;  // (PAIR: the last step may have an entry for group 0 only)
+    const uint32_t stage = active ? stage_at(index) : 0;
     // The mask values of this stage were requested a stage ago and landed with that stage's copies
     // (stage_landed waits for everything): they are turned into bits before anything new is
     // requested, so that no wait for them stands behind the next stage's copies.
@@ -422,17 +439,18 @@ __global__ __launch_bounds__(WAVES * 64)
 #pragma unroll
     for (int t = 0; t < TILES; ++t) {
       allowed_bits[t] = MASKED ? mask_bits(mask_raw[t]) : 0xffffu;
-      live[t] = tile_key0(stage, t) < key_end && (!MASKED || __builtin_amdgcn_ballot_w64(allowed_bits[t] != 0) != 0);
+      live[t] = active && tile_key0(stage, t) < key_end &&
+                (!MASKED || __builtin_amdgcn_ballot_w64(allowed_bits[t] != 0) != 0);
     }
-    if (index + 1 < walk) {
-      const uint32_t next = stage_at(index + 1);
-      copy_stage(next, (index + 1) & 1);  // into the buffer every wave left at the last barrier
+    if (walk_index(step + 1) < walk) {
+      const uint32_t next = stage_at(walk_index(step + 1));
+      copy_stage(next, (step + 1) & 1);  // into the buffer every wave left at the last barrier
       if constexpr (MASKED) {
 #pragma unroll
         for (int t = 0; t < TILES; ++t) mask_request(tile_key0(next, t), mask_raw[t]);
       }
     }
-    const unsigned char *k_stage = stage_lds + (index & 1) * 2 * STAGE_BYTES;
+    const unsigned char *k_stage = group_lds + (step & 1) * 2 * STAGE_BYTES;
     const unsigned char *v_stage = k_stage + STAGE_BYTES;
     if constexpr (KEYSPLIT) {
       if (live[0])
@@ -444,7 +462,7 @@ __global__ __launch_bounds__(WAVES * 64)
     const uint32_t key0 = stage * STAGE_KEYS;
     if constexpr (!MASKED && STAGE_KEYS == 64) {
       // (without a mask the second tile exists whenever the first does, except at the very end)
-      if (key0 < key_end) {
+      if (active && key0 < key_end) {
         const f16x_t first_scores = tile_scores(k_stage, 0);
         const bool second = key0 + 32 < key_end;
         f16x_t second_scores = first_scores;
@@ -522,6 +540,34 @@ __global__ __launch_bounds__(WAVES * 64)
       *reinterpret_cast<uint2 *>(out_row + d0 + e) = packed;
     }
     return;
+  }
+  if constexpr (PAIR) {
+    // Group 1 leaves its share in LDS (the stages are read to the end: the loop's last barrier), register
+    // by register with the lanes side by side, and group 0's wave of the same rows folds it into its own:
+    // both hold the same (row, head_dim) in the same lane and register.
+    float *share = reinterpret_cast<float *>(stage_lds) + wave * (JJ * 16 + 2) * 64;
+    static_assert((size_t)WAVES * (JJ * 16 + 2) * 64 * sizeof(float) <= 8 * (size_t)STAGE_BYTES, "the shares fit the stages");
+    if (group == 1) {
+      share[lane] = running_max;
+      share[64 + lane] = running_sum;
+#pragma unroll
+      for (int jj = 0; jj < JJ; ++jj)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) share[(2 + jj * 16 + r) * 64 + lane] = out_acc[jj][r];
+    }
+    __syncthreads();
+    if (group == 1) return;
+    const float other_max = share[lane], other_sum = share[64 + lane];
+    const float best = fmaxf(running_max, other_max);
+    const float reference = best == -INFINITY ? 0.0f : best;
+    const float own_weight = __builtin_amdgcn_exp2f((running_max - reference) * score_scale);  // 0 for a share without keys
+    const float other_weight = __builtin_amdgcn_exp2f((other_max - reference) * score_scale);
+    running_sum = running_sum * own_weight + other_sum * other_weight;
+#pragma unroll
+    for (int jj = 0; jj < JJ; ++jj)
+#pragma unroll
+      for (int r = 0; r < 16; ++r)
+        out_acc[jj][r] = out_acc[jj][r] * own_weight + share[(2 + jj * 16 + r) * 64 + lane] * other_weight;
   }
   if (!has_rows) return;
 
@@ -690,10 +736,10 @@ __global__ __launch_bounds__(256) void dense_attention_rows_kernel(DenseAttentio
   }
 }
 
-template <int D, int WAVES, int STAGE_KEYS, int MASK, bool KEYSPLIT>
+template <int D, int WAVES, int STAGE_KEYS, int MASK, bool KEYSPLIT, bool PAIR = false>
 hipError_t launch_tile32_instance(uint32_t grid, const DenseAttentionArgs &a, hipStream_t stream) {
-  constexpr size_t bytes = 2 * 2 * (size_t)STAGE_KEYS * D * 2;  // two stages of K and V
-  auto kernel = &dense_attention_tile32_kernel<D, WAVES, STAGE_KEYS, MASK, KEYSPLIT>;
+  constexpr size_t bytes = (PAIR ? 2 : 1) * 2 * 2 * (size_t)STAGE_KEYS * D * 2;  // two stages of K and V per group
+  auto kernel = &dense_attention_tile32_kernel<D, WAVES, STAGE_KEYS, MASK, KEYSPLIT, PAIR>;
   if constexpr (bytes >= 64 * 1024) {
     static bool configured = false;  // the attribute is per device function
     if (!configured) {
@@ -703,16 +749,16 @@ hipError_t launch_tile32_instance(uint32_t grid, const DenseAttentionArgs &a, hi
       configured = true;
     }
   }
-  hipLaunchKernelGGL(kernel, dim3(grid), dim3(WAVES * 64), bytes, stream, a);
+  hipLaunchKernelGGL(kernel, dim3(grid), dim3(WAVES * 64 * (PAIR ? 2 : 1)), bytes, stream, a);
   return hipGetLastError();
 }
 
 // mask: 0 none, 1 bytes, 2 halves
-template <int D, int WAVES, int STAGE_KEYS, bool KEYSPLIT>
+template <int D, int WAVES, int STAGE_KEYS, bool KEYSPLIT, bool PAIR = false>
 hipError_t launch_tile32(int mask, uint32_t grid, const DenseAttentionArgs &a, hipStream_t stream) {
-  if (mask == 2) return launch_tile32_instance<D, WAVES, STAGE_KEYS, 2, KEYSPLIT>(grid, a, stream);
-  if (mask == 1) return launch_tile32_instance<D, WAVES, STAGE_KEYS, 1, KEYSPLIT>(grid, a, stream);
-  return launch_tile32_instance<D, WAVES, STAGE_KEYS, 0, KEYSPLIT>(grid, a, stream);
+  if (mask == 2) return launch_tile32_instance<D, WAVES, STAGE_KEYS, 2, KEYSPLIT, PAIR>(grid, a, stream);
+  if (mask == 1) return launch_tile32_instance<D, WAVES, STAGE_KEYS, 1, KEYSPLIT, PAIR>(grid, a, stream);
+  return launch_tile32_instance<D, WAVES, STAGE_KEYS, 0, KEYSPLIT, PAIR>(grid, a, stream);
 }
 
 // Which kernel a launch takes and the slabs and stages it works in.
@@ -798,6 +844,15 @@ hipError_t launch_dense_attention(const DenseAttentionArgs &a, hipStream_t strea
       // tokens - one tile per barrier, half the sharing.)  Heads of 256: 128 KB of stages, one
       // workgroup per CU with all of its registers.
       if (a.head_dim == 256) return launch_tile32<256, 4, 64, false>(mask, (uint32_t)workgroups, scheduled, stream);
+      // One or two workgroups per CU: two groups of four waves per slab, each with half of the stages (a
+      // CU then holds one workgroup at a time, at the same two waves per SIMD): 32 heads x 2048 tokens,
+      // 512 workgroups, 72.9 -> 67.6 us.  The groups meet at every stage's barrier, so two of them get
+      // less out of a CU than two workgroups of four waves that run side by side freely - launches with
+      // enough of those keep them.
+      if (workgroups <= 2 * (uint64_t)device_compute_units() && a.key_length >= 256) {
+        if (a.head_dim == 64) return launch_tile32<64, 4, 64, false, true>(mask, (uint32_t)workgroups, scheduled, stream);
+        return launch_tile32<128, 4, 64, false, true>(mask, (uint32_t)workgroups, scheduled, stream);
+      }
       if (a.head_dim == 64) return launch_tile32<64, 4, 64, false>(mask, (uint32_t)workgroups, scheduled, stream);
       return launch_tile32<128, 4, 64, false>(mask, (uint32_t)workgroups, scheduled, stream);
     }
