@@ -162,6 +162,7 @@ def test_filters_reduce_to_the_best_tokens():
         assert sample(Params.create(temperature=1.0, top_k=50, top_p=1e-4, seed=seed), 900, data) in best
         # min_p = 1: only tokens as probable as the best one survive
         assert sample(Params.create(temperature=1.0, top_k=50, min_p=1.0, seed=seed), 900, data) in best
-    # seed 0 draws from the clock: any kept candidate
-    top40 = {token for token, _ in Float16Logits.top(40 + len(best), 900, data)}
-    assert sample(Params.create(temperature=1.0, top_k=40, seed=0), 900, data) in top40
+    # seed 0 draws from the clock: any kept candidate, i.e. a token at least as good as the 40th best
+    # (which of the tokens tied at that value are kept is the heap's business)
+    drawn = sample(Params.create(temperature=1.0, top_k=40, seed=0), 900, data)
+    assert values[drawn] >= np.sort(values.astype(np.float32))[-40]
