@@ -79,7 +79,8 @@ constexpr int kWavesPerBlock = 4;  // consecutive 32-row slabs of one head
 // instead of four times.
 // WAVES x 32 query rows per workgroup, STAGE_KEYS keys per LDS stage (launched as 4 x 64: 64 KB at
 // D = 128, two workgroups per CU).
-// MASK: 0 no mask, 1 a mask of bytes, 2 of halves (every score is then tested; without one the instantiation carries
+// MASK: 0 no mask, 1 a mask of bytes, 2 of halves, 3 the mask as one bit per (row, key), which the pass over the
+// mask ahead of this kernel leaves (every score is then tested; without one the instantiation carries
 // nothing of it).
 // KEYSPLIT: the four waves of a workgroup share ONE slab of 32 query rows and take a quarter of every
 // 128-key stage each; their partial results meet in LDS at the end.  For launches with fewer
@@ -178,16 +179,19 @@ __global__ __launch_bounds__(WAVES * 64 * (PAIR ? 2 : 1))
   // element; a tile whose 32 x 32 mask values allow nothing is skipped whole.
   constexpr int TILES = KEYSPLIT ? 1 : STAGE_KEYS / 32;  // tiles of a stage this wave works on
   struct MaskRaw {
-    uint32_t w[MASK == 2 ? 8 : MASK == 1 ? 4 : 1];
+    uint32_t w[MASK == 2 ? 8 : MASK == 1 ? 4 : 1];  // (bits: the 32 keys of the lane's row in one dword)
   };
-  [[maybe_unused]] const size_t mask_row =
-      masked ? (((size_t)(a.mask_batches == 1 ? 0 : batch) * a.mask_heads + (a.mask_heads == 1 ? 0 : head)) *
-                    a.query_length + min(q0 + row_lane, a.query_length - 1)) * L
+  [[maybe_unused]] const size_t mask_row_index =
+      masked ? ((size_t)(a.mask_batches == 1 ? 0 : batch) * a.mask_heads + (a.mask_heads == 1 ? 0 : head)) *
+                       a.query_length + min(q0 + row_lane, a.query_length - 1)
              : 0;
+  [[maybe_unused]] const size_t mask_row = mask_row_index * L;
   [[maybe_unused]] const bool mask_runs =
       masked && L % 4 == 0 && L >= 4 && reinterpret_cast<uintptr_t>(a.mask) % 8 == 0;  // the same for every lane
   [[maybe_unused]] auto mask_request = [&](uint32_t key0, MaskRaw &raw) __attribute__((always_inline)) {
-    if constexpr (MASK == 2) {
+    if constexpr (MASK == 3) {
+      raw.w[0] = a.mask_bits[mask_row_index * a.mask_words_per_row + (min(key0, L - 1) >> 5)];
+    } else if constexpr (MASK == 2) {
       {
         const uint16_t *row = reinterpret_cast<const uint16_t *>(a.mask) + mask_row;
 #pragma unroll
@@ -223,14 +227,35 @@ __global__ __launch_bounds__(WAVES * 64 * (PAIR ? 2 : 1))
   [[maybe_unused]] auto mask_bits = [&](const MaskRaw &raw) __attribute__((always_inline)) {
     uint32_t bits = 0;
     if constexpr (MASKED) {
+      // Most tiles of the masks a prefill builds are allowed as a whole, and their values are all +0.0
+      // (halves) or all 1 (bytes): one OR / AND over the lane's words and a vote say so, and only the
+      // tiles the mask's edge runs through pay for the value-by-value conversion.
+      if constexpr (MASK == 3) {
+        // bit k of the dword is key key0 + k of this lane's row; score r is key (r / 4) * 8 + half * 4 + r % 4
+        if (__builtin_amdgcn_ballot_w64(raw.w[0] != 0xffffffffu) == 0) return 0xffffu;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        bool allowed;
-        if constexpr (MASK == 2)
-          allowed = half_bits_to_float((uint16_t)(raw.w[2 * (r >> 2) + ((r & 3) >> 1)] >> (16 * (r & 1)))) >= 0.0f;
-        else
-          allowed = ((raw.w[r >> 2] >> (8 * (r & 3))) & 0xffu) != 0;
-        bits |= allowed ? (1u << r) : 0u;
+        for (int g = 0; g < 4; ++g) bits |= ((raw.w[0] >> (8 * g + 4 * half)) & 0xfu) << (4 * g);
+        return bits;
+      } else {
+        bool plain;
+        if constexpr (MASK == 2) {
+          uint32_t any = 0;
+#pragma unroll
+          for (int i = 0; i < 8; ++i) any |= raw.w[i];
+          plain = any == 0;
+        } else {
+          plain = raw.w[0] == 0x01010101u && raw.w[1] == 0x01010101u && raw.w[2] == 0x01010101u && raw.w[3] == 0x01010101u;
+        }
+        if (__builtin_amdgcn_ballot_w64(!plain) == 0) return 0xffffu;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          bool allowed;
+          if constexpr (MASK == 2)
+            allowed = half_bits_to_float((uint16_t)(raw.w[2 * (r >> 2) + ((r & 3) >> 1)] >> (16 * (r & 1)))) >= 0.0f;
+          else
+            allowed = ((raw.w[r >> 2] >> (8 * (r & 3))) & 0xffu) != 0;
+          bits |= allowed ? (1u << r) : 0u;
+        }
       }
     }
     return bits;
@@ -591,77 +616,71 @@ __global__ __launch_bounds__(WAVES * 64 * (PAIR ? 2 : 1))
     }
 }
 
-// ---- which stages of keys a mask leaves to a slab of query rows ------------------------------
+// ---- the pass over a mask ahead of the attention kernel ---------------------------------------
 //
-// One workgroup of 1024 threads per (eight stages of keys, slab of query rows, mask row group): a thread
-// ORs one run of four consecutive keys down its share of the slab's rows (sixteen or eight), the lanes of a stage vote, and
-// the workgroup stores the eight answers as one byte of the map the attention kernel reads.
-// rows_per_slab x stage_keys is the attention launch's geometry: 128 x 64, or 32 x 128 when the
-// keys of a slab are split over the waves.
-__global__ __launch_bounds__(1024) void mask_stage_map_kernel(DenseAttentionArgs a, uint32_t rows_per_slab,
-                                                              uint32_t stage_keys, uint32_t map_stride) {
+// Leaves (1) the mask as one bit per (mask row, key), words_per_row dwords a row - what the attention
+// kernel reads instead of the bytes or halves: one dword per lane and tile of 32 keys - and (2) one bit
+// per (mask row group, slab of query rows, stage of keys) that says whether the mask allows anything
+// there.  One workgroup per (eight stages, slab, mask row group) = one byte of that map; a thread takes
+// 64 consecutive keys of one row (every request out before the first value is looked at).
+// rows_per_slab x stage_keys is the attention launch's geometry: 128 x 64, or 32 x 128 when the keys
+// of a slab are split over the waves; the workgroup has rows_per_slab * stage_keys / 8 threads.
+__global__ __launch_bounds__(1024) void mask_bits_kernel(DenseAttentionArgs a, uint32_t rows_per_slab, uint32_t stage_keys,
+                                                         uint32_t map_stride, uint32_t *bits_out, uint32_t words_per_row) {
   __shared__ uint32_t chunk_bits;
   const uint32_t chunk = blockIdx.x, slab = blockIdx.y, group = blockIdx.z;
   const uint32_t L = a.key_length;
-  const uint32_t runs = 2 * stage_keys;                   // runs of four keys in eight stages: 128 or 256
-  const uint32_t row_groups = 1024 / runs;                // 8 or 4
-  const uint32_t rows_each = rows_per_slab / row_groups;  // 16 or 8
-  const uint32_t run = threadIdx.x % runs, row_group = threadIdx.x / runs;
-  const uint32_t key = chunk * 8 * stage_keys + run * 4;
-  const uint32_t row0 = slab * rows_per_slab + row_group * rows_each;
-  const bool whole_runs = L % 4 == 0 && L >= 4 && reinterpret_cast<uintptr_t>(a.mask) % 8 == 0;
-  const size_t group_base = (size_t)group * a.query_length * L;
+  const uint32_t units = stage_keys / 8;  // 64-key units in eight stages: 8 or 16
+  const uint32_t unit = threadIdx.x % units, row = slab * rows_per_slab + threadIdx.x / units;
+  const uint32_t key = chunk * 8 * stage_keys + unit * 64;
   if (threadIdx.x == 0) chunk_bits = 0;
-  // every request goes out before the first value is looked at (rows past the end repeat the last one,
-  // a run past the end the last whole run: what they say is dropped below)
-  constexpr int kRows = 16;
-  uint32_t any = 0;
-  const uint32_t last_row = a.query_length - 1;
-  if (whole_runs) {
-    const uint32_t at_key = min(key, L - 4);
+  uint32_t word[2] = {0, 0};  // keys key .. key + 31, key + 32 .. key + 63
+  const bool inside = row < a.query_length && key < L;
+  if (inside) {
+    const size_t first = ((size_t)group * a.query_length + row) * L + key;
+    const bool whole = key + 64 <= L && reinterpret_cast<uintptr_t>(a.mask) % 16 == 0;
     if (a.mask_dtype == 2) {
-      const uint16_t *mask = reinterpret_cast<const uint16_t *>(a.mask) + group_base + at_key;
-      uint2 four[kRows];
+      const uint16_t *values = reinterpret_cast<const uint16_t *>(a.mask) + first;
+      if (whole && L % 8 == 0) {
+        uint4 piece[8];
 #pragma unroll
-      for (int r = 0; r < kRows; ++r) four[r] = *reinterpret_cast<const uint2 *>(mask + (size_t)min(row0 + r, last_row) * L);
+        for (int i = 0; i < 8; ++i) piece[i] = reinterpret_cast<const uint4 *>(values)[i];
 #pragma unroll
-      for (int r = 0; r < kRows; ++r) {
-        const bool counts = (uint32_t)r < rows_each && row0 + r <= last_row;
-        const bool allowed = half_bits_to_float((uint16_t)four[r].x) >= 0.0f || half_bits_to_float((uint16_t)(four[r].x >> 16)) >= 0.0f ||
-                             half_bits_to_float((uint16_t)four[r].y) >= 0.0f || half_bits_to_float((uint16_t)(four[r].y >> 16)) >= 0.0f;
-        any |= counts && allowed ? 1u : 0u;
+        for (int i = 0; i < 8; ++i) {
+          const uint32_t four[4] = {piece[i].x, piece[i].y, piece[i].z, piece[i].w};
+#pragma unroll
+          for (int e = 0; e < 8; ++e) {
+            const bool allowed = half_bits_to_float((uint16_t)(four[e >> 1] >> (16 * (e & 1)))) >= 0.0f;
+            word[i >> 2] |= allowed ? 1u << ((i & 3) * 8 + e) : 0u;
+          }
+        }
+      } else {
+        for (uint32_t e = 0; e < 64 && key + e < L; ++e)
+          word[e >> 5] |= half_bits_to_float(values[e]) >= 0.0f ? 1u << (e & 31) : 0u;
       }
     } else {
-      const uint8_t *mask = a.mask + group_base + at_key;
-      uint32_t four[kRows];
+      const uint8_t *values = a.mask + first;
+      if (whole && L % 16 == 0) {
+        uint4 piece[4];
 #pragma unroll
-      for (int r = 0; r < kRows; ++r) four[r] = *reinterpret_cast<const uint32_t *>(mask + (size_t)min(row0 + r, last_row) * L);
+        for (int i = 0; i < 4; ++i) piece[i] = reinterpret_cast<const uint4 *>(values)[i];
 #pragma unroll
-      for (int r = 0; r < kRows; ++r) any |= ((uint32_t)r < rows_each && row0 + r <= last_row && four[r] != 0) ? 1u : 0u;
-    }
-    if (key >= L) any = 0;
-  } else {
-    // rows of the mask that are not whole runs: element by element
-    for (uint32_t r = 0; r < rows_each && row0 + r <= last_row; ++r)
-      for (uint32_t e = 0; e < 4 && key + e < L; ++e) {
-        const size_t at = group_base + (size_t)(row0 + r) * L + key + e;
-        const bool allowed = a.mask_dtype == 2 ? half_bits_to_float(reinterpret_cast<const uint16_t *>(a.mask)[at]) >= 0.0f
-                                               : a.mask[at] != 0;
-        any |= allowed ? 1u : 0u;
+        for (int i = 0; i < 4; ++i) {
+          const uint32_t four[4] = {piece[i].x, piece[i].y, piece[i].z, piece[i].w};
+#pragma unroll
+          for (int e = 0; e < 16; ++e)
+            word[i >> 1] |= ((four[e >> 2] >> (8 * (e & 3))) & 0xffu) != 0 ? 1u << ((i & 1) * 16 + e) : 0u;
+        }
+      } else {
+        for (uint32_t e = 0; e < 64 && key + e < L; ++e) word[e >> 5] |= values[e] != 0 ? 1u << (e & 31) : 0u;
       }
+    }
+    uint32_t *out = bits_out + ((size_t)group * a.query_length + row) * words_per_row + (key >> 5);
+    out[0] = word[0];
+    out[1] = word[1];
   }
   __syncthreads();
-  // the lanes of one stage are stage_keys / 4 neighbours (16 or 32) of one wave
-  const uint64_t votes = __builtin_amdgcn_ballot_w64(any != 0);
-  if ((threadIdx.x & 63) == 0) {
-    const uint32_t lanes_per_stage = stage_keys / 4, stages_per_wave = 64 / lanes_per_stage;
-    const uint32_t first_stage = run / lanes_per_stage;
-    const uint64_t lanes = lanes_per_stage == 32 ? 0xffffffffull : 0xffffull;
-    uint32_t bits = 0;
-    for (uint32_t j = 0; j < stages_per_wave; ++j)
-      if ((votes >> (j * lanes_per_stage)) & lanes) bits |= 1u << (first_stage + j);
-    if (bits != 0) atomicOr(&chunk_bits, bits);
-  }
+  if ((word[0] | word[1]) != 0) atomicOr(&chunk_bits, 1u << (unit * 64 / stage_keys));
   __syncthreads();
   if (threadIdx.x == 0) a.stage_map[((size_t)group * gridDim.y + slab) * map_stride + chunk] = (uint8_t)chunk_bits;
 }
@@ -753,9 +772,10 @@ hipError_t launch_tile32_instance(uint32_t grid, const DenseAttentionArgs &a, hi
   return hipGetLastError();
 }
 
-// mask: 0 none, 1 bytes, 2 halves
+// mask: 0 none, 1 bytes, 2 halves, 3 bits
 template <int D, int WAVES, int STAGE_KEYS, bool KEYSPLIT, bool PAIR = false>
 hipError_t launch_tile32(int mask, uint32_t grid, const DenseAttentionArgs &a, hipStream_t stream) {
+  if (mask == 3) return launch_tile32_instance<D, WAVES, STAGE_KEYS, 3, KEYSPLIT, PAIR>(grid, a, stream);
   if (mask == 2) return launch_tile32_instance<D, WAVES, STAGE_KEYS, 2, KEYSPLIT, PAIR>(grid, a, stream);
   if (mask == 1) return launch_tile32_instance<D, WAVES, STAGE_KEYS, 1, KEYSPLIT, PAIR>(grid, a, stream);
   return launch_tile32_instance<D, WAVES, STAGE_KEYS, 0, KEYSPLIT, PAIR>(grid, a, stream);
@@ -795,6 +815,13 @@ uint32_t stage_map_stride(const DenseAttentionArgs &a, const Tile32Geometry &g) 
   return ((a.key_length + g.stage_keys - 1) / g.stage_keys + 7) / 8;
 }
 
+// the map comes first in the scratch memory, rounded up so that the bit words behind it are aligned
+size_t stage_map_region(const DenseAttentionArgs &a, const Tile32Geometry &g) {
+  return ((size_t)a.mask_batches * a.mask_heads * g.slabs * stage_map_stride(a, g) + 255) & ~(size_t)255;
+}
+
+uint32_t mask_words_per_row(const DenseAttentionArgs &a) { return 2 * ((a.key_length + 63) / 64); }
+
 }  // namespace
 
 size_t dense_attention_workspace_bytes(const DenseAttentionArgs &a) {
@@ -804,7 +831,7 @@ size_t dense_attention_workspace_bytes(const DenseAttentionArgs &a) {
   // a few stages only: walking them all (their arithmetic is skipped where the mask forbids it) costs
   // less than another launch ahead of the attention kernel
   if ((a.key_length + g.stage_keys - 1) / g.stage_keys <= 4) return 0;
-  return (size_t)a.mask_batches * a.mask_heads * g.slabs * stage_map_stride(a, g);
+  return stage_map_region(a, g) + (size_t)a.mask_batches * a.mask_heads * a.query_length * mask_words_per_row(a) * 4;
 }
 
 hipError_t launch_dense_attention(const DenseAttentionArgs &a, hipStream_t stream) {
@@ -818,43 +845,48 @@ hipError_t launch_dense_attention(const DenseAttentionArgs &a, hipStream_t strea
       const int mask = dense_masked(a) ? (a.mask_dtype == 2 ? 2 : 1) : 0;
       DenseAttentionArgs scheduled = a;
       scheduled.cus_per_xcd = (uint32_t)device_compute_units() / 8;
-      // the pass over the mask that says which stages of keys each slab of rows has to walk
+      // the pass over the mask: which stages of keys each slab of rows has to walk, and the mask as bits
+      int mask_kind = mask;
       if (mask != 0 && a.stage_map != nullptr) {
         const uint32_t stride = stage_map_stride(a, geometry);
         const uint64_t groups = (uint64_t)a.mask_batches * a.mask_heads;
-        if (a.stage_map_bytes < groups * geometry.slabs * stride || geometry.slabs > 65535 || groups > 65535)
+        const size_t map_region = stage_map_region(a, geometry);
+        const size_t wanted = map_region + (size_t)groups * a.query_length * mask_words_per_row(a) * 4;
+        if (a.stage_map_bytes < wanted || geometry.slabs > 65535 || groups > 65535 ||
+            (reinterpret_cast<uintptr_t>(a.stage_map) & 3) != 0) {
           scheduled.stage_map = nullptr;
-        else
-          hipLaunchKernelGGL(mask_stage_map_kernel, dim3(stride, geometry.slabs, (uint32_t)groups), dim3(1024), 0, stream, a,
-                             geometry.rows_per_slab, geometry.stage_keys, stride);
+        } else {
+          uint32_t *bits = reinterpret_cast<uint32_t *>(a.stage_map + map_region);
+          hipLaunchKernelGGL(mask_bits_kernel, dim3(stride, geometry.slabs, (uint32_t)groups),
+                             dim3(geometry.rows_per_slab * geometry.stage_keys / 8), 0, stream, a, geometry.rows_per_slab,
+                             geometry.stage_keys, stride, bits, mask_words_per_row(a));
+          scheduled.mask_bits = bits;
+          scheduled.mask_words_per_row = mask_words_per_row(a);
+          mask_kind = 3;
+        }
       }
-      // Fewer workgroups of 128 rows than CUs: the launch lasts as long as one wave's walk over the
-      // keys of its slab, so the waves of a workgroup share 32 rows and a quarter of the keys each
-      // (four times the workgroups, a quarter of the walk): 9 heads x 2048 tokens of 64, causal,
-      // 45.0 -> 22.9 us.  Larger launches keep 128 rows a workgroup: a stage of K and V then serves
-      // four times as many rows.
       if (geometry.key_split) {
         const uint32_t grid = (uint32_t)((a.query_length + 31) / 32) * a.heads * a.batches;
-        if (a.head_dim == 64) return launch_tile32<64, 4, 128, true>(mask, grid, scheduled, stream);
-        return launch_tile32<128, 4, 128, true>(mask, grid, scheduled, stream);
+        if (a.head_dim == 64) return launch_tile32<64, 4, 128, true>(mask_kind, grid, scheduled, stream);
+        return launch_tile32<128, 4, 128, true>(mask_kind, grid, scheduled, stream);
       }
       // 32 x 32 wave tiles over shared LDS stages, four waves and 64 keys a stage.  (Workgroups of two
       // waves with 32-key stages, twice as many and four per CU, so that short causal launches are not
       // as long as their longest workgroup, measured slower: 105.6 against 91.2 us at 32 heads x 2048
       // tokens - one tile per barrier, half the sharing.)  Heads of 256: 128 KB of stages, one
       // workgroup per CU with all of its registers.
-      if (a.head_dim == 256) return launch_tile32<256, 4, 64, false>(mask, (uint32_t)workgroups, scheduled, stream);
+      if (a.head_dim == 256) return launch_tile32<256, 4, 64, false>(mask_kind, (uint32_t)workgroups, scheduled, stream);
       // One or two workgroups per CU: two groups of four waves per slab, each with half of the stages (a
       // CU then holds one workgroup at a time, at the same two waves per SIMD): 32 heads x 2048 tokens,
       // 512 workgroups, 72.9 -> 67.6 us.  The groups meet at every stage's barrier, so two of them get
       // less out of a CU than two workgroups of four waves that run side by side freely - launches with
       // enough of those keep them.
       if (workgroups <= 2 * (uint64_t)device_compute_units() && a.key_length >= 256) {
-        if (a.head_dim == 64) return launch_tile32<64, 4, 64, false, true>(mask, (uint32_t)workgroups, scheduled, stream);
-        return launch_tile32<128, 4, 64, false, true>(mask, (uint32_t)workgroups, scheduled, stream);
+        if (a.head_dim == 64) return launch_tile32<64, 4, 64, false, true>(mask_kind, (uint32_t)workgroups, scheduled, stream);
+        return launch_tile32<128, 4, 64, false, true>(mask_kind, (uint32_t)workgroups, scheduled, stream);
       }
-      if (a.head_dim == 64) return launch_tile32<64, 4, 64, false>(mask, (uint32_t)workgroups, scheduled, stream);
-      return launch_tile32<128, 4, 64, false>(mask, (uint32_t)workgroups, scheduled, stream);
+      if (a.head_dim == 64) return launch_tile32<64, 4, 64, false>(mask_kind, (uint32_t)workgroups, scheduled, stream);
+      return launch_tile32<128, 4, 64, false>(mask_kind, (uint32_t)workgroups, scheduled, stream);
     }
   }
   const uint64_t blocks = (rows + 3) / 4;

@@ -179,6 +179,10 @@ struct DenseAttentionArgs {
   // anything there, written by a pass over the mask ahead of the attention kernel.
   uint8_t *stage_map = nullptr;
   size_t stage_map_bytes = 0;
+  // Set by the launcher: the same pass also leaves the mask as one bit per (mask row, key) behind the
+  // map, mask_words_per_row dwords a row, which is what the attention kernel then reads.
+  const uint32_t *mask_bits = nullptr;
+  uint32_t mask_words_per_row = 0;
 };
 size_t dense_attention_workspace_bytes(const DenseAttentionArgs &args);
 hipError_t launch_dense_attention(const DenseAttentionArgs &args, hipStream_t stream);
