@@ -372,3 +372,34 @@ def test_masks_that_forbid_whole_stages(runtime, dim, heads, kv_heads, batches, 
               (batches, heads, tokens, dim))
     want = expected(query, key, value, allowed, scale)
     assert_close_to_oracle(got, want, f"mask of whole stages D={dim} {heads}/{kv_heads} x {tokens} after {past}, window {window}")
+
+
+@pytest.mark.parametrize("dim,heads,kv_heads,batches,tokens,mask_dtype", [
+    (128, 16, 4, 3, 700, 1),   # 288 workgroups: two groups of four waves per slab
+    (64, 24, 8, 4, 680, 2),    # 576 workgroups: four waves per slab
+    (64, 4, 2, 2, 1100, 1),    # 32-row slabs with the keys split over the waves
+])
+def test_masks_of_every_batch_and_head(runtime, dim, heads, kv_heads, batches, tokens, mask_dtype):
+    """A mask of its own for every (batch, head): causal with a sliding window whose width depends on
+    the head and a band of forbidden keys that depends on the batch - so the stages a slab has to
+    walk differ from one mask row group to the next."""
+    rng = np.random.default_rng(dim + heads + tokens)
+    query = rng.standard_normal((batches, heads, tokens, dim)).astype(np.float16)
+    key = rng.standard_normal((batches, kv_heads, tokens, dim)).astype(np.float16)
+    value = rng.standard_normal((batches, kv_heads, tokens, dim)).astype(np.float16)
+    scale = 1.0 / math.sqrt(dim)
+    rows = np.arange(tokens)[:, None]
+    keys = np.arange(tokens)[None, :]
+    allowed = np.empty((batches, heads, tokens, tokens), dtype=bool)
+    for b in range(batches):
+        for h in range(heads):
+            visible = (keys <= rows) & (keys > rows - (90 + 37 * h))
+            visible &= ~((keys >= 100 + 64 * b) & (keys < 230 + 64 * b))
+            allowed[b, h] = visible
+    mask = np.where(allowed, 0.0, -np.inf).astype(np.float16) if mask_dtype == 2 else allowed.astype(np.uint8)
+    params = attention_params(batches, heads, tokens, tokens, dim, batches, heads, False, scale, kv_heads,
+                              mask_dtype=mask_dtype)
+    got = run(runtime, f"llmopt_attention_f16_simd_h{dim}", query, key, value, mask, params,
+              (batches, heads, tokens, dim))
+    want = expected(query, key, value, allowed, scale)
+    assert_close_to_oracle(got, want, f"per-head masks D={dim} {heads}/{kv_heads} x {tokens}")
