@@ -322,7 +322,7 @@ __global__ __launch_bounds__(WAVES * 64 * (PAIR ? 2 : 1))
     return stage * STAGE_KEYS + (KEYSPLIT ? wave * 32 : (uint32_t)t * 32);
   };
   // With a mask, the stages of keys that have anything for this slab of rows come from a map a pass
-  // over the mask left (one bit per mask row group, slab and stage): wave 0 turns the slab's bits
+  // over the mask left (one byte per mask row group, slab and stage): wave 0 turns the slab's bytes
   // into the list of its live stages, and the loop below walks that list - a stage the mask forbids
   // costs nothing.  Without a map (no scratch given, or more stages than the list holds) every stage
   // is walked and only its arithmetic is skipped.
@@ -334,14 +334,14 @@ __global__ __launch_bounds__(WAVES * 64 * (PAIR ? 2 : 1))
   if constexpr (MASKED) {
     listed = a.stage_map != nullptr && stages <= kMaxLive;
     if (listed) {
-      const uint32_t total_stages = (L + STAGE_KEYS - 1) / STAGE_KEYS, map_stride = (total_stages + 7) / 8;
+      const uint32_t map_stride = (L + STAGE_KEYS - 1) / STAGE_KEYS;  // a byte per stage
       const uint32_t mask_group = (a.mask_batches == 1 ? 0 : batch) * a.mask_heads + (a.mask_heads == 1 ? 0 : head);
       const uint8_t *map = a.stage_map + ((size_t)mask_group * slabs + slab) * map_stride;
       if (wave_of_all == 0) {
         uint32_t count = 0;
         for (uint32_t base = 0; base < stages; base += 64) {
           const uint32_t stage = base + lane;
-          const bool live = stage < stages && ((map[min(stage, stages - 1) >> 3] >> (stage & 7)) & 1u) != 0;
+          const bool live = stage < stages && map[min(stage, stages - 1)] != 0;
           const uint64_t votes = __builtin_amdgcn_ballot_w64(live);
           if (live) live_list[count + __builtin_popcountll(votes & ((1ull << lane) - 1))] = (uint16_t)stage;
           count += (uint32_t)__builtin_popcountll(votes);
@@ -619,20 +619,21 @@ __global__ __launch_bounds__(WAVES * 64 * (PAIR ? 2 : 1))
 // ---- the pass over a mask ahead of the attention kernel ---------------------------------------
 //
 // Leaves (1) the mask as one bit per (mask row, key), words_per_row dwords a row - what the attention
-// kernel reads instead of the bytes or halves: one dword per lane and tile of 32 keys - and (2) one bit
+// kernel reads instead of the bytes or halves: one dword per lane and tile of 32 keys - and (2) one byte
 // per (mask row group, slab of query rows, stage of keys) that says whether the mask allows anything
-// there.  One workgroup per (eight stages, slab, mask row group) = one byte of that map; a thread takes
-// 64 consecutive keys of one row (every request out before the first value is looked at).
+// there.  One workgroup per (two stages, slab, mask row group); a thread takes 64 consecutive keys of
+// one row (every request out before the first value is looked at).  (One workgroup per eight stages and
+// a bit per stage left three quarters of the CUs without work: 9.8 us for 2048 x 2048 halves.)
 // rows_per_slab x stage_keys is the attention launch's geometry: 128 x 64, or 32 x 128 when the keys
-// of a slab are split over the waves; the workgroup has rows_per_slab * stage_keys / 8 threads.
-__global__ __launch_bounds__(1024) void mask_bits_kernel(DenseAttentionArgs a, uint32_t rows_per_slab, uint32_t stage_keys,
+// of a slab are split over the waves; the workgroup has rows_per_slab * stage_keys / 32 threads.
+__global__ __launch_bounds__(256) void mask_bits_kernel(DenseAttentionArgs a, uint32_t rows_per_slab, uint32_t stage_keys,
                                                          uint32_t map_stride, uint32_t *bits_out, uint32_t words_per_row) {
   __shared__ uint32_t chunk_bits;
   const uint32_t chunk = blockIdx.x, slab = blockIdx.y, group = blockIdx.z;
   const uint32_t L = a.key_length;
-  const uint32_t units = stage_keys / 8;  // 64-key units in eight stages: 8 or 16
+  const uint32_t units = stage_keys / 32;  // 64-key units in two stages: 2 or 4
   const uint32_t unit = threadIdx.x % units, row = slab * rows_per_slab + threadIdx.x / units;
-  const uint32_t key = chunk * 8 * stage_keys + unit * 64;
+  const uint32_t key = chunk * 2 * stage_keys + unit * 64;
   if (threadIdx.x == 0) chunk_bits = 0;
   uint32_t word[2] = {0, 0};  // keys key .. key + 31, key + 32 .. key + 63
   const bool inside = row < a.query_length && key < L;
@@ -682,7 +683,9 @@ __global__ __launch_bounds__(1024) void mask_bits_kernel(DenseAttentionArgs a, u
   __syncthreads();
   if ((word[0] | word[1]) != 0) atomicOr(&chunk_bits, 1u << (unit * 64 / stage_keys));
   __syncthreads();
-  if (threadIdx.x == 0) a.stage_map[((size_t)group * gridDim.y + slab) * map_stride + chunk] = (uint8_t)chunk_bits;
+  if (threadIdx.x < 2 && chunk * 2 + threadIdx.x < map_stride)
+    a.stage_map[((size_t)group * gridDim.y + slab) * map_stride + chunk * 2 + threadIdx.x] =
+        (uint8_t)((chunk_bits >> threadIdx.x) & 1u);
 }
 
 // ---- row-serial kernel (every other configuration) ---------------------------
@@ -811,8 +814,9 @@ Tile32Geometry tile32_geometry(const DenseAttentionArgs &a) {
 
 bool dense_masked(const DenseAttentionArgs &a) { return a.mask != nullptr && a.mask_batches > 0; }
 
+// bytes of the stage map per (mask row group, slab): one per stage of keys
 uint32_t stage_map_stride(const DenseAttentionArgs &a, const Tile32Geometry &g) {
-  return ((a.key_length + g.stage_keys - 1) / g.stage_keys + 7) / 8;
+  return (a.key_length + g.stage_keys - 1) / g.stage_keys;
 }
 
 // the map comes first in the scratch memory, rounded up so that the bit words behind it are aligned
@@ -857,8 +861,8 @@ hipError_t launch_dense_attention(const DenseAttentionArgs &a, hipStream_t strea
           scheduled.stage_map = nullptr;
         } else {
           uint32_t *bits = reinterpret_cast<uint32_t *>(a.stage_map + map_region);
-          hipLaunchKernelGGL(mask_bits_kernel, dim3(stride, geometry.slabs, (uint32_t)groups),
-                             dim3(geometry.rows_per_slab * geometry.stage_keys / 8), 0, stream, a, geometry.rows_per_slab,
+          hipLaunchKernelGGL(mask_bits_kernel, dim3((stride + 1) / 2, geometry.slabs, (uint32_t)groups),
+                             dim3(geometry.rows_per_slab * geometry.stage_keys / 32), 0, stream, a, geometry.rows_per_slab,
                              geometry.stage_keys, stride, bits, mask_words_per_row(a));
           scheduled.mask_bits = bits;
           scheduled.mask_words_per_row = mask_words_per_row(a);

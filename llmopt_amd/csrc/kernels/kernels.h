@@ -174,7 +174,7 @@ struct DenseAttentionArgs {
   float scale;
   uint32_t kv_heads, token_first_output, past_length, token_first_value, mask_dtype;
   uint32_t cus_per_xcd = 0;  // set by the launcher (workgroup order of the causal launch)
-  // Scratch for masked launches (may be null: every stage of keys is then walked): one bit per
+  // Scratch for masked launches (may be null: every stage of keys is then walked): one byte per
   // (mask batch, mask head, slab of query rows, stage of keys) that says whether the mask allows
   // anything there, written by a pass over the mask ahead of the attention kernel.
   uint8_t *stage_map = nullptr;
