@@ -403,3 +403,47 @@ def test_masks_of_every_batch_and_head(runtime, dim, heads, kv_heads, batches, t
               (batches, heads, tokens, dim))
     want = expected(query, key, value, allowed, scale)
     assert_close_to_oracle(got, want, f"per-head masks D={dim} {heads}/{kv_heads} x {tokens}")
+
+
+@pytest.mark.parametrize("case", range(10))
+def test_random_block_masks(runtime, case):
+    """Masks made of random rectangles of allowed keys (so that whole stages, whole tiles, single rows
+    and single keys are forbidden in no particular pattern), random geometry: every slab layout, both
+    mask types, masks shared or per batch / head, rows of the mask that are and are not whole runs."""
+    rng = np.random.default_rng(9000 + case)
+    dim = int(rng.choice([64, 128, 256]))
+    kv_heads = int(rng.integers(1, 4))
+    heads = kv_heads * int(rng.integers(1, 4))
+    batches = int(rng.integers(1, 3))
+    new = int(rng.integers(16, 700))
+    past = int(rng.integers(0, 900))
+    if case % 3 == 0:  # enough workgroups of 128 rows for the four- and eight-wave slabs
+        heads, kv_heads, batches, new = 16 * int(rng.integers(1, 3)), 8, int(rng.integers(2, 4)), int(rng.integers(500, 800))
+        dim = int(rng.choice([64, 128]))
+    length = past + new
+    if case % 2 == 0:
+        length = (length + 7) // 8 * 8
+        past = length - new
+    query = rng.standard_normal((batches, heads, new, dim)).astype(np.float16)
+    key = rng.standard_normal((batches, kv_heads, length, dim)).astype(np.float16)
+    value = rng.standard_normal((batches, kv_heads, length, dim)).astype(np.float16)
+    mask_batches = batches if rng.random() < 0.5 else 1
+    mask_heads = heads if rng.random() < 0.5 else 1
+    allowed = np.zeros((mask_batches, mask_heads, new, length), dtype=bool)
+    for b in range(mask_batches):
+        for h in range(mask_heads):
+            for _ in range(int(rng.integers(1, 6))):
+                r0, k0 = int(rng.integers(0, new)), int(rng.integers(0, length))
+                r1 = min(new, r0 + int(rng.integers(1, new + 1)))
+                k1 = min(length, k0 + int(rng.integers(1, length + 1)))
+                allowed[b, h, r0:r1, k0:k1] = True
+    allowed[:, :, new // 2, :] = False
+    mask_dtype = 1 + case % 2
+    mask = allowed.astype(np.uint8) if mask_dtype == 1 else np.where(allowed, 0.0, -np.inf).astype(np.float16)
+    scale = 1.0 / math.sqrt(dim)
+    params = attention_params(batches, heads, new, length, dim, mask_batches, mask_heads, False, scale, kv_heads,
+                              mask_dtype=mask_dtype)
+    got = run(runtime, f"llmopt_attention_f16_simd_h{dim}", query, key, value, mask, params, (batches, heads, new, dim))
+    want = expected(query, key, value, np.broadcast_to(allowed, (batches, heads, new, length)), scale)
+    assert np.all(got[:, :, new // 2].view(np.uint16) == 0)
+    assert_close_to_oracle(got, want, f"random block mask {case}: D={dim} {heads}/{kv_heads} x{batches}, {new} after {past}")
