@@ -554,3 +554,38 @@ def test_suffix_prefill_over_cached_tokens(runtime, name, b, h, kvh, dim, past, 
     expected = oracle.paged_attention_q8(query, ck, cv, pool, slots, mask, params)
     assert np.all(out[:, 2].view(np.uint16) == 0)
     assert_close_to_oracle(out, expected, f"suffix prefill {name} {q_len} new after {past}")
+
+
+@pytest.mark.parametrize("case", range(8))
+def test_random_suffix_prefill(runtime, case):
+    """Random paged attention with sixteen query tokens or more: head sizes 64 / 128 / 256, any layer of a
+    pool of several layers, contexts from nothing to several hundred tokens, masks of either type, shared
+    or per head, with random holes."""
+    rng = np.random.default_rng(7000 + case)
+    dim = int(rng.choice([64, 128, 256]))
+    kvh = int(rng.integers(1, 4))
+    h = kvh * int(rng.integers(1, 5))
+    b = int(rng.integers(1, 3))
+    layers = int(rng.integers(1, 4))
+    layer = int(rng.integers(0, layers))
+    past = int(rng.integers(0, 800)) if case else 0
+    q_len = int(rng.integers(16, 200))
+    pool, slots, _, te, stride, ko, vo = build_pool(rng, kvh, dim, [max(past, 1)], layers=layers, layer=layer)
+    slots = slots[:past]
+    query = rng.standard_normal((b, h, q_len, dim)).astype(np.float16)
+    ck = rng.standard_normal((b, kvh, q_len, dim)).astype(np.float16)
+    cv = rng.standard_normal((b, kvh, q_len, dim)).astype(np.float16)
+    mask_heads = h if rng.random() < 0.5 else 1
+    visible = np.arange(past + q_len)[None, :] <= past + np.arange(q_len)[:, None]
+    visible = np.broadcast_to(visible, (b, mask_heads, q_len, past + q_len)).copy()
+    visible &= rng.random(visible.shape) > 0.1
+    mask_dtype = 1 + case % 2
+    mask = visible.astype(np.uint8) if mask_dtype == 1 else np.where(visible, 0.0, -np.inf).astype(np.float16)
+    params = PagedParams(batches=b, query_heads=h, kv_heads=kvh, past_length=past, head_dim=dim,
+                         mask_batches=b, mask_heads=mask_heads, token_elements=te, key_offset=ko, value_offset=vo,
+                         group_size=64, token_stride=stride, scale=1.0 / math.sqrt(dim), query_length=q_len,
+                         mask_dtype=mask_dtype, window=0)
+    out = run_paged(runtime, "llmopt_attention_q8_paged_simd_generic", query, ck, cv, pool, slots, mask, params)
+    expected = oracle.paged_attention_q8(query, ck, cv, pool, slots, mask, params)
+    assert_close_to_oracle(out, expected, f"random suffix prefill {case}: D={dim} {h}/{kvh} x{b}, {q_len} after {past}, "
+                                          f"layer {layer} of {layers}")
