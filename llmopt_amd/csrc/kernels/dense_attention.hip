@@ -639,13 +639,16 @@ __global__ __launch_bounds__(256) void mask_bits_kernel(DenseAttentionArgs a, ui
   const bool inside = row < a.query_length && key < L;
   if (inside) {
     const size_t first = ((size_t)group * a.query_length + row) * L + key;
-    const bool whole = key + 64 <= L && reinterpret_cast<uintptr_t>(a.mask) % 16 == 0;
+    // 16-byte requests at whatever alignment the row has (rows of a suffix's mask start anywhere);
+    // only a row's last, partial unit goes element by element
+    typedef uint32_t unaligned_u32x4_t __attribute__((ext_vector_type(4), aligned(1)));
+    const bool whole = key + 64 <= L;
     if (a.mask_dtype == 2) {
       const uint16_t *values = reinterpret_cast<const uint16_t *>(a.mask) + first;
-      if (whole && L % 8 == 0) {
-        uint4 piece[8];
+      if (whole) {
+        unaligned_u32x4_t piece[8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) piece[i] = reinterpret_cast<const uint4 *>(values)[i];
+        for (int i = 0; i < 8; ++i) piece[i] = reinterpret_cast<const unaligned_u32x4_t *>(values)[i];
 #pragma unroll
         for (int i = 0; i < 8; ++i) {
           const uint32_t four[4] = {piece[i].x, piece[i].y, piece[i].z, piece[i].w};
@@ -661,10 +664,10 @@ __global__ __launch_bounds__(256) void mask_bits_kernel(DenseAttentionArgs a, ui
       }
     } else {
       const uint8_t *values = a.mask + first;
-      if (whole && L % 16 == 0) {
-        uint4 piece[4];
+      if (whole) {
+        unaligned_u32x4_t piece[4];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) piece[i] = reinterpret_cast<const uint4 *>(values)[i];
+        for (int i = 0; i < 4; ++i) piece[i] = reinterpret_cast<const unaligned_u32x4_t *>(values)[i];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
           const uint32_t four[4] = {piece[i].x, piece[i].y, piece[i].z, piece[i].w};
@@ -796,7 +799,9 @@ Tile32Geometry tile32_geometry(const DenseAttentionArgs &a) {
   Tile32Geometry g = {false, false, 128, 64, 0, 0};
   const bool aligned = reinterpret_cast<uintptr_t>(a.query) % 16 == 0 && reinterpret_cast<uintptr_t>(a.key) % 16 == 0 &&
                        reinterpret_cast<uintptr_t>(a.value) % 8 == 0 && reinterpret_cast<uintptr_t>(a.output) % 8 == 0;
-  if (!((a.head_dim == 64 || a.head_dim == 128 || a.head_dim == 256) && aligned && a.query_length >= 16)) return g;
+  if (!((a.head_dim == 64 || a.head_dim == 128 || a.head_dim == 256) && aligned &&
+        (a.query_length >= 16 || (a.query_length >= 2 && a.key_length >= 256))))
+    return g;
   // K and V stages are copied as 16-byte pieces of whole rows (16-byte aligned K and V rows), and the
   // maxima are taken before scaling (a positive, finite scale); anything else takes the row kernel
   const size_t value_row_halfs = a.token_first_value ? (size_t)(a.kv_heads > 0 ? a.kv_heads : a.heads) * a.head_dim

@@ -529,6 +529,9 @@ def test_attention_int8_decoders_are_bit_exact(runtime, decoder, name):
     ("llmopt_attention_q8_paged_simd_h64", 1, 4, 4, 64, 1000, 200, 2),
     ("llmopt_attention_q8_paged_simd_h256", 1, 4, 2, 256, 130, 33, 1),
     ("llmopt_attention_q8_paged_simd_generic", 1, 32, 8, 128, 515, 140, 1),
+    # a few new tokens over a long context take the copy as well
+    ("llmopt_attention_q8_paged_simd_h64_gqa3", 1, 9, 3, 64, 700, 3, 1),
+    ("llmopt_attention_q8_paged_simd_generic", 2, 8, 4, 128, 300, 9, 2),
 ])
 def test_suffix_prefill_over_cached_tokens(runtime, name, b, h, kvh, dim, past, q_len, mask_dtype):
     """Sixteen query tokens or more over a Q8 context, with the mask the reference builds for a suffix
