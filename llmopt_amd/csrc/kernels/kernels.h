@@ -217,9 +217,10 @@ struct RotaryQkArgs {
 };
 hipError_t launch_rotary_qk(const RotaryQkArgs &args, hipStream_t stream);
 
-// The rotation of one token per sequence (tokens = 1) and, in the same launch, the Q8
-// quantisation of the rotated keys (pack.source[0] is rotary.k_output) and of the values
-// into their pool slots; pack.item_major is set.  Same arithmetic as the two launches.
+// The rotation (token-major in, head-major out; one token per sequence in a decode step, a
+// prompt's tokens in a prefill) and, in the same launch, the Q8 quantisation of the rotated keys
+// and of the values (pack.source[1], token-major) into the pool slot of every (sequence, token);
+// pack.item_major is set and pack.items = batches * tokens.  Same arithmetic as the separate launches.
 struct RotaryPackArgs {
   RotaryQkArgs rotary;
   Q8PackArgs pack;

@@ -57,9 +57,13 @@ __global__ __launch_bounds__(256) void q8_pack_kernel(Q8PackArgs a) {
 }
 
 // One wave per row of head_dim values, four rows per workgroup: the query rows of every
-// sequence (rotated), then the key rows (rotated, stored as fp16 for this step's attention and
-// as Q8 in the sequence's new pool slot), then the value rows (Q8 only).  A row is walked in
-// 64-wide pieces, which are the Q8 groups.
+// (sequence, token) (rotated), then the key rows (rotated, stored as fp16 for this step's attention
+// and as Q8 in the token's pool slot), then the value rows (Q8 only).  A row is walked in 64-wide
+// pieces, which are the Q8 groups.  Inputs are token-major [sequence, token, head, width], the
+// rotated outputs head-major [sequence, head, token, width] as llmopt_rotary_qk_f16_simd_h64
+// leaves them (lib/metal_normalization_source.ml:765-802); with one token per sequence - a decode
+// step - the two are the same.  Slot and, when the table is not shared, cosine / sine row of item
+// sequence * tokens + token.
 __global__ __launch_bounds__(256) void rotary_qk_pack_kernel(RotaryPackArgs a) {
   const RotaryQkArgs &r = a.rotary;
   const Q8PackArgs &p = a.pack;
@@ -69,22 +73,25 @@ __global__ __launch_bounds__(256) void rotary_qk_pack_kernel(RotaryPackArgs a) {
   // load - left to per-lane values they were vector loads from the argument block and the slot
   // table, each a trip to memory the row's own loads had to wait for
   const uint32_t row = blockIdx.x * 4 + __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  const uint32_t q_rows = r.batches * r.q_heads, kv_rows = r.batches * r.k_heads;
+  const uint32_t items = r.batches * r.tokens;
+  const uint32_t q_rows = items * r.q_heads, kv_rows = items * r.k_heads;
   if (row >= q_rows + 2 * kv_rows) return;
   const bool is_q = row < q_rows;
   const bool is_v = row >= q_rows + kv_rows;
-  const uint32_t local_row = is_q ? row : is_v ? row - q_rows - kv_rows : row - q_rows;  // [sequence, head]
+  const uint32_t local_row = is_q ? row : is_v ? row - q_rows - kv_rows : row - q_rows;  // [sequence, token, head]
   const uint32_t heads = is_q ? r.q_heads : r.k_heads;
-  const uint32_t batch = local_row / heads;
-  const uint32_t head = local_row - batch * heads;
+  const uint32_t item = local_row / heads;
+  const uint32_t head = local_row - item * heads;
+  const uint32_t batch = item / r.tokens, token = item - batch * r.tokens;
   const size_t base = (size_t)local_row * r.width;
   const _Float16 *input = reinterpret_cast<const _Float16 *>(is_q ? r.q_input : is_v ? p.source[1] : r.k_input) + base;
-  _Float16 *output = reinterpret_cast<_Float16 *>(is_q ? r.q_output : r.k_output) + base;
-  const size_t trig_base = (size_t)(r.trig_batches == 1 ? 0 : batch) * r.width;
+  _Float16 *output = reinterpret_cast<_Float16 *>(is_q ? r.q_output : r.k_output) +
+                     (((size_t)batch * heads + head) * r.tokens + token) * r.width;
+  const size_t trig_base = ((size_t)(r.trig_batches == 1 ? 0 : batch) * r.tokens + token) * r.width;
   const _Float16 *cosine = reinterpret_cast<const _Float16 *>(r.cosine) + trig_base;
   const _Float16 *sine = reinterpret_cast<const _Float16 *>(r.sine) + trig_base;
   size_t slot_base = 0;
-  if (!is_q) slot_base = (size_t)p.slots[batch] * p.token_stride;
+  if (!is_q) slot_base = (size_t)p.slots[item] * p.token_stride;
   int8_t *values = reinterpret_cast<int8_t *>(p.pool + slot_base);
   uint16_t *scales = reinterpret_cast<uint16_t *>(p.pool + slot_base + p.token_elements);
   const uint32_t segment_offset = p.segment_offset[is_v ? 1 : 0];
@@ -144,10 +151,10 @@ hipError_t launch_q8_pack(const Q8PackArgs &args, bool pair, hipStream_t stream)
 
 hipError_t launch_rotary_qk_pack(const RotaryPackArgs &args, hipStream_t stream) {
   const RotaryQkArgs &r = args.rotary;
-  if (r.tokens != 1 || r.width % 64 != 0 || args.pack.items != r.batches || args.pack.heads != r.k_heads ||
+  if (r.tokens == 0 || r.width % 64 != 0 || args.pack.items != r.batches * r.tokens || args.pack.heads != r.k_heads ||
       args.pack.head_dim != r.width || !args.pack.item_major)
     return hipErrorInvalidValue;
-  const uint32_t rows = r.batches * (r.q_heads + 2 * r.k_heads);
+  const uint32_t rows = r.batches * r.tokens * (r.q_heads + 2 * r.k_heads);
   if (rows == 0) return hipSuccess;
   hipLaunchKernelGGL(rotary_qk_pack_kernel, dim3((rows + 3) / 4), dim3(256), 0, stream, args);
   return hipGetLastError();

@@ -132,9 +132,9 @@ int rotary_qk_pack_batched(llmopt_hip_context *context, const DispatchRecord &re
   RotaryPackArgs args = {};
   if (int status = parse_rotary_qk(record, &args.rotary)) return status;
   if (int status = parse_pack_pair(record, 28, 5, 6, 7, 8, true, &args.pack)) return status;
-  if (args.rotary.tokens != 1 || args.pack.items != args.rotary.batches || args.pack.heads != args.rotary.k_heads ||
-      args.pack.head_dim != args.rotary.width)
-    return fail(LLMOPT_ERR_INVALID, "%s requires one token per sequence and the same sequences, KV heads and width "
+  if ((uint64_t)args.pack.items != (uint64_t)args.rotary.batches * args.rotary.tokens ||
+      args.pack.heads != args.rotary.k_heads || args.pack.head_dim != args.rotary.width)
+    return fail(LLMOPT_ERR_INVALID, "%s requires the same tokens (sequences x tokens items), KV heads and width "
                 "in both parameter blocks", record.name.c_str());
   return launched(launch_rotary_qk_pack(args, context->stream), record.name.c_str());
 }

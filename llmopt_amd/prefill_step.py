@@ -9,8 +9,10 @@ does this after a prefill), causal dense fp16 attention over the fresh K/V
 and the LM-head argmax of the last token gives the first generated token.  Afterwards the pool
 holds the prompt, and a `DecodeStep` over the same pool and slot table continues from there.
 
-Only reference entry points and the two normalising projection entries `decode_step.py` also
-uses; every entry is (kernel name, buffers, parameter block, grid, threadgroup).  V leaves the QKV
+Reference entry points plus the extensions `decode_step.py` also uses - the two normalising
+projection entries and, unless `reference_entries` is set, the rotation fused with the Q8 pack
+(`llmopt_rotary_qk_pack_q8_batched` in place of the rotation and two cache packs: the same bytes
+out); every entry is (kernel name, buffers, parameter block, grid, threadgroup).  V leaves the QKV
 projection token-major [tokens, kv_heads * head_dim]: the attention entry takes it as it is
 (token_first_value), and the cache pack reads it as ONE head of kv_heads * head_dim values, whose
 64-wide groups are the same bytes and scales as the per-head groups of the head-major layout.
@@ -31,12 +33,13 @@ class PrefillStep:
     into pool slots `slots[0 .. tokens)` (positions 0 .. tokens - 1)."""
 
     def __init__(self, runtime: Runtime, config: DecodeConfig, weights: dict, tokens: int, pool: Buffer,
-                 slots: Buffer, device_weights: dict | None = None):
+                 slots: Buffer, device_weights: dict | None = None, reference_entries: bool = False):
         if tokens < 2:
             raise ValueError("a prefill has at least two tokens (one token is a decode step)")
         if config.head_dim not in (64, 128, 256, 512):
             raise ValueError("dense attention entries exist for head sizes 64, 128, 256 and 512")
         self.runtime, self.config, self.token_count = runtime, config, tokens
+        self.reference_entries = reference_entries
         b = runtime.buffer_of_bytes
         c = config
         self.pool, self.slots = pool, slots
@@ -83,14 +86,24 @@ class PrefillStep:
             out.append(("llmopt_rms_w4a16_qkv_linear_f16_g64",
                         [x_in, layer["attn_norm"], *layer["q"], *layer["k"], *layer["v"], w["q"], w["k"], w["v"]],
                         u32s(t, h, qd, kvd, kvd) + struct.pack("<f", c.epsilon), rows_grid(qd + 2 * kvd), group))
-            out.append(("llmopt_rotary_qk_f16_simd_h64", [w["q"], w["k"], self.cos, self.sin, w["q_rot"], w["k_rot"]],
-                        u32s(1, t, c.q_heads, c.kv_heads, c.head_dim, c.head_dim // 2, 1),
-                        (((t * (c.q_heads + c.kv_heads) + 3) // 4) * 256, 1, 1), group))
-            # K head-major [kv_heads, tokens, d]; V token-major = one head of kv_heads * d values
-            out.append(("llmopt_cache_pack_attention_q8_simd", [w["k_rot"], self.slots, self.pool],
-                        pack(key_offset, c.kv_heads, c.head_dim), (t * kvd // 64 * 32, 1, 1), group))
-            out.append(("llmopt_cache_pack_attention_q8_simd", [w["v"], self.slots, self.pool],
-                        pack(value_offset, 1, kvd), (t * kvd // 64 * 32, 1, 1), group))
+            if self.reference_entries:
+                out.append(("llmopt_rotary_qk_f16_simd_h64",
+                            [w["q"], w["k"], self.cos, self.sin, w["q_rot"], w["k_rot"]],
+                            u32s(1, t, c.q_heads, c.kv_heads, c.head_dim, c.head_dim // 2, 1),
+                            (((t * (c.q_heads + c.kv_heads) + 3) // 4) * 256, 1, 1), group))
+                # K head-major [kv_heads, tokens, d]; V token-major = one head of kv_heads * d values
+                out.append(("llmopt_cache_pack_attention_q8_simd", [w["k_rot"], self.slots, self.pool],
+                            pack(key_offset, c.kv_heads, c.head_dim), (t * kvd // 64 * 32, 1, 1), group))
+                out.append(("llmopt_cache_pack_attention_q8_simd", [w["v"], self.slots, self.pool],
+                            pack(value_offset, 1, kvd), (t * kvd // 64 * 32, 1, 1), group))
+            else:
+                # rotation and every token's Q8 slot in one launch: the same bytes out, two launches fewer a layer
+                out.append(("llmopt_rotary_qk_pack_q8_batched",
+                            [w["q"], w["k"], self.cos, self.sin, w["q_rot"], w["k_rot"], w["v"], self.slots, self.pool],
+                            u32s(1, t, c.q_heads, c.kv_heads, c.head_dim, c.head_dim // 2, 1) +
+                            u32s(t, key_offset, value_offset, c.kv_heads, c.head_dim, 64, c.token_elements,
+                                 c.token_elements // 64, c.token_stride, t, 0),
+                            (((t * (c.q_heads + 2 * c.kv_heads) + 3) // 4) * 256, 1, 1), group))
             out.append((f"llmopt_attention_f16_simd_h{c.head_dim}",
                         [w["q_rot"], w["k_rot"], w["v"], w["q_rot"], w["attention"]], attention_params,
                         (t * c.q_heads, 1, 1), (64, 1, 1)))

@@ -166,6 +166,61 @@ def test_rotary_pack_in_one_launch_equals_the_two_launches(runtime, batches, q_h
     np.testing.assert_array_equal(first[value_offset + 64:value_offset + 128].view(np.int8), expected)
 
 
+@pytest.mark.parametrize("batches,tokens,q_heads,k_heads,d,trig_batches", [(1, 37, 9, 3, 64, 1), (2, 5, 8, 2, 128, 2),
+                                                                            (1, 300, 9, 3, 64, 1)])
+def test_rotary_pack_of_a_prompt_equals_the_separate_launches(runtime, batches, tokens, q_heads, k_heads, d,
+                                                              trig_batches):
+    """Several tokens per sequence (a prefill): token-major Q, K and V in, head-major rotated Q and K
+    out as llmopt_rotary_qk_f16_simd_h64 leaves them, and every token's K and V in its pool slot as
+    two llmopt_cache_pack_attention_q8_simd launches leave them (K from the head-major rotated rows,
+    V - token-major - as one head of k_heads * d values) - bit for bit."""
+    rng = np.random.default_rng(tokens * 100 + d)
+    elements = 2 * 2 * k_heads * d  # two layers; the second one is written
+    stride = elements + 2 * (elements // 64)
+    key_offset, value_offset = 2 * k_heads * d, 3 * k_heads * d
+    items = batches * tokens
+    capacity = items + 4
+    q = rng.standard_normal((batches, tokens, q_heads, d)).astype(np.float16)
+    k = rng.standard_normal((batches, tokens, k_heads, d)).astype(np.float16)
+    v = rng.standard_normal((batches, tokens, k_heads, d)).astype(np.float16)
+    cos = np.concatenate([rope_tables(tokens, d, rng)[0] for _ in range(trig_batches)])
+    sin = np.concatenate([rope_tables(tokens, d, rng)[1] for _ in range(trig_batches)])
+    slots = rng.permutation(capacity)[:items].astype(np.uint32)
+    start = rng.integers(0, 256, size=capacity * stride, dtype=np.uint8)
+    rotary_params = u32s(batches, tokens, q_heads, k_heads, d, d // 2, trig_batches)
+    inputs = [runtime.buffer_of_bytes(x) for x in (q, k, cos, sin)]
+    v_buffer, slot_buffer = runtime.buffer_of_bytes(v), runtime.buffer_of_bytes(slots)
+
+    def outputs():
+        return (runtime.buffer_of_bytes(np.full(q.size, np.nan, dtype=np.float16)),
+                runtime.buffer_of_bytes(np.full(k.size, np.nan, dtype=np.float16)),
+                runtime.buffer_of_bytes(start))
+
+    q_two, k_two, pool_two = outputs()
+    rows = items * (q_heads + k_heads)
+    runtime.dispatch("llmopt_rotary_qk_f16_simd_h64", [*inputs, q_two, k_two], rotary_params,
+                     grid=(((rows + 7) // 8) * 256, 1, 1), group=(256, 1, 1))
+    # K head-major [k_heads, tokens, d] per sequence; V token-major as one head of k_heads * d values
+    for b in range(batches):
+        seq_slots = runtime.buffer_of_bytes(slots[b * tokens:(b + 1) * tokens])
+        k_rows = k_two.view(b * k_heads * tokens * d * 2, k_heads * tokens * d * 2)
+        v_rows = v_buffer.view(b * tokens * k_heads * d * 2, tokens * k_heads * d * 2)
+        runtime.dispatch("llmopt_cache_pack_attention_q8_simd", [k_rows, seq_slots, pool_two],
+                         u32s(tokens, key_offset, k_heads, d, 64, elements, elements // 64, stride, tokens, 0),
+                         grid=(tokens * k_heads * (d // 64) * 64, 1, 1), group=(256, 1, 1))
+        runtime.dispatch("llmopt_cache_pack_attention_q8_simd", [v_rows, seq_slots, pool_two],
+                         u32s(tokens, value_offset, 1, k_heads * d, 64, elements, elements // 64, stride, tokens, 0),
+                         grid=(tokens * k_heads * (d // 64) * 64, 1, 1), group=(256, 1, 1))
+    q_one, k_one, pool_one = outputs()
+    pack_params = u32s(items, key_offset, value_offset, k_heads, d, 64, elements, elements // 64, stride, items, 0)
+    runtime.dispatch("llmopt_rotary_qk_pack_q8_batched",
+                     [*inputs, q_one, k_one, v_buffer, slot_buffer, pool_one], rotary_params + pack_params,
+                     grid=(((items * (q_heads + 2 * k_heads) + 3) // 4) * 256, 1, 1), group=(256, 1, 1))
+    np.testing.assert_array_equal(q_one.numpy(np.uint16, (q.size,)), q_two.numpy(np.uint16, (q.size,)))
+    np.testing.assert_array_equal(k_one.numpy(np.uint16, (k.size,)), k_two.numpy(np.uint16, (k.size,)))
+    np.testing.assert_array_equal(pool_one.numpy(np.uint8, (capacity, stride)), pool_two.numpy(np.uint8, (capacity, stride)))
+
+
 def test_rotary_pack_rejects_blocks_that_disagree(runtime):
     d, batches, heads = 64, 2, 3
     elements = 2 * heads * d
@@ -178,8 +233,8 @@ def test_rotary_pack_rejects_blocks_that_disagree(runtime):
     pack = lambda items, kv: u32s(items, 0, heads * d, kv, d, 64, elements, elements // 64, stride, items, 0)
     for rotary, cache in ((u32s(batches, 1, 9, heads, d, d // 2, 1), pack(batches, 2)),
                           (u32s(batches, 1, 9, heads, d, d // 2, 1), pack(1, heads)),
-                          (u32s(1, 2, 9, heads, d, d // 2, 1), pack(batches, heads))):
-        with pytest.raises(Exception, match="requires one token per sequence"):
+                          (u32s(1, 1, 9, heads, d, d // 2, 1), pack(batches, heads))):
+        with pytest.raises(Exception, match="requires the same tokens"):
             runtime.dispatch("llmopt_rotary_qk_pack_q8_batched", buffers, rotary + cache,
                              grid=(256, 1, 1), group=(256, 1, 1))
 

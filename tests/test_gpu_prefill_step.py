@@ -142,3 +142,31 @@ def test_prefill_matches_oracle_chain_and_decode_continues(runtime, tokens, laye
                            "decode step after the prefill", rel_l2_tol=2e-2)
     decode_rms = float(np.sqrt(np.mean(decode_logits.astype(np.float64) ** 2)))
     assert float(decode_logits[0, next_token[0]]) >= float(decode_logits[0].max()) - 2e-2 * decode_rms
+
+
+def test_fused_rotation_and_pack_leave_the_same_bytes_as_the_reference_entries(runtime):
+    """The prefill with the rotation fused into the Q8 pack against the one built from the reference's
+    own entries (rotation, pack of K, pack of V): the same residual stream, the same pool, the same
+    first token - bit for bit."""
+    from llmopt_amd.decode_step import DecodeConfig, random_weights
+    from llmopt_amd.prefill_step import PrefillStep
+    rng = np.random.default_rng(77)
+    tokens = 70
+    config = DecodeConfig(layers=2, vocabulary=1000)
+    weights = random_weights(config, rng)
+    capacity = tokens + 3
+    order = rng.permutation(capacity).astype(np.uint32)
+    pool = rng.integers(0, 256, size=capacity * config.token_stride, dtype=np.uint8)
+    prompt = rng.integers(0, config.vocabulary, tokens)
+    results = []
+    for reference_entries in (False, True):
+        device_pool = runtime.buffer_of_bytes(pool)
+        step = PrefillStep(runtime, config, weights, tokens, device_pool, runtime.buffer_of_bytes(order),
+                           reference_entries=reference_entries)
+        assert len(step.dispatches) == (2 + config.layers * (8 if reference_entries else 6))
+        token = step.run(prompt)
+        results.append((token, step.work["x"][0].numpy(np.uint16, (tokens, config.hidden)),
+                        device_pool.numpy(np.uint8, (capacity, config.token_stride))))
+    assert results[0][0] == results[1][0]
+    np.testing.assert_array_equal(results[0][1], results[1][1])
+    np.testing.assert_array_equal(results[0][2], results[1][2])
