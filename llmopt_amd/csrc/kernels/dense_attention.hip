@@ -691,6 +691,28 @@ __global__ __launch_bounds__(256) void mask_bits_kernel(DenseAttentionArgs a, ui
         (uint8_t)((chunk_bits >> threadIdx.x) & 1u);
 }
 
+// ---- the mask of the speculative tree attention entries ---------------------------------------
+struct TreeMaskArgs {
+  uint8_t *mask;
+  uint32_t query_length, key_length, past_length;
+  uint32_t tree_masks[8];
+};
+
+__global__ __launch_bounds__(256) void tree_mask_kernel(TreeMaskArgs a) {
+  const uint64_t index = (uint64_t)blockIdx.x * 256 + threadIdx.x;
+  if (index >= (uint64_t)a.query_length * a.key_length) return;
+  const uint32_t query = (uint32_t)(index / a.key_length), key = (uint32_t)(index % a.key_length);
+  bool allowed = key < a.past_length;
+  if (!allowed) {
+    const uint32_t draft = key - a.past_length;
+    uint32_t bits = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) bits = query == (uint32_t)i ? a.tree_masks[i] : bits;
+    allowed = draft < a.query_length && draft < 32 && ((bits >> draft) & 1u) != 0;
+  }
+  a.mask[index] = allowed ? 1 : 0;
+}
+
 // ---- row-serial kernel (every other configuration) ---------------------------
 
 constexpr int kMaxFragments = 8;  // head_dim <= 512
@@ -832,6 +854,17 @@ size_t stage_map_region(const DenseAttentionArgs &a, const Tile32Geometry &g) {
 uint32_t mask_words_per_row(const DenseAttentionArgs &a) { return 2 * ((a.key_length + 63) / 64); }
 
 }  // namespace
+
+hipError_t launch_tree_mask(uint8_t *mask, uint32_t query_length, uint32_t key_length, uint32_t past_length,
+                            const uint32_t tree_masks[8], hipStream_t stream) {
+  const uint64_t elements = (uint64_t)query_length * key_length;
+  if (elements == 0) return hipSuccess;
+  if ((elements + 255) / 256 > 0x7fffffffull) return hipErrorInvalidValue;
+  TreeMaskArgs args = {mask, query_length, key_length, past_length, {}};
+  for (int i = 0; i < 8; ++i) args.tree_masks[i] = tree_masks[i];
+  hipLaunchKernelGGL(tree_mask_kernel, dim3((uint32_t)((elements + 255) / 256)), dim3(256), 0, stream, args);
+  return hipGetLastError();
+}
 
 size_t dense_attention_workspace_bytes(const DenseAttentionArgs &a) {
   if (!dense_masked(a) || a.batches == 0 || a.heads == 0 || a.query_length == 0 || a.key_length == 0) return 0;

@@ -187,6 +187,13 @@ struct DenseAttentionArgs {
 size_t dense_attention_workspace_bytes(const DenseAttentionArgs &args);
 hipError_t launch_dense_attention(const DenseAttentionArgs &args, hipStream_t stream);
 
+// The mask of llmopt_attention_tree_speculative_f16 (llmopt_speculative_tree_allowed,
+// lib/metal_attention_source.ml:361-381) as bytes [query_length, key_length]: every key before
+// past_length is visible; draft key i (key past_length + i, i < query_length) is visible to query
+// token q when bit i of tree_masks[q] is set (q < 8; later query tokens see the past only).
+hipError_t launch_tree_mask(uint8_t *mask, uint32_t query_length, uint32_t key_length, uint32_t past_length,
+                            const uint32_t tree_masks[8], hipStream_t stream);
+
 // ---- decode glue ---------------------------------------------------------------
 
 // out[row, i] = half(x[row, i] * rsqrt(mean(x[row]^2) + eps) * w[i]), one wave per row.

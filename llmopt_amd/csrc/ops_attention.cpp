@@ -333,6 +333,65 @@ int dense_attention(llmopt_hip_context *context, const DispatchRecord &record) {
   return launched(launch_dense_attention(args, context->stream), name);
 }
 
+// llmopt_attention_tree_speculative_f16{,_simd_h64} (lib/metal_attention_source.ml:351-512, dispatch
+// lib/metal_dispatch_attention.ml:219-245): dense attention of a few draft tokens over past_length
+// cached keys and each other, who sees whom among the drafts given by eight bit masks.
+// SpeculativeAttentionParams, 64 bytes: batches 0, heads 4, query_length 8, key_length 12,
+// head_dimension 16, kv_heads 20, past_length 24, scale(f32) 28, tree_mask_0..7 at 32..60.
+// buffers: query [b, h, q, D], key [b, kvh, L, D], value [b, L, kvh, D] (token-major), output
+// [b, q, h, D] (token-major).  The masks are written out as a byte mask [q, L] in the context's
+// scratch memory and the dense attention kernels run with it.
+int speculative_attention(llmopt_hip_context *context, const DispatchRecord &record) {
+  if (int status = require_buffer_count(record, 4)) return status;
+  if (int status = require_parameter_bytes(record, 64)) return status;
+  const char *name = record.name.c_str();
+  DenseAttentionArgs args = {};
+  args.batches = param_u32(record, 0);
+  args.heads = param_u32(record, 4);
+  args.query_length = param_u32(record, 8);
+  args.key_length = param_u32(record, 12);
+  args.head_dim = param_u32(record, 16);
+  args.kv_heads = param_u32(record, 20);
+  const uint32_t past_length = param_u32(record, 24);
+  args.scale = param_f32(record, 28);
+  uint32_t tree_masks[8];
+  for (int i = 0; i < 8; ++i) tree_masks[i] = param_u32(record, 32 + 4 * i);
+  if (args.head_dim == 0 || args.head_dim > 512)
+    return fail(LLMOPT_ERR_INVALID, "%s supports head dimensions 1..512, got %u", name, args.head_dim);
+  const uint32_t kv_heads = args.kv_heads > 0 ? args.kv_heads : args.heads;
+  if (kv_heads == 0 || (kv_heads < args.heads && args.heads % kv_heads != 0) || kv_heads > args.heads)
+    return fail(LLMOPT_ERR_INVALID, "%s requires heads to be a multiple of kv_heads", name);
+  const uint64_t rows = (uint64_t)args.batches * args.heads * args.query_length;
+  if (rows != 0 && args.key_length == 0) return fail(LLMOPT_ERR_INVALID, "%s requires at least one key", name);
+  const uint64_t kv_elements = (uint64_t)args.batches * kv_heads * args.key_length * args.head_dim;
+  if (int status = require_buffer_size(record.buffers[0], rows * args.head_dim * 2, "attention query")) return status;
+  if (int status = require_buffer_size(record.buffers[1], kv_elements * 2, "attention key")) return status;
+  if (int status = require_buffer_size(record.buffers[2], kv_elements * 2, "attention value")) return status;
+  if (int status = require_buffer_size(record.buffers[3], rows * args.head_dim * 2, "attention output")) return status;
+  if (rows == 0) return LLMOPT_OK;
+  args.query = reinterpret_cast<const uint16_t *>(record.buffers[0].device);
+  args.key = reinterpret_cast<const uint16_t *>(record.buffers[1].device);
+  args.value = reinterpret_cast<const uint16_t *>(record.buffers[2].device);
+  args.output = reinterpret_cast<uint16_t *>(record.buffers[3].device);
+  args.mask_batches = 1, args.mask_heads = 1, args.mask_dtype = 1, args.causal = 0;
+  args.token_first_output = 1, args.token_first_value = 1;
+  const size_t mask_bytes = ((size_t)args.query_length * args.key_length + 255) & ~(size_t)255;
+  // the dense kernels' own scratch is sized for any 16-byte aligned mask address
+  args.mask = reinterpret_cast<const uint8_t *>((uintptr_t)4096);
+  const size_t map_bytes = dense_attention_workspace_bytes(args);
+  uint8_t *scratch = static_cast<uint8_t *>(context_workspace(context, mask_bytes + map_bytes));
+  if (scratch == nullptr) return LLMOPT_ERR_FAILURE;
+  args.mask = scratch;
+  if (map_bytes > 0) {
+    args.stage_map = scratch + mask_bytes;
+    args.stage_map_bytes = map_bytes;
+  }
+  if (int status = launched(launch_tree_mask(scratch, args.query_length, args.key_length, past_length, tree_masks,
+                                             context->stream), name))
+    return status;
+  return launched(launch_dense_attention(args, context->stream), name);
+}
+
 }  // namespace
 
 void register_cache_kernels(std::vector<KernelEntryPoint> &table) {
@@ -360,6 +419,8 @@ void register_attention_kernels(std::vector<KernelEntryPoint> &table) {
                                       "llmopt_attention_f16_simd_h128", "llmopt_attention_f16_simd_h256",
                                       "llmopt_attention_f16_simd_h512"};
   for (const char *name : dense) table.push_back({name, attention, dense_attention});
+  table.push_back({"llmopt_attention_tree_speculative_f16", attention, speculative_attention});
+  table.push_back({"llmopt_attention_tree_speculative_f16_simd_h64", attention, speculative_attention});
   // Extension: per-sequence context lengths and slot tables in one launch.
   table.push_back({"llmopt_attention_q8_paged_batched", attention, paged_attention_batched});
 }

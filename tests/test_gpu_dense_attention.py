@@ -447,3 +447,39 @@ def test_random_block_masks(runtime, case):
     want = expected(query, key, value, np.broadcast_to(allowed, (batches, heads, new, length)), scale)
     assert np.all(got[:, :, new // 2].view(np.uint16) == 0)
     assert_close_to_oracle(got, want, f"random block mask {case}: D={dim} {heads}/{kv_heads} x{batches}, {new} after {past}")
+
+
+@pytest.mark.parametrize("dim,heads,kv_heads,batches,q_len,past,masks", [
+    (64, 9, 3, 1, 4, 300, [1, 3, 7, 15, 0, 0, 0, 0]),          # the default chain of four drafts
+    (64, 4, 4, 2, 8, 0, [1, 3, 5, 11, 21, 37, 69, 133]),       # a tree; nothing cached
+    (128, 8, 2, 1, 6, 1000, [1, 3, 5, 9, 19, 35, 0, 0]),
+    (128, 2, 1, 1, 10, 40, [1, 2, 4, 8, 16, 32, 64, 128]),     # query tokens 8 and 9 see the past only
+    (256, 2, 2, 1, 3, 500, [1, 1, 5, 0, 0, 0, 0, 0]),
+])
+def test_speculative_tree_attention(runtime, dim, heads, kv_heads, batches, q_len, past, masks):
+    """llmopt_attention_tree_speculative_f16{,_simd_h64}: draft tokens over the cached keys and over each
+    other as eight bit masks say (lib/metal_attention_source.ml:361-381); token-major V and output.
+    The expected rows are the oracle's dense attention under the mask that function describes."""
+    rng = np.random.default_rng(dim + q_len + past)
+    length = past + q_len
+    query = rng.standard_normal((batches, heads, q_len, dim)).astype(np.float16)
+    key = rng.standard_normal((batches, kv_heads, length, dim)).astype(np.float16)
+    value = rng.standard_normal((batches, kv_heads, length, dim)).astype(np.float16)
+    scale = 1.0 / math.sqrt(dim)
+    allowed = np.zeros((q_len, length), dtype=bool)
+    allowed[:, :past] = True
+    for q in range(min(q_len, 8)):
+        for draft in range(q_len):
+            allowed[q, past + draft] = bool((masks[q] >> draft) & 1)
+    params = struct.pack("<7If8I", batches, heads, q_len, length, dim, kv_heads, past, scale, *masks)
+    name = "llmopt_attention_tree_speculative_f16_simd_h64" if dim == 64 else "llmopt_attention_tree_speculative_f16"
+    out = runtime.buffer_of_bytes(np.full((batches, q_len, heads, dim), np.nan, dtype=np.float16))
+    value_token_major = np.ascontiguousarray(value.transpose(0, 2, 1, 3))
+    runtime.dispatch(name, [runtime.buffer_of_bytes(query), runtime.buffer_of_bytes(key),
+                            runtime.buffer_of_bytes(value_token_major), out], params,
+                     grid=(((batches * heads * q_len + 7) // 8) * 256, 1, 1), group=(256, 1, 1))
+    got = out.numpy(np.float16, (batches, q_len, heads, dim)).transpose(0, 2, 1, 3)
+    want = expected(query, key, value, np.broadcast_to(allowed[None, None], (batches, heads, q_len, length)), scale)
+    if past == 40:  # rows without a visible key at all do not occur here; rows 8, 9 see exactly the past
+        assert np.all(np.isfinite(got))
+    assert_close_to_oracle(got, want, f"tree attention D={dim} {heads}/{kv_heads}, {q_len} drafts after {past}")
