@@ -222,8 +222,10 @@ int llmopt_hip_prebaked_create(llmopt_hip_library *library,
 void llmopt_hip_release_prebaked(llmopt_hip_prebaked *plan);
 /* caml_llmopt_prebaked_execute (:2167-2560): writes `token` (int64) at the
  * start of the token buffer, makes past_tokens the context length of every
- * paged attention record (:2182-2195), replays all records in order, waits,
- * and returns the first int32 of the output buffer in *out_token.
+ * paged attention record (:2182-2195) and `checkpoint` the slot of every
+ * llmopt_cache_pack_checkpoint_q8_simd record (byte 0 of its parameter block,
+ * :2186-2188), replays all records in order, waits, and returns the first
+ * int32 of the output buffer in *out_token.
  * past_tokens beyond the slot tables' capacity is LLMOPT_ERR_INVALID.
  * Debug replays of the reference, switched on by the same environment
  * variables (:2203-2347): LLMOPT_PROFILE_BREAKDOWN runs the records one at a

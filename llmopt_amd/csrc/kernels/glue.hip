@@ -404,8 +404,10 @@ namespace {
 // the input token (given, or the previous step's output token: llmopt_chain_token_id,
 // native/ocaml_metal_stubs.m:1570-1577) and the context length every sequence attends to.
 __global__ void plan_state_kernel(int64_t *token, int64_t value, const int32_t *chain_from, uint32_t *past,
-                                  uint32_t past_value, uint32_t past_count) {
+                                  uint32_t past_value, uint32_t past_count, uint32_t *checkpoint,
+                                  uint32_t checkpoint_value) {
   if (threadIdx.x == 0 && token != nullptr) *token = chain_from != nullptr ? (int64_t)*chain_from : value;
+  if (threadIdx.x == 0 && checkpoint != nullptr) *checkpoint = checkpoint_value;
   for (uint32_t i = threadIdx.x; i < past_count; i += blockDim.x) past[i] = past_value;
 }
 
@@ -435,9 +437,10 @@ hipError_t launch_nan_scan(const void *data, size_t bytes, bool f32, uint32_t *f
 }
 
 hipError_t launch_plan_state(int64_t *token, int64_t value, const int32_t *chain_from, uint32_t *past,
-                             uint32_t past_value, uint32_t past_count, hipStream_t stream) {
+                             uint32_t past_value, uint32_t past_count, uint32_t *checkpoint, uint32_t checkpoint_value,
+                             hipStream_t stream) {
   hipLaunchKernelGGL(plan_state_kernel, dim3(1), dim3(256), 0, stream, token, value, chain_from, past, past_value,
-                     past_count);
+                     past_count, checkpoint, checkpoint_value);
   return hipGetLastError();
 }
 

@@ -127,6 +127,22 @@ struct Q8UnpackArgs {
 hipError_t launch_q8_pack(const Q8PackArgs &args, bool pair, hipStream_t stream);
 hipError_t launch_q8_unpack(const Q8UnpackArgs &args, hipStream_t stream);
 
+// llmopt_cache_{pack,unpack}_checkpoint_q8* (lib/metal_cache_source.ml:245-343,
+// CheckpointCacheParams :36-44): one layer's flat f16 state of layer_elements values to or from
+// checkpoint slot `checkpoint` of a pool of checkpoint_stride-byte slots, the same group-64
+// quantiser as the attention cache (int8 values of all layers, then their f16 scales).
+// device_checkpoint, when not null, holds the slot index instead (a retained plan writes it per
+// step); it is held to max_checkpoint, the last slot the pool has room for.
+struct Q8CheckpointArgs {
+  const uint16_t *source;  // pack
+  uint16_t *destination;   // unpack
+  uint8_t *pool;
+  const uint32_t *device_checkpoint;
+  uint32_t checkpoint, max_checkpoint, layer, layer_elements, checkpoint_elements, checkpoint_stride;
+};
+hipError_t launch_q8_checkpoint_pack(const Q8CheckpointArgs &args, hipStream_t stream);
+hipError_t launch_q8_checkpoint_unpack(const Q8CheckpointArgs &args, hipStream_t stream);
+
 // Q8PagedAttentionParams (lib/metal_cache_source.ml:352-369) plus the
 // per-sequence extension: when past_lengths is not null, sequence b attends to
 // past_lengths[b] pool tokens whose slot indices start at
@@ -259,7 +275,8 @@ hipError_t launch_copy_bytes(void *destination, const void *source, size_t bytes
 // One small launch that sets a retained plan's per-step state: *token = *chain_from (when not
 // null; int32 widened) or `value` (token may be null), and past[0..past_count) = past_value.
 hipError_t launch_plan_state(int64_t *token, int64_t value, const int32_t *chain_from, uint32_t *past,
-                             uint32_t past_value, uint32_t past_count, hipStream_t stream);
+                             uint32_t past_value, uint32_t past_count, uint32_t *checkpoint, uint32_t checkpoint_value,
+                             hipStream_t stream);
 
 // Sets *found (device memory) to 1 when [data, data + bytes) holds a NaN, read as fp16 words or
 // (f32) as float32 words; leaves it alone otherwise.

@@ -110,6 +110,41 @@ __global__ __launch_bounds__(256) void rotary_qk_pack_kernel(RotaryPackArgs a) {
   }
 }
 
+// One wave per 64-wide group of the layer's state.
+__global__ __launch_bounds__(256) void q8_checkpoint_pack_kernel(Q8CheckpointArgs a) {
+  const uint32_t lane = threadIdx.x & 63;
+  const uint32_t layer_groups = a.layer_elements >> 6;
+  const uint32_t group = blockIdx.x * (blockDim.x >> 6) + (threadIdx.x >> 6);
+  if (group >= layer_groups) return;
+  const uint32_t checkpoint = min(a.device_checkpoint ? *a.device_checkpoint : a.checkpoint, a.max_checkpoint);
+  uint8_t *slot = a.pool + (size_t)checkpoint * a.checkpoint_stride;
+  int8_t *values = reinterpret_cast<int8_t *>(slot);
+  uint16_t *scales = reinterpret_cast<uint16_t *>(slot + a.checkpoint_elements);
+  uint16_t stored;
+  values[(size_t)a.layer * a.layer_elements + group * 64 + lane] =
+      q8_quantize(half_bits_to_float(a.source[(size_t)group * 64 + lane]), &stored);
+  if (lane == 0) scales[(size_t)a.layer * layer_groups + group] = stored;
+}
+
+// One thread per four consecutive values.
+__global__ __launch_bounds__(256) void q8_checkpoint_unpack_kernel(Q8CheckpointArgs a) {
+  const size_t index = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (index >= a.layer_elements / 4) return;
+  const uint32_t local = (uint32_t)index * 4;
+  const uint32_t checkpoint = min(a.device_checkpoint ? *a.device_checkpoint : a.checkpoint, a.max_checkpoint);
+  const uint8_t *slot = a.pool + (size_t)checkpoint * a.checkpoint_stride;
+  // (a checkpoint slot is only 2-byte aligned: its stride is elements + 2 * groups)
+  typedef uint32_t unaligned_u32_t __attribute__((aligned(1)));
+  const uint32_t packed = *reinterpret_cast<const unaligned_u32_t *>(slot + (size_t)a.layer * a.layer_elements + local);
+  const uint16_t *scales = reinterpret_cast<const uint16_t *>(slot + a.checkpoint_elements);
+  const float scale = half_bits_to_float(scales[(size_t)a.layer * (a.layer_elements >> 6) + (local >> 6)]);
+  uint16_t out[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) out[i] = float_to_half_bits((float)(int8_t)((packed >> (8 * i)) & 0xffu) * scale);
+  *reinterpret_cast<uint2 *>(a.destination + local) =
+      make_uint2((uint32_t)out[0] | ((uint32_t)out[1] << 16), (uint32_t)out[2] | ((uint32_t)out[3] << 16));
+}
+
 __global__ __launch_bounds__(256) void q8_unpack_kernel(Q8UnpackArgs a) {
   // one thread per 4 consecutive elements of one (item, head)
   const size_t index = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -157,6 +192,20 @@ hipError_t launch_rotary_qk_pack(const RotaryPackArgs &args, hipStream_t stream)
   const uint32_t rows = r.batches * r.tokens * (r.q_heads + 2 * r.k_heads);
   if (rows == 0) return hipSuccess;
   hipLaunchKernelGGL(rotary_qk_pack_kernel, dim3((rows + 3) / 4), dim3(256), 0, stream, args);
+  return hipGetLastError();
+}
+
+hipError_t launch_q8_checkpoint_pack(const Q8CheckpointArgs &args, hipStream_t stream) {
+  const uint32_t groups = args.layer_elements >> 6;
+  if (groups == 0) return hipSuccess;
+  hipLaunchKernelGGL(q8_checkpoint_pack_kernel, dim3((groups + 3) / 4), dim3(256), 0, stream, args);
+  return hipGetLastError();
+}
+
+hipError_t launch_q8_checkpoint_unpack(const Q8CheckpointArgs &args, hipStream_t stream) {
+  const uint32_t vectors = args.layer_elements / 4;
+  if (vectors == 0) return hipSuccess;
+  hipLaunchKernelGGL(q8_checkpoint_unpack_kernel, dim3((vectors + 255) / 256), dim3(256), 0, stream, args);
   return hipGetLastError();
 }
 

@@ -2,6 +2,8 @@
 // buffer order and parameter-block layout of lib/metal_cache_source.ml:9-34,
 // 46-243,352-583 (host side lib/metal_cache.ml:230-511,
 // lib/metal_dispatch_attention.ml:104-217, lib/metal_parameters.ml:119-140).
+#include <algorithm>
+
 #include "kernels/kernels.h"
 #include "runtime.h"
 
@@ -166,6 +168,58 @@ int cache_unpack(llmopt_hip_context *context, const DispatchRecord &record) {
   args.slots = reinterpret_cast<const uint32_t *>(record.buffers[1].device);
   args.destination = reinterpret_cast<uint16_t *>(record.buffers[2].device);
   return launched(launch_q8_unpack(args, context->stream), record.name.c_str());
+}
+
+// CheckpointCacheParams, 28 bytes (lib/metal_cache_source.ml:36-44): checkpoint 0, layer 4,
+// layer_elements 8, group_size 12, checkpoint_elements 16, checkpoint_groups 20, checkpoint_stride 24.
+// pack buffers: source, pool; unpack buffers: pool, destination.
+int cache_checkpoint(llmopt_hip_context *context, const DispatchRecord &record, bool pack) {
+  if (int status = require_buffer_count(record, 2)) return status;
+  if (int status = require_parameter_bytes(record, 28)) return status;
+  const char *name = record.name.c_str();
+  Q8CheckpointArgs args = {};
+  args.checkpoint = param_u32(record, 0);
+  args.layer = param_u32(record, 4);
+  args.layer_elements = param_u32(record, 8);
+  const uint32_t group_size = param_u32(record, 12);
+  args.checkpoint_elements = param_u32(record, 16);
+  const uint32_t checkpoint_groups = param_u32(record, 20);
+  args.checkpoint_stride = param_u32(record, 24);
+  if (group_size != 64) return fail(LLMOPT_ERR_INVALID, "%s supports the Q8 group size 64 only, got %u", name, group_size);
+  if (args.layer_elements % 64 != 0 || args.checkpoint_elements % 64 != 0 ||
+      checkpoint_groups != args.checkpoint_elements / 64 ||
+      (uint64_t)args.checkpoint_stride < (uint64_t)args.checkpoint_elements + 2ull * checkpoint_groups ||
+      args.checkpoint_stride % 2 != 0)
+    return fail(LLMOPT_ERR_INVALID, "%s received an inconsistent Q8 checkpoint layout", name);
+  if (((uint64_t)args.layer + 1) * args.layer_elements > args.checkpoint_elements)
+    return fail(LLMOPT_ERR_INVALID, "%s layer lies outside the checkpoint", name);
+  const BoundBuffer &pool = record.buffers[pack ? 1 : 0];
+  const BoundBuffer &state = record.buffers[pack ? 0 : 1];
+  if (int status = require_buffer_size(pool, args.checkpoint_stride, "checkpoint pool")) return status;
+  args.max_checkpoint = (uint32_t)std::min<uint64_t>(pool.length / args.checkpoint_stride - 1, 0xffffffffull);
+  if (record.device_checkpoint == nullptr && args.checkpoint > args.max_checkpoint)
+    return fail(LLMOPT_ERR_INVALID, "HIP checkpoint pool buffer is too small: required=%llu actual=%llu",
+                (unsigned long long)(args.checkpoint + 1ull) * args.checkpoint_stride, (unsigned long long)pool.length);
+  if (int status = require_buffer_size(state, (uint64_t)args.layer_elements * 2, pack ? "checkpoint source" : "checkpoint destination"))
+    return status;
+  if ((reinterpret_cast<uintptr_t>(pool.device) & 1) != 0 || (reinterpret_cast<uintptr_t>(state.device) & 7) != 0)
+    return fail(LLMOPT_ERR_INVALID, "%s requires 2-byte aligned pools and 8-byte aligned states", name);
+  args.pool = pool.device;
+  args.device_checkpoint = record.device_checkpoint;
+  if (pack) {
+    args.source = reinterpret_cast<const uint16_t *>(state.device);
+    return launched(launch_q8_checkpoint_pack(args, context->stream), name);
+  }
+  args.destination = reinterpret_cast<uint16_t *>(state.device);
+  return launched(launch_q8_checkpoint_unpack(args, context->stream), name);
+}
+
+int cache_pack_checkpoint(llmopt_hip_context *context, const DispatchRecord &record) {
+  return cache_checkpoint(context, record, true);
+}
+
+int cache_unpack_checkpoint(llmopt_hip_context *context, const DispatchRecord &record) {
+  return cache_checkpoint(context, record, false);
 }
 
 // Q8PagedAttentionParams, 64 bytes (lib/metal_cache_source.ml:352-369):
@@ -403,6 +457,10 @@ void register_cache_kernels(std::vector<KernelEntryPoint> &table) {
   table.push_back({"llmopt_rotary_qk_pack_q8_batched", cache, rotary_qk_pack_batched});
   table.push_back({"llmopt_cache_unpack_attention_q8", cache, cache_unpack});
   table.push_back({"llmopt_cache_unpack_attention_q8_vec4", cache, cache_unpack});
+  table.push_back({"llmopt_cache_pack_checkpoint_q8", cache, cache_pack_checkpoint});
+  table.push_back({"llmopt_cache_pack_checkpoint_q8_simd", cache, cache_pack_checkpoint});
+  table.push_back({"llmopt_cache_unpack_checkpoint_q8", cache, cache_unpack_checkpoint});
+  table.push_back({"llmopt_cache_unpack_checkpoint_q8_vec4", cache, cache_unpack_checkpoint});
 }
 
 void register_attention_kernels(std::vector<KernelEntryPoint> &table) {

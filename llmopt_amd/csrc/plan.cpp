@@ -32,6 +32,11 @@ struct llmopt_hip_prebaked : llmopt::RefCounted {
   llmopt_hip_library *library = nullptr;
   std::vector<DispatchRecord> records;
   std::vector<bool> is_paged_attention;
+  // llmopt_cache_pack_checkpoint_q8_simd: byte 0 of its parameter block is the step's checkpoint slot
+  // (native/ocaml_metal_stubs.m:1965, 2186-2199)
+  std::vector<bool> is_checkpoint_pack;
+  uint32_t *device_checkpoint = nullptr;  // the word behind device_past's, when the plan packs a checkpoint
+  uint32_t checkpoint = 0;                // of the step being enqueued
   llmopt_hip_buffer *token_buffer = nullptr;
   llmopt_hip_buffer *output_buffer = nullptr;
   // context length of the step, one word per sequence of the widest attention record
@@ -109,6 +114,7 @@ int capture_plan(llmopt_hip_prebaked *plan) {
 // after).  chain: the input token is the output token the previous step left in the output
 // buffer (the reference's llmopt_chain_token_id launch).
 int enqueue_step(llmopt_hip_prebaked *plan, int64_t token, bool chain, int64_t past_tokens, int32_t *host_token) {
+  const uint32_t checkpoint = plan->checkpoint;
   llmopt_hip_context *context = plan->library->context;
   if (int status = use_device(context)) return status;
   if (past_tokens < 0 || (uint64_t)past_tokens > plan->past_capacity)
@@ -129,14 +135,15 @@ int enqueue_step(llmopt_hip_prebaked *plan, int64_t token, bool chain, int64_t p
     if (plan->executable == nullptr || plan->workspace_generation != context->workspace_generation)
       if (int status = capture_plan(plan)) return status;
     LLMOPT_HIP_TRY(launch_plan_state(token_slot, token, chain_from, plan->device_past, (uint32_t)past_tokens,
-                                     plan->past_count, context->stream),
+                                     plan->past_count, plan->device_checkpoint, checkpoint, context->stream),
                    "HIP could not write the decode step's state");
     LLMOPT_HIP_TRY(hipGraphLaunch(plan->executable, context->stream), "HIP graph launch failed");
   } else {
-    LLMOPT_HIP_TRY(launch_plan_state(token_slot, token, chain_from, nullptr, 0, 0, context->stream),
+    LLMOPT_HIP_TRY(launch_plan_state(token_slot, token, chain_from, nullptr, 0, 0, nullptr, 0, context->stream),
                    "HIP could not write the decode token");
     for (size_t i = 0; i < plan->records.size(); ++i) {
       DispatchRecord &record = plan->records[i];
+      if (plan->is_checkpoint_pack[i] && record.parameters.size() >= 4) memcpy(record.parameters.data(), &checkpoint, 4);
       if (plan->is_paged_attention[i] && record.parameters.size() >= 16) {
         const uint32_t past = (uint32_t)past_tokens;
         memcpy(record.parameters.data() + 12, &past, 4);
@@ -201,6 +208,7 @@ int debug_step(llmopt_hip_prebaked *plan, int64_t token, int64_t past_tokens, bo
   // frozen records read the context length from the plan's device words, the others from byte 12
   LLMOPT_HIP_TRY(launch_plan_state(token_slot, token, nullptr, plan->single_submission ? plan->device_past : nullptr,
                                    (uint32_t)past_tokens, plan->single_submission ? plan->past_count : 0,
+                                   plan->single_submission ? plan->device_checkpoint : nullptr, plan->checkpoint,
                                    context->stream),
                  "HIP could not write the decode step's state");
   hipEvent_t before = nullptr, after = nullptr;
@@ -221,6 +229,8 @@ int debug_step(llmopt_hip_prebaked *plan, int64_t token, int64_t past_tokens, bo
       const uint32_t past = (uint32_t)past_tokens;
       memcpy(record.parameters.data() + 12, &past, 4);
     }
+    if (!plan->single_submission && plan->is_checkpoint_pack[i] && record.parameters.size() >= 4)
+      memcpy(record.parameters.data(), &plan->checkpoint, 4);
     std::vector<bool> bad_before(record.buffers.size(), false);
     if (nan_check)
       for (size_t b = 0; b < record.buffers.size() && status == LLMOPT_OK; ++b) {
@@ -349,6 +359,7 @@ int llmopt_hip_prebaked_create(llmopt_hip_library *library, const llmopt_hip_dis
     if (status != LLMOPT_OK) break;
     const bool paged = is_reference_paged_attention(items[i].name);
     plan->is_paged_attention.push_back(paged);
+    plan->is_checkpoint_pack.push_back(strcmp(items[i].name, "llmopt_cache_pack_checkpoint_q8_simd") == 0);
     const DispatchRecord &record = plan->records[i];
     if (!paged || record.parameters.size() < 64 || record.buffers.size() < 7) continue;
     plan->past_count = std::max(plan->past_count, param_u32(record, 0));
@@ -358,19 +369,26 @@ int llmopt_hip_prebaked_create(llmopt_hip_library *library, const llmopt_hip_dis
     plan->past_capacity = (uint32_t)std::min<uint64_t>(plan->past_capacity, std::min<uint64_t>(slots, kQ8AttentionSplitTokens));
   }
   plan->is_paged_attention.resize(count, false);
+  plan->is_checkpoint_pack.resize(count, false);
   if (status == LLMOPT_OK && plan->single_submission) {
-    const uint32_t words = std::max<uint32_t>(plan->past_count, 1);
+    const uint32_t past_words = std::max<uint32_t>(plan->past_count, 1);
+    const uint32_t words = past_words + 1;  // the step's checkpoint slot behind the context lengths
     void *block = nullptr;
     if (hipMalloc(&block, (size_t)words * 4) != hipSuccess || hipMemset(block, 0, (size_t)words * 4) != hipSuccess) {
       if (block) (void)hipFree(block);
       status = fail(LLMOPT_ERR_FAILURE, "HIP could not allocate the plan's step state");
     } else {
       plan->device_past = static_cast<uint32_t *>(block);
-      for (size_t i = 0; i < count; ++i)
+      for (size_t i = 0; i < count; ++i) {
         if (plan->is_paged_attention[i]) {
           plan->records[i].device_past_lengths = plan->device_past;
           plan->records[i].device_past_capacity = plan->past_capacity;
         }
+        if (plan->is_checkpoint_pack[i]) {
+          plan->device_checkpoint = plan->device_past + past_words;
+          plan->records[i].device_checkpoint = plan->device_checkpoint;
+        }
+      }
       status = capture_plan(plan);
     }
   }
@@ -399,8 +417,10 @@ void llmopt_hip_release_prebaked(llmopt_hip_prebaked *plan) {
 
 int llmopt_hip_prebaked_execute(llmopt_hip_prebaked *plan, int64_t token, int64_t past_tokens, int64_t checkpoint,
                                 int64_t *out_token) {
-  (void)checkpoint;  // recurrent-state checkpoints (llmopt_cache_pack_checkpoint_q8_simd) are not part of this backend
   if (plan == nullptr) return fail(LLMOPT_ERR_FAILURE, "HIP prebaked plan has been finalized");
+  // the slot llmopt_cache_pack_checkpoint_q8_simd launches of the plan write this step (as the reference:
+  // the low 32 bits of the argument; the ring queue has no such argument and keeps the last one)
+  plan->checkpoint = (uint32_t)(int32_t)checkpoint;
   int32_t next_token = 0;
   const bool nan_check =
       getenv("LLMOPT_DEBUG_NAN_CHECK") != nullptr && (past_tokens > 0 || getenv("LLMOPT_CHECK_PREFILL") != nullptr);

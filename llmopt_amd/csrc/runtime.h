@@ -97,6 +97,10 @@ struct DispatchRecord {
   // step of a sequence.
   const uint32_t *device_past_lengths = nullptr;
   uint32_t device_past_capacity = 0;
+  // Set by a retained plan on its llmopt_cache_pack_checkpoint_q8_simd launches: the checkpoint slot of
+  // the step lives in device memory (the reference rewrites byte 0 of the parameter block per step,
+  // native/ocaml_metal_stubs.m:2186-2188).
+  const uint32_t *device_checkpoint = nullptr;
 };
 
 // A kernel handler checks buffer count, parameter length and buffer sizes

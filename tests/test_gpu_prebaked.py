@@ -233,3 +233,35 @@ def test_nan_check_replay_names_the_first_record_that_produces_a_nan(runtime, mo
     plan.execute(5, 0)  # a clean row again (a buffer that held a NaN before a record is not blamed on it)
     with pytest.raises(Exception):
         plan.execute(7, 0)
+
+
+def test_plan_writes_the_checkpoint_slot_of_each_step(runtime):
+    """llmopt_hip_prebaked_execute's checkpoint argument: the llmopt_cache_pack_checkpoint_q8_simd
+    records of a plan write the slot the step names (native/ocaml_metal_stubs.m:2186-2188 rewrites
+    byte 0 of their parameter block), the other checkpoint entry keeps the slot it was created with."""
+    from llmopt_amd.native import Prebaked
+    from tests.gpu_util import u32s
+    rng = np.random.default_rng(23)
+    layers, layer_elements, slots = 2, 4 * 64, 5
+    elements = layers * layer_elements
+    stride = elements + 2 * (elements // 64)
+    state = (rng.standard_normal(layer_elements) * 2).astype(np.float16)
+    start = np.zeros(slots * stride, dtype=np.uint8)
+    pool = runtime.buffer_of_bytes(start)
+    source = runtime.buffer_of_bytes(state)
+    token = runtime.buffer_of_bytes(np.zeros(1, dtype=np.int64))
+    output = runtime.buffer_of_bytes(np.zeros(1, dtype=np.int32))
+    params = lambda slot, layer: u32s(slot, layer, layer_elements, 64, elements, elements // 64, stride)
+    grid = (layer_elements // 64 * 32, 1, 1)
+    plan = Prebaked(runtime, [("llmopt_cache_pack_checkpoint_q8_simd", [source, pool], params(0, 0), grid, (256, 1, 1)),
+                              ("llmopt_cache_pack_checkpoint_q8", [source, pool], params(4, 1), grid, (256, 1, 1))],
+                    token, output)
+    assert plan.single_submission
+    for slot in (3, 1):
+        plan.execute(0, 0, checkpoint=slot)
+    got = pool.numpy(np.uint8, (slots, stride))
+    written = got[:, :layer_elements].any(axis=1)
+    np.testing.assert_array_equal(written, [False, True, False, True, False])   # layer 0: the slots of the two steps
+    np.testing.assert_array_equal(got[3, :layer_elements], got[1, :layer_elements])
+    assert got[4, layer_elements:elements].any() and not got[:4, layer_elements:elements].any()  # layer 1: slot 4 only
+    del plan

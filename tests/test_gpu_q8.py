@@ -592,3 +592,54 @@ def test_random_suffix_prefill(runtime, case):
     expected = oracle.paged_attention_q8(query, ck, cv, pool, slots, mask, params)
     assert_close_to_oracle(out, expected, f"random suffix prefill {case}: D={dim} {h}/{kvh} x{b}, {q_len} after {past}, "
                                           f"layer {layer} of {layers}")
+
+
+def checkpoint_layout(layers, layer_elements):
+    elements = layers * layer_elements
+    return elements, elements + 2 * (elements // 64)
+
+
+def quantize_groups(state):
+    """The quantiser of lib/metal_cache_source.ml:245-272 on a flat f16 state, group by group."""
+    groups = state.astype(np.float32).reshape(-1, 64)
+    maximum = np.abs(groups).max(axis=1)
+    scale = np.where(maximum == 0, np.float32(1.0), maximum / np.float32(127.0)).astype(np.float16)
+    values = np.clip(np.rint(groups / scale.astype(np.float32)[:, None]), -127, 127).astype(np.int8)
+    return values.reshape(-1), scale
+
+
+@pytest.mark.parametrize("name", ["llmopt_cache_pack_checkpoint_q8", "llmopt_cache_pack_checkpoint_q8_simd"])
+def test_checkpoint_pack_and_unpack_are_bit_exact(runtime, name):
+    """One layer's recurrent state into slot `checkpoint` of a pool of checkpoints and back
+    (lib/metal_cache_source.ml:245-343): int8 values and f16 scales against the quantiser's definition,
+    the other layers and the other slots untouched, the unpacked halves against int8 x scale."""
+    rng = np.random.default_rng(17)
+    layers, layer_elements, slots = 3, 5 * 64, 4
+    elements, stride = checkpoint_layout(layers, layer_elements)
+    state = (rng.standard_normal(layer_elements) * 3).astype(np.float16)
+    state[64:128] = 0  # an all-zero group stores scale 1.0
+    start = rng.integers(0, 256, size=slots * stride, dtype=np.uint8)
+    pool = runtime.buffer_of_bytes(start)
+    layer, checkpoint = 1, 2
+    params = u32s(checkpoint, layer, layer_elements, 64, elements, elements // 64, stride)
+    runtime.dispatch(name, [runtime.buffer_of_bytes(state), pool], params,
+                     grid=(layer_elements // 64 * 32, 1, 1), group=(256, 1, 1))
+    got = pool.numpy(np.uint8, (slots, stride))
+    values, scales = quantize_groups(state)
+    expected = start.reshape(slots, stride).copy()
+    expected[checkpoint, layer * layer_elements:(layer + 1) * layer_elements] = values.view(np.uint8)
+    groups = layer_elements // 64
+    expected[checkpoint, elements + 2 * layer * groups:elements + 2 * (layer + 1) * groups] = scales.view(np.uint8)
+    np.testing.assert_array_equal(got, expected)
+    assert scales[1] == np.float16(1.0)
+    want = (values.astype(np.float32).reshape(-1, 64) * scales.astype(np.float32)[:, None]).astype(np.float16)
+    for unpack in ("llmopt_cache_unpack_checkpoint_q8", "llmopt_cache_unpack_checkpoint_q8_vec4"):
+        destination = runtime.buffer_of_bytes(np.full(layer_elements, np.nan, dtype=np.float16))
+        runtime.dispatch(unpack, [pool, destination], params, grid=(layer_elements, 1, 1), group=(256, 1, 1))
+        np.testing.assert_array_equal(destination.numpy(np.uint16, (layer_elements,)), want.reshape(-1).view(np.uint16))
+    with pytest.raises(Exception, match="pool buffer is too small"):
+        runtime.dispatch(name, [runtime.buffer_of_bytes(state), pool],
+                         u32s(slots, layer, layer_elements, 64, elements, elements // 64, stride))
+    with pytest.raises(Exception, match="layer lies outside"):
+        runtime.dispatch(name, [runtime.buffer_of_bytes(state), pool],
+                         u32s(0, layers, layer_elements, 64, elements, elements // 64, stride))
