@@ -372,6 +372,7 @@ def check_tokens(tokens, expected_logits):
 @pytest.mark.parametrize("m,n,k,dtype,extra,staged", [
     (1, 49152, 576, np.float16, False, True),   # the decode LM head, two-stage form
     (1, 1000, 576, np.float16, True, False),
+    (2, 16400, 576, np.float16, True, False),   # a wide head with its logits
     (3, 2048, 640, np.float32, True, True),
     (8, 520, 2048, np.float16, False, False),
     (11, 300, 128, np.float16, True, False),    # more rows than one GEMV launch takes

@@ -136,7 +136,9 @@ def test_runtime_smoke_is_exact(runtime, golden, with_bias):
 
 
 GEMV_SHAPES = [(1, 1536, 576), (1, 4096, 4096), (2, 512, 4096), (3, 260, 1024), (4, 96, 14336),
-               (5, 64, 640), (8, 200, 4096), (8, 33, 14336), (7, 1, 64)]
+               (5, 64, 640), (8, 200, 4096), (8, 33, 14336), (7, 1, 64),
+               # many short rows: one and two activation rows on the matrix-core kernel
+               (1, 16384, 576), (2, 20008, 1024), (2, 16385, 64)]
 
 
 @pytest.mark.parametrize("m,n,k", GEMV_SHAPES)
