@@ -199,6 +199,12 @@ int llmopt_hip_commit_batch_async(llmopt_hip_batch *batch);
  * on the first, in recorded order). */
 int llmopt_hip_commit_batch_profiled(llmopt_hip_batch *batch, int use_graph, int repeats,
                                      float *gpu_milliseconds);
+/* The same commit with every one of the `repeats` timed runs measured on its own (a HIP
+ * event between consecutive runs): gpu_milliseconds_each[0 .. repeats) receives their GPU
+ * milliseconds, so that a caller can report a median.  No reference counterpart (the
+ * reference reports one command buffer's GPU time per commit, :1337-1347). */
+int llmopt_hip_commit_batch_profiled_each(llmopt_hip_batch *batch, int use_graph, int repeats,
+                                          float *gpu_milliseconds_each);
 /* caml_llmopt_metal_abort_batch (:1372-1382). */
 int llmopt_hip_abort_batch(llmopt_hip_batch *batch);
 

@@ -129,6 +129,27 @@ int llmopt_op_parameters_paged_attention_q8(uint8_t out[64], int64_t batches, in
                                             int64_t key_offset, int64_t value_offset,
                                             int64_t group_size, int64_t token_stride, double scale,
                                             int64_t mask_dtype, int64_t query_length, int64_t window);
+/* Kv_cache.Format.bytes_for_elements (lib/kv_cache.ml:16-21): `elements` int8 values plus one
+ * f16 scale per group of 64 (the last group may be partial); -1 for a negative count or on
+ * overflow (the reference raises Invalid_argument). */
+int64_t llmopt_op_kv_bytes_for_elements(int64_t elements);
+
+/* Kv_cache.Layout.Attention_layer (lib/kv_cache.ml:27-42) and the region Layout.create_heterogeneous
+ * gives it (lib/kv_cache.ml:44-50,126-152). */
+typedef struct llmopt_op_kv_layer {
+  int64_t kv_heads, head_dim;
+} llmopt_op_kv_layer;
+typedef struct llmopt_op_kv_region {
+  int64_t key_offset, value_offset, segment_elements, segment_bytes;
+} llmopt_op_kv_region;
+/* Kv_cache.Layout.create_heterogeneous for attention layers (lib/kv_cache.ml:80-166): every
+ * token's pool slot holds each layer's keys, then its values, layers side by side, then all
+ * f16 group scales.  Writes the per-layer regions (regions may be NULL), token_elements and
+ * bytes_per_token (the slot stride).  Same checks and messages: positive kv_heads / head_dim,
+ * "Q8 KV group_size must divide each attention head dimension", "... overflows". */
+int llmopt_op_kv_layout(const llmopt_op_kv_layer *layers, size_t layer_count, llmopt_op_kv_region *regions,
+                        int64_t *token_elements, int64_t *bytes_per_token);
+
 /* Kernel_abi.Operation.to_string of an entry name this library implements
  * (lib/kernel_abi.ml:37-70), NULL for an unknown name. */
 const char *llmopt_op_kernel_operation(const char *kernel_name);

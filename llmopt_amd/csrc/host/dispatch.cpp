@@ -526,6 +526,44 @@ int llmopt_op_parameters_paged_attention_q8(uint8_t out[64], int64_t batches, in
   return LLMOPT_OK;
 }
 
+// Kv_cache.Format.bytes_for_elements (lib/kv_cache.ml:10-21).
+int64_t llmopt_op_kv_bytes_for_elements(int64_t elements) {
+  if (elements < 0) return -1;
+  const int64_t groups = elements / 64 + (elements % 64 == 0 ? 0 : 1);
+  if (groups > (kMaxInt - elements) / 2) return -1;
+  return elements + 2 * groups;
+}
+
+// Kv_cache.Layout.create_heterogeneous, attention layers only (lib/kv_cache.ml:80-166).
+int llmopt_op_kv_layout(const llmopt_op_kv_layer *layers, size_t layer_count, llmopt_op_kv_region *regions,
+                        int64_t *token_elements, int64_t *bytes_per_token) {
+  if (layers == nullptr && layer_count != 0) return fail(LLMOPT_ERR_INVALID, "KV layout needs its attention layers");
+  for (size_t i = 0; i < layer_count; ++i) {  // Attention_layer.create, :33-38
+    if (layers[i].kv_heads <= 0) return fail(LLMOPT_ERR_FAILURE, "attention KV layer requires positive kv_heads");
+    if (layers[i].head_dim <= 0) return fail(LLMOPT_ERR_FAILURE, "attention KV layer requires positive head_dim");
+  }
+  for (size_t i = 0; i < layer_count; ++i)
+    if (layers[i].head_dim % 64 != 0)
+      return fail(LLMOPT_ERR_FAILURE, "Q8 KV group_size must divide each attention head dimension");
+  int64_t offset = 0;
+  for (size_t i = 0; i < layer_count; ++i) {
+    if (layers[i].kv_heads > kMaxInt / layers[i].head_dim)
+      return fail(LLMOPT_ERR_FAILURE, "attention KV layer element count overflows");
+    const int64_t elements = layers[i].kv_heads * layers[i].head_dim;
+    const int64_t segment_bytes = llmopt_op_kv_bytes_for_elements(elements);
+    if (segment_bytes < 0) return fail(LLMOPT_ERR_FAILURE, "attention KV segment byte length overflows");
+    if (elements > kMaxInt - offset || elements > kMaxInt - (offset + elements))
+      return fail(LLMOPT_ERR_FAILURE, "KV token element count overflows");
+    if (regions != nullptr) regions[i] = {offset, offset + elements, elements, segment_bytes};
+    offset += 2 * elements;
+  }
+  const int64_t bytes = llmopt_op_kv_bytes_for_elements(offset);
+  if (bytes < 0) return fail(LLMOPT_ERR_FAILURE, "KV token byte length overflows");
+  if (token_elements != nullptr) *token_elements = offset;
+  if (bytes_per_token != nullptr) *bytes_per_token = bytes;
+  return LLMOPT_OK;
+}
+
 const char *llmopt_op_kernel_operation(const char *kernel_name) {
   if (kernel_name == nullptr) return nullptr;
   const llmopt::KernelEntryPoint *entry = llmopt::find_kernel(kernel_name);

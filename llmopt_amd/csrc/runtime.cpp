@@ -695,8 +695,13 @@ static int submit_batch(llmopt_hip_batch *batch, bool wait) {
 int llmopt_hip_commit_batch(llmopt_hip_batch *batch) { return submit_batch(batch, true); }
 int llmopt_hip_commit_batch_async(llmopt_hip_batch *batch) { return submit_batch(batch, false); }
 
-int llmopt_hip_commit_batch_profiled(llmopt_hip_batch *batch, int use_graph, int repeats,
-                                     float *gpu_milliseconds) {
+}  // extern "C"
+
+namespace {
+
+// The profiled commit: `each`, when not null, receives the GPU milliseconds of every one of the
+// `repeats` timed runs (an event between consecutive runs); `total` their sum from first to last event.
+int commit_profiled(llmopt_hip_batch *batch, int use_graph, int repeats, float *gpu_milliseconds, float *each) {
   if (int status = require_active_batch(batch)) return status;
   if (repeats <= 0) return fail(LLMOPT_ERR_INVALID, "profiled commit needs a positive repeat count");
   constexpr int kMaxBranches = 4;  // hardware queues a process gets by default
@@ -758,6 +763,7 @@ int llmopt_hip_commit_batch_profiled(llmopt_hip_batch *batch, int use_graph, int
   hipGraph_t graph = nullptr;
   hipGraphExec_t executable = nullptr;
   hipEvent_t start = nullptr, stop = nullptr, fork = nullptr, joined[kMaxBranches] = {};
+  std::vector<hipEvent_t> between;  // after every run but the last, when each run is timed
   if (status == LLMOPT_OK && use_graph) {
     for (int b = 1; b < branches && status == LLMOPT_OK; ++b)
       if (hipStreamCreateWithFlags(&side[b], hipStreamNonBlocking) != hipSuccess ||
@@ -789,6 +795,12 @@ int llmopt_hip_commit_batch_profiled(llmopt_hip_batch *batch, int use_graph, int
   if (status == LLMOPT_OK &&
       (hipEventCreate(&start) != hipSuccess || hipEventCreate(&stop) != hipSuccess))
     status = fail(LLMOPT_ERR_FAILURE, "HIP could not create timing events");
+  if (status == LLMOPT_OK && each != nullptr) {
+    between.assign((size_t)repeats - 1, nullptr);
+    for (hipEvent_t &event : between)
+      if (status == LLMOPT_OK && hipEventCreate(&event) != hipSuccess)
+        status = fail(LLMOPT_ERR_FAILURE, "HIP could not create timing events");
+  }
   if (status == LLMOPT_OK) {
     (void)hipEventRecord(start, stream);
     for (int i = 0; i < repeats && status == LLMOPT_OK; ++i) {
@@ -798,6 +810,7 @@ int llmopt_hip_commit_batch_profiled(llmopt_hip_batch *batch, int use_graph, int
       } else {
         status = launch_all(false, false);
       }
+      if (each != nullptr && i + 1 < repeats) (void)hipEventRecord(between[(size_t)i], stream);
     }
     (void)hipEventRecord(stop, stream);
     if (hipStreamSynchronize(stream) != hipSuccess && status == LLMOPT_OK)
@@ -806,7 +819,14 @@ int llmopt_hip_commit_batch_profiled(llmopt_hip_batch *batch, int use_graph, int
     if (status == LLMOPT_OK && hipEventElapsedTime(&elapsed, start, stop) != hipSuccess)
       status = fail(LLMOPT_ERR_FAILURE, "HIP could not read the timing events");
     if (gpu_milliseconds) *gpu_milliseconds = elapsed;
+    for (int i = 0; i < repeats && status == LLMOPT_OK && each != nullptr; ++i) {
+      hipEvent_t from = i == 0 ? start : between[(size_t)i - 1], to = i + 1 == repeats ? stop : between[(size_t)i];
+      if (hipEventElapsedTime(&each[i], from, to) != hipSuccess)
+        status = fail(LLMOPT_ERR_FAILURE, "HIP could not read the timing events");
+    }
   }
+  for (hipEvent_t event : between)
+    if (event) (void)hipEventDestroy(event);
   if (start) (void)hipEventDestroy(start);
   if (stop) (void)hipEventDestroy(stop);
   if (executable) (void)hipGraphExecDestroy(executable);
@@ -819,6 +839,21 @@ int llmopt_hip_commit_batch_profiled(llmopt_hip_batch *batch, int use_graph, int
   }
   clear_batch(batch);
   return status;
+}
+
+}  // namespace
+
+extern "C" {
+
+int llmopt_hip_commit_batch_profiled(llmopt_hip_batch *batch, int use_graph, int repeats,
+                                     float *gpu_milliseconds) {
+  return commit_profiled(batch, use_graph, repeats, gpu_milliseconds, nullptr);
+}
+
+int llmopt_hip_commit_batch_profiled_each(llmopt_hip_batch *batch, int use_graph, int repeats,
+                                          float *gpu_milliseconds_each) {
+  if (gpu_milliseconds_each == nullptr) return fail(LLMOPT_ERR_INVALID, "profiled commit needs room for the timings");
+  return commit_profiled(batch, use_graph, repeats, nullptr, gpu_milliseconds_each);
 }
 
 int llmopt_hip_abort_batch(llmopt_hip_batch *batch) {

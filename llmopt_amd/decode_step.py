@@ -19,6 +19,7 @@ rewrites those buffers after a step.
 """
 from __future__ import annotations
 
+import functools
 import math
 import struct
 from dataclasses import dataclass
@@ -38,6 +39,12 @@ def linear_grid(columns: int) -> int:
     return ((columns + 7) // 8) * 8 * 32
 
 
+@functools.lru_cache(maxsize=None)
+def _kv_layout(layers: int, kv_heads: int, head_dim: int):
+    from . import ops
+    return ops.kv_layout([(kv_heads, head_dim)] * layers)
+
+
 @dataclass(frozen=True)
 class DecodeConfig:
     hidden: int = 576
@@ -51,17 +58,26 @@ class DecodeConfig:
     rope_theta: float = 10000.0
 
     @property
+    def kv_layout(self):
+        """Kv_cache.Layout of this model's attention layers (lib/kv_cache.ml:126-166), from the
+        library's llmopt_op_kv_layout."""
+        return _kv_layout(self.layers, self.kv_heads, self.head_dim)
+
+    @property
     def layer_elements(self) -> int:
-        return 2 * self.kv_heads * self.head_dim
+        """Keys plus values of one layer in a token's slot (layers are uniform here: the key offset
+        of layer i is i * layer_elements, its values follow its keys)."""
+        key_offset, value_offset, segment, _ = self.kv_layout.regions[0]
+        return 2 * segment
 
     @property
     def token_elements(self) -> int:
-        return self.layers * self.layer_elements
+        return self.kv_layout.token_elements
 
     @property
     def token_stride(self) -> int:
-        """Kv_cache.Layout bytes per token: int8 values + one f16 scale per 64 (lib/kv_cache.ml:126-166)."""
-        return self.token_elements + 2 * (self.token_elements // 64)
+        """Bytes per token: int8 values + one f16 scale per 64."""
+        return self.kv_layout.bytes_per_token
 
 
 def rope_rows(config: DecodeConfig, positions) -> tuple[np.ndarray, np.ndarray]:

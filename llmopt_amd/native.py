@@ -103,6 +103,8 @@ def lib() -> ctypes.CDLL:
         "llmopt_hip_commit_batch_async": (ctypes.c_int, [vp]),
         "llmopt_hip_commit_batch_profiled": (ctypes.c_int, [vp, ctypes.c_int, ctypes.c_int,
                                                            ctypes.POINTER(ctypes.c_float)]),
+        "llmopt_hip_commit_batch_profiled_each": (ctypes.c_int, [vp, ctypes.c_int, ctypes.c_int,
+                                                                ctypes.POINTER(ctypes.c_float)]),
         "llmopt_hip_abort_batch": (ctypes.c_int, [vp]),
         "llmopt_hip_prebaked_create": (ctypes.c_int, [vp, item_p, sz, vp, vp, pp]),
         "llmopt_hip_release_prebaked": (None, [vp]),
@@ -142,7 +144,7 @@ EXPORTED_SYMBOLS = (
     "llmopt_hip_begin_batch", "llmopt_hip_release_batch", "llmopt_hip_batch_dispatch",
     "llmopt_hip_batch_dispatch_all", "llmopt_hip_batch_copy", "llmopt_hip_batch_barrier",
     "llmopt_hip_commit_batch", "llmopt_hip_commit_batch_async",
-    "llmopt_hip_commit_batch_profiled", "llmopt_hip_abort_batch",
+    "llmopt_hip_commit_batch_profiled", "llmopt_hip_commit_batch_profiled_each", "llmopt_hip_abort_batch",
     "llmopt_hip_prebaked_create", "llmopt_hip_release_prebaked", "llmopt_hip_prebaked_execute",
     "llmopt_hip_prebaked_is_single_submission",
     "llmopt_hip_ring_create", "llmopt_hip_ring_submit", "llmopt_hip_ring_wait_completion",
@@ -398,6 +400,12 @@ class Batch:
         _check(lib().llmopt_hip_commit_batch_profiled(self._handle, int(use_graph), repeats,
                                                       ctypes.byref(elapsed)))
         return float(elapsed.value)
+
+    def commit_profiled_each(self, repeats: int = 3, use_graph=True) -> list[float]:
+        """The same with every one of the `repeats` runs timed on its own: GPU milliseconds of each."""
+        elapsed = (ctypes.c_float * repeats)()
+        _check(lib().llmopt_hip_commit_batch_profiled_each(self._handle, int(use_graph), repeats, elapsed))
+        return [float(value) for value in elapsed]
 
     def abort(self) -> None:
         _check(lib().llmopt_hip_abort_batch(self._handle))

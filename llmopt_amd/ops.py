@@ -36,6 +36,25 @@ class _CValue(ctypes.Structure):
                 ("dims", ctypes.c_int64 * 8)]
 
 
+class _CKvLayer(ctypes.Structure):
+    _fields_ = [("kv_heads", ctypes.c_int64), ("head_dim", ctypes.c_int64)]
+
+
+class _CKvRegion(ctypes.Structure):
+    _fields_ = [("key_offset", ctypes.c_int64), ("value_offset", ctypes.c_int64),
+                ("segment_elements", ctypes.c_int64), ("segment_bytes", ctypes.c_int64)]
+
+
+@dataclass(frozen=True)
+class KvLayout:
+    """Kv_cache.Layout of attention layers (lib/kv_cache.ml:52-61): token_elements int8 values per
+    token, bytes_per_token (the pool slot stride) and (key_offset, value_offset, segment_elements,
+    segment_bytes) per layer."""
+    token_elements: int
+    bytes_per_token: int
+    regions: tuple
+
+
 class _CPagedConfig(ctypes.Structure):
     _fields_ = [("token_elements", ctypes.c_int64), ("key_offset", ctypes.c_int64),
                 ("value_offset", ctypes.c_int64), ("group_size", ctypes.c_int64),
@@ -49,6 +68,7 @@ OPERATOR_SYMBOLS = (
     "llmopt_op_attention",
     "llmopt_op_paged_attention_kernel_name", "llmopt_op_linear_f16_grid", "llmopt_op_simd_rows_grid",
     "llmopt_op_parameters_paged_attention_q8", "llmopt_op_kernel_operation",
+    "llmopt_op_kv_bytes_for_elements", "llmopt_op_kv_layout",
 )
 
 _configured = False
@@ -82,6 +102,10 @@ def _lib() -> ctypes.CDLL:
         handle.llmopt_op_parameters_paged_attention_q8.argtypes = [ctypes.c_char_p] + [i64] * 12 + [dbl] + [i64] * 3
         handle.llmopt_op_kernel_operation.argtypes = [ctypes.c_char_p]
         handle.llmopt_op_kernel_operation.restype = ctypes.c_char_p
+        handle.llmopt_op_kv_bytes_for_elements.argtypes = [i64]
+        handle.llmopt_op_kv_bytes_for_elements.restype = i64
+        handle.llmopt_op_kv_layout.argtypes = [ctypes.POINTER(_CKvLayer), sz, ctypes.POINTER(_CKvRegion),
+                                               ctypes.POINTER(i64), ctypes.POINTER(i64)]
         _configured = True
     return handle
 
@@ -113,6 +137,27 @@ def parameters_paged_attention_q8(*, batches, query_heads, kv_heads, past_length
         token_elements, key_offset, value_offset, group_size, token_stride, float(scale), mask_dtype,
         query_length, window))
     return out.raw
+
+
+def kv_bytes_for_elements(elements: int) -> int:
+    """Kv_cache.Format.bytes_for_elements (lib/kv_cache.ml:16-21)."""
+    result = _lib().llmopt_op_kv_bytes_for_elements(elements)
+    if result < 0:
+        raise LlmoptError("KV element count cannot be negative" if elements < 0 else "Q8 KV byte length overflows")
+    return result
+
+
+def kv_layout(layers: Sequence[tuple]) -> KvLayout:
+    """Kv_cache.Layout.create_heterogeneous over attention layers given as (kv_heads, head_dim)
+    (lib/kv_cache.ml:80-166): where each layer's keys and values sit in a token's pool slot."""
+    count = len(layers)
+    c_layers = (_CKvLayer * max(1, count))(*[_CKvLayer(int(h), int(d)) for h, d in layers])
+    regions = (_CKvRegion * max(1, count))()
+    elements, stride = ctypes.c_int64(), ctypes.c_int64()
+    native._check(_lib().llmopt_op_kv_layout(c_layers, count, regions, ctypes.byref(elements), ctypes.byref(stride)))
+    return KvLayout(elements.value, stride.value,
+                    tuple((r.key_offset, r.value_offset, r.segment_elements, r.segment_bytes)
+                          for r in regions[:count]))
 
 
 def kernel_operation(name: str) -> Optional[str]:

@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 from tests.gpu_util import assert_close_to_oracle
-from tests.test_gpu_decode_step import oracle_step
+from oracle.chain import decode_chain as oracle_step
 
 pytestmark = pytest.mark.gpu
 

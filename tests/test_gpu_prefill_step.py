@@ -2,15 +2,11 @@
 pack of every token and causal dense attention -> LM-head argmax of the last token) built by
 llmopt_amd.prefill_step against the same chain composed from the CPU oracle, and of the decode
 step that continues from the pool the prefill filled."""
-import math
-
 import numpy as np
 import pytest
 
-import oracle
-from oracle import CacheParams
 from tests.gpu_util import assert_close_to_oracle
-from tests.test_gpu_decode_step import f16, oracle_step
+from oracle.chain import decode_chain as oracle_step, prefill_chain as oracle_prefill
 
 pytestmark = pytest.mark.gpu
 
@@ -21,46 +17,6 @@ def runtime():
     rt = Runtime()
     yield rt
     rt.close()
-
-
-def oracle_prefill(config, weights, tokens, slots, pool):
-    """The whole prompt through the oracle, every kernel boundary rounded to half as the kernels
-    store it; returns the residual stream [tokens, hidden], the last token's logits and the pool."""
-    from llmopt_amd.decode_step import rope_rows
-    c = config
-    t = len(tokens)
-    pool = pool.copy()
-    cos, sin = rope_rows(c, np.arange(t))
-    x = weights["embedding"][np.asarray(tokens)]
-    causal = np.tril(np.ones((t, t), dtype=np.float32))[None, None]
-    for index, layer in enumerate(weights["layers"]):
-        key_offset = index * c.layer_elements
-        value_offset = key_offset + c.kv_heads * c.head_dim
-        n1 = f16(oracle.rms_norm(x, layer["attn_norm"], c.epsilon))
-        q = f16(oracle.w4a16_linear(n1, *layer["q"], None)).reshape(t, c.q_heads, c.head_dim)
-        k = f16(oracle.w4a16_linear(n1, *layer["k"], None)).reshape(t, c.kv_heads, c.head_dim)
-        v = f16(oracle.w4a16_linear(n1, *layer["v"], None)).reshape(t, c.kv_heads, c.head_dim)
-        q_rot = f16(oracle.rotary_h(q, cos, sin))  # [heads, tokens, d]
-        k_rot = f16(oracle.rotary_h(k, cos, sin))
-        v_heads = np.ascontiguousarray(v.transpose(1, 0, 2))
-        for source, offset in ((k_rot, key_offset), (v_heads, value_offset)):
-            oracle.q8_pack(source, slots, pool,
-                           CacheParams(items=t, segment_offset=offset, heads=c.kv_heads, head_dim=c.head_dim,
-                                       group_size=64, token_elements=c.token_elements,
-                                       token_groups=c.token_elements // 64, token_stride=c.token_stride,
-                                       source_items=t, source_offset=0))
-        repeat = c.q_heads // c.kv_heads
-        attention = oracle.attention(q_rot[None], np.repeat(k_rot, repeat, axis=0)[None],
-                                     np.repeat(v_heads, repeat, axis=0)[None], causal, 1.0 / math.sqrt(c.head_dim))
-        attention = f16(attention[0].transpose(1, 0, 2).reshape(t, -1))  # token-major [tokens, heads * d]
-        x_mid = f16(oracle.add(oracle.w4a16_linear(attention, *layer["o"], None), x.astype(np.float32)))
-        n2 = f16(oracle.rms_norm(x_mid, layer["ffn_norm"], c.epsilon))
-        product = f16(oracle.silu_mul(oracle.w4a16_linear(n2, *layer["gate"], None),
-                                      oracle.w4a16_linear(n2, *layer["up"], None)))
-        x = f16(oracle.add(oracle.w4a16_linear(product, *layer["down"], None), x_mid.astype(np.float32)))
-    final = oracle.rms_norm(x[-1:], weights["final_norm"], c.epsilon)
-    logits = oracle.w4a16_linear(final, *weights["lm_head"], None)[0]
-    return x, logits, pool
 
 
 @pytest.mark.parametrize("tokens,layers", [(5, 2), (48, 2), (133, 2), (133, 1), (300, 1)])

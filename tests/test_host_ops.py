@@ -93,3 +93,39 @@ def test_header_and_python_list_the_same_operator_symbols():
     text = re.sub(r"/\*.*?\*/", "", open(os.path.join(root, "include", "llmopt_hip_ops.h")).read(), flags=re.S)
     declared = sorted(set(re.findall(r"\b(llmopt_op_[a-z0-9_]+)\s*\(", text)))
     assert declared == sorted(ops.OPERATOR_SYMBOLS)
+
+
+def test_kv_layout_matches_the_reference_gemma_numbers():
+    """test/test_cache.ml:183-320: 48 layers, every sixth one global (1 KV head of 512), the others
+    sliding (8 KV heads of 256): 172 032 elements and 177 408 bytes per token, layer 5's keys at
+    20 480 and values at 20 992, layer 6's keys at 21 504, a pool of 8 tokens 1 419 264 bytes."""
+    import json
+    import os
+    golden = json.load(open(os.path.join(os.path.dirname(__file__), "golden", "reference_vectors.json")))
+    layers = [(1, 512) if (layer + 1) % 6 == 0 else (8, 256) for layer in range(48)]
+    layout = ops.kv_layout(layers)
+    assert layout.token_elements == golden["kv_layout_gemma"]["token_elements"] == 172032
+    assert layout.bytes_per_token == golden["kv_layout_gemma"]["bytes_per_token"] == 177408
+    assert layout.regions[5][:2] == (20480, 20992)
+    assert layout.regions[6][0] == 21504
+    assert layout.regions[5][2:] == (512, 512 + 2 * 8) and layout.regions[0][2:] == (2048, 2048 + 2 * 32)
+    assert 8 * layout.bytes_per_token == 1419264
+
+
+def test_kv_layout_of_the_benchmark_shapes_and_its_errors():
+    from llmopt_amd.decode_step import DecodeConfig
+    # C4: one layer of 8 KV heads of 128 -> 2048 + 64 bytes; C5: 30 layers of 3 KV heads of 64 -> 11 520 + 360
+    assert ops.kv_layout([(8, 128)]).bytes_per_token == 2112
+    config = DecodeConfig()
+    assert (config.token_elements, config.token_stride, config.layer_elements) == (11520, 11880, 384)
+    assert config.kv_layout.regions[7][:2] == (7 * 384, 7 * 384 + 192)
+    # Kv_cache.Format.bytes_for_elements (lib/kv_cache.ml:10-21): a partial last group has a scale of its own
+    assert [ops.kv_bytes_for_elements(n) for n in (0, 1, 64, 65, 128)] == [0, 3, 66, 69, 132]
+    for layers, message in (([(0, 64)], "attention KV layer requires positive kv_heads"),
+                            ([(2, 0)], "attention KV layer requires positive head_dim"),
+                            ([(2, 96)], "Q8 KV group_size must divide each attention head dimension"),
+                            ([(2 ** 40, 2 ** 30)], "attention KV layer element count overflows")):
+        with pytest.raises(ops.LlmoptError, match=message):
+            ops.kv_layout(layers)
+    with pytest.raises(ops.LlmoptError):
+        ops.kv_bytes_for_elements(-1)
