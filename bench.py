@@ -432,7 +432,7 @@ def pool_block(rng, config, context):
     return block
 
 
-def verify_decode_chain(runtime, batch, context, rng):
+def verify_decode_chain(runtime, batch, context, rng, fused=None):
     """Checker: a two-layer copy of the timed decode step (same batch, same context, same kernels
     per layer; vocabulary 2048) against the oracle's chain on up to six of its sequences."""
     from llmopt_amd.decode_step import DecodeConfig, DecodeStep, random_weights
@@ -442,7 +442,7 @@ def verify_decode_chain(runtime, batch, context, rng):
     block = pool_block(rng, small, context)
     pool, slots, offsets, new_slots = decode_inputs(runtime, small, batch, context, block)
     step = DecodeStep(runtime, small, weights, batch, pool, runtime.buffer_of_bytes(slots), offsets,
-                      [context] * batch, new_slots, [context] * batch)
+                      [context] * batch, new_slots, [context] * batch, fused=fused)
     tokens = rng.integers(0, small.vocabulary, batch)
     got_tokens = step.run(tokens)
     got_hidden = step.work["x"][0].numpy(np.float16, (batch, small.hidden)).astype(np.float64)
@@ -462,7 +462,7 @@ def verify_decode_chain(runtime, batch, context, rng):
     return bool(np.all(np.isfinite(got_hidden)) and rel_l2 <= 4e-3 and tokens_ok), rel_l2, len(sample)
 
 
-def bench_decode_step(runtime, batches=(1, 8, 32, 128), context=2048, use_graph=True):
+def bench_decode_step(runtime, batches=(1, 8, 32, 128), context=2048, use_graph=True, fused=None):
     """C5: one decode step of the 30-layer model (hidden 576, 9/3 heads of 64, MLP 1536,
     vocabulary 49152), every sequence with `context` tokens in the Q8 pool, replayed as a
     HIP graph.  tokens/s = batch / step time.  Checked outside the timed region: what the replayed
@@ -477,7 +477,7 @@ def bench_decode_step(runtime, batches=(1, 8, 32, 128), context=2048, use_graph=
     for batch in batches:
         pool, slots, offsets, new_slots = decode_inputs(runtime, config, batch, context, block)
         step = DecodeStep(runtime, config, weights, batch, pool, runtime.buffer_of_bytes(slots), offsets,
-                          [context] * batch, new_slots, [context] * batch)
+                          [context] * batch, new_slots, [context] * batch, fused=fused)
         tokens = rng.integers(0, config.vocabulary, batch)
         eager_tokens = step.run(tokens)  # first-use allocations; and the eager result the replay must repeat
         eager_hidden = step.work["x"][0].numpy(np.uint16, (batch, config.hidden))
@@ -510,9 +510,10 @@ def bench_decode_step(runtime, batches=(1, 8, 32, 128), context=2048, use_graph=
             single = plan.single_submission
             del plan
         launches, weight_bytes, kv_bytes = len(step.dispatches), step.weight_bytes(), step.kv_bytes()
+        fused_step = step.fused
         del step, pool
-        chain_ok, chain_rel_l2, chain_sequences = verify_decode_chain(runtime, batch, context, rng)
-        results.append({"batch": batch, "context": context, "launches": launches,
+        chain_ok, chain_rel_l2, chain_sequences = verify_decode_chain(runtime, batch, context, rng, fused)
+        results.append({"batch": batch, "context": context, "launches": launches, "launches_per_layer": 4 if fused_step else 6,
                         "ms_per_step": round(ms, 4), "tokens_per_s": round(batch / (ms * 1e-3), 1),
                         "prebaked_execute_wall_ms": None if execute_ms is None else round(execute_ms, 4),
                         "prebaked_execute_tokens_per_s": None if execute_ms is None
@@ -743,6 +744,8 @@ def main():
     parser.add_argument("--decode-eager", action="store_true",
                         help="launch the decode step from the host instead of replaying a HIP graph")
     parser.add_argument("--decode-batches", default="1,8,32,128", help="batch sizes of the decode-step extra")
+    parser.add_argument("--decode-fused", choices=("auto", "on", "off"), default="auto",
+                        help="the decode step as four launches a layer (on), six (off), or whichever the step picks")
     parser.add_argument("--serial-only", action="store_true",
                         help="leave out the concurrent-branch graphs and the warm (cached) per-case loops: every "
                              "launch of the run then is a serial, cold one (for kernel traces)")
@@ -804,7 +807,8 @@ def main():
         extras["prefill_attention"] = bench_prefill_attention(runtime)
     if "decode" in wanted:
         extras["decode_step"] = bench_decode_step(
-            runtime, batches=tuple(int(b) for b in args.decode_batches.split(",")), use_graph=not args.decode_eager)
+            runtime, batches=tuple(int(b) for b in args.decode_batches.split(",")), use_graph=not args.decode_eager,
+            fused={"auto": None, "on": True, "off": False}[args.decode_fused])
     if "prefill" in wanted:
         extras["prefill_step"] = bench_prefill(runtime)
     # refuse to print numbers whose outputs did not match the oracle

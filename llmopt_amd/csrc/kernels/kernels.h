@@ -83,6 +83,62 @@ hipError_t launch_w4a16_linear(const W4LinearArgs &args, hipStream_t stream);
 hipError_t launch_w4a16_qkv(const W4QkvArgs &args, hipStream_t stream);
 hipError_t launch_w4a16_dual_swiglu(const W4DualSwigluArgs &args, hipStream_t stream);
 
+// ---- fused decode-step launches (no reference kernels; small activations: k <= 2048) ----------
+//
+// A decode step at small batch is bound by the number of its launches, not by their bytes: these
+// kernels do in one launch what several reference kernels do in a row, with the same arithmetic
+// at every rounding point.
+
+// The residual stream of a layer arrives as x plus, when partial_count != 0, the pending partial
+// sums of the previous layer's down projection: row r of the stream is
+// half(sum_p partials[p][r][:] (p ascending, float32) + float(x[r][:])), the value
+// llmopt_w4a16_down_add_f16_g64 would have stored.  Every workgroup forms the rows it needs; the
+// first writes them to x_out (may be null).
+struct FusedResidual {
+  const uint16_t *x;      // f16 [m, k]
+  const float *partials;  // f32 [partial_count, m, k], may be null when partial_count == 0
+  uint32_t partial_count;
+  uint16_t *x_out;        // f16 [m, k]
+};
+constexpr uint32_t kFusedMaxPartials = 32;
+constexpr uint32_t kFusedMaxWidth = 2048;
+
+// llmopt_rms_norm_f16_simd + llmopt_w4a16_qkv_linear_f16_g64 + llmopt_rotary_qk_f16_simd_h64 +
+// llmopt_cache_pack_attention_q8_pair_simd for one new token per sequence, heads of 64: a
+// workgroup owns one head of one sequence - both halves of every rotation pair and the whole
+// Q8 group - so nothing is handed over between workgroups.
+struct FusedQkvArgs {
+  FusedResidual in;
+  W4Norm norm;              // weight_first = 0
+  W4Matrix w[3];            // q, k, v
+  uint32_t n[3];            // multiples of 64
+  const uint16_t *cosine, *sine;  // f16 [m, 64]
+  uint16_t *q_out, *k_out;  // rotated, f16 [m, n[0]], [m, n[1]]
+  uint16_t *v_out;          // f16 [m, n[2]]
+  const uint32_t *slots;    // [m]: pool slot of every sequence's new token
+  uint8_t *pool;
+  uint32_t m, k;
+  uint32_t key_offset, value_offset, token_elements, token_stride;
+};
+bool fused_qkv_ok(const FusedQkvArgs &args);
+hipError_t launch_fused_qkv(const FusedQkvArgs &args, hipStream_t stream);
+
+// llmopt_w4a16_swiglu_rms_f16_g64 + llmopt_w4a16_dual_swiglu_f16_g64 + the contraction of
+// llmopt_w4a16_down_add_f16_g64: workgroup j owns the 64 intermediate columns [64 j, 64 j + 64),
+// computes product = half(silu(gate) * up) for them and multiplies it into the down projection's
+// partial sum over those 64 columns, partials[j][r][:] (float32, scale applied).  The sums over j
+// and the residual are taken by the launch that reads the stream next (FusedResidual).
+struct FusedFfnArgs {
+  const uint16_t *x;   // f16 [m, k]
+  W4Norm norm;         // weight_first = 1
+  W4Matrix gate, up;   // [n, k/2]
+  W4Matrix down;       // [k, n/2]
+  float *partials;     // f32 [n / 64, m, k]
+  uint32_t m, n, k;
+};
+bool fused_ffn_ok(uint32_t m, uint32_t n, uint32_t k);
+hipError_t launch_fused_ffn(const FusedFfnArgs &args, hipStream_t stream);
+
 // The product kernels' own nibble decoders run over a whole matrix, as float32 [n, k]:
 // decoder 0 = w4_decode_pairs and 1 = w4_decode_biased (minus its bias), each times the float32
 // scale, i.e. the exact q * s of python/llmopt_backend/quantization.py:91-121; decoder 2 = the

@@ -17,16 +17,6 @@
 namespace llmopt {
 namespace {
 
-// One 64-wide group, one element per lane: the stored scale and this lane's int8 value.
-__device__ __forceinline__ int8_t q8_quantize(float x, uint16_t *stored_scale) {
-  const float maximum = wave_max(fabsf(x));
-  const uint16_t stored = float_to_half_bits(maximum == 0.0f ? 1.0f : maximum / 127.0f);
-  const float scale = half_bits_to_float(stored);
-  const float rounded = rintf(x / scale);
-  *stored_scale = stored;
-  return (int8_t)(int)fminf(fmaxf(rounded, -127.0f), 127.0f);
-}
-
 template <bool PAIR>
 __global__ __launch_bounds__(256) void q8_pack_kernel(Q8PackArgs a) {
   const uint32_t lane = threadIdx.x & 63;

@@ -37,8 +37,8 @@ __device__ __forceinline__ uint16_t float_to_half_bits(float value) {
 //
 // XOR with 8 turns a two's-complement nibble into offset binary (q + 8).  A 4-bit field in the
 // mantissa of 1024.0 (0x6400, ulp 1) or of 64.0 (0x5400, ulp 1/16, field at bits 4..7) reads as
-// 1024 + (q + 8) or 64 + (q + 8) exactly.  Both steps are one XOR after the mask:
-// (w & mask) ^ (magic | (0x88888888 & mask)), the magic bits lying outside the mask.  The four
+// 1024 + (q + 8) or 64 + (q + 8) exactly: ((w ^ 0x88888888) & mask) | magic, the magic bits lying
+// outside the mask.  The four
 // results hold the pairs (k0,k4) (k1,k5) (k2,k6) (k3,k7): the activation is arranged to match.
 struct W4Pairs {
   h2_t p04, p15, p26, p37;
@@ -48,12 +48,14 @@ struct W4Pairs {
 // corrected afterwards by 1032 * sum(x at K offsets 0,4,2,6) + 72 * sum(x at K offsets 1,5,3,7),
 // which does not depend on the weight row.
 __device__ __forceinline__ W4Pairs w4_decode_biased(uint32_t word) {
-  const uint32_t hi = word >> 8;
+  // the sign-bit flip of all eight nibbles at once, then one and-or per pair (six operations a dword)
+  const uint32_t flipped = word ^ 0x88888888u;
+  const uint32_t hi = flipped >> 8;
   W4Pairs out;
-  out.p04 = as_h2((word & 0x000F000Fu) ^ 0x64086408u);
-  out.p15 = as_h2((word & 0x00F000F0u) ^ 0x54805480u);
-  out.p26 = as_h2((hi & 0x000F000Fu) ^ 0x64086408u);
-  out.p37 = as_h2((hi & 0x00F000F0u) ^ 0x54805480u);
+  out.p04 = as_h2((flipped & 0x000F000Fu) | 0x64006400u);
+  out.p15 = as_h2((flipped & 0x00F000F0u) | 0x54005400u);
+  out.p26 = as_h2((hi & 0x000F000Fu) | 0x64006400u);
+  out.p37 = as_h2((hi & 0x00F000F0u) | 0x54005400u);
   return out;
 }
 
@@ -131,16 +133,22 @@ __device__ __forceinline__ float wave_sum(float value) {
 // Rotate-half position encoding of one element (lib/metal_normalization_source.ml:765-802):
 // half(half(x[col] * cos[col]) + half(+-x[col -+ half_dimension] * sin[col])), every product and
 // the sum rounded to half separately.
+// The same on values already in registers: `partner` is the element half_dimension away, negated
+// for the columns of the first half.
+__device__ __forceinline__ _Float16 rotate_half_value(_Float16 value, _Float16 partner, _Float16 cosine,
+                                                      _Float16 sine, bool first_half) {
+#pragma clang fp contract(off)
+  const _Float16 rotated = first_half ? -partner : partner;
+  const _Float16 direct = value * cosine;
+  const _Float16 turned = rotated * sine;
+  return direct + turned;
+}
+
 __device__ __forceinline__ _Float16 rotate_half_element(const _Float16 *input, const _Float16 *cosine,
                                                         const _Float16 *sine, uint32_t col,
                                                         uint32_t half_dimension) {
-#pragma clang fp contract(off)
   const uint32_t rotated_col = col < half_dimension ? col + half_dimension : col - half_dimension;
-  _Float16 rotated = input[rotated_col];
-  if (col < half_dimension) rotated = -rotated;
-  const _Float16 direct = input[col] * cosine[col];
-  const _Float16 turned = rotated * sine[col];
-  return direct + turned;
+  return rotate_half_value(input[col], input[rotated_col], cosine[col], sine[col], col < half_dimension);
 }
 
 __device__ __forceinline__ float wave_max(float value) {
@@ -158,6 +166,18 @@ __device__ __forceinline__ float wave_max(float value) {
   const float r2 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 32));
   const float r3 = __builtin_bit_cast(float, __builtin_amdgcn_readlane(bits, 48));
   return fmaxf(fmaxf(r0, r1), fmaxf(r2, r3));
+}
+
+// Q8 cache quantiser of one 64-wide group, one element per lane (lib/metal_cache_source.ml:62-80):
+// the stored scale half(max|x| / 127) (1.0 for an all-zero group) and this lane's int8 value
+// clamp(rint(x / float(scale)), -127, 127).
+__device__ __forceinline__ int8_t q8_quantize(float x, uint16_t *stored_scale) {
+  const float maximum = wave_max(fabsf(x));
+  const uint16_t stored = float_to_half_bits(maximum == 0.0f ? 1.0f : maximum / 127.0f);
+  const float scale = half_bits_to_float(stored);
+  const float rounded = rintf(x / scale);
+  *stored_scale = stored;
+  return (int8_t)(int)fminf(fmaxf(rounded, -127.0f), 127.0f);
 }
 
 }  // namespace llmopt

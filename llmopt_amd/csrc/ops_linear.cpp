@@ -217,6 +217,111 @@ int w4a16_down_add(llmopt_hip_context *context, const DispatchRecord &record) {
   return launched(launch_w4a16_linear(args, context->stream), record.name.c_str());
 }
 
+// Extension (no reference kernel): one new token per sequence through llmopt_rms_norm_f16_simd,
+// llmopt_w4a16_qkv_linear_f16_g64, llmopt_rotary_qk_f16_simd_h64 and
+// llmopt_cache_pack_attention_q8_pair_simd as ONE launch, heads of 64.  The residual stream comes in as
+// `input` plus `partial_count` pending partial sums of the previous layer's down projection
+// (llmopt_rms_w4a16_swiglu_down_partial_f16_g64), and is written out whole to `stream`.
+// buffers: input f16 [m,k], partials f32 [partial_count,m,k] (any buffer when partial_count = 0),
+// stream f16 [m,k], norm weight, qW, qS, kW, kS, vW, vS, trig f16 [2,m,64] (cosine rows, then sine rows),
+// qOut f16 [m,n_q] (rotated), kOut f16 [m,n_k] (rotated), vOut f16 [m,n_v], slots u32 [m], pool.
+// parameters: u32 m, k, n_q, n_k, n_v; f32 epsilon; u32 partial_count, key_offset, value_offset,
+// token_elements, token_stride.
+int rms_w4a16_qkv_rotary_pack(llmopt_hip_context *context, const DispatchRecord &record) {
+  if (int status = require_buffer_count(record, 16)) return status;
+  if (int status = require_parameter_bytes(record, 44)) return status;
+  const char *name = record.name.c_str();
+  FusedQkvArgs args = {};
+  args.m = param_u32(record, 0);
+  args.k = param_u32(record, 4);
+  args.norm = {as_f16(record.buffers[3]), param_f32(record, 20), 0};
+  args.in.partial_count = param_u32(record, 24);
+  args.key_offset = param_u32(record, 28);
+  args.value_offset = param_u32(record, 32);
+  args.token_elements = param_u32(record, 36);
+  args.token_stride = param_u32(record, 40);
+  static const char *const labels[3] = {"query", "key", "value"};
+  for (int i = 0; i < 3; ++i) {
+    args.n[i] = param_u32(record, 8 + 4 * i);
+    if (int status = check_w4_shape(name, args.m, args.n[i], args.k)) return status;
+    if (args.n[i] % 64 != 0) return fail(LLMOPT_ERR_INVALID, "%s requires whole heads of 64 columns, got %u", name, args.n[i]);
+    if (int status = check_w4_matrix(record.buffers[4 + 2 * i], record.buffers[5 + 2 * i], args.n[i], args.k, labels[i]))
+      return status;
+    if (int status = require_buffer_size(record.buffers[11 + i], (uint64_t)args.m * args.n[i] * 2, "output")) return status;
+    args.w[i] = {record.buffers[4 + 2 * i].device, as_f16(record.buffers[5 + 2 * i])};
+  }
+  if (args.k > kFusedMaxWidth) return fail(LLMOPT_ERR_INVALID, "%s takes activations of at most %u values, got %u", name, kFusedMaxWidth, args.k);
+  if (args.in.partial_count > kFusedMaxPartials)
+    return fail(LLMOPT_ERR_INVALID, "%s takes at most %u partial sums, got %u", name, kFusedMaxPartials, args.in.partial_count);
+  if (!std::isfinite(args.norm.epsilon) || args.norm.epsilon <= 0.0f)
+    return fail(LLMOPT_ERR_INVALID, "%s requires a positive finite epsilon", name);
+  if (args.token_elements % 64 != 0 || args.token_stride % 2 != 0 ||
+      (uint64_t)args.token_stride < (uint64_t)args.token_elements + 2ull * (args.token_elements / 64) ||
+      args.key_offset % 64 != 0 || args.value_offset % 64 != 0 ||
+      (uint64_t)args.key_offset + args.n[1] > args.token_elements ||
+      (uint64_t)args.value_offset + args.n[2] > args.token_elements)
+    return fail(LLMOPT_ERR_INVALID, "%s received an inconsistent Q8 token layout", name);
+  const uint64_t stream_bytes = (uint64_t)args.m * args.k * 2;
+  if (int status = require_buffer_size(record.buffers[0], stream_bytes, "input")) return status;
+  if (args.in.partial_count != 0)
+    if (int status = require_buffer_size(record.buffers[1], (uint64_t)args.in.partial_count * args.m * args.k * 4, "partial sums"))
+      return status;
+  if (int status = require_buffer_size(record.buffers[2], stream_bytes, "stream")) return status;
+  if (int status = require_buffer_size(record.buffers[3], (uint64_t)args.k * 2, "norm weight")) return status;
+  if (int status = require_buffer_size(record.buffers[10], (uint64_t)args.m * 64 * 2 * 2, "cosine and sine rows")) return status;
+  if (int status = require_buffer_size(record.buffers[14], (uint64_t)args.m * 4, "slots")) return status;
+  if (int status = require_buffer_size(record.buffers[15], args.token_stride, "pool")) return status;
+  args.in.x = as_f16(record.buffers[0]);
+  args.in.partials = reinterpret_cast<const float *>(record.buffers[1].device);
+  args.in.x_out = reinterpret_cast<uint16_t *>(record.buffers[2].device);
+  args.cosine = as_f16(record.buffers[10]);
+  args.sine = args.cosine + (size_t)args.m * 64;
+  args.q_out = reinterpret_cast<uint16_t *>(record.buffers[11].device);
+  args.k_out = reinterpret_cast<uint16_t *>(record.buffers[12].device);
+  args.v_out = reinterpret_cast<uint16_t *>(record.buffers[13].device);
+  args.slots = reinterpret_cast<const uint32_t *>(record.buffers[14].device);
+  args.pool = record.buffers[15].device;
+  if (args.in.x == args.in.x_out)
+    return fail(LLMOPT_ERR_INVALID, "%s writes the stream while other workgroups still read the input: two buffers", name);
+  if (!fused_qkv_ok(args)) return fail(LLMOPT_ERR_INVALID, "%s requires 16-byte aligned buffers", name);
+  return launched(launch_fused_qkv(args, context->stream), name);
+}
+
+// Extension (no reference kernel): llmopt_w4a16_swiglu_rms_f16_g64, llmopt_w4a16_dual_swiglu_f16_g64 and
+// the contraction of llmopt_w4a16_down_add_f16_g64 as ONE launch that leaves, per 64 columns of the
+// intermediate, a float32 partial sum of every output; the launch that reads the stream next adds them
+// and the residual (llmopt_rms_w4a16_qkv_rotary_pack_q8_f16_g64).  W4A16SwiGLUFFNParams {u32 m, n, k; f32 eps}.
+// buffers: input f16 [m,k], norm weight, gateW, gateS, upW, upS, downW, downS, partials f32 [n/64,m,k].
+int rms_w4a16_swiglu_down_partial(llmopt_hip_context *context, const DispatchRecord &record) {
+  if (int status = require_buffer_count(record, 9)) return status;
+  if (int status = require_parameter_bytes(record, 16)) return status;
+  const char *name = record.name.c_str();
+  const uint32_t m = param_u32(record, 0), n = param_u32(record, 4), k = param_u32(record, 8);
+  const float epsilon = param_f32(record, 12);
+  if (int status = check_w4_shape(name, m, n, k)) return status;
+  if (!fused_ffn_ok(m, n, k))
+    return fail(LLMOPT_ERR_INVALID, "%s takes a hidden width k whose slice of the three matrices fits a workgroup's "
+                "memory (k <= 1472) and n a multiple of 64 up to %u, got k = %u, n = %u", name, 64 * kFusedMaxPartials, k, n);
+  if (!std::isfinite(epsilon) || epsilon <= 0.0f) return fail(LLMOPT_ERR_INVALID, "%s requires a positive finite epsilon", name);
+  if (int status = require_buffer_size(record.buffers[0], (uint64_t)m * k * 2, "input")) return status;
+  if (int status = require_buffer_size(record.buffers[1], (uint64_t)k * 2, "norm weight")) return status;
+  if (int status = check_w4_matrix(record.buffers[2], record.buffers[3], n, k, "gate")) return status;
+  if (int status = check_w4_matrix(record.buffers[4], record.buffers[5], n, k, "up")) return status;
+  if (int status = check_w4_matrix(record.buffers[6], record.buffers[7], k, n, "down")) return status;
+  if (int status = require_buffer_size(record.buffers[8], (uint64_t)(n / 64) * m * k * 4, "partial sums")) return status;
+  FusedFfnArgs args = {};
+  args.x = as_f16(record.buffers[0]);
+  args.norm = {as_f16(record.buffers[1]), epsilon, 1};
+  args.gate = {record.buffers[2].device, as_f16(record.buffers[3])};
+  args.up = {record.buffers[4].device, as_f16(record.buffers[5])};
+  args.down = {record.buffers[6].device, as_f16(record.buffers[7])};
+  args.partials = reinterpret_cast<float *>(record.buffers[8].device);
+  args.m = m;
+  args.n = n;
+  args.k = k;
+  return launched(launch_fused_ffn(args, context->stream), name);
+}
+
 // Extension (no reference kernel): float32 [n,k] from the product kernels' own nibble decoders,
 // for checking the unpack arithmetic bit for bit.  Parameters {u32 n, k} or {u32 n, k, decoder}:
 // decoder 0 (default) = w4_decode_pairs x scale, 1 = w4_decode_biased minus its bias x scale, 2 = the
@@ -275,6 +380,8 @@ void register_linear_kernels(std::vector<KernelEntryPoint> &table) {
   table.push_back({"llmopt_w4a16_down_add_f16_g64", ffn, w4a16_down_add});
   table.push_back({"llmopt_w4a16_down_add_f16_g64_m4", ffn, w4a16_down_add});
   table.push_back({"llmopt_w4a16_down_add_f16_g64_m8", ffn, w4a16_down_add});
+  table.push_back({"llmopt_rms_w4a16_qkv_rotary_pack_q8_f16_g64", qkv, rms_w4a16_qkv_rotary_pack});
+  table.push_back({"llmopt_rms_w4a16_swiglu_down_partial_f16_g64", ffn, rms_w4a16_swiglu_down_partial});
   table.push_back({"llmopt_w4_dequant_f32", linear, w4_dequant_f32});
   table.push_back({"llmopt_q8_decode_f32", "cache", q8_decode_f32});
 }

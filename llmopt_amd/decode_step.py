@@ -29,6 +29,13 @@ import numpy as np
 from .native import Buffer, Runtime
 
 
+# Above this many sequences the fused launches (one or two sequences per workgroup, every workgroup
+# reading and decoding its weights again) cost more than the launches they save: measured at 2048
+# tokens of context, ms per step fused / not: batch 1 0.794 / 0.794, 2 0.852 / 0.977, 8 0.923 / 1.048,
+# 16 1.132 / 1.169, 24 1.372 / 1.302, 32 1.418 / 1.346, 64 2.08 / 1.93.
+FUSED_MAX_BATCH = 16
+
+
 def u32s(*values) -> bytes:
     """Metal_parameters.u32s (lib/metal_parameters.ml:14-22)."""
     return struct.pack("<%dI" % len(values), *values)
@@ -127,17 +134,25 @@ class DecodeStep:
 
     def __init__(self, runtime: Runtime, config: DecodeConfig, weights: dict, batch: int, pool: Buffer,
                  slots: Buffer, slot_offsets, past_lengths, new_slots, positions, max_context=None,
-                 slots_host=None, reference_entries: bool = False):
+                 slots_host=None, reference_entries: bool = False, fused: bool | None = None):
         """max_context: the longest context any later step will have (sizes the attention launch;
         default: the longest now).  slots_host: the host copy of the slot table, with room behind
         every sequence's slots for the tokens `advance` will add.  reference_entries (batch 1):
         rotation, cache pack and attention as the reference's own three kernels
         (llmopt_rotary_qk_f16_simd_h64, llmopt_cache_pack_attention_q8_pair_simd,
-        llmopt_attention_q8_paged_simd_h64_gqa3) instead of the batched extension entries."""
+        llmopt_attention_q8_paged_simd_h64_gqa3) instead of the batched extension entries.
+        fused (default: whenever the shapes allow and reference_entries is off): four launches a
+        layer - norm + QKV + rotation + cache pack as one, attention, output projection, and the
+        SwiGLU FFN as one that leaves partial sums for the next layer's first launch - instead of six."""
         self.runtime, self.config, self.batch = runtime, config, batch
         self.reference_entries = reference_entries
         if reference_entries and batch != 1:
             raise ValueError("the reference's paged attention entries share one slot table: batch 1")
+        can_fuse = (config.head_dim == 64 and config.hidden % 64 == 0 and config.hidden <= 1472 and
+                    config.mlp % 64 == 0 and config.mlp // 64 <= 32)
+        if fused and (reference_entries or not can_fuse):
+            raise ValueError("the fused launches take heads of 64, hidden <= 1472 and mlp <= 2048")
+        self.fused = can_fuse and not reference_entries and batch <= FUSED_MAX_BATCH if fused is None else fused
         self.host_lengths = np.asarray(past_lengths, dtype=np.uint32).copy()
         self.host_offsets = np.asarray(slot_offsets, dtype=np.uint32).copy()
         self.host_positions = np.asarray(positions, dtype=np.int64).copy()
@@ -152,7 +167,10 @@ class DecodeStep:
         self.slot_offsets = b(np.asarray(slot_offsets, dtype=np.uint32))
         self.new_slots = b(np.asarray(new_slots, dtype=np.uint32))
         cos, sin = rope_rows(c, positions)
-        self.cos, self.sin = b(cos), b(sin)
+        # cosine rows, then sine rows, in one buffer (the fused launch takes them as one)
+        self.trig = b(np.concatenate([cos, sin]))
+        self.cos = self.trig.view(0, cos.nbytes)
+        self.sin = self.trig.view(cos.nbytes, sin.nbytes)
         self.max_past = int(max(past_lengths)) if max_context is None else int(max_context)
         self.device = {
             "embedding": b(weights["embedding"]),
@@ -170,6 +188,9 @@ class DecodeStep:
             "attention": create(q_bytes),
             "product": create(batch * c.mlp * 2),
         }
+        if self.fused:
+            self.work["stream"] = create(batch * h * 2)
+            self.work["partials"] = create((c.mlp // 64) * batch * h * 4)
         self.dispatches = self._build()
 
     def _linear_entry(self, columns_of_one_row: int):
@@ -192,6 +213,9 @@ class DecodeStep:
             x_in, x_mid = w["x"][0], w["x"][1]
             key_offset = index * c.layer_elements
             value_offset = key_offset + kvd
+            if self.fused:
+                out += self._fused_layer(index, layer, key_offset, value_offset)
+                continue
             # each RMSNorm rides in the projection launch that reads it
             suffix, grid = self._linear_entry(qd + 2 * kvd)
             out.append(("llmopt_rms_w4a16_qkv_linear_f16_g64",
@@ -208,14 +232,7 @@ class DecodeStep:
                             u32s(m, key_offset, value_offset, c.kv_heads, c.head_dim, 64, c.token_elements,
                                  c.token_elements // 64, c.token_stride, m, 0),
                             (((m * (c.q_heads + 2 * c.kv_heads) + 3) // 4) * 256, 1, 1), group))
-                attention_params = struct.pack(
-                    "<12IfIII", m, c.q_heads, c.kv_heads, 0, c.head_dim, 0, 0, c.token_elements, key_offset,
-                    value_offset, 64, c.token_stride, 1.0 / math.sqrt(c.head_dim), 1, 0, 0)
-                attention_params += struct.pack("<I", self.max_past)
-                out.append(("llmopt_attention_q8_paged_batched",
-                            [w["q_rot"], w["k_rot"], w["v"], self.pool, self.slots, self.slots, w["attention"],
-                             self.past_lengths, self.slot_offsets],
-                            attention_params, (((m * c.q_heads + 7) // 8) * 256, 1, 1), group))
+                out.append(self._batched_attention(key_offset, value_offset))
             suffix, grid = self._linear_entry(h)
             out.append(("llmopt_w4a16_linear_f16_g64" + suffix,
                         [w["attention"], *layer["o"], x_in, x_mid], u32s(m, h, qd, 1, h), grid, group))
@@ -230,6 +247,52 @@ class DecodeStep:
         out.append(("llmopt_w4a16_lm_head_argmax_f16",
                     [w["x"][0], self.device["final_norm"], *self.device["lm_head"], self.token_ids],
                     u32s(m, c.vocabulary, h) + struct.pack("<f", c.epsilon), (m * 256, 1, 1), group))
+        return out
+
+    def _batched_attention(self, key_offset: int, value_offset: int) -> tuple:
+        c, m, w = self.config, self.batch, self.work
+        attention_params = struct.pack(
+            "<12IfIII", m, c.q_heads, c.kv_heads, 0, c.head_dim, 0, 0, c.token_elements, key_offset,
+            value_offset, 64, c.token_stride, 1.0 / math.sqrt(c.head_dim), 1, 0, 0)
+        attention_params += struct.pack("<I", self.max_past)
+        return ("llmopt_attention_q8_paged_batched",
+                [w["q_rot"], w["k_rot"], w["v"], self.pool, self.slots, self.slots, w["attention"],
+                 self.past_lengths, self.slot_offsets],
+                attention_params, (((m * c.q_heads + 7) // 8) * 256, 1, 1), (256, 1, 1))
+
+    def _fused_layer(self, index: int, layer: dict, key_offset: int, value_offset: int) -> list[tuple]:
+        """Four launches: the residual stream enters as the previous layer's `x_mid` plus the partial
+        sums its FFN launch left (the first layer: the embedding rows, no sums); the last layer's FFN
+        runs as the two reference entries, so that the LM head finds a whole stream."""
+        c, m, w = self.config, self.batch, self.work
+        h, qd, kvd = c.hidden, c.q_heads * c.head_dim, c.kv_heads * c.head_dim
+        group = (256, 1, 1)
+        first, last = index == 0, index == c.layers - 1
+        slices = c.mlp // 64
+        stream_in = w["x"][0] if first else w["x"][1]
+        out = [("llmopt_rms_w4a16_qkv_rotary_pack_q8_f16_g64",
+                [stream_in, w["partials"], w["stream"], layer["attn_norm"], *layer["q"], *layer["k"], *layer["v"],
+                 self.trig, w["q_rot"], w["k_rot"], w["v"], self.new_slots, self.pool],
+                u32s(m, h, qd, kvd, kvd) + struct.pack("<f", c.epsilon) +
+                u32s(0 if first else slices, key_offset, value_offset, c.token_elements, c.token_stride),
+                (((qd + 2 * kvd) // 64) * 256, m, 1), group),
+               self._batched_attention(key_offset, value_offset)]
+        suffix, grid = self._linear_entry(h)
+        out.append(("llmopt_w4a16_linear_f16_g64" + suffix,
+                    [w["attention"], *layer["o"], w["stream"], w["x"][1]], u32s(m, h, qd, 1, h), grid, group))
+        ffn_params = u32s(m, c.mlp, h) + struct.pack("<f", c.epsilon)
+        if not last:
+            out.append(("llmopt_rms_w4a16_swiglu_down_partial_f16_g64",
+                        [w["x"][1], layer["ffn_norm"], *layer["gate"], *layer["up"], *layer["down"], w["partials"]],
+                        ffn_params, (slices * 256, m, 1), group))
+            return out
+        suffix, grid = self._linear_entry(c.mlp)
+        out.append(("llmopt_rms_w4a16_dual_swiglu_f16_g64",
+                    [w["x"][1], layer["ffn_norm"], *layer["gate"], *layer["up"], w["product"]], ffn_params, grid,
+                    group))
+        suffix, grid = self._linear_entry(h)
+        out.append(("llmopt_w4a16_down_add_f16_g64" + suffix,
+                    [w["product"], *layer["down"], w["x"][1], w["x"][0]], ffn_params, grid, group))
         return out
 
     def _reference_attention(self, key_offset: int, value_offset: int) -> list[tuple]:

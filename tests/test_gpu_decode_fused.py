@@ -1,0 +1,256 @@
+"""The fused decode-step launches (llmopt_rms_w4a16_qkv_rotary_pack_q8_f16_g64,
+llmopt_rms_w4a16_swiglu_down_partial_f16_g64) against the launches they stand for and against the
+CPU oracle, and the decode step built from them against the oracle's chain."""
+import struct
+
+import numpy as np
+import pytest
+
+import oracle
+from oracle import CacheParams
+from oracle.chain import decode_chain, f16, rope_rows
+from tests.gpu_util import assert_close_to_oracle, u32s
+
+pytestmark = pytest.mark.gpu
+
+GROUP = (256, 1, 1)
+
+
+@pytest.fixture(scope="module")
+def runtime():
+    from llmopt_amd.native import Runtime
+    rt = Runtime()
+    yield rt
+    rt.close()
+
+
+def random_w4(rng, n, k):
+    return (rng.integers(0, 256, size=(n, k // 2), dtype=np.uint8),
+            rng.uniform(0.005, 0.02, size=(n, k // 64)).astype(np.float16))
+
+
+def pending_stream(rng, m, k, partial_count):
+    """A residual stream as the fused launches hand it over: rows plus pending float32 partial sums,
+    and the rows a reader forms from them (sums in ascending order, float32, one rounding to half)."""
+    x = rng.standard_normal((m, k)).astype(np.float16)
+    partials = (rng.standard_normal((max(1, partial_count), m, k)) * 0.2).astype(np.float32)
+    total = np.zeros((m, k), dtype=np.float32)
+    for p in range(partial_count):
+        total = total + partials[p]
+    stream = (total + x.astype(np.float32)).astype(np.float16) if partial_count else x
+    return x, partials, stream
+
+
+@pytest.mark.parametrize("m,k,heads,partial_count", [(1, 576, (9, 3, 3), 0), (1, 576, (9, 3, 3), 24), (3, 576, (9, 3, 3), 24),
+                                                     (8, 576, (9, 3, 3), 24), (5, 1024, (4, 2, 2), 7), (2, 2048, (2, 1, 1), 32),
+                                                     (40, 576, (9, 3, 3), 24), (37, 1536, (3, 1, 1), 3), (2, 64, (1, 1, 1), 1)])
+def test_fused_qkv_rotary_pack_against_separate_launches_and_oracle(runtime, m, k, heads, partial_count):
+    rng = np.random.default_rng(1000 * m + k + partial_count)
+    q_heads, k_heads, v_heads = heads
+    assert k_heads == v_heads
+    n = [64 * q_heads, 64 * k_heads, 64 * v_heads]
+    layers, layer = 3, 1  # the new token's K / V go into the middle layer of a three-layer slot
+    layer_elements = 2 * n[1]
+    token_elements = layers * layer_elements
+    stride = token_elements + 2 * (token_elements // 64)
+    key_offset, value_offset = layer * layer_elements, layer * layer_elements + n[1]
+    capacity = m + 3
+    new_slots = rng.permutation(capacity).astype(np.uint32)[:m]
+    pool = rng.integers(0, 256, size=capacity * stride, dtype=np.uint8)
+    x, partials, stream = pending_stream(rng, m, k, partial_count)
+    gain = rng.uniform(0.5, 1.5, k).astype(np.float16)
+    weights = [random_w4(rng, count, k) for count in n]
+    positions = rng.integers(0, 5000, size=m)
+
+    class Rope:
+        head_dim, rope_theta = 64, 10000.0
+    cos, sin = rope_rows(Rope, positions)
+    b = runtime.buffer_of_bytes
+    device_w = [(b(w), b(s)) for w, s in weights]
+    outputs = {name: b(np.full(m * width, np.nan, dtype=np.float16)) for name, width in zip("qkv", n)}
+    stream_out = b(np.full(m * k, np.nan, dtype=np.float16))
+    device_pool = b(pool)
+    epsilon = 1e-5
+    runtime.dispatch("llmopt_rms_w4a16_qkv_rotary_pack_q8_f16_g64",
+                     [b(x), b(partials), stream_out, b(gain), *device_w[0], *device_w[1], *device_w[2],
+                      b(np.concatenate([cos, sin])), outputs["q"], outputs["k"], outputs["v"], b(new_slots), device_pool],
+                     u32s(m, k, *n) + struct.pack("<f", epsilon) +
+                     u32s(partial_count, key_offset, value_offset, token_elements, stride), grid=(256, 1, 1), group=GROUP)
+    # the stream the launch formed and stored: the partial sums are added in float32 in a fixed order of
+    # the kernel's own (groups of threads share them), then rounded once: the half nearest the exact sum,
+    # or its neighbour where float32 rounding moved a sum across a rounding boundary
+    got_stream = stream_out.numpy(np.float16, (m, k))
+    assert np.all(np.isfinite(got_stream))
+    step = np.spacing(np.abs(stream)).astype(np.float64)  # one half ulp step at the expected value
+    # (where the operands cancel, the float32 rounding of another summation order - 2^-23 of the operands -
+    # is itself several steps of the small result)
+    operands = np.abs(x).astype(np.float64) + np.abs(partials[:partial_count]).astype(np.float64).sum(axis=0)
+    assert np.all(np.abs(got_stream.astype(np.float64) - stream.astype(np.float64)) <= step + 4e-7 * operands)
+    assert np.mean(got_stream != stream) < 0.01
+    stream = got_stream  # what the rest of the launch worked on
+    got = {name: outputs[name].numpy(np.float16, (m, width)) for name, width in zip("qkv", n)}
+    got_pool = device_pool.numpy(np.uint8, (capacity, stride))
+
+    # the launches it stands for, on the same stream
+    separate = {name: b(np.zeros(m * width, dtype=np.float16)) for name, width in zip("qkv", n)}
+    rotated = {name: b(np.zeros(m * width, dtype=np.float16)) for name, width in zip("qk", n)}
+    separate_pool = b(pool)
+    runtime.dispatch("llmopt_rms_w4a16_qkv_linear_f16_g64",
+                     [b(stream), b(gain), *device_w[0], *device_w[1], *device_w[2], separate["q"], separate["k"],
+                      separate["v"]], u32s(m, k, *n) + struct.pack("<f", epsilon), grid=(256, 1, 1), group=GROUP)
+    runtime.dispatch("llmopt_rotary_qk_pack_q8_batched",
+                     [separate["q"], separate["k"], b(cos), b(sin), rotated["q"], rotated["k"], separate["v"],
+                      b(new_slots), separate_pool],
+                     u32s(m, 1, q_heads, k_heads, 64, 32, m) +
+                     u32s(m, key_offset, value_offset, k_heads, 64, 64, token_elements, token_elements // 64, stride, m, 0),
+                     grid=(256, 1, 1), group=GROUP)
+    want = {"q": rotated["q"].numpy(np.float16, (m, n[0])), "k": rotated["k"].numpy(np.float16, (m, n[1])),
+            "v": separate["v"].numpy(np.float16, (m, n[2]))}
+    for name in "qkv":
+        # the same arithmetic but for the order of the float32 sums over K: a last half bit here and there
+        assert_close_to_oracle(got[name], want[name].astype(np.float32), f"{name} vs separate launches", rel_l2_tol=3e-4)
+    want_pool = separate_pool.numpy(np.uint8, (capacity, stride))
+    untouched = np.setdiff1d(np.arange(capacity), new_slots)
+    np.testing.assert_array_equal(got_pool[untouched], pool.reshape(capacity, stride)[untouched])
+    segment = slice(key_offset, key_offset + 2 * n[1])
+    difference = got_pool[new_slots, segment].view(np.int8).astype(np.int32) - \
+        want_pool[new_slots, segment].view(np.int8).astype(np.int32)
+    assert np.abs(difference).max() <= 1
+    # the other layers' bytes of the new tokens' slots stay what they were
+    for lo, hi in ((0, key_offset), (key_offset + 2 * n[1], token_elements)):
+        np.testing.assert_array_equal(got_pool[new_slots, lo:hi], pool.reshape(capacity, stride)[new_slots, lo:hi])
+    scale_lo, scale_hi = token_elements + 2 * (key_offset // 64), token_elements + 2 * ((key_offset + 2 * n[1]) // 64)
+    got_scales = got_pool[new_slots, scale_lo:scale_hi].copy().view(np.uint16).astype(np.int32)
+    want_scales = want_pool[new_slots, scale_lo:scale_hi].copy().view(np.uint16).astype(np.int32)
+    assert np.abs(got_scales - want_scales).max() <= 2
+    np.testing.assert_array_equal(got_pool[new_slots, token_elements:scale_lo],
+                                  pool.reshape(capacity, stride)[new_slots, token_elements:scale_lo])
+
+    # the oracle on the same stream; the cache bytes are exactly the quantiser's for the K / V this launch stored
+    normalised = f16(oracle.rms_norm(stream, gain, epsilon))
+    for name, (packed, scale), count in zip("qkv", weights, heads):
+        projected = f16(oracle.w4a16_linear(normalised, packed, scale, None)).reshape(m, count, 64)
+        if name != "v":
+            projected = f16(oracle.rotary_h(projected, cos, sin)).transpose(1, 0, 2)  # back to [m, heads, 64]
+        assert_close_to_oracle(got[name], projected.reshape(m, -1).astype(np.float32), f"{name} vs oracle")
+    exact_pool = pool.copy()
+    for name, offset in (("k", key_offset), ("v", value_offset)):
+        source = np.ascontiguousarray(got[name].reshape(m, k_heads, 64).transpose(1, 0, 2))
+        oracle.q8_pack(source, new_slots, exact_pool,
+                       CacheParams(items=m, segment_offset=offset, heads=k_heads, head_dim=64, group_size=64,
+                                   token_elements=token_elements, token_groups=token_elements // 64,
+                                   token_stride=stride, source_items=m, source_offset=0))
+    np.testing.assert_array_equal(got_pool, exact_pool.reshape(capacity, stride))
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 1536, 576), (2, 1536, 576), (8, 1536, 576), (33, 1536, 576), (3, 2048, 1024),
+                                   (5, 128, 1408), (2, 64, 64), (4, 1024, 704)])
+def test_fused_ffn_partial_sums_against_separate_launches_and_oracle(runtime, m, n, k):
+    rng = np.random.default_rng(7 * m + n + k)
+    x = rng.standard_normal((m, k)).astype(np.float16)
+    gain = rng.uniform(0.5, 1.5, k).astype(np.float16)
+    gate, up, down = random_w4(rng, n, k), random_w4(rng, n, k), random_w4(rng, k, n)
+    b = runtime.buffer_of_bytes
+    device = [b(a) for pair in (gate, up, down) for a in pair]
+    slices = n // 64
+    partials = b(np.full(slices * m * k, np.nan, dtype=np.float32))
+    params = u32s(m, n, k) + struct.pack("<f", 1e-5)
+    runtime.dispatch("llmopt_rms_w4a16_swiglu_down_partial_f16_g64", [b(x), b(gain), *device, partials], params,
+                     grid=(256, 1, 1), group=GROUP)
+    got_partials = partials.numpy(np.float32, (slices, m, k))
+    assert np.all(np.isfinite(got_partials))
+    total = np.zeros((m, k), dtype=np.float32)
+    for p in range(slices):
+        total = total + got_partials[p]
+    got = (total + x.astype(np.float32)).astype(np.float16)  # what the next reader of the stream forms
+
+    product = b(np.zeros(m * n, dtype=np.float16))
+    separate = b(np.zeros(m * k, dtype=np.float16))
+    runtime.dispatch("llmopt_rms_w4a16_dual_swiglu_f16_g64", [b(x), b(gain), *device[:4], product], params,
+                     grid=(256, 1, 1), group=GROUP)
+    runtime.dispatch("llmopt_w4a16_down_add_f16_g64" + ("" if m == 1 else "_m4"),
+                     [product, *device[4:], b(x), separate], params, grid=(256, 1, 1), group=GROUP)
+    assert_close_to_oracle(got, separate.numpy(np.float16, (m, k)).astype(np.float32), "vs separate launches",
+                           rel_l2_tol=3e-4)
+
+    normalised = f16(oracle.rms_norm(x, gain, 1e-5))
+    want_product = f16(oracle.silu_mul(oracle.w4a16_linear(normalised, *gate, None),
+                                       oracle.w4a16_linear(normalised, *up, None)))
+    want = oracle.add(oracle.w4a16_linear(want_product, *down, None), x.astype(np.float32))
+    assert_close_to_oracle(got, want, "vs oracle")
+    # every partial sum is its own 64 columns of the contraction
+    for p in sorted({0, slices // 2, slices - 1}):
+        columns = slice(64 * p, 64 * p + 64)
+        packed = np.ascontiguousarray(down[0][:, 32 * p:32 * p + 32])
+        want_partial = oracle.w4a16_linear(want_product[:, columns], packed, np.ascontiguousarray(down[1][:, p:p + 1]), None)
+        error = np.linalg.norm(got_partials[p] - want_partial) / max(np.linalg.norm(want_partial), 1e-30)
+        assert error <= 2e-3, f"partial sum {p}: {error:.3e}"  # the product's half rounding carries over
+
+
+def test_fused_entries_reject_what_they_cannot_take(runtime):
+    from llmopt_amd.native import LlmoptError
+    b = runtime.buffer_of_bytes
+    any_buffer = b(np.zeros(4096, dtype=np.uint8))
+    with pytest.raises(LlmoptError, match="k <= 1472"):
+        runtime.dispatch("llmopt_rms_w4a16_swiglu_down_partial_f16_g64", [any_buffer] * 9,
+                         u32s(1, 64, 4096) + struct.pack("<f", 1e-5), grid=(256, 1, 1), group=GROUP)
+    with pytest.raises(LlmoptError, match="whole heads of 64"):
+        runtime.dispatch("llmopt_rms_w4a16_qkv_rotary_pack_q8_f16_g64", [any_buffer] * 16,
+                         u32s(1, 64, 64, 32, 32) + struct.pack("<f", 1e-5) + u32s(0, 0, 64, 128, 132),
+                         grid=(256, 1, 1), group=GROUP)
+    with pytest.raises(LlmoptError, match="two buffers"):
+        big = b(np.zeros(1 << 16, dtype=np.uint8))
+        runtime.dispatch("llmopt_rms_w4a16_qkv_rotary_pack_q8_f16_g64", [big] * 16,
+                         u32s(1, 64, 64, 64, 64) + struct.pack("<f", 1e-5) + u32s(0, 0, 64, 128, 132),
+                         grid=(256, 1, 1), group=GROUP)
+
+
+@pytest.mark.parametrize("batch", [1, 2, 8, 32])
+def test_fused_step_leaves_what_the_unfused_step_leaves(runtime, batch):
+    """The same step as four launches a layer and as six: tokens equal, hidden state and cache within
+    the half roundings the two orders of float32 sums allow; three layers, so that the partial sums
+    pass from layer to layer twice and the last layer's whole stream feeds the LM head."""
+    from llmopt_amd.decode_step import DecodeConfig, DecodeStep, random_weights
+    rng = np.random.default_rng(40 + batch)
+    config = DecodeConfig(layers=3, vocabulary=1000)
+    weights = random_weights(config, rng)
+    lengths = [int(v) for v in rng.integers(1, 200, size=batch)]
+    total = sum(lengths)
+    capacity = total + batch
+    order = rng.permutation(capacity).astype(np.uint32)
+    slots, new_slots = order[:total], order[total:]
+    offsets = np.concatenate([[0], np.cumsum(lengths)[:-1]]).astype(np.uint32)
+    stride, elements = config.token_stride, config.token_elements
+    pool = np.zeros((capacity, stride), dtype=np.uint8)
+    pool[:, :elements] = np.clip(np.rint(rng.standard_normal((capacity, elements)) * 38), -127, 127) \
+        .astype(np.int8).view(np.uint8)
+    pool[:, elements:] = rng.uniform(0.02, 0.035, (capacity, elements // 64)).astype(np.float16) \
+        .view(np.uint8).reshape(capacity, -1)
+    tokens = rng.integers(0, config.vocabulary, batch)
+    results = {}
+    for fused in (False, True):
+        device_pool = runtime.buffer_of_bytes(pool)
+        step = DecodeStep(runtime, config, weights, batch, device_pool, runtime.buffer_of_bytes(slots), offsets,
+                          lengths, new_slots, lengths, fused=fused)
+        assert step.fused == fused
+        assert len(step.dispatches) == (2 + 4 * config.layers + 1 if fused else 2 + 6 * config.layers)
+        got_tokens = step.run(tokens)
+        results[fused] = (got_tokens, step.work["x"][0].numpy(np.float16, (batch, config.hidden)),
+                          device_pool.numpy(np.uint8, (capacity, stride)))
+    assert_close_to_oracle(results[True][1], results[False][1].astype(np.float32), "fused vs unfused hidden state",
+                           rel_l2_tol=2e-3)
+    difference = results[True][2][:, :elements].view(np.int8).astype(np.int32) - \
+        results[False][2][:, :elements].view(np.int8).astype(np.int32)
+    assert np.abs(difference).max() <= 1
+    hidden, logits, _ = decode_chain(config, weights, pool.reshape(-1), slots, offsets, lengths, new_slots, lengths, tokens)
+    # three layers of chained kernels that each store half: 2e-3 a layer in relative L2, as the two-layer
+    # chains are held to 4e-3, and the largest single difference at 1e-2 x RMS a layer
+    want = hidden.astype(np.float64)
+    rms_hidden = float(np.sqrt(np.mean(want ** 2)))
+    for fused in (True, False):
+        difference = results[fused][1].astype(np.float64) - want
+        assert np.linalg.norm(difference) <= 6e-3 * np.linalg.norm(want), f"fused={fused}"
+        assert np.abs(difference).max() <= 3e-2 * rms_hidden, f"fused={fused}"
+    rms = float(np.sqrt(np.mean(logits.astype(np.float64) ** 2)))
+    for b in range(batch):
+        assert float(logits[b, results[True][0][b]]) >= float(logits[b].max()) - 2e-2 * rms

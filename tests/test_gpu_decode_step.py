@@ -30,7 +30,8 @@ def ragged_lengths(batch, seed):
 # itself), 9-32 its row-grouped form: batch 8 and 32 are the sizes the decode-step benchmark times.
 @pytest.mark.parametrize("batch,lengths", [(1, [37]), (2, [130, 9]), (3, [64, 5, 300]), (8, ragged_lengths(8, 5)),
                                            (32, ragged_lengths(32, 6))])
-def test_decode_step_matches_oracle_chain(runtime, batch, lengths):
+@pytest.mark.parametrize("fused", [False, True], ids=["six_launches_a_layer", "four_launches_a_layer"])
+def test_decode_step_matches_oracle_chain(runtime, batch, lengths, fused):
     from llmopt_amd.decode_step import DecodeConfig, DecodeStep, random_weights
     rng = np.random.default_rng(17 + batch)
     config = DecodeConfig(layers=2, vocabulary=1000)
@@ -52,7 +53,7 @@ def test_decode_step_matches_oracle_chain(runtime, batch, lengths):
 
     device_pool = runtime.buffer_of_bytes(pool)
     step = DecodeStep(runtime, config, weights, batch, device_pool, runtime.buffer_of_bytes(slots), offsets,
-                      lengths, new_slots, positions)
+                      lengths, new_slots, positions, fused=fused)
     got_tokens = step.run(tokens)
     got_hidden = step.work["x"][0].numpy(np.float16, (batch, config.hidden))
 
