@@ -62,6 +62,7 @@ def copies_for(k, n):
 
 GEMV_SHAPES = [(4096, 4096), (4096, 14336), (14336, 4096)]
 GEMV_ROWS = [1, 2, 4, 8]
+OTHER_GEMV_SHAPES = [(8192, 8192), (4096, 11008), (11008, 4096), (5120, 5120), (4096, 28672)]  # (K, N)
 
 
 def gemv_bytes(m, k, n):
@@ -244,9 +245,27 @@ def bench_gemv(runtime, steps, warmup, serial_only=False):
     c1 = {"m": 1, "k": k, "n": n, "bytes": gemv_bytes(1, k, n), "us_per_launch": round(c1_us, 3),
           "GBps": round(gemv_bytes(1, k, n) / (c1_us * 1e-6) / 1e9, 1), "verified": ok,
           "rel_l2": float("%.3g" % rel_l2)}
+    # shapes beside the sweep's (other models' projections): the same method, every launch on another HBM copy
+    other = []
+    for k, n in (() if serial_only else OTHER_GEMV_SHAPES):
+        x4, packed, scale = w4_inputs(rng, 4, n, k)
+        copies = [(runtime.buffer_of_bytes(packed), runtime.buffer_of_bytes(scale)) for _ in range(copies_for(k, n))]
+        for m in (1, 4):
+            bx = runtime.buffer_of_bytes(x4[:m])
+            out = runtime.buffer_of_bytes(np.full(m * n, np.nan, dtype=np.float16))
+            batch = runtime.begin_batch()
+            for bw, bs in copies:
+                record_linear(batch, m, n, k, bx, bw, bs, out)
+            us = batch.commit_profiled(repeats=2, use_graph=True) * 1e3 / (2 * len(copies))
+            ok, rel_l2 = verify_linear(out, m, n, x4[:m], packed, scale, check_rng)
+            other.append({"m": m, "k": k, "n": n, "bytes": gemv_bytes(m, k, n), "us_per_launch": round(us, 3),
+                          "GBps": round(gemv_bytes(m, k, n) / (us * 1e-6) / 1e9, 1),
+                          "hbm_frac": round(gemv_bytes(m, k, n) / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4),
+                          "verified": ok, "rel_l2": float("%.3g" % rel_l2)})
+        del copies
     return {"bytes_per_step": bytes_per_step, "ms_per_step": ms_per_step,
             "graph_ms_per_step": graph_ms_per_step, "graph_replays_ms": [round(ms / steps, 4) for ms in replays],
-            "concurrent_ms_per_step": concurrent, "cases": cases, "c1": c1}
+            "concurrent_ms_per_step": concurrent, "cases": cases, "c1": c1, "other": other}
 
 
 def bench_gemm(runtime):
@@ -789,7 +808,7 @@ def main():
     extras = {"gemv_cases": gemv["cases"],
               "gemv_sweep_serial_graph": {"ms_per_step": round(gemv["graph_ms_per_step"], 4),
                                           "GBps": round(value, 1), "replays_ms_per_step": gemv["graph_replays_ms"]},
-              "gemv_kernels": kernels, "gemv_c1_1x576x1536": gemv["c1"],
+              "gemv_kernels": kernels, "gemv_c1_1x576x1536": gemv["c1"], "gemv_other_shapes": gemv["other"],
               "gemv_eager_host_launch_GBps":
                   round(gemv["bytes_per_step"] / (gemv["ms_per_step"] * 1e-3) / 1e9, 1),
               "gemv_eager_host_launch_ms_per_step": round(gemv["ms_per_step"], 4),
@@ -814,6 +833,7 @@ def main():
     # refuse to print numbers whose outputs did not match the oracle
     checked = [("gemv %(m)dx%(k)dx%(n)d" % c, c["verified"]) for c in gemv["cases"]]
     checked.append(("gemv c1", gemv["c1"]["verified"]))
+    checked += [("gemv %(m)dx%(k)dx%(n)d" % c, c["verified"]) for c in gemv["other"]]
     checked += [("%(kind)s %(m)dx%(n)dx%(k)d" % c, c["verified"]) for c in extras.get("prefill_gemm", [])]
     if "q8_attention" in extras:
         checked.append(("q8 attention", extras["q8_attention"]["verified"]))

@@ -475,19 +475,6 @@ uint32_t rows_per_workgroup(uint32_t m, uint32_t k, uint32_t column_blocks) {
              : 1;
 }
 
-// Kernels that take more dynamic LDS than the default limit say so once per device.
-template <typename Kernel>
-hipError_t allow_dynamic_lds(Kernel kernel, size_t bytes) {
-  static bool configured[64] = {};
-  int device = 0;
-  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= 64) return hipErrorInvalidDevice;
-  if (bytes <= 64 * 1024 || configured[device]) return hipSuccess;
-  const hipError_t status =
-      hipFuncSetAttribute(reinterpret_cast<const void *>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024 - 2048);
-  if (status == hipSuccess) configured[device] = true;
-  return status;
-}
-
 uint32_t padded(uint32_t bytes) { return (bytes + 15) & ~15u; }
 
 size_t qkv_lds_bytes(uint32_t rows, uint32_t k, bool partials) {
@@ -506,25 +493,33 @@ uint32_t partials_per_thread(uint32_t rows, uint32_t k, uint32_t partial_count) 
   return (partial_count + groups - 1) / groups;
 }
 
+template <int M, int PER>
+hipError_t launch_qkv_instance(const FusedQkvArgs &a, dim3 grid, size_t lds, hipStream_t stream) {
+  static bool configured[kMaxDevices] = {};
+  if (lds > 64 * 1024)
+    if (hipError_t status = allow_dynamic_lds(reinterpret_cast<const void *>(fused_qkv_kernel<M, PER>), 158 * 1024, configured))
+      return status;
+  hipLaunchKernelGGL((fused_qkv_kernel<M, PER>), grid, dim3(kThreads), lds, stream, a);
+  return hipGetLastError();
+}
+
 template <int M>
 hipError_t launch_qkv_rows(const FusedQkvArgs &a, dim3 grid, hipStream_t stream) {
   const uint32_t per = partials_per_thread(M, a.k, a.in.partial_count);
   const size_t lds = qkv_lds_bytes(M, a.k, per != 0);
-  const auto launch = [&](auto kernel) {
-    if (hipError_t status = allow_dynamic_lds(kernel, lds)) return status;
-    hipLaunchKernelGGL(kernel, grid, dim3(kThreads), lds, stream, a);
-    return hipGetLastError();
-  };
-  if (per == 0) return launch(fused_qkv_kernel<M, 0>);
-  if (per <= 8) return launch(fused_qkv_kernel<M, 8>);
-  if (per <= 16) return launch(fused_qkv_kernel<M, 16>);
-  return launch(fused_qkv_kernel<M, 32>);
+  if (per == 0) return launch_qkv_instance<M, 0>(a, grid, lds, stream);
+  if (per <= 8) return launch_qkv_instance<M, 8>(a, grid, lds, stream);
+  if (per <= 16) return launch_qkv_instance<M, 16>(a, grid, lds, stream);
+  return launch_qkv_instance<M, 32>(a, grid, lds, stream);
 }
 
 template <int M>
 hipError_t launch_ffn_rows(const FusedFfnArgs &a, dim3 grid, hipStream_t stream) {
   const size_t lds = ffn_lds_bytes(M, a.k);
-  if (hipError_t status = allow_dynamic_lds(fused_ffn_kernel<M>, lds)) return status;
+  static bool configured[kMaxDevices] = {};
+  if (lds > 64 * 1024)
+    if (hipError_t status = allow_dynamic_lds(reinterpret_cast<const void *>(fused_ffn_kernel<M>), 158 * 1024, configured))
+      return status;
   hipLaunchKernelGGL(fused_ffn_kernel<M>, grid, dim3(kThreads), lds, stream, a);
   return hipGetLastError();
 }

@@ -788,13 +788,8 @@ hipError_t launch_tile32_instance(uint32_t grid, const DenseAttentionArgs &a, hi
   constexpr size_t bytes = (PAIR ? 2 : 1) * 2 * 2 * (size_t)STAGE_KEYS * D * 2;  // two stages of K and V per group
   auto kernel = &dense_attention_tile32_kernel<D, WAVES, STAGE_KEYS, MASK, KEYSPLIT, PAIR>;
   if constexpr (bytes >= 64 * 1024) {
-    static bool configured = false;  // the attribute is per device function
-    if (!configured) {
-      const hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)bytes);
-      if (status != hipSuccess) return status;
-      configured = true;
-    }
+    static bool configured[kMaxDevices] = {};  // the attribute is per device function and device
+    if (hipError_t status = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), (int)bytes, configured)) return status;
   }
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(WAVES * 64 * (PAIR ? 2 : 1)), bytes, stream, a);
   return hipGetLastError();

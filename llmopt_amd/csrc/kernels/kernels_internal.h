@@ -9,6 +9,25 @@ namespace llmopt {
 
 int device_compute_units();
 
+// hipFuncSetAttribute applies to one device: launchers that raise a kernel's dynamic LDS limit keep
+// one "done" flag per device (a process may hold a context on each).
+constexpr int kMaxDevices = 64;
+inline int current_device() {
+  int device = -1;
+  if (hipGetDevice(&device) != hipSuccess || device < 0 || device >= kMaxDevices) return -1;
+  return device;
+}
+// Raises `kernel`'s dynamic LDS limit to `bytes` on the current device, once per device (`done`: the
+// launcher's own flags).
+inline hipError_t allow_dynamic_lds(const void *kernel, int bytes, bool (&done)[kMaxDevices]) {
+  const int device = current_device();
+  if (device < 0) return hipErrorInvalidDevice;
+  if (done[device]) return hipSuccess;
+  const hipError_t status = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+  if (status == hipSuccess) done[device] = true;
+  return status;
+}
+
 hipError_t launch_w4a16_gemv_linear(const W4LinearArgs &args, hipStream_t stream);
 hipError_t launch_w4a16_gemv_qkv(const W4QkvArgs &args, hipStream_t stream);
 hipError_t launch_w4a16_gemv_dual_swiglu(const W4DualSwigluArgs &args, hipStream_t stream);

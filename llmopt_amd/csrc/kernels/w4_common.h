@@ -37,8 +37,8 @@ __device__ __forceinline__ uint16_t float_to_half_bits(float value) {
 //
 // XOR with 8 turns a two's-complement nibble into offset binary (q + 8).  A 4-bit field in the
 // mantissa of 1024.0 (0x6400, ulp 1) or of 64.0 (0x5400, ulp 1/16, field at bits 4..7) reads as
-// 1024 + (q + 8) or 64 + (q + 8) exactly: ((w ^ 0x88888888) & mask) | magic, the magic bits lying
-// outside the mask.  The four
+// 1024 + (q + 8) or 64 + (q + 8) exactly.  Both steps are one XOR after the mask:
+// (w & mask) ^ (magic | (0x88888888 & mask)), the magic bits lying outside the mask.  The four
 // results hold the pairs (k0,k4) (k1,k5) (k2,k6) (k3,k7): the activation is arranged to match.
 struct W4Pairs {
   h2_t p04, p15, p26, p37;
@@ -48,14 +48,12 @@ struct W4Pairs {
 // corrected afterwards by 1032 * sum(x at K offsets 0,4,2,6) + 72 * sum(x at K offsets 1,5,3,7),
 // which does not depend on the weight row.
 __device__ __forceinline__ W4Pairs w4_decode_biased(uint32_t word) {
-  // the sign-bit flip of all eight nibbles at once, then one and-or per pair (six operations a dword)
-  const uint32_t flipped = word ^ 0x88888888u;
-  const uint32_t hi = flipped >> 8;
+  const uint32_t hi = word >> 8;
   W4Pairs out;
-  out.p04 = as_h2((flipped & 0x000F000Fu) | 0x64006400u);
-  out.p15 = as_h2((flipped & 0x00F000F0u) | 0x54005400u);
-  out.p26 = as_h2((hi & 0x000F000Fu) | 0x64006400u);
-  out.p37 = as_h2((hi & 0x00F000F0u) | 0x54005400u);
+  out.p04 = as_h2((word & 0x000F000Fu) ^ 0x64086408u);
+  out.p15 = as_h2((word & 0x00F000F0u) ^ 0x54805480u);
+  out.p26 = as_h2((hi & 0x000F000Fu) ^ 0x64086408u);
+  out.p37 = as_h2((hi & 0x00F000F0u) ^ 0x54805480u);
   return out;
 }
 

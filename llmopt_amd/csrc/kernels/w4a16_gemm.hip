@@ -458,13 +458,10 @@ hipError_t launch_tile(GemmParams &p, hipStream_t stream, uint32_t splits = 1) {
   constexpr int BN = 2 * WN * 32;
   constexpr size_t lds_bytes = ((size_t)XS * BM * BK + 2 * (size_t)NW * BN * LDS_STRIDE) * sizeof(_Float16);
   static_assert(lds_bytes <= 160 * 1024, "a workgroup's stages must fit the CU's LDS");
-  static bool configured = false;
-  if (!configured) {
-    hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(&w4a16_gemm_kernel<WM, WN, DUAL, XS, SPLITK>),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
-    if (status != hipSuccess) return status;
-    configured = true;
-  }
+  static bool configured[kMaxDevices] = {};
+  if (hipError_t status = allow_dynamic_lds(reinterpret_cast<const void *>(&w4a16_gemm_kernel<WM, WN, DUAL, XS, SPLITK>),
+                                            (int)lds_bytes, configured))
+    return status;
   p.tiles_m = (p.m + BM - 1) / BM;
   p.tiles_n = (p.n + BN - 1) / BN;
   if (p.segments > 1) {

@@ -442,13 +442,10 @@ Plan make_plan(uint32_t k, uint32_t max_n, uint32_t matrices, bool dual) {
 
 template <int NB, bool DUAL>
 hipError_t launch_ring(const MfmaGemvParams &p, uint32_t matrices, const Plan &plan, hipStream_t stream) {
-  static bool configured = false;  // the attribute is per device function
-  if (!configured) {
-    hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(&w4a16_gemv_mfma_kernel<NB, DUAL>),
-                                            hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    if (status != hipSuccess) return status;
-    configured = true;
-  }
+  static bool configured[kMaxDevices] = {};  // the attribute is per device function and device
+  if (hipError_t status = allow_dynamic_lds(reinterpret_cast<const void *>(&w4a16_gemv_mfma_kernel<NB, DUAL>), 160 * 1024,
+                                            configured))
+    return status;
   const dim3 grid(plan.blocks, p.row_groups > 1 ? p.row_groups : plan.slices, matrices);
   hipLaunchKernelGGL((w4a16_gemv_mfma_kernel<NB, DUAL>), grid, dim3(plan.waves_k * plan.waves_t * 64),
                      plan.lds_bytes, stream, p);

@@ -26,9 +26,14 @@
 // of another wave's activation request would hold the whole workgroup at its barrier - and the
 // rest of the ring of DEPTH loads right after.
 //
-// K is a template parameter (KL ranges of 512): strides in LDS, the ring indices and the loop
-// are compile-time.  Instantiated for K = 4096 and K = 14336; other shapes keep the kernels of
-// w4a16_gemv.hip / w4a16_gemv_mfma.hip.
+// The K ranges of 512 are a template parameter: strides in LDS, the ring indices and the (unrolled)
+// walk over K are compile-time.  K = 4096 and K = 14336 have instantiations of exactly their length;
+// at three and four activation rows every other multiple of 128 from 2048 to 8192 runs an
+// instantiation whose LDS layout and unrolled walk are cut for the longest such row, with the row's
+// real length a launch argument: what lies beyond the row's end is skipped.  (Walking K in a real loop
+// was measured twice, with the compiler's waits and with requests in assembly waited for by count:
+// 1.3 - 2.6 TB/s against the unrolled walk's 3.9 - 4.4 - a loop's back edge costs the ring its depth.)  Other shapes keep the kernels of w4a16_gemv.hip /
+// w4a16_gemv_mfma.hip.  N from 3072 up: beyond one round of workgroups the launch makes several.
 #include <algorithm>
 
 #include "kernels.h"
@@ -45,7 +50,7 @@ struct QuadParams {
   uint16_t *y;
   const uint16_t *addend;
   uint32_t has_addend, addend_stride;
-  uint32_t m, n;
+  uint32_t m, n, k;
 };
 
 __device__ __forceinline__ h4_t pack_h4(uint32_t lo, uint32_t hi) {
@@ -65,9 +70,11 @@ constexpr size_t quad_lds_bytes(uint32_t waves) {
   return (size_t)MR * (2 * KL * 512 + 16) + (size_t)KL * 16 * 16 + (size_t)waves * RQ * 4 * (KL * 16 + 16);
 }
 
-// MR: activation rows staged (m <= MR <= 4); KL: K / 512; RQ: row quads per wave; DEPTH: weight
-// loads in flight per wave; EARLY: how many of them go out before the staging waits;
-// THREADS: workgroup size (waves beyond units_per_wg only help staging).
+// MR: activation rows staged (m <= MR <= 4); KL: K / 512 (EXACT) or the most K ranges the
+// instantiation's LDS layout holds (K = p.k is then any multiple of 512 up to 512 KL, and the walk
+// over K stops where the row ends); RQ: row quads per wave; DEPTH: weight loads in flight per wave;
+// EARLY: how many of them go out before the staging waits; THREADS: workgroup size (waves beyond
+// units_per_wg only help staging).
 // Registers: a workgroup is one wave per SIMD, and told only that, the compiler spreads itself over
 // the 512 registers a lone wave may have (220 at one row of K = 14336, half of them accumulator
 // registers used as spill space) - a CU then holds nothing beside this workgroup, and launches that
@@ -81,19 +88,27 @@ constexpr int quad_waves_per_simd() {
   return (KL > 8 && RQ == 2) ? 1 : MR <= 2 ? 3 : 2;
 }
 
-template <int MR, int KL, int RQ, int DEPTH, int EARLY, int THREADS>
+template <int MR, int KL, int RQ, int DEPTH, int EARLY, int THREADS, bool EXACT = true>
 __global__ __launch_bounds__(THREADS)
     __attribute__((amdgpu_waves_per_eu(quad_waves_per_simd<MR, KL, RQ>(), quad_waves_per_simd<MR, KL, RQ>()))) void
     w4a16_gemv_quad_kernel(QuadParams p, uint32_t units_per_wg) {
   static_assert(MR >= 1 && MR <= 4 && EARLY >= 1 && EARLY <= DEPTH && DEPTH <= KL * RQ && THREADS % 64 == 0, "shape");
-  constexpr uint32_t K = KL * 512, row_bytes = K / 2, groups = K / 64;
-  constexpr uint32_t kRowStride = 2 * K + 16;         // bytes between activation rows in LDS
-  constexpr uint32_t kScaleStride = groups * 2 + 16;  // bytes between scale rows in LDS
-  constexpr uint32_t kXUnits = MR * (K / 8);          // 16-byte units of activation to stage
+  constexpr uint32_t KMAX = KL * 512;                  // what the LDS layout is cut for
+  const uint32_t K = EXACT ? KMAX : p.k;               // a constant in the exact instantiations
+  const uint32_t row_bytes = K / 2, groups = K / 64;
+  constexpr uint32_t kRowStride = 2 * KMAX + 16;         // bytes between activation rows in LDS
+  constexpr uint32_t kScaleStride = (KMAX / 64) * 2 + 16;  // bytes between scale rows in LDS
+  constexpr uint32_t kXUnits = MR * (KMAX / 8);          // 16-byte units of activation to stage
   constexpr int XPER = (kXUnits + THREADS - 1) / THREADS;
-  constexpr uint32_t kScaleUnitsPerRow = groups * 2 / 16;
-  constexpr int SPER = ((THREADS / 64) * RQ * 4 * kScaleUnitsPerRow + THREADS - 1) / THREADS;
-  constexpr int TOTAL = KL * RQ;
+  const uint32_t kScaleUnitsPerRow = groups * 2 / 16;
+  constexpr int SPER = ((THREADS / 64) * RQ * 4 * ((KMAX / 64) * 2 / 16) + THREADS - 1) / THREADS;
+  constexpr int TOTAL_MAX = KL * RQ;
+  // K ranges of the row: the last one may be partly there (K a multiple of 128): its missing
+  // activations are staged as zeros, its weight requests held inside the row, its scales to the
+  // row's last group
+  const uint32_t ranges = EXACT ? KL : (K + 511) / 512;
+  const int TOTAL = EXACT ? TOTAL_MAX : (int)ranges * RQ;
+  const uint32_t scale_pitch = EXACT ? kScaleStride : groups * 2;  // other K: rows side by side, as in memory
   extern __shared__ __attribute__((aligned(16))) unsigned char lds_raw[];
   unsigned char *xs = lds_raw;
   float *cin = reinterpret_cast<float *>(lds_raw + MR * kRowStride);  // [piece of 32 K][activation row 0..3]
@@ -109,18 +124,19 @@ __global__ __launch_bounds__(THREADS)
   // Unit e of a thread is 16-byte unit `u` of activation row `row`.  When a row is a whole
   // number of passes of the workgroup both are known without a division: the staging runs once
   // per unit, and every vector instruction in it costs four cycles a wave.
-  constexpr bool kWholePasses = (K / 8) % THREADS == 0;
-  constexpr uint32_t kPassesPerRow = kWholePasses ? (K / 8) / THREADS : 1;
+  // (Rows are laid out for KMAX values; of a shorter row only the first K / 8 units exist.)
+  constexpr bool kWholePasses = (KMAX / 8) % THREADS == 0;
+  constexpr uint32_t kPassesPerRow = kWholePasses ? (KMAX / 8) / THREADS : 1;
   auto unit_of = [&](int e, uint32_t &row, uint32_t &u, bool &inside) __attribute__((always_inline)) {
     if constexpr (kWholePasses) {
       row = (uint32_t)e / kPassesPerRow;
       u = threadIdx.x + ((uint32_t)e % kPassesPerRow) * THREADS;
-      inside = true;
+      inside = EXACT || u < ranges * 64;
     } else {
       const uint32_t idx = threadIdx.x + e * THREADS;
-      inside = idx < kXUnits;
-      row = min(idx, kXUnits - 1) / (K / 8);
-      u = min(idx, kXUnits - 1) % (K / 8);
+      row = min(idx, kXUnits - 1) / (KMAX / 8);
+      u = min(idx, kXUnits - 1) % (KMAX / 8);
+      inside = idx < kXUnits && (EXACT || u < ranges * 64);
     }
   };
   uint4 xin[XPER];
@@ -129,9 +145,9 @@ __global__ __launch_bounds__(THREADS)
     uint32_t row, u;
     bool inside;
     unit_of(e, row, u, inside);
-    xin[e] = reinterpret_cast<const uint4 *>(p.x + (size_t)min(row, p.m - 1) * K)[u];
+    xin[e] = reinterpret_cast<const uint4 *>(p.x + (size_t)min(row, p.m - 1) * K)[EXACT ? u : min(u, K / 8 - 1)];
   }
-  const uint32_t scale_units = rows_per_wg * kScaleUnitsPerRow;
+  const uint32_t scale_units = EXACT ? rows_per_wg * kScaleUnitsPerRow : rows_per_wg * groups * 2 / 16;
   const size_t s_first = (size_t)row0 * groups * 2, s_last = (size_t)p.n * groups * 2 - 16;
   // (four named registers, not an array: left as an array the compiler kept it in scratch memory
   // and waited for these loads right here, before the first weight request, to store them there)
@@ -149,24 +165,36 @@ __global__ __launch_bounds__(THREADS)
   const uint32_t unit = __builtin_amdgcn_readfirstlane(blockIdx.x * units_per_wg + min(wave, units_per_wg - 1));
   u32x4_t wreg[DEPTH];
   const uint32_t w_lane = j * row_bytes + b * 16;
+  // the lane's piece of the row's last K range, held inside the row when that range is partly there
+  const uint32_t w_lane_last = EXACT ? w_lane : j * row_bytes + min(b * 16, row_bytes - (ranges - 1) * 256 - 16);
   const uint8_t *w_quad[RQ];
 #pragma unroll
   for (int rq = 0; rq < RQ; ++rq) {
     const uint32_t quad = __builtin_amdgcn_readfirstlane(min(unit * RQ + rq, quads - 1));
     w_quad[rq] = p.w + (size_t)quad * 4 * row_bytes;
   }
+  auto ring_request = [&](u32x4_t &into, const uint8_t *address) __attribute__((always_inline)) {
+    into = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(address));
+  };
+  uint16_t addend_bits[RQ][MR] = {};
+  if (!EXACT && p.has_addend) {
+    // (other K: the addend goes out first and lands first; nothing but the ring is then requested in the walk)
+#pragma unroll
+    for (int q = 0; q < RQ; ++q)
+#pragma unroll
+      for (int i = 0; i < MR; ++i)
+        addend_bits[q][i] = p.addend[(size_t)min((uint32_t)i, p.m - 1) * p.addend_stride + min(unit * RQ + q, quads - 1) * 4 + j];
+  }
   __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-  for (int n = 0; n < EARLY; ++n)
-    wreg[n] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(w_quad[n % RQ] + (n / RQ) * 256 + w_lane));
+  for (int n = 0; n < EARLY; ++n) ring_request(wreg[n], w_quad[n % RQ] + (n / RQ) * 256 + w_lane);
   __builtin_amdgcn_sched_barrier(0);
   if (EARLY < DEPTH) {
     // loads return in issue order: with only the early weights outstanding, the activation and
     // the scales have landed
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(EARLY) : "memory");
 #pragma unroll
-    for (int n = EARLY; n < DEPTH; ++n)
-      wreg[n] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(w_quad[n % RQ] + (n / RQ) * 256 + w_lane));
+    for (int n = EARLY; n < DEPTH; ++n) ring_request(wreg[n], w_quad[n % RQ] + (n / RQ) * 256 + w_lane);
     __builtin_amdgcn_sched_barrier(0);
   }
   // 3. stage: pair order, the decode-bias correction of every 32-K piece, the scales
@@ -177,7 +205,7 @@ __global__ __launch_bounds__(THREADS)
     bool inside;
     unit_of(e, row, u, inside);
     uint4 v = pair_order(xin[e]);
-    if (row >= p.m) v = make_uint4(0, 0, 0, 0);
+    if (row >= p.m || (!EXACT && u >= K / 8)) v = make_uint4(0, 0, 0, 0);
     // 1032 * (x0 + x4 + x2 + x6) + 72 * (x1 + x5 + x3 + x7): exact products, float32 sums
     float corr = __builtin_amdgcn_fdot2(as_h2(v.x), bias_even, 0.0f, false);
     corr = __builtin_amdgcn_fdot2(as_h2(v.z), bias_even, corr, false);
@@ -194,8 +222,12 @@ __global__ __launch_bounds__(THREADS)
   // (corrections of A rows beyond MR are never written: those rows of D are never read)
   auto scale_store = [&](int e, const uint4 &value) __attribute__((always_inline)) {
     const uint32_t idx = threadIdx.x + e * THREADS;
-    if (idx < scale_units)
-      *reinterpret_cast<uint4 *>(ss + (idx / kScaleUnitsPerRow) * kScaleStride + (idx % kScaleUnitsPerRow) * 16) = value;
+    if (idx < scale_units) {
+      if constexpr (EXACT)
+        *reinterpret_cast<uint4 *>(ss + (idx / kScaleUnitsPerRow) * kScaleStride + (idx % kScaleUnitsPerRow) * 16) = value;
+      else
+        *reinterpret_cast<uint4 *>(ss + idx * 16) = value;
+    }
   };
   scale_store(0, scale_in0);
   if constexpr (SPER > 1) scale_store(1, scale_in1);
@@ -212,45 +244,80 @@ __global__ __launch_bounds__(THREADS)
   for (int rq = 0; rq < RQ; ++rq) acc[rq] = f4_t{0.f, 0.f, 0.f, 0.f};
   uint4 xa[4];
   f4_t cinit;
-  uint16_t addend_bits[RQ][MR] = {};
-  const unsigned char *my_scales = ss + (wave * RQ * 4 + j) * kScaleStride + (b >> 1) * 2;
+  const unsigned char *my_scales = ss + (wave * RQ * 4 + j) * scale_pitch + (EXACT ? (b >> 1) * 2 : 0);
+  if constexpr (EXACT) {
+  #pragma unroll
+    for (int n = 0; n < TOTAL_MAX; ++n) {
+      const int kp = n / RQ, rq = n % RQ;
+      if (rq == 0) {
+  #pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          xa[t] = make_uint4(0, 0, 0, 0);
+          if (j < MR) xa[t] = *reinterpret_cast<const uint4 *>(xs + j * kRowStride + (kp * 64 + 4 * b + t) * 16);
+        }
+        cinit = *reinterpret_cast<const f4_t *>(cin + (kp * 16 + b) * 4);
+      }
+      const uint16_t scale_bits = *reinterpret_cast<const uint16_t *>(
+          my_scales + rq * 4 * scale_pitch + (uint32_t)kp * 16);
+      const u32x4_t words = wreg[n % DEPTH];
+      f4_t d = cinit;
+  #pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const W4Pairs pr = w4_decode_biased(words[t]);
+        d = __builtin_amdgcn_mfma_f32_4x4x4f16(pack_h4(xa[t].x, xa[t].y), pack_h4(as_u32(pr.p04), as_u32(pr.p15)), d, 0, 0, 0);
+        d = __builtin_amdgcn_mfma_f32_4x4x4f16(pack_h4(xa[t].z, xa[t].w), pack_h4(as_u32(pr.p26), as_u32(pr.p37)), d, 0, 0, 0);
+      }
+      if (n + DEPTH < TOTAL)
+        wreg[n % DEPTH] = __builtin_nontemporal_load(
+            reinterpret_cast<const u32x4_t *>(w_quad[(n + DEPTH) % RQ] + ((n + DEPTH) / RQ) * 256 + w_lane));
+      if (n + DEPTH == TOTAL && p.has_addend) {
+        // The addend of this wave's outputs is requested right behind its last weights: it lands
+        // with them, and the store path has no load of its own to wait for.  Every lane reads
+        // (lanes 0..3 hold row 4 * quad + j; the others repeat them), clamped into the buffer.
+  #pragma unroll
+        for (int q = 0; q < RQ; ++q)
+  #pragma unroll
+          for (int i = 0; i < MR; ++i)
+            addend_bits[q][i] = p.addend[(size_t)min((uint32_t)i, p.m - 1) * p.addend_stride +
+                                         min(unit * RQ + q, quads - 1) * 4 + j];
+      }
+      const float scale = half_bits_to_float(scale_bits);
+  #pragma unroll
+      for (int i = 0; i < 4; ++i) acc[rq][i] = fmaf(d[i], scale, acc[rq][i]);
+    }
+  } else {
+    // The unrolled walk of the longest row this instantiation's LDS layout holds; what lies beyond the
+    // row's real end is skipped (the same for every wave).
 #pragma unroll
-  for (int n = 0; n < TOTAL; ++n) {
-    const int kp = n / RQ, rq = n % RQ;
-    if (rq == 0) {
+    for (int n = 0; n < TOTAL_MAX; ++n) {
+      if (n >= TOTAL) continue;
+      const int kp = n / RQ, rq = n % RQ;
+      if (rq == 0) {
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          xa[t] = make_uint4(0, 0, 0, 0);
+          if (j < MR) xa[t] = *reinterpret_cast<const uint4 *>(xs + j * kRowStride + (kp * 64 + 4 * b + t) * 16);
+        }
+        cinit = *reinterpret_cast<const f4_t *>(cin + (kp * 16 + b) * 4);
+      }
+      const uint16_t scale_bits = *reinterpret_cast<const uint16_t *>(
+          my_scales + rq * 4 * scale_pitch + min((uint32_t)kp * 8 + (b >> 1), groups - 1) * 2);
+      const u32x4_t words = wreg[n % DEPTH];
+      f4_t d = cinit;
 #pragma unroll
       for (int t = 0; t < 4; ++t) {
-        xa[t] = make_uint4(0, 0, 0, 0);
-        if (j < MR) xa[t] = *reinterpret_cast<const uint4 *>(xs + j * kRowStride + (kp * 64 + 4 * b + t) * 16);
+        const W4Pairs pr = w4_decode_biased(words[t]);
+        d = __builtin_amdgcn_mfma_f32_4x4x4f16(pack_h4(xa[t].x, xa[t].y), pack_h4(as_u32(pr.p04), as_u32(pr.p15)), d, 0, 0, 0);
+        d = __builtin_amdgcn_mfma_f32_4x4x4f16(pack_h4(xa[t].z, xa[t].w), pack_h4(as_u32(pr.p26), as_u32(pr.p37)), d, 0, 0, 0);
       }
-      cinit = *reinterpret_cast<const f4_t *>(cin + (kp * 16 + b) * 4);
+      if (n + DEPTH < TOTAL)
+        wreg[n % DEPTH] = __builtin_nontemporal_load(reinterpret_cast<const u32x4_t *>(
+            w_quad[(n + DEPTH) % RQ] + ((n + DEPTH) / RQ) * 256 +
+            ((uint32_t)((n + DEPTH) / RQ) == ranges - 1 ? w_lane_last : w_lane)));
+      const float scale = half_bits_to_float(scale_bits);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) acc[rq][i] = fmaf(d[i], scale, acc[rq][i]);
     }
-    const uint16_t scale_bits = *reinterpret_cast<const uint16_t *>(my_scales + rq * 4 * kScaleStride + kp * 16);
-    const u32x4_t words = wreg[n % DEPTH];
-    f4_t d = cinit;
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      const W4Pairs pr = w4_decode_biased(words[t]);
-      d = __builtin_amdgcn_mfma_f32_4x4x4f16(pack_h4(xa[t].x, xa[t].y), pack_h4(as_u32(pr.p04), as_u32(pr.p15)), d, 0, 0, 0);
-      d = __builtin_amdgcn_mfma_f32_4x4x4f16(pack_h4(xa[t].z, xa[t].w), pack_h4(as_u32(pr.p26), as_u32(pr.p37)), d, 0, 0, 0);
-    }
-    if (n + DEPTH < TOTAL)
-      wreg[n % DEPTH] = __builtin_nontemporal_load(
-          reinterpret_cast<const u32x4_t *>(w_quad[(n + DEPTH) % RQ] + ((n + DEPTH) / RQ) * 256 + w_lane));
-    if (n + DEPTH == TOTAL && p.has_addend) {
-      // The addend of this wave's outputs is requested right behind its last weights: it lands
-      // with them, and the store path has no load of its own to wait for.  Every lane reads
-      // (lanes 0..3 hold row 4 * quad + j; the others repeat them), clamped into the buffer.
-#pragma unroll
-      for (int q = 0; q < RQ; ++q)
-#pragma unroll
-        for (int i = 0; i < MR; ++i)
-          addend_bits[q][i] = p.addend[(size_t)min((uint32_t)i, p.m - 1) * p.addend_stride +
-                                       min(unit * RQ + q, quads - 1) * 4 + j];
-    }
-    const float scale = half_bits_to_float(scale_bits);
-#pragma unroll
-    for (int i = 0; i < 4; ++i) acc[rq][i] = fmaf(d[i], scale, acc[rq][i]);
   }
   // 5. sum over the sixteen blocks (lanes j + 4 b) and store
 #pragma unroll
@@ -270,17 +337,12 @@ __global__ __launch_bounds__(THREADS)
   }
 }
 
-template <int MR, int KL, int RQ, int DEPTH, int EARLY, int THREADS>
+template <int MR, int KL, int RQ, int DEPTH, int EARLY, int THREADS, bool EXACT = true>
 hipError_t launch_instance(const QuadParams &p, uint32_t grid, uint32_t units_per_wg, hipStream_t stream) {
   const size_t lds = quad_lds_bytes<MR, KL, RQ>(units_per_wg);
-  auto kernel = &w4a16_gemv_quad_kernel<MR, KL, RQ, DEPTH, EARLY, THREADS>;
-  static bool configured = false;  // once per process: the kernel may use more than the default 64 KB of LDS
-  if (!configured) {
-    const hipError_t status = hipFuncSetAttribute(reinterpret_cast<const void *>(kernel),
-                                                  hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    if (status != hipSuccess) return status;
-    configured = true;
-  }
+  auto kernel = &w4a16_gemv_quad_kernel<MR, KL, RQ, DEPTH, EARLY, THREADS, EXACT>;
+  static bool configured[kMaxDevices] = {};  // once per device: the kernel may use more than the default 64 KB of LDS
+  if (hipError_t status = allow_dynamic_lds(reinterpret_cast<const void *>(kernel), 160 * 1024, configured)) return status;
   hipLaunchKernelGGL(kernel, dim3(grid), dim3(THREADS), lds, stream, p, units_per_wg);
   return hipGetLastError();
 }
@@ -290,16 +352,51 @@ struct QuadPlan {
   uint32_t rq, waves, grid;
 };
 
-QuadPlan quad_plan(uint32_t n) {
+// most: row quads a workgroup takes at most (14 = seven waves of two).
+QuadPlan quad_plan(uint32_t n, uint32_t most = 14) {
   const uint32_t quads = n / 4;
   const uint32_t cus = (uint32_t)device_compute_units();
-  const uint32_t per_wg = (quads + cus - 1) / cus;
+  uint32_t per_wg = (quads + cus - 1) / cus;
   QuadPlan plan = {0, 0, 0};
-  if (per_wg < 3 || per_wg > 14) return plan;  // too little work per CU, or more than seven waves of two quads
+  if (per_wg < 3) return plan;  // too little work per CU
+  if (per_wg > most) {
+    // several rounds of workgroups, the same number of quads in each
+    const uint32_t rounds = (per_wg + most - 1) / most;
+    per_wg = (quads + cus * rounds - 1) / (cus * rounds);
+  }
   plan.rq = per_wg <= 7 ? 1 : 2;
   plan.waves = (per_wg + plan.rq - 1) / plan.rq;
   plan.grid = (quads + plan.waves * plan.rq - 1) / (plan.waves * plan.rq);
   return plan;
+}
+
+// Any K that is a multiple of 512 within the instantiation's KL ranges: the ring depths of the
+// benchmark shapes' instantiations, chosen by the row length (six loads in flight for every long row).
+// Long rows other than the benchmark's: one quad per wave (a wave that alternates between two quads of
+// 8192 values measured 18.7 us at 8192 x 8192 and four rows against 13.2 with twice the workgroups of one
+// quad per wave).
+uint32_t any_k_most_quads(uint32_t k) { return k > 4096 ? 7 : 14; }
+
+template <int MR, int KL>
+hipError_t launch_rows_any_k(const QuadParams &p, hipStream_t stream) {
+  const QuadPlan plan = quad_plan(p.n, any_k_most_quads(p.k));
+  const bool wide = plan.waves > 4;
+  if (plan.rq == 2) {
+    if constexpr (MR == 4 && KL > 16) {
+      return hipErrorInvalidValue;
+    } else {
+      if (wide) return launch_instance<MR, KL, 2, 8, 2, 448, false>(p, plan.grid, plan.waves, stream);
+      return launch_instance<MR, KL, 2, 8, 2, 256, false>(p, plan.grid, plan.waves, stream);
+    }
+  }
+  if constexpr (KL <= 16) {
+    if (p.k <= 4096) {
+      if (wide) return launch_instance<MR, KL, 1, 4, 4, 448, false>(p, plan.grid, plan.waves, stream);
+      return launch_instance<MR, KL, 1, 4, 4, 256, false>(p, plan.grid, plan.waves, stream);
+    }
+  }
+  if (wide) return launch_instance<MR, KL, 1, 6, 2, 448, false>(p, plan.grid, plan.waves, stream);
+  return launch_instance<MR, KL, 1, 6, 2, 256, false>(p, plan.grid, plan.waves, stream);
 }
 
 template <int MR, int KL>
@@ -338,15 +435,33 @@ hipError_t launch_k(const QuadParams &p, hipStream_t stream) {
   return launch_rows<4, KL>(p, stream);
 }
 
+template <int KL>
+hipError_t launch_any_k(const QuadParams &p, hipStream_t stream) {
+  return launch_rows_any_k<4, KL>(p, stream);
+}
+
+// Rows of up to 8192 values (four rows of more do not fit the LDS block next to their scales; K = 14336
+// has its own instantiation).
+constexpr uint32_t kAnyK = 16 * 512;
+
 }  // namespace
 
 bool w4a16_gemv_quad_ok(const W4LinearArgs &a) {
   if (a.m == 0 || a.m > 4 || a.y == nullptr || a.y_f32 != nullptr) return false;
-  if (a.k != 4096 && a.k != 14336) return false;
   if (a.n % 4 != 0) return false;
   const QuadPlan plan = quad_plan(a.n);
   if (plan.rq == 0) return false;
-  if (a.k == 14336 && a.m > 2 && plan.rq == 2 && plan.waves > 4) return false;  // no instantiation without spills
+  if (a.k == 14336) {
+    if (a.m > 2 && plan.rq == 2 && plan.waves > 4) return false;  // no instantiation without spills
+  } else if (a.k != 4096) {
+    // Other K: three and four activation rows only (at one and two the v_dot2 kernel of
+    // w4a16_gemv.hip measured faster on every such shape: 9.9 against 18.7 us at 16384 x 4096, 9.1 against
+    // 11.7 at 8192 x 8192; at four rows this one wins, 7.4 against 9.7 us at 5120 x 5120, 13.7 against
+    // 15.9 at 5120 x 13824).  K ranges of 512 of which the last may be partly there, at least as many as
+    // the ring's first requests reach; four scale rows a whole number of 16-byte units.
+    if (a.m < 3 || a.k % 128 != 0 || a.k < 2048 || a.k > kAnyK) return false;
+    if (quad_plan(a.n, any_k_most_quads(a.k)).rq == 0) return false;
+  }
   // 16-byte loads of activation rows, weight row pieces and scale rows
   if (((reinterpret_cast<uintptr_t>(a.x) | reinterpret_cast<uintptr_t>(a.w.weight) |
         reinterpret_cast<uintptr_t>(a.w.scale)) & 15) != 0)
@@ -356,9 +471,10 @@ bool w4a16_gemv_quad_ok(const W4LinearArgs &a) {
 
 hipError_t launch_w4a16_gemv_quad_linear(const W4LinearArgs &a, hipStream_t stream) {
   if (!w4a16_gemv_quad_ok(a)) return hipErrorInvalidValue;
-  QuadParams p = {a.x, a.w.weight, a.w.scale, a.y, a.addend, a.has_addend, a.addend_row_stride, a.m, a.n};
+  QuadParams p = {a.x, a.w.weight, a.w.scale, a.y, a.addend, a.has_addend, a.addend_row_stride, a.m, a.n, a.k};
   if (a.k == 4096) return launch_k<8>(p, stream);
-  return launch_k<28>(p, stream);
+  if (a.k == 14336) return launch_k<28>(p, stream);
+  return launch_any_k<16>(p, stream);
 }
 
 }  // namespace llmopt

@@ -354,7 +354,22 @@ QUAD_CELLS = [(3, 4096, 4096, "bias"), (2, 4100, 4096, "residual"), (4, 6144, 40
               (1, 4100, 14336, "bias"), (3, 6144, 14336, "residual"), (4, 4096, 14336, "bias"),
               (2, 9004, 14336, None), (4, 3072, 14336, None),
               # three and four rows of K = 14336 beyond N = 8192 leave the quad kernel (no instantiation without spills)
-              (3, 9004, 14336, "bias")]
+              (3, 9004, 14336, "bias"),
+              # three and four rows at any K that is a multiple of 128 up to 8192 (the instantiations cut for rows
+              # of 8192 values, the walk over K stopping at the row's end, the last 512-wide range partly
+              # there): short and long rings, one and two quads per wave, the shortest and the longest rows;
+              # one and two rows of such K, and longer rows, run the kernels of w4a16_gemv.hip / _mfma.hip
+              (1, 8192, 8192, None), (4, 8192, 8192, "residual"), (1, 5120, 5120, "bias"), (4, 5120, 5120, None),
+              (2, 4096, 2048, "residual"), (3, 12288, 2560, None), (4, 3100, 7680, "bias"), (1, 4096, 11264, None),
+              (2, 9004, 16384, "residual"), (1, 3072, 16384, "bias"), (2, 4096, 10240, None),
+              # N beyond one round of workgroups (28672 rows: two rounds; 49152: four)
+              (1, 28672, 4096, None), (4, 28672, 4096, "residual"), (2, 49152, 2048, "bias"), (1, 30000, 14336, None),
+              # a last K range that is partly there (11008 = 21.5 ranges, 2176 = 4.25, 5248 = 10.25, 16256 = 31.75)
+              (2, 4096, 11008, "bias"), (1, 11008, 11008, None), (4, 4096, 2176, "residual"), (3, 5120, 5248, None),
+              (4, 9004, 7808, "bias"), (2, 3072, 16256, None),
+              (3, 4096, 2048, "bias"), (4, 8192, 4096 + 128, None), (3, 28672, 8192, "residual"),
+              # K not a multiple of 128, four rows beyond 8192
+              (4, 4096, 4160, "bias"), (4, 4096, 11264, None)]
 
 
 @pytest.mark.parametrize("m,n,k,addend", QUAD_CELLS)
