@@ -40,6 +40,7 @@
 #include "kernels.h"
 #include "kernels_internal.h"
 #include "w4_common.h"
+#include "w4_piece.h"
 
 // Time stamps of one workgroup's phases for a scratch timing program (compiled out of the library).
 #ifdef LLMOPT_FUSED_STAMPS
@@ -109,58 +110,6 @@ __device__ __forceinline__ void wait_for_copies_and_meet() {
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
 #endif
   __syncthreads();
-}
-
-// 32 activations of M rows in pair order, and what the biased decode adds to a dot product with them.
-template <int M>
-struct Held {
-  uint4 x[M][4];
-  float correction[M];
-};
-
-// The lane's 32 values [32 piece, 32 piece + 32) of every row, from halves in LDS (row stride `stride` halves).
-template <int M>
-__device__ __forceinline__ void hold_rows(Held<M> &held, const uint16_t *rows, uint32_t stride, uint32_t piece,
-                                          bool present) {
-  // the correction as dot products with the constant pairs (1032, 1032) and (72, 72): exact products,
-  // float32 sums, sixteen instructions instead of a conversion and an addition per value
-  const h2_t bias_a = {(_Float16)1032.0f, (_Float16)1032.0f}, bias_b = {(_Float16)72.0f, (_Float16)72.0f};
-#pragma unroll
-  for (int m = 0; m < M; ++m) {
-    float sum_a = 0.0f, sum_b = 0.0f;
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const uint4 natural = *reinterpret_cast<const uint4 *>(rows + m * stride + piece * 32 + j * 8);
-      const uint4 v = present ? pair_order(natural) : make_uint4(0, 0, 0, 0);
-      held.x[m][j] = v;
-      sum_a = __builtin_amdgcn_fdot2(as_h2(v.x), bias_a, sum_a, false);
-      sum_b = __builtin_amdgcn_fdot2(as_h2(v.y), bias_b, sum_b, false);
-      sum_a = __builtin_amdgcn_fdot2(as_h2(v.z), bias_a, sum_a, false);
-      sum_b = __builtin_amdgcn_fdot2(as_h2(v.w), bias_b, sum_b, false);
-    }
-    held.correction[m] = sum_a + sum_b;
-  }
-}
-
-// One 16-byte piece of a weight row against the held activations: q . x * scale per row, this lane's share.
-template <int M>
-__device__ __forceinline__ void piece_dot(const u32x4_t weights, float scale, const Held<M> &held, float (&out)[M]) {
-  // one accumulator per dword: four short chains instead of one of sixteen
-  float part[M][4];
-#pragma unroll
-  for (int j = 0; j < 4; ++j) {
-    const W4Pairs q = w4_decode_biased(weights[j]);
-#pragma unroll
-    for (int m = 0; m < M; ++m) {
-      float a = __builtin_amdgcn_fdot2(q.p04, as_h2(held.x[m][j].x), 0.0f, false);
-      a = __builtin_amdgcn_fdot2(q.p15, as_h2(held.x[m][j].y), a, false);
-      a = __builtin_amdgcn_fdot2(q.p26, as_h2(held.x[m][j].z), a, false);
-      part[m][j] = __builtin_amdgcn_fdot2(q.p37, as_h2(held.x[m][j].w), a, false);
-    }
-  }
-#pragma unroll
-  for (int m = 0; m < M; ++m)
-    out[m] = (((part[m][0] + part[m][1]) + (part[m][2] + part[m][3])) - held.correction[m]) * scale;
 }
 
 // How the lanes of a wave share whole weight rows of `pieces` 16-byte pieces: `rows_per_step` rows per
@@ -378,7 +327,8 @@ __global__ __launch_bounds__(kThreads) void fused_qkv_kernel(FusedQkvArgs a) {
   FUSED_STAMP(8);
 }
 
-template <int M>
+// PER: pending partial sums a thread adds to the stream on the way in (0: none), as in fused_qkv_kernel.
+template <int M, int PER>
 __global__ __launch_bounds__(kThreads) void fused_ffn_kernel(FusedFfnArgs a) {
   extern __shared__ __attribute__((aligned(16))) uint8_t fused_lds[];
   __shared__ float square_lds[M][kWaves];
@@ -392,6 +342,7 @@ __global__ __launch_bounds__(kThreads) void fused_ffn_kernel(FusedFfnArgs a) {
   uint8_t *down_lds = carve.take(a.k * 32);  // 32 bytes a row: the slice's 64 columns
   uint16_t *down_scales_lds = reinterpret_cast<uint16_t *>(carve.take(a.k * 2));
   uint16_t *x_lds = reinterpret_cast<uint16_t *>(carve.take(M * a.k * 2));
+  f4_t *group_lds = reinterpret_cast<f4_t *>(carve.take(PER > 0 ? kThreads * 16 : 0));
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const uint32_t row0 = blockIdx.y * M;
@@ -415,8 +366,8 @@ __global__ __launch_bounds__(kThreads) void fused_ffn_kernel(FusedFfnArgs a) {
 #pragma unroll
   for (int pass = 0; pass < kScalePasses; ++pass)
     down_scales[pass] = a.down.scale[(size_t)min(threadIdx.x + pass * kThreads, a.k - 1) * (a.n >> 6) + slice];
-  const FusedResidual in = {a.x, nullptr, 0, nullptr};
-  stage_normalised_rows<M, 0>(in, a.norm, a.m, a.k, row0, false, x_lds, nullptr, square_lds);
+  stage_normalised_rows<M, PER>(a.in, a.norm, a.m, a.k, row0, blockIdx.x == 0 && a.in.x_out != nullptr, x_lds, group_lds,
+                                square_lds);
 #pragma unroll
   for (int pass = 0; pass < kScalePasses; ++pass)
     if (threadIdx.x + pass * kThreads < a.k) down_scales_lds[threadIdx.x + pass * kThreads] = down_scales[pass];
@@ -464,13 +415,13 @@ __global__ __launch_bounds__(kThreads) void fused_ffn_kernel(FusedFfnArgs a) {
 bool aligned16(const void *pointer) { return (reinterpret_cast<uintptr_t>(pointer) & 15) == 0; }
 
 constexpr size_t kLdsBudget = 150 * 1024;
-size_t ffn_lds_bytes(uint32_t rows, uint32_t k);
+size_t ffn_lds_bytes(uint32_t rows, uint32_t k, bool partials);
 
 // Sequences per workgroup: one, until the launch has more workgroups than the device holds at once
 // (two share a workgroup's decoded weights; their rows must fit one pass of the staging).
 uint32_t rows_per_workgroup(uint32_t m, uint32_t k, uint32_t column_blocks) {
   return (uint64_t)m * column_blocks > 2ull * (uint32_t)device_compute_units() && 2 * (k >> 2) <= (uint32_t)kThreads &&
-                 ffn_lds_bytes(2, k) <= kLdsBudget
+                 ffn_lds_bytes(2, k, true) <= kLdsBudget
              ? 2
              : 1;
 }
@@ -481,8 +432,9 @@ size_t qkv_lds_bytes(uint32_t rows, uint32_t k, bool partials) {
   return padded(kHead * (k >> 1)) + padded(kHead * (k >> 6) * 2) + padded(rows * k * 2) + (partials ? kThreads * 16 : 0);
 }
 
-size_t ffn_lds_bytes(uint32_t rows, uint32_t k) {
-  return 2 * padded(kHead * (k >> 1)) + 2 * padded(kHead * (k >> 6) * 2) + padded(k * 32) + padded(k * 2) + padded(rows * k * 2);
+size_t ffn_lds_bytes(uint32_t rows, uint32_t k, bool partials) {
+  return 2 * padded(kHead * (k >> 1)) + 2 * padded(kHead * (k >> 6) * 2) + padded(k * 32) + padded(k * 2) +
+         padded(rows * k * 2) + (partials ? kThreads * 16 : 0);
 }
 
 // Partial sums a thread adds on the way in: groups of threads share them (stage_normalised_rows).
@@ -513,15 +465,24 @@ hipError_t launch_qkv_rows(const FusedQkvArgs &a, dim3 grid, hipStream_t stream)
   return launch_qkv_instance<M, 32>(a, grid, lds, stream);
 }
 
-template <int M>
-hipError_t launch_ffn_rows(const FusedFfnArgs &a, dim3 grid, hipStream_t stream) {
-  const size_t lds = ffn_lds_bytes(M, a.k);
+template <int M, int PER>
+hipError_t launch_ffn_instance(const FusedFfnArgs &a, dim3 grid, size_t lds, hipStream_t stream) {
   static bool configured[kMaxDevices] = {};
   if (lds > 64 * 1024)
-    if (hipError_t status = allow_dynamic_lds(reinterpret_cast<const void *>(fused_ffn_kernel<M>), 158 * 1024, configured))
+    if (hipError_t status = allow_dynamic_lds(reinterpret_cast<const void *>(fused_ffn_kernel<M, PER>), 158 * 1024, configured))
       return status;
-  hipLaunchKernelGGL(fused_ffn_kernel<M>, grid, dim3(kThreads), lds, stream, a);
+  hipLaunchKernelGGL((fused_ffn_kernel<M, PER>), grid, dim3(kThreads), lds, stream, a);
   return hipGetLastError();
+}
+
+template <int M>
+hipError_t launch_ffn_rows(const FusedFfnArgs &a, dim3 grid, hipStream_t stream) {
+  const uint32_t per = partials_per_thread(M, a.k, a.in.partial_count);
+  const size_t lds = ffn_lds_bytes(M, a.k, per != 0);
+  if (per == 0) return launch_ffn_instance<M, 0>(a, grid, lds, stream);
+  if (per <= 8) return launch_ffn_instance<M, 8>(a, grid, lds, stream);
+  if (per <= 16) return launch_ffn_instance<M, 16>(a, grid, lds, stream);
+  return launch_ffn_instance<M, 32>(a, grid, lds, stream);
 }
 
 }  // namespace
@@ -544,13 +505,16 @@ hipError_t launch_fused_qkv(const FusedQkvArgs &a, hipStream_t stream) {
   return per == 1 ? launch_qkv_rows<1>(a, grid, stream) : launch_qkv_rows<2>(a, grid, stream);
 }
 
-bool fused_ffn_ok(uint32_t m, uint32_t n, uint32_t k) {
-  return m != 0 && k != 0 && k % 64 == 0 && k <= kFusedMaxWidth && ffn_lds_bytes(1, k) <= kLdsBudget && n != 0 &&
+bool fused_ffn_ok(uint32_t m, uint32_t n, uint32_t k, bool pending) {
+  return m != 0 && k != 0 && k % 64 == 0 && k <= kFusedMaxWidth && ffn_lds_bytes(1, k, pending) <= kLdsBudget && n != 0 &&
          n % kHead == 0 && n / kHead <= kFusedMaxPartials;
 }
 
 hipError_t launch_fused_ffn(const FusedFfnArgs &a, hipStream_t stream) {
-  if (!fused_ffn_ok(a.m, a.n, a.k) || !aligned16(a.x) || !aligned16(a.norm.weight) || !aligned16(a.gate.weight) ||
+  if (a.in.partial_count > kFusedMaxPartials) return hipErrorInvalidValue;
+  if (a.in.partial_count != 0 && (a.in.partials == nullptr || !aligned16(a.in.partials))) return hipErrorInvalidValue;
+  if (a.in.x_out != nullptr && (!aligned16(a.in.x_out) || a.in.x_out == a.in.x)) return hipErrorInvalidValue;
+  if (!fused_ffn_ok(a.m, a.n, a.k, a.in.partial_count != 0) || !aligned16(a.in.x) || !aligned16(a.norm.weight) || !aligned16(a.gate.weight) ||
       !aligned16(a.up.weight) || !aligned16(a.down.weight) || !aligned16(a.partials) || !aligned16(a.gate.scale) ||
       !aligned16(a.up.scale))
     return hipErrorInvalidValue;

@@ -129,14 +129,15 @@ hipError_t launch_fused_qkv(const FusedQkvArgs &args, hipStream_t stream);
 // partial sum over those 64 columns, partials[j][r][:] (float32, scale applied).  The sums over j
 // and the residual are taken by the launch that reads the stream next (FusedResidual).
 struct FusedFfnArgs {
-  const uint16_t *x;   // f16 [m, k]
+  FusedResidual in;    // the stream: rows plus pending partial sums (e.g. of the projecting attention merge)
   W4Norm norm;         // weight_first = 1
   W4Matrix gate, up;   // [n, k/2]
   W4Matrix down;       // [k, n/2]
   float *partials;     // f32 [n / 64, m, k]
   uint32_t m, n, k;
 };
-bool fused_ffn_ok(uint32_t m, uint32_t n, uint32_t k);
+// pending: the input arrives with partial sums to add (their staging takes 8 KiB of the workgroup's memory)
+bool fused_ffn_ok(uint32_t m, uint32_t n, uint32_t k, bool pending = false);
 hipError_t launch_fused_ffn(const FusedFfnArgs &args, hipStream_t stream);
 
 // The product kernels' own nibble decoders run over a whole matrix, as float32 [n, k]:
@@ -223,7 +224,19 @@ struct Q8AttentionArgs {
   uint32_t max_past_length;  // >= every past length (bounds the split grid)
   void *workspace;           // split-context partials
   size_t workspace_bytes;
+  // Optional (no reference kernel; split-context launches with heads of 64 only, see
+  // q8_attention_can_project): instead of storing the output rows, every (sequence, head) row -
+  // rounded to half, as it would have been stored - is multiplied into that head's 64 columns of the
+  // W4 output projection `projection` [projected_width, query_heads * 64 / 2], and the float32
+  // partial sums go to projected[head][sequence][projected_width] (group scale applied).  The sum over
+  // heads and the residual are taken by the launch that reads the stream next (FusedResidual);
+  // `output` may then be null.
+  W4Matrix projection = {nullptr, nullptr};
+  float *projected = nullptr;
+  uint32_t projected_width = 0;
 };
+// True when launch_q8_attention can take args.projected for these arguments.
+bool q8_attention_can_project(const Q8AttentionArgs &args);
 
 // The longest context the split-context kernels take (longer ones run the row-serial kernel).
 constexpr uint32_t kQ8AttentionSplitTokens = 128 * 1024;

@@ -28,6 +28,7 @@
 #include "kernels.h"
 #include "kernels_internal.h"
 #include "w4_common.h"
+#include "w4_piece.h"
 
 namespace llmopt {
 namespace {
@@ -517,19 +518,37 @@ constexpr int kMergeSlices = 4;  // chunk slices summed in parallel per output r
 // finds the global maximum and the per-chunk weights exp2(max_c - max) in
 // parallel over chunks; phase 2 is an independent-load weighted sum over a
 // quarter of the chunks per thread, finished through LDS.
-template <int D>
+// PASSES > 0 (D = 64): the row is not stored but multiplied into the head's 64 columns of an output
+// projection (Q8AttentionArgs::projection): lane pair p of pass i owns output column p + 128 i and
+// the two 16-byte pieces of that weight row that belong to this head (one scale group); the requests
+// for them go out first and land while the partial results are being merged.
+template <int D, int PASSES = 0>
 __global__ __launch_bounds__(kMergeSlices *D) void q8_attention_merge_kernel(Q8AttentionArgs a,
                                                                              uint32_t chunks_max,
                                                                              uint32_t chunk_tokens,
                                                                              uint32_t balanced_slots) {
   constexpr int THREADS = kMergeSlices * D;
   constexpr int WAVES = THREADS / 64;
+  static_assert(PASSES == 0 || D == 64, "a head's columns are one 64-wide scale group of the projection");
   __shared__ float reduce_lds[3][WAVES];
   __shared__ float weight_lds[kMaxSplitChunks];
   __shared__ float slice_lds[kMergeSlices][D];
+  __shared__ __attribute__((aligned(16))) uint16_t row_lds[D];
   const uint32_t head = blockIdx.x;
   const uint32_t batch = blockIdx.y;
   const uint32_t tid = threadIdx.x;
+  u32x4_t projection_weights[PASSES > 0 ? PASSES : 1];
+  uint16_t projection_scales[PASSES > 0 ? PASSES : 1];
+  if constexpr (PASSES > 0) {
+    const uint32_t row_bytes = a.query_heads * (D / 2);
+#pragma unroll
+    for (int i = 0; i < PASSES; ++i) {
+      const size_t column = min((tid >> 1) + (uint32_t)(THREADS / 2) * i, a.projected_width - 1);
+      projection_weights[i] =
+          *reinterpret_cast<const u32x4_t *>(a.projection.weight + column * row_bytes + head * (D / 2) + (tid & 1) * 16);
+      projection_scales[i] = a.projection.scale[column * a.query_heads + head];
+    }
+  }
   const uint32_t d = tid % D;
   const uint32_t slice = tid / D;
   const uint32_t heads_per_kv = a.query_heads / a.kv_heads;
@@ -636,7 +655,26 @@ __global__ __launch_bounds__(kMergeSlices *D) void q8_attention_merge_kernel(Q8A
     float total = 0.0f;
 #pragma unroll
     for (int s = 0; s < kMergeSlices; ++s) total += slice_lds[s][d];
-    a.output[((size_t)batch * a.query_heads + head) * D + d] = float_to_half_bits(total / denominator);
+    const uint16_t stored = float_to_half_bits(total / denominator);
+    if constexpr (PASSES == 0)
+      a.output[((size_t)batch * a.query_heads + head) * D + d] = stored;
+    else
+      row_lds[d] = stored;
+  }
+  if constexpr (PASSES > 0) {
+    __syncthreads();
+    Held<1> held;
+    hold_rows<1>(held, row_lds, D, tid & 1, true);
+    float *out = a.projected + ((size_t)head * a.batches + batch) * a.projected_width;
+#pragma unroll
+    for (int i = 0; i < PASSES; ++i) {
+      float share[1];
+      piece_dot<1>(projection_weights[i], half_bits_to_float(projection_scales[i]), held, share);
+      const float total = share[0] + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
+                                         0, __builtin_bit_cast(int, share[0]), 0xB1, 0xF, 0xF, false));
+      const uint32_t column = (tid >> 1) + (uint32_t)(THREADS / 2) * i;
+      if ((tid & 1) == 0 && column < a.projected_width) out[column] = total;
+    }
   }
 }
 
@@ -1062,7 +1100,14 @@ size_t q8_attention_workspace_bytes(const Q8AttentionArgs &a) {
   return (size_t)a.batches * a.kv_heads * split_chunks(a) * per_partial * sizeof(float);
 }
 
+bool q8_attention_can_project(const Q8AttentionArgs &a) {
+  return a.head_dim == 64 && !use_dense_copy_path(a) && use_split_path(a) && a.projected_width != 0 &&
+         a.projected_width <= 1024 && a.projection.weight != nullptr && a.projection.scale != nullptr &&
+         (reinterpret_cast<uintptr_t>(a.projection.weight) & 15) == 0;
+}
+
 hipError_t launch_q8_attention(const Q8AttentionArgs &a, hipStream_t stream) {
+  if (a.projected != nullptr && !q8_attention_can_project(a)) return hipErrorInvalidValue;
   if (use_dense_copy_path(a)) {
     if (a.batches == 0 || a.query_heads == 0) return hipSuccess;
     const DenseCopyPlan plan = dense_copy_plan(a, a.workspace);
@@ -1099,6 +1144,17 @@ hipError_t launch_q8_attention(const Q8AttentionArgs &a, hipStream_t stream) {
         hipLaunchKernelGGL((q8_attention_split_kernel<D, false, true>), grid, block, 0, stream, a, chunks, chunk_tokens, slots);
       else
         hipLaunchKernelGGL((q8_attention_split_kernel<D, false, false>), grid, block, 0, stream, a, chunks, chunk_tokens, slots);
+      if constexpr (D == 64) {
+        if (a.projected != nullptr) {
+          if (a.projected_width <= 640)
+            hipLaunchKernelGGL((q8_attention_merge_kernel<64, 5>), merge_grid, dim3(kMergeSlices * 64), 0, stream, a, chunks,
+                               chunk_tokens, slots);
+          else
+            hipLaunchKernelGGL((q8_attention_merge_kernel<64, 8>), merge_grid, dim3(kMergeSlices * 64), 0, stream, a, chunks,
+                               chunk_tokens, slots);
+          return;
+        }
+      }
       hipLaunchKernelGGL(q8_attention_merge_kernel<D>, merge_grid, dim3(kMergeSlices * D), 0, stream, a, chunks,
                          chunk_tokens, slots);
     };

@@ -232,9 +232,13 @@ int cache_unpack_checkpoint(llmopt_hip_context *context, const DispatchRecord &r
 //
 // The batched extension appends u32 max_past_length at byte 64 and two
 // buffers: past_lengths u32[batches], slot_offsets u32[batches].
-int paged_attention(llmopt_hip_context *context, const DispatchRecord &record, bool batched) {
-  if (int status = require_buffer_count(record, batched ? 9 : 7)) return status;
-  if (int status = require_parameter_bytes(record, batched ? 68 : 64)) return status;
+// projecting (extension llmopt_attention_q8_paged_batched_w4a16_partial_g64, batched only): the output rows
+// are not stored but multiplied, head by head, into an output projection; buffer 6 receives the float32
+// partial sums [query_heads, batches, hidden] instead, two more buffers hold the projection's packed
+// weights [hidden, query_heads * 64 / 2] and scales, and u32 hidden follows the batched parameter words.
+int paged_attention(llmopt_hip_context *context, const DispatchRecord &record, bool batched, bool projecting = false) {
+  if (int status = require_buffer_count(record, projecting ? 11 : batched ? 9 : 7)) return status;
+  if (int status = require_parameter_bytes(record, projecting ? 72 : batched ? 68 : 64)) return status;
   Q8AttentionArgs args = {};
   args.batches = param_u32(record, 0);
   args.query_heads = param_u32(record, 4);
@@ -288,7 +292,20 @@ int paged_attention(llmopt_hip_context *context, const DispatchRecord &record, b
     if (batched && args.mask_batches != 0)
       return fail(LLMOPT_ERR_INVALID, "%s does not take a mask", name);
   }
-  if (int status = require_buffer_size(record.buffers[6], q_bytes, "output")) return status;
+  if (projecting) {
+    args.projected_width = param_u32(record, 68);
+    const uint64_t hidden = args.projected_width, width = (uint64_t)args.query_heads * args.head_dim;
+    if (hidden == 0 || args.head_dim != 64)
+      return fail(LLMOPT_ERR_INVALID, "%s takes heads of 64 and a positive projection width", name);
+    if (int status = require_buffer_size(record.buffers[6], (uint64_t)args.query_heads * args.batches * hidden * 4, "partial sums"))
+      return status;
+    if (int status = require_buffer_size(record.buffers[9], hidden * (width / 2), "projection packed weight")) return status;
+    if (int status = require_buffer_size(record.buffers[10], hidden * (width / 64) * 2, "projection scale")) return status;
+    args.projection = {record.buffers[9].device, reinterpret_cast<const uint16_t *>(record.buffers[10].device)};
+    args.projected = reinterpret_cast<float *>(record.buffers[6].device);
+  } else if (int status = require_buffer_size(record.buffers[6], q_bytes, "output")) {
+    return status;
+  }
   args.query = reinterpret_cast<const uint16_t *>(record.buffers[0].device);
   args.current_key = reinterpret_cast<const uint16_t *>(record.buffers[1].device);
   args.current_value = reinterpret_cast<const uint16_t *>(record.buffers[2].device);
@@ -296,7 +313,7 @@ int paged_attention(llmopt_hip_context *context, const DispatchRecord &record, b
   args.pool_bytes = record.buffers[3].length;
   args.slots = reinterpret_cast<const uint32_t *>(record.buffers[4].device);
   args.mask = masked ? record.buffers[5].device : nullptr;
-  args.output = reinterpret_cast<uint16_t *>(record.buffers[6].device);
+  args.output = projecting ? nullptr : reinterpret_cast<uint16_t *>(record.buffers[6].device);
   if (retained) {
     if (masked) return fail(LLMOPT_ERR_INVALID, "%s with a mask cannot read its context length from device memory", name);
     args.past_lengths = record.device_past_lengths;
@@ -307,6 +324,9 @@ int paged_attention(llmopt_hip_context *context, const DispatchRecord &record, b
     args.past_lengths = reinterpret_cast<const uint32_t *>(record.buffers[7].device);
     args.slot_offsets = reinterpret_cast<const uint32_t *>(record.buffers[8].device);
   }
+  if (projecting && !q8_attention_can_project(args))
+    return fail(LLMOPT_ERR_INVALID, "%s takes what the split-context kernels take (one query token, no mask, contexts of "
+                "64 tokens and more in the launch) and a projection of at most 1024 rows", name);
   const size_t workspace_bytes = q8_attention_workspace_bytes(args);
   if (workspace_bytes > 0) {
     args.workspace = context_workspace(context, workspace_bytes);
@@ -322,6 +342,10 @@ int paged_attention_reference(llmopt_hip_context *context, const DispatchRecord 
 
 int paged_attention_batched(llmopt_hip_context *context, const DispatchRecord &record) {
   return paged_attention(context, record, true);
+}
+
+int paged_attention_batched_projecting(llmopt_hip_context *context, const DispatchRecord &record) {
+  return paged_attention(context, record, true, true);
 }
 
 // AttentionParams, 14 x 4 bytes (lib/metal_attention_source.ml:251-256,
@@ -481,6 +505,8 @@ void register_attention_kernels(std::vector<KernelEntryPoint> &table) {
   table.push_back({"llmopt_attention_tree_speculative_f16_simd_h64", attention, speculative_attention});
   // Extension: per-sequence context lengths and slot tables in one launch.
   table.push_back({"llmopt_attention_q8_paged_batched", attention, paged_attention_batched});
+  // Extension: the same with every head's output row multiplied into its columns of a W4 output projection.
+  table.push_back({"llmopt_attention_q8_paged_batched_w4a16_partial_g64", attention, paged_attention_batched_projecting});
 }
 
 }  // namespace llmopt

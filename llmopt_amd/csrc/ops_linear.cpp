@@ -292,34 +292,60 @@ int rms_w4a16_qkv_rotary_pack(llmopt_hip_context *context, const DispatchRecord 
 // intermediate, a float32 partial sum of every output; the launch that reads the stream next adds them
 // and the residual (llmopt_rms_w4a16_qkv_rotary_pack_q8_f16_g64).  W4A16SwiGLUFFNParams {u32 m, n, k; f32 eps}.
 // buffers: input f16 [m,k], norm weight, gateW, gateS, upW, upS, downW, downS, partials f32 [n/64,m,k].
-int rms_w4a16_swiglu_down_partial(llmopt_hip_context *context, const DispatchRecord &record) {
-  if (int status = require_buffer_count(record, 9)) return status;
-  if (int status = require_parameter_bytes(record, 16)) return status;
+// `summing` (llmopt_sum_rms_w4a16_swiglu_down_partial_f16_g64): the input itself arrives as rows plus
+// pending partial sums (of the projecting attention entry) and is written out whole: buffers input,
+// pending f32 [pending_count,m,k], stream f16 [m,k], then as above; u32 pending_count follows epsilon.
+int swiglu_down_partial(llmopt_hip_context *context, const DispatchRecord &record, bool summing) {
+  const size_t b = summing ? 2 : 0;
+  if (int status = require_buffer_count(record, 9 + b)) return status;
+  if (int status = require_parameter_bytes(record, summing ? 20 : 16)) return status;
   const char *name = record.name.c_str();
   const uint32_t m = param_u32(record, 0), n = param_u32(record, 4), k = param_u32(record, 8);
   const float epsilon = param_f32(record, 12);
   if (int status = check_w4_shape(name, m, n, k)) return status;
-  if (!fused_ffn_ok(m, n, k))
+  if (!fused_ffn_ok(m, n, k, summing && param_u32(record, 16) != 0))
     return fail(LLMOPT_ERR_INVALID, "%s takes a hidden width k whose slice of the three matrices fits a workgroup's "
-                "memory (k <= 1472) and n a multiple of 64 up to %u, got k = %u, n = %u", name, 64 * kFusedMaxPartials, k, n);
+                "memory (k <= 1472, with pending sums k <= 1344) and n a multiple of 64 up to %u, got k = %u, n = %u", name,
+                64 * kFusedMaxPartials, k, n);
   if (!std::isfinite(epsilon) || epsilon <= 0.0f) return fail(LLMOPT_ERR_INVALID, "%s requires a positive finite epsilon", name);
   if (int status = require_buffer_size(record.buffers[0], (uint64_t)m * k * 2, "input")) return status;
-  if (int status = require_buffer_size(record.buffers[1], (uint64_t)k * 2, "norm weight")) return status;
-  if (int status = check_w4_matrix(record.buffers[2], record.buffers[3], n, k, "gate")) return status;
-  if (int status = check_w4_matrix(record.buffers[4], record.buffers[5], n, k, "up")) return status;
-  if (int status = check_w4_matrix(record.buffers[6], record.buffers[7], k, n, "down")) return status;
-  if (int status = require_buffer_size(record.buffers[8], (uint64_t)(n / 64) * m * k * 4, "partial sums")) return status;
+  if (int status = require_buffer_size(record.buffers[b + 1], (uint64_t)k * 2, "norm weight")) return status;
+  if (int status = check_w4_matrix(record.buffers[b + 2], record.buffers[b + 3], n, k, "gate")) return status;
+  if (int status = check_w4_matrix(record.buffers[b + 4], record.buffers[b + 5], n, k, "up")) return status;
+  if (int status = check_w4_matrix(record.buffers[b + 6], record.buffers[b + 7], k, n, "down")) return status;
+  if (int status = require_buffer_size(record.buffers[b + 8], (uint64_t)(n / 64) * m * k * 4, "partial sums")) return status;
   FusedFfnArgs args = {};
-  args.x = as_f16(record.buffers[0]);
-  args.norm = {as_f16(record.buffers[1]), epsilon, 1};
-  args.gate = {record.buffers[2].device, as_f16(record.buffers[3])};
-  args.up = {record.buffers[4].device, as_f16(record.buffers[5])};
-  args.down = {record.buffers[6].device, as_f16(record.buffers[7])};
-  args.partials = reinterpret_cast<float *>(record.buffers[8].device);
+  args.in.x = as_f16(record.buffers[0]);
+  if (summing) {
+    args.in.partial_count = param_u32(record, 16);
+    if (args.in.partial_count > kFusedMaxPartials)
+      return fail(LLMOPT_ERR_INVALID, "%s takes at most %u pending partial sums, got %u", name, kFusedMaxPartials, args.in.partial_count);
+    if (args.in.partial_count != 0)
+      if (int status = require_buffer_size(record.buffers[1], (uint64_t)args.in.partial_count * m * k * 4, "pending partial sums"))
+        return status;
+    if (int status = require_buffer_size(record.buffers[2], (uint64_t)m * k * 2, "stream")) return status;
+    args.in.partials = reinterpret_cast<const float *>(record.buffers[1].device);
+    args.in.x_out = reinterpret_cast<uint16_t *>(record.buffers[2].device);
+    if (args.in.x_out == args.in.x)
+      return fail(LLMOPT_ERR_INVALID, "%s writes the stream while other workgroups still read the input: two buffers", name);
+  }
+  args.norm = {as_f16(record.buffers[b + 1]), epsilon, 1};
+  args.gate = {record.buffers[b + 2].device, as_f16(record.buffers[b + 3])};
+  args.up = {record.buffers[b + 4].device, as_f16(record.buffers[b + 5])};
+  args.down = {record.buffers[b + 6].device, as_f16(record.buffers[b + 7])};
+  args.partials = reinterpret_cast<float *>(record.buffers[b + 8].device);
   args.m = m;
   args.n = n;
   args.k = k;
   return launched(launch_fused_ffn(args, context->stream), name);
+}
+
+int rms_w4a16_swiglu_down_partial(llmopt_hip_context *context, const DispatchRecord &record) {
+  return swiglu_down_partial(context, record, false);
+}
+
+int sum_rms_w4a16_swiglu_down_partial(llmopt_hip_context *context, const DispatchRecord &record) {
+  return swiglu_down_partial(context, record, true);
 }
 
 // Extension (no reference kernel): float32 [n,k] from the product kernels' own nibble decoders,
@@ -382,6 +408,7 @@ void register_linear_kernels(std::vector<KernelEntryPoint> &table) {
   table.push_back({"llmopt_w4a16_down_add_f16_g64_m8", ffn, w4a16_down_add});
   table.push_back({"llmopt_rms_w4a16_qkv_rotary_pack_q8_f16_g64", qkv, rms_w4a16_qkv_rotary_pack});
   table.push_back({"llmopt_rms_w4a16_swiglu_down_partial_f16_g64", ffn, rms_w4a16_swiglu_down_partial});
+  table.push_back({"llmopt_sum_rms_w4a16_swiglu_down_partial_f16_g64", ffn, sum_rms_w4a16_swiglu_down_partial});
   table.push_back({"llmopt_w4_dequant_f32", linear, w4_dequant_f32});
   table.push_back({"llmopt_q8_decode_f32", "cache", q8_decode_f32});
 }

@@ -34,6 +34,8 @@ from .native import Buffer, Runtime
 # tokens of context, ms per step fused / not: batch 1 0.794 / 0.794, 2 0.852 / 0.977, 8 0.923 / 1.048,
 # 16 1.132 / 1.169, 24 1.372 / 1.302, 32 1.418 / 1.346, 64 2.08 / 1.93.
 FUSED_MAX_BATCH = 16
+# The attention launch multiplies its heads into the output projection where it can (three launches a layer).
+PROJECTING_ATTENTION = True
 
 
 def u32s(*values) -> bytes:
@@ -134,16 +136,19 @@ class DecodeStep:
 
     def __init__(self, runtime: Runtime, config: DecodeConfig, weights: dict, batch: int, pool: Buffer,
                  slots: Buffer, slot_offsets, past_lengths, new_slots, positions, max_context=None,
-                 slots_host=None, reference_entries: bool = False, fused: bool | None = None):
+                 slots_host=None, reference_entries: bool = False, fused: bool | None = None,
+                 projecting: bool | None = None):
         """max_context: the longest context any later step will have (sizes the attention launch;
         default: the longest now).  slots_host: the host copy of the slot table, with room behind
         every sequence's slots for the tokens `advance` will add.  reference_entries (batch 1):
         rotation, cache pack and attention as the reference's own three kernels
         (llmopt_rotary_qk_f16_simd_h64, llmopt_cache_pack_attention_q8_pair_simd,
         llmopt_attention_q8_paged_simd_h64_gqa3) instead of the batched extension entries.
-        fused (default: whenever the shapes allow and reference_entries is off): four launches a
-        layer - norm + QKV + rotation + cache pack as one, attention, output projection, and the
-        SwiGLU FFN as one that leaves partial sums for the next layer's first launch - instead of six."""
+        fused (default: whenever the shapes allow and reference_entries is off): norm + QKV + rotation
+        + cache pack as one launch, attention, output projection, and the SwiGLU FFN as one that leaves
+        partial sums for the next layer's first launch - four launches a layer instead of six; three
+        where the attention launch can multiply its heads into the output projection itself
+        (`self.projecting`: contexts of 64 tokens and more, hidden <= 1024, at most 32 query heads)."""
         self.runtime, self.config, self.batch = runtime, config, batch
         self.reference_entries = reference_entries
         if reference_entries and batch != 1:
@@ -153,6 +158,12 @@ class DecodeStep:
         if fused and (reference_entries or not can_fuse):
             raise ValueError("the fused launches take heads of 64, hidden <= 1472 and mlp <= 2048")
         self.fused = can_fuse and not reference_entries and batch <= FUSED_MAX_BATCH if fused is None else fused
+        self.max_past = int(max(past_lengths)) if max_context is None else int(max_context)
+        can_project = bool(self.fused and self.max_past >= 64 and config.hidden <= 1024 and config.q_heads <= 32)
+        if projecting and not can_project:
+            raise ValueError("the projecting attention takes a fused step, contexts of 64 tokens and more, "
+                             "hidden <= 1024 and at most 32 query heads")
+        self.projecting = can_project and PROJECTING_ATTENTION if projecting is None else projecting
         self.host_lengths = np.asarray(past_lengths, dtype=np.uint32).copy()
         self.host_offsets = np.asarray(slot_offsets, dtype=np.uint32).copy()
         self.host_positions = np.asarray(positions, dtype=np.int64).copy()
@@ -171,7 +182,6 @@ class DecodeStep:
         self.trig = b(np.concatenate([cos, sin]))
         self.cos = self.trig.view(0, cos.nbytes)
         self.sin = self.trig.view(cos.nbytes, sin.nbytes)
-        self.max_past = int(max(past_lengths)) if max_context is None else int(max_context)
         self.device = {
             "embedding": b(weights["embedding"]),
             "final_norm": b(weights["final_norm"]),
@@ -191,6 +201,8 @@ class DecodeStep:
         if self.fused:
             self.work["stream"] = create(batch * h * 2)
             self.work["partials"] = create((c.mlp // 64) * batch * h * 4)
+        if self.projecting:
+            self.work["head_partials"] = create(c.q_heads * batch * h * 4)
         self.dispatches = self._build()
 
     def _linear_entry(self, columns_of_one_row: int):
@@ -249,16 +261,24 @@ class DecodeStep:
                     u32s(m, c.vocabulary, h) + struct.pack("<f", c.epsilon), (m * 256, 1, 1), group))
         return out
 
-    def _batched_attention(self, key_offset: int, value_offset: int) -> tuple:
+    def _batched_attention(self, key_offset: int, value_offset: int, projection=None) -> tuple:
+        """projection: the output projection's (weights, scales) for the entry that leaves every head's
+        share of it as float32 partial sums instead of the attention rows."""
         c, m, w = self.config, self.batch, self.work
         attention_params = struct.pack(
             "<12IfIII", m, c.q_heads, c.kv_heads, 0, c.head_dim, 0, 0, c.token_elements, key_offset,
             value_offset, 64, c.token_stride, 1.0 / math.sqrt(c.head_dim), 1, 0, 0)
         attention_params += struct.pack("<I", self.max_past)
+        grid = (((m * c.q_heads + 7) // 8) * 256, 1, 1)
+        if projection is not None:
+            return ("llmopt_attention_q8_paged_batched_w4a16_partial_g64",
+                    [w["q_rot"], w["k_rot"], w["v"], self.pool, self.slots, self.slots, w["head_partials"],
+                     self.past_lengths, self.slot_offsets, *projection],
+                    attention_params + struct.pack("<I", c.hidden), grid, (256, 1, 1))
         return ("llmopt_attention_q8_paged_batched",
                 [w["q_rot"], w["k_rot"], w["v"], self.pool, self.slots, self.slots, w["attention"],
                  self.past_lengths, self.slot_offsets],
-                attention_params, (((m * c.q_heads + 7) // 8) * 256, 1, 1), (256, 1, 1))
+                attention_params, grid, (256, 1, 1))
 
     def _fused_layer(self, index: int, layer: dict, key_offset: int, value_offset: int) -> list[tuple]:
         """Four launches: the residual stream enters as the previous layer's `x_mid` plus the partial
@@ -275,12 +295,21 @@ class DecodeStep:
                  self.trig, w["q_rot"], w["k_rot"], w["v"], self.new_slots, self.pool],
                 u32s(m, h, qd, kvd, kvd) + struct.pack("<f", c.epsilon) +
                 u32s(0 if first else slices, key_offset, value_offset, c.token_elements, c.token_stride),
-                (((qd + 2 * kvd) // 64) * 256, m, 1), group),
-               self._batched_attention(key_offset, value_offset)]
+                (((qd + 2 * kvd) // 64) * 256, m, 1), group)]
+        ffn_params = u32s(m, c.mlp, h) + struct.pack("<f", c.epsilon)
+        if self.projecting and not last:
+            # three launches: the attention leaves each head's share of the output projection, the
+            # FFN launch adds them to the stream on its way in
+            out.append(self._batched_attention(key_offset, value_offset, projection=layer["o"]))
+            out.append(("llmopt_sum_rms_w4a16_swiglu_down_partial_f16_g64",
+                        [w["stream"], w["head_partials"], w["x"][1], layer["ffn_norm"], *layer["gate"], *layer["up"],
+                         *layer["down"], w["partials"]],
+                        ffn_params + u32s(c.q_heads), (slices * 256, m, 1), group))
+            return out
+        out.append(self._batched_attention(key_offset, value_offset))
         suffix, grid = self._linear_entry(h)
         out.append(("llmopt_w4a16_linear_f16_g64" + suffix,
                     [w["attention"], *layer["o"], w["stream"], w["x"][1]], u32s(m, h, qd, 1, h), grid, group))
-        ffn_params = u32s(m, c.mlp, h) + struct.pack("<f", c.epsilon)
         if not last:
             out.append(("llmopt_rms_w4a16_swiglu_down_partial_f16_g64",
                         [w["x"][1], layer["ffn_norm"], *layer["gate"], *layer["up"], *layer["down"], w["partials"]],

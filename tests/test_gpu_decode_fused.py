@@ -1,6 +1,8 @@
 """The fused decode-step launches (llmopt_rms_w4a16_qkv_rotary_pack_q8_f16_g64,
-llmopt_rms_w4a16_swiglu_down_partial_f16_g64) against the launches they stand for and against the
-CPU oracle, and the decode step built from them against the oracle's chain."""
+llmopt_rms_w4a16_swiglu_down_partial_f16_g64, llmopt_sum_rms_w4a16_swiglu_down_partial_f16_g64,
+llmopt_attention_q8_paged_batched_w4a16_partial_g64) against the launches they stand for and against
+the CPU oracle, and the decode step built from them against the oracle's chain."""
+import math
 import struct
 
 import numpy as np
@@ -187,17 +189,118 @@ def test_fused_ffn_partial_sums_against_separate_launches_and_oracle(runtime, m,
         assert error <= 2e-3, f"partial sum {p}: {error:.3e}"  # the product's half rounding carries over
 
 
+@pytest.mark.parametrize("m,n,k,pending", [(1, 1536, 576, 9), (2, 1536, 576, 9), (8, 1536, 576, 9), (5, 128, 1024, 32),
+                                           (3, 256, 704, 1), (16, 1536, 576, 9), (4, 64, 576, 0)])
+def test_summing_ffn_forms_the_stream_and_leaves_the_partial_sums_of_the_plain_entry(runtime, m, n, k, pending):
+    rng = np.random.default_rng(11 * m + n + k + pending)
+    x, pending_sums, stream = pending_stream(rng, m, k, pending)
+    gain = rng.uniform(0.5, 1.5, k).astype(np.float16)
+    b = runtime.buffer_of_bytes
+    device = [b(a) for pair in (random_w4(rng, n, k), random_w4(rng, n, k), random_w4(rng, k, n)) for a in pair]
+    slices = n // 64
+    params = u32s(m, n, k) + struct.pack("<f", 1e-5)
+    stream_out = b(np.full(m * k, np.nan, dtype=np.float16))
+    partials = b(np.full(slices * m * k, np.nan, dtype=np.float32))
+    runtime.dispatch("llmopt_sum_rms_w4a16_swiglu_down_partial_f16_g64",
+                     [b(x), b(pending_sums), stream_out, b(gain), *device, partials], params + u32s(pending),
+                     grid=(256, 1, 1), group=GROUP)
+    got_stream = stream_out.numpy(np.float16, (m, k))
+    assert np.all(np.isfinite(got_stream))
+    step = np.spacing(np.abs(stream)).astype(np.float64)
+    operands = np.abs(x).astype(np.float64) + np.abs(pending_sums[:pending]).astype(np.float64).sum(axis=0)
+    assert np.all(np.abs(got_stream.astype(np.float64) - stream.astype(np.float64)) <= step + 4e-7 * operands)
+    assert np.mean(got_stream != stream) < 0.01
+    # the plain entry on the stream this launch formed: the same kernel from there on, bit for bit
+    plain = b(np.full(slices * m * k, np.nan, dtype=np.float32))
+    runtime.dispatch("llmopt_rms_w4a16_swiglu_down_partial_f16_g64", [b(got_stream), b(gain), *device, plain], params,
+                     grid=(256, 1, 1), group=GROUP)
+    np.testing.assert_array_equal(partials.numpy(np.uint32, (slices, m, k)), plain.numpy(np.uint32, (slices, m, k)))
+
+
+def paged_case(rng, batch, q_heads, kv_heads, lengths):
+    """A ragged batch over a pool of one layer's slots: (pool, slots, offsets, stride, token_elements)."""
+    token_elements = 2 * kv_heads * 64
+    stride = token_elements + 2 * (token_elements // 64)
+    total = int(np.sum(lengths))
+    capacity = total + 5
+    slots = rng.permutation(capacity).astype(np.uint32)[:total]
+    offsets = np.concatenate([[0], np.cumsum(lengths)[:-1]]).astype(np.uint32)
+    pool = np.zeros((capacity, stride), dtype=np.uint8)
+    pool[:, :token_elements] = np.clip(np.rint(rng.standard_normal((capacity, token_elements)) * 38), -127, 127) \
+        .astype(np.int8).view(np.uint8)
+    pool[:, token_elements:] = rng.uniform(0.02, 0.035, (capacity, token_elements // 64)).astype(np.float16) \
+        .view(np.uint8).reshape(capacity, -1)
+    return pool, slots, offsets, stride, token_elements
+
+
+@pytest.mark.parametrize("batch,q_heads,kv_heads,hidden,longest", [(1, 9, 3, 576, 2048), (1, 9, 3, 576, 64), (2, 9, 3, 576, 300),
+                                                                   (8, 9, 3, 576, 2048), (5, 8, 2, 1024, 700),
+                                                                   (16, 9, 3, 576, 500), (3, 4, 4, 64, 150),
+                                                                   (33, 2, 1, 704, 260)])
+def test_projecting_attention_leaves_each_heads_share_of_the_output_projection(runtime, batch, q_heads, kv_heads, hidden,
+                                                                               longest):
+    rng = np.random.default_rng(batch * 1000 + hidden + longest)
+    lengths = rng.integers(1, longest + 1, size=batch).astype(np.uint32)
+    lengths[rng.integers(0, batch)] = longest
+    pool, slots, offsets, stride, token_elements = paged_case(rng, batch, q_heads, kv_heads, lengths)
+    width = q_heads * 64
+    query = rng.standard_normal((batch, width)).astype(np.float16)
+    key = rng.standard_normal((batch, kv_heads * 64)).astype(np.float16)
+    value = rng.standard_normal((batch, kv_heads * 64)).astype(np.float16)
+    projection = random_w4(rng, hidden, width)
+    b = runtime.buffer_of_bytes
+    shared = [b(query), b(key), b(value), b(pool), b(slots)]
+    tail = [b(lengths), b(offsets)]
+    device_projection = [b(a) for a in projection]
+    params = struct.pack("<12IfIII", batch, q_heads, kv_heads, 0, 64, 0, 0, token_elements, 0, kv_heads * 64, 64, stride,
+                         1.0 / math.sqrt(64), 1, 0, 0) + struct.pack("<I", longest)
+    rows = b(np.full(batch * width, np.nan, dtype=np.float16))
+    runtime.dispatch("llmopt_attention_q8_paged_batched", [*shared, shared[4], rows, *tail], params, grid=(256, 1, 1), group=GROUP)
+    attention = rows.numpy(np.float16, (batch, width))
+    partials = b(np.full(q_heads * batch * hidden, np.nan, dtype=np.float32))
+    runtime.dispatch("llmopt_attention_q8_paged_batched_w4a16_partial_g64",
+                     [*shared, shared[4], partials, *tail, *device_projection], params + u32s(hidden), grid=(256, 1, 1), group=GROUP)
+    got = partials.numpy(np.float32, (q_heads, batch, hidden))
+    assert np.all(np.isfinite(got))
+    # every head's 64 columns of the contraction, on the rows the plain entry stores (the same merge, rounded to half)
+    for head in range(q_heads):
+        packed = np.ascontiguousarray(projection[0][:, 32 * head:32 * head + 32])
+        scale = np.ascontiguousarray(projection[1][:, head:head + 1])
+        want = oracle.w4a16_linear(attention[:, 64 * head:64 * head + 64], packed, scale, None)
+        error = np.linalg.norm(got[head] - want) / max(np.linalg.norm(want), 1e-30)
+        # (the two instantiations of the merge may round an element of a row to neighbouring halves: 5e-4 of
+        # one element in 64)
+        assert error <= 2e-4, f"head {head}: {error:.3e}"
+    # and their sum in ascending order against the output-projection launch
+    total = np.zeros((batch, hidden), dtype=np.float32)
+    for head in range(q_heads):
+        total = total + got[head]
+    projected = b(np.zeros(batch * hidden, dtype=np.float16))
+    runtime.dispatch("llmopt_w4a16_linear_f16_g64" + ("" if batch == 1 else "_m4"), [rows, *device_projection, rows, projected],
+                     u32s(batch, hidden, width, 0, hidden), grid=(256, 1, 1), group=GROUP)
+    assert_close_to_oracle(total.astype(np.float16), projected.numpy(np.float16, (batch, hidden)).astype(np.float32),
+                           "sum of the shares vs the projection launch", rel_l2_tol=3e-4)
+
+
 def test_fused_entries_reject_what_they_cannot_take(runtime):
     from llmopt_amd.native import LlmoptError
     b = runtime.buffer_of_bytes
     any_buffer = b(np.zeros(4096, dtype=np.uint8))
-    with pytest.raises(LlmoptError, match="k <= 1472"):
+    with pytest.raises(LlmoptError, match="k <= 1472,"):
         runtime.dispatch("llmopt_rms_w4a16_swiglu_down_partial_f16_g64", [any_buffer] * 9,
                          u32s(1, 64, 4096) + struct.pack("<f", 1e-5), grid=(256, 1, 1), group=GROUP)
     with pytest.raises(LlmoptError, match="whole heads of 64"):
         runtime.dispatch("llmopt_rms_w4a16_qkv_rotary_pack_q8_f16_g64", [any_buffer] * 16,
                          u32s(1, 64, 64, 32, 32) + struct.pack("<f", 1e-5) + u32s(0, 0, 64, 128, 132),
                          grid=(256, 1, 1), group=GROUP)
+    with pytest.raises(LlmoptError, match="contexts of 64 tokens and more"):
+        big = b(np.zeros(1 << 16, dtype=np.uint8))
+        runtime.dispatch("llmopt_attention_q8_paged_batched_w4a16_partial_g64", [big] * 11,
+                         struct.pack("<12IfIII", 1, 1, 1, 0, 64, 0, 0, 128, 0, 64, 64, 132, 0.125, 1, 0, 0) + u32s(10, 64),
+                         grid=(256, 1, 1), group=GROUP)
+    with pytest.raises(LlmoptError, match="at most 32 pending"):
+        runtime.dispatch("llmopt_sum_rms_w4a16_swiglu_down_partial_f16_g64", [any_buffer] * 11,
+                         u32s(1, 64, 64) + struct.pack("<f", 1e-5) + u32s(33), grid=(256, 1, 1), group=GROUP)
     with pytest.raises(LlmoptError, match="two buffers"):
         big = b(np.zeros(1 << 16, dtype=np.uint8))
         runtime.dispatch("llmopt_rms_w4a16_qkv_rotary_pack_q8_f16_g64", [big] * 16,
@@ -207,7 +310,7 @@ def test_fused_entries_reject_what_they_cannot_take(runtime):
 
 @pytest.mark.parametrize("batch", [1, 2, 8, 32])
 def test_fused_step_leaves_what_the_unfused_step_leaves(runtime, batch):
-    """The same step as four launches a layer and as six: tokens equal, hidden state and cache within
+    """The same step as three or four launches a layer and as six: hidden state and cache within
     the half roundings the two orders of float32 sums allow; three layers, so that the partial sums
     pass from layer to layer twice and the last layer's whole stream feeds the LM head."""
     from llmopt_amd.decode_step import DecodeConfig, DecodeStep, random_weights
@@ -215,6 +318,7 @@ def test_fused_step_leaves_what_the_unfused_step_leaves(runtime, batch):
     config = DecodeConfig(layers=3, vocabulary=1000)
     weights = random_weights(config, rng)
     lengths = [int(v) for v in rng.integers(1, 200, size=batch)]
+    lengths[0] = max(lengths[0], 70)  # long enough for the projecting attention
     total = sum(lengths)
     capacity = total + batch
     order = rng.permutation(capacity).astype(np.uint32)
@@ -228,29 +332,33 @@ def test_fused_step_leaves_what_the_unfused_step_leaves(runtime, batch):
         .view(np.uint8).reshape(capacity, -1)
     tokens = rng.integers(0, config.vocabulary, batch)
     results = {}
-    for fused in (False, True):
+    # six launches a layer, four, and three (the last layer of a fused step: five)
+    launches = {"unfused": 2 + 6 * config.layers, "fused": 2 + 4 * config.layers + 1, "projecting": 2 + 3 * (config.layers - 1) + 5}
+    for mode in launches:
         device_pool = runtime.buffer_of_bytes(pool)
         step = DecodeStep(runtime, config, weights, batch, device_pool, runtime.buffer_of_bytes(slots), offsets,
-                          lengths, new_slots, lengths, fused=fused)
-        assert step.fused == fused
-        assert len(step.dispatches) == (2 + 4 * config.layers + 1 if fused else 2 + 6 * config.layers)
+                          lengths, new_slots, lengths, fused=mode != "unfused", projecting=mode == "projecting")
+        assert step.fused == (mode != "unfused") and step.projecting == (mode == "projecting")
+        assert len(step.dispatches) == launches[mode]
         got_tokens = step.run(tokens)
-        results[fused] = (got_tokens, step.work["x"][0].numpy(np.float16, (batch, config.hidden)),
-                          device_pool.numpy(np.uint8, (capacity, stride)))
-    assert_close_to_oracle(results[True][1], results[False][1].astype(np.float32), "fused vs unfused hidden state",
-                           rel_l2_tol=2e-3)
-    difference = results[True][2][:, :elements].view(np.int8).astype(np.int32) - \
-        results[False][2][:, :elements].view(np.int8).astype(np.int32)
-    assert np.abs(difference).max() <= 1
+        results[mode] = (got_tokens, step.work["x"][0].numpy(np.float16, (batch, config.hidden)),
+                         device_pool.numpy(np.uint8, (capacity, stride)))
+    for mode in ("fused", "projecting"):
+        assert_close_to_oracle(results[mode][1], results["unfused"][1].astype(np.float32), f"{mode} vs unfused hidden state",
+                               rel_l2_tol=2e-3)
+        difference = results[mode][2][:, :elements].view(np.int8).astype(np.int32) - \
+            results["unfused"][2][:, :elements].view(np.int8).astype(np.int32)
+        assert np.abs(difference).max() <= 1
     hidden, logits, _ = decode_chain(config, weights, pool.reshape(-1), slots, offsets, lengths, new_slots, lengths, tokens)
     # three layers of chained kernels that each store half: 2e-3 a layer in relative L2, as the two-layer
     # chains are held to 4e-3, and the largest single difference at 1e-2 x RMS a layer
     want = hidden.astype(np.float64)
     rms_hidden = float(np.sqrt(np.mean(want ** 2)))
-    for fused in (True, False):
-        difference = results[fused][1].astype(np.float64) - want
-        assert np.linalg.norm(difference) <= 6e-3 * np.linalg.norm(want), f"fused={fused}"
-        assert np.abs(difference).max() <= 3e-2 * rms_hidden, f"fused={fused}"
+    for mode in launches:
+        difference = results[mode][1].astype(np.float64) - want
+        assert np.linalg.norm(difference) <= 6e-3 * np.linalg.norm(want), mode
+        assert np.abs(difference).max() <= 3e-2 * rms_hidden, mode
     rms = float(np.sqrt(np.mean(logits.astype(np.float64) ** 2)))
-    for b in range(batch):
-        assert float(logits[b, results[True][0][b]]) >= float(logits[b].max()) - 2e-2 * rms
+    for mode in launches:
+        for b in range(batch):
+            assert float(logits[b, results[mode][0][b]]) >= float(logits[b].max()) - 2e-2 * rms, mode

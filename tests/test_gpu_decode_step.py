@@ -28,11 +28,13 @@ def ragged_lengths(batch, seed):
 
 # Batch 1-2 run the register-activation GEMV, 3-8 the matrix-core GEMV (normalising its rows
 # itself), 9-32 its row-grouped form: batch 8 and 32 are the sizes the decode-step benchmark times.
-@pytest.mark.parametrize("batch,lengths", [(1, [37]), (2, [130, 9]), (3, [64, 5, 300]), (8, ragged_lengths(8, 5)),
+@pytest.mark.parametrize("batch,lengths", [(1, [37]), (1, [77]), (2, [130, 9]), (3, [64, 5, 300]), (8, ragged_lengths(8, 5)),
                                            (32, ragged_lengths(32, 6))])
-@pytest.mark.parametrize("fused", [False, True], ids=["six_launches_a_layer", "four_launches_a_layer"])
-def test_decode_step_matches_oracle_chain(runtime, batch, lengths, fused):
+@pytest.mark.parametrize("launches", [6, 4, 3], ids=["six_launches_a_layer", "four_launches_a_layer", "three_launches_a_layer"])
+def test_decode_step_matches_oracle_chain(runtime, batch, lengths, launches):
     from llmopt_amd.decode_step import DecodeConfig, DecodeStep, random_weights
+    if launches == 3 and max(lengths) < 64:
+        pytest.skip("the projecting attention takes contexts of 64 tokens and more")
     rng = np.random.default_rng(17 + batch)
     config = DecodeConfig(layers=2, vocabulary=1000)
     weights = random_weights(config, rng)
@@ -53,7 +55,8 @@ def test_decode_step_matches_oracle_chain(runtime, batch, lengths, fused):
 
     device_pool = runtime.buffer_of_bytes(pool)
     step = DecodeStep(runtime, config, weights, batch, device_pool, runtime.buffer_of_bytes(slots), offsets,
-                      lengths, new_slots, positions, fused=fused)
+                      lengths, new_slots, positions, fused=launches < 6, projecting=launches == 3)
+    assert len(step.dispatches) == {6: 14, 4: 11, 3: 10}[launches]  # (the last layer of a fused step: five)
     got_tokens = step.run(tokens)
     got_hidden = step.work["x"][0].numpy(np.float16, (batch, config.hidden))
 
@@ -75,9 +78,14 @@ def test_decode_step_matches_oracle_chain(runtime, batch, lengths, fused):
         got_q = got_pool[new_slots[b], :elements].view(np.int8).astype(np.int32)
         want_q = want_pool[new_slots[b], :elements].view(np.int8).astype(np.int32)
         assert np.abs(got_q - want_q).max() <= 1
-        got_s = got_pool[new_slots[b], elements:].view(np.uint16).astype(np.int32)
-        want_s = want_pool[new_slots[b], elements:].view(np.uint16).astype(np.int32)
-        assert np.abs(got_s - want_s).max() <= 2
+        got_s = got_pool[new_slots[b], elements:].copy().view(np.uint16)
+        want_s = want_pool[new_slots[b], elements:].copy().view(np.uint16)
+        first = config.layer_elements // 64  # scale groups of the first layer
+        assert np.abs(got_s[:first].astype(np.int32) - want_s[:first].astype(np.int32)).max() <= 2
+        # a later layer's keys and values carry what the chain before them is allowed: their largest (the scale
+        # is it / 127) within the hidden state's own 4e-3
+        later_got, later_want = got_s[first:].view(np.float16).astype(np.float64), want_s[first:].view(np.float16).astype(np.float64)
+        assert np.all(np.abs(later_got - later_want) <= 4e-3 * later_want)
     untouched = np.setdiff1d(np.arange(capacity), new_slots)
     np.testing.assert_array_equal(got_pool[untouched], want_pool[untouched])
 
