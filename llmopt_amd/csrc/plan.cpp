@@ -37,6 +37,10 @@ struct llmopt_hip_prebaked : llmopt::RefCounted {
   std::vector<bool> is_checkpoint_pack;
   uint32_t *device_checkpoint = nullptr;  // the word behind device_past's, when the plan packs a checkpoint
   uint32_t checkpoint = 0;                // of the step being enqueued
+  // the highest checkpoint slot every checkpoint pack of the plan has room for in its pool (a retained
+  // plan reads the step's slot from device memory, where the launch can only clamp it: the host
+  // refuses a step beyond this before anything is queued)
+  uint32_t checkpoint_limit = 0xffffffffu;
   llmopt_hip_buffer *token_buffer = nullptr;
   llmopt_hip_buffer *output_buffer = nullptr;
   // context length of the step, one word per sequence of the widest attention record
@@ -361,6 +365,12 @@ int llmopt_hip_prebaked_create(llmopt_hip_library *library, const llmopt_hip_dis
     plan->is_paged_attention.push_back(paged);
     plan->is_checkpoint_pack.push_back(strcmp(items[i].name, "llmopt_cache_pack_checkpoint_q8_simd") == 0);
     const DispatchRecord &record = plan->records[i];
+    if (plan->is_checkpoint_pack[i] && record.parameters.size() >= 28 && record.buffers.size() >= 2) {
+      // CheckpointCacheParams: checkpoint_stride at byte 24; buffers: source, pool
+      const uint32_t stride = param_u32(record, 24);
+      const uint64_t slots = stride != 0 ? record.buffers[1].length / stride : 0;
+      plan->checkpoint_limit = (uint32_t)std::min<uint64_t>(plan->checkpoint_limit, slots != 0 ? slots - 1 : 0);
+    }
     if (!paged || record.parameters.size() < 64 || record.buffers.size() < 7) continue;
     plan->past_count = std::max(plan->past_count, param_u32(record, 0));
     if (param_u32(record, 20) != 0 && param_u32(record, 56) != 0) plan->single_submission = false;  // masked
@@ -420,6 +430,9 @@ int llmopt_hip_prebaked_execute(llmopt_hip_prebaked *plan, int64_t token, int64_
   if (plan == nullptr) return fail(LLMOPT_ERR_FAILURE, "HIP prebaked plan has been finalized");
   // the slot llmopt_cache_pack_checkpoint_q8_simd launches of the plan write this step (as the reference:
   // the low 32 bits of the argument; the ring queue has no such argument and keeps the last one)
+  if (plan->checkpoint_limit != 0xffffffffu && (uint32_t)(int32_t)checkpoint > plan->checkpoint_limit)
+    return fail(LLMOPT_ERR_INVALID, "HIP checkpoint pool buffer is too small: the plan's pools hold checkpoints 0..%u, step asks for %u",
+                plan->checkpoint_limit, (uint32_t)(int32_t)checkpoint);
   plan->checkpoint = (uint32_t)(int32_t)checkpoint;
   int32_t next_token = 0;
   const bool nan_check =

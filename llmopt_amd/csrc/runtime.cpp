@@ -109,7 +109,15 @@ void *context_workspace(llmopt_hip_context *context, size_t bytes) {
   context->scratch_touched = true;
   if (bytes <= context->workspace_bytes) return context->workspace;
   if (context->sizing_capture) {
-    // the launch being captured is never run: any non-null address will do
+    // The launch being captured is never run: any non-null address will do.  Only for a launch that
+    // really is being captured: one that would run (another thread using the context while a plan is
+    // being captured, which the interface does not allow) must not get a placeholder for an address.
+    hipStreamCaptureStatus capturing = hipStreamCaptureStatusNone;
+    if (hipStreamIsCapturing(context->stream, &capturing) != hipSuccess || capturing != hipStreamCaptureStatusActive) {
+      (void)hipGetLastError();
+      fail(LLMOPT_ERR_FAILURE, "HIP context is capturing a plan on another thread: a context serves one thread at a time");
+      return nullptr;
+    }
     context->sizing_wanted = std::max(context->sizing_wanted, bytes);
     return context->workspace ? context->workspace : static_cast<void *>(context);
   }

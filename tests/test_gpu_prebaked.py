@@ -264,4 +264,111 @@ def test_plan_writes_the_checkpoint_slot_of_each_step(runtime):
     np.testing.assert_array_equal(written, [False, True, False, True, False])   # layer 0: the slots of the two steps
     np.testing.assert_array_equal(got[3, :layer_elements], got[1, :layer_elements])
     assert got[4, layer_elements:elements].any() and not got[:4, layer_elements:elements].any()  # layer 1: slot 4 only
+    # a slot the pool has no room for: refused on the host, nothing queued (the launch itself, reading
+    # the slot from device memory, could only clamp it)
+    from llmopt_amd.native import LlmoptError
+    with pytest.raises(LlmoptError, match=r"checkpoints 0\.\.4, step asks for 5") as error:
+        plan.execute(0, 0, checkpoint=slots)
+    assert error.value.code == -2
+    np.testing.assert_array_equal(pool.numpy(np.uint8, (slots, stride)), got)
+    del plan
+
+
+def test_plan_is_captured_again_after_the_kernel_workspace_moved(runtime):
+    """A plan's graph holds the address of the context's kernel workspace (the attention launches'
+    partial results).  An eager launch that needs more grows the workspace - the old block is freed -
+    and the next step of the plan must capture its records again: tokens, hidden state and pool equal
+    to eager steps bit for bit, before and after."""
+    import math
+    import struct
+    from llmopt_amd.decode_step import DecodeConfig, random_weights
+    from llmopt_amd.native import Prebaked, Runtime
+    own = Runtime()  # a context of its own: what other tests left in the shared one's workspace is not known
+    try:
+        rng = np.random.default_rng(77)
+        config = DecodeConfig(layers=2, vocabulary=1000)
+        weights = random_weights(config, rng)
+        lengths, room = [120, 70], 6
+        case = make_case(rng, config, lengths, room)
+        eager, eager_pool = build_step(own, config, weights, case, lengths, room)
+        frozen, frozen_pool = build_step(own, config, weights, case, lengths, room)
+        plan = Prebaked(own, frozen.dispatches, frozen.tokens, frozen.token_ids)
+        assert plan.single_submission
+        tokens = rng.integers(0, config.vocabulary, len(lengths))
+
+        def both_step(label):
+            nonlocal tokens
+            want = eager.run(tokens)
+            frozen.tokens.write(np.asarray(tokens, dtype=np.int64))
+            plan.execute(int(tokens[0]), int(frozen.host_lengths[0]))
+            np.testing.assert_array_equal(frozen.token_ids.numpy(np.uint32, (len(lengths),)), want, err_msg=label)
+            np.testing.assert_array_equal(frozen.work["x"][0].numpy(np.uint16), eager.work["x"][0].numpy(np.uint16),
+                                          err_msg=label)
+            np.testing.assert_array_equal(frozen_pool.numpy(np.uint8), eager_pool.numpy(np.uint8), err_msg=label)
+            tokens = want.astype(np.int64)
+            eager.advance()
+            frozen.advance()
+
+        both_step("before the workspace moved")
+        # 64 sequences of 8 KV heads of 128: about 18 MB of partial results, many times what the two
+        # short sequences of the plan asked for
+        batch, q_heads, kv_heads, dim, context = 64, 32, 8, 128, 80
+        elements = 2 * kv_heads * dim
+        stride = elements + 2 * (elements // 64)
+        big_pool = own.buffer_of_bytes(rng.integers(0, 256, size=context * stride, dtype=np.uint8))
+        big_slots = own.buffer_of_bytes(np.tile(np.arange(context, dtype=np.uint32), batch))
+        rows = lambda heads: own.buffer_of_bytes(rng.standard_normal(batch * heads * dim).astype(np.float16))
+        out = own.create_buffer(batch * q_heads * dim * 2)
+        own.dispatch("llmopt_attention_q8_paged_batched",
+                     [rows(q_heads), rows(kv_heads), rows(kv_heads), big_pool, big_slots, big_slots, out,
+                      own.buffer_of_bytes(np.full(batch, context, dtype=np.uint32)),
+                      own.buffer_of_bytes(np.arange(batch, dtype=np.uint32) * context)],
+                     struct.pack("<12IfIII", batch, q_heads, kv_heads, 0, dim, 0, 0, elements, 0, kv_heads * dim, 64, stride,
+                                 1.0 / math.sqrt(dim), 1, 0, 0) + struct.pack("<I", context),
+                     grid=(256, 1, 1), group=(256, 1, 1))
+        own.synchronize()
+        for index in range(2):
+            both_step(f"step {index} after the workspace moved")
+        del plan
+    finally:
+        own.close()
+
+
+def test_plan_with_a_masked_attention_is_launched_from_the_host(runtime):
+    """A masked paged attention cannot read its context length from device memory (the mask's row
+    length follows it): such a plan is not one graph but the records launched one by one, the length
+    patched into parameter byte 12 on the host - as the reference does for every plan.  Two steps at
+    different context lengths against the oracle."""
+    import math
+    import oracle
+    from oracle import PagedParams
+    from llmopt_amd.native import Prebaked
+    from tests.test_gpu_q8 import build_pool, paged_params_bytes
+    rng = np.random.default_rng(5)
+    b, h, kvh, dim, capacity = 1, 4, 2, 64, 90
+    pool, slots, _, te, stride, ko, vo = build_pool(rng, kvh, dim, [capacity])
+    query = rng.standard_normal((b, h, 1, dim)).astype(np.float16)
+    ck = rng.standard_normal((b, kvh, 1, dim)).astype(np.float16)
+    cv = rng.standard_normal((b, kvh, 1, dim)).astype(np.float16)
+    params = lambda past: PagedParams(batches=b, query_heads=h, kv_heads=kvh, past_length=past, head_dim=dim,
+                                      mask_batches=1, mask_heads=1, token_elements=te, key_offset=ko, value_offset=vo,
+                                      group_size=64, token_stride=stride, scale=1.0 / math.sqrt(dim), query_length=1,
+                                      mask_dtype=1, window=0)
+    mask_buffer = runtime.create_buffer(capacity + 1)
+    out = runtime.buffer_of_bytes(np.full((b, 1, h, dim), np.nan, dtype=np.float16))
+    slot_buffer = runtime.buffer_of_bytes(slots)
+    token = runtime.buffer_of_bytes(np.zeros(1, dtype=np.int64))
+    output = runtime.buffer_of_bytes(np.zeros(1, dtype=np.int32))
+    plan = Prebaked(runtime, [("llmopt_attention_q8_paged_simd_generic",
+                               [runtime.buffer_of_bytes(query), runtime.buffer_of_bytes(ck), runtime.buffer_of_bytes(cv),
+                                runtime.buffer_of_bytes(pool), slot_buffer, mask_buffer, out],
+                               paged_params_bytes(params(0)), (256, 1, 1), (256, 1, 1))], token, output)
+    assert not plan.single_submission
+    for past in (70, 33):
+        mask = (rng.random((1, 1, 1, past + 1)) > 0.3).astype(np.uint8)
+        mask[..., past] = 1
+        mask_buffer.write(np.concatenate([mask.reshape(-1), np.zeros(capacity - past, dtype=np.uint8)]))
+        plan.execute(0, past)
+        expected = oracle.paged_attention_q8(query, ck, cv, pool, slots[:past], mask, params(past))
+        assert_close_to_oracle(out.numpy(np.float16, (b, 1, h, dim)), expected, f"masked plan at {past} tokens")
     del plan
