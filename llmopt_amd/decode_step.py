@@ -31,10 +31,12 @@ from .native import Buffer, Runtime
 
 # Above this many sequences the fused launches (one or two sequences per workgroup, every workgroup
 # reading and decoding its weights again) cost more than the launches they save: measured at 2048
-# tokens of context, ms per step fused / not: batch 1 0.794 / 0.794, 2 0.852 / 0.977, 8 0.923 / 1.048,
-# 16 1.132 / 1.169, 24 1.372 / 1.302, 32 1.418 / 1.346, 64 2.08 / 1.93.
-FUSED_MAX_BATCH = 16
-# The attention launch multiplies its heads into the output projection where it can (three launches a layer).
+# tokens of context, ms per step as three launches a layer / as six: batch 1 0.742 / 0.794, 2 0.785 / 0.977,
+# 8 0.856 / 1.048, 12 1.011 / 1.072, 16 1.050 / 1.136, 20 1.161 / 1.260, 24 1.292 / 1.279, 28 1.313 / 1.299,
+# 32 1.361 / 1.321.
+FUSED_MAX_BATCH = 20
+# The attention launch multiplies its heads into the output projection where it can (three launches a
+# layer instead of four: batch 1 0.742 against 0.771 ms, 8 0.856 / 0.907, 16 1.052 / 1.096, 32 1.364 / 1.379).
 PROJECTING_ATTENTION = True
 
 
