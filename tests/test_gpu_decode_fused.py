@@ -18,6 +18,27 @@ pytestmark = pytest.mark.gpu
 GROUP = (256, 1, 1)
 
 
+def drawn_cases():
+    """Seeded random shapes for the fused entries, beside the hand-picked ones: rows, widths, head counts and
+    pending sums anywhere the entries accept them."""
+    rng = np.random.default_rng(20240607)
+    qkv, ffn, summing, projecting = [], [], [], []
+    for _ in range(10):
+        kv = int(rng.integers(1, 5))
+        qkv.append((int(rng.integers(1, 41)), 64 * int(rng.integers(1, 33)), (kv * int(rng.integers(1, 5)), kv, kv),
+                    int(rng.integers(0, 33))))
+        ffn.append((int(rng.integers(1, 41)), 64 * int(rng.integers(1, 33)), 64 * int(rng.integers(1, 24))))
+        summing.append((int(rng.integers(1, 41)), 64 * int(rng.integers(1, 33)), 64 * int(rng.integers(1, 22)),
+                        int(rng.integers(0, 33))))
+        kv = int(rng.integers(1, 5))
+        projecting.append((int(rng.integers(1, 41)), kv * int(rng.integers(1, 7)), kv, 64 * int(rng.integers(1, 17)),
+                           int(rng.integers(64, 700))))
+    return qkv, ffn, summing, projecting
+
+
+DRAWN_QKV, DRAWN_FFN, DRAWN_SUMMING, DRAWN_PROJECTING = drawn_cases()
+
+
 @pytest.fixture(scope="module")
 def runtime():
     from llmopt_amd.native import Runtime
@@ -45,7 +66,8 @@ def pending_stream(rng, m, k, partial_count):
 
 @pytest.mark.parametrize("m,k,heads,partial_count", [(1, 576, (9, 3, 3), 0), (1, 576, (9, 3, 3), 24), (3, 576, (9, 3, 3), 24),
                                                      (8, 576, (9, 3, 3), 24), (5, 1024, (4, 2, 2), 7), (2, 2048, (2, 1, 1), 32),
-                                                     (40, 576, (9, 3, 3), 24), (37, 1536, (3, 1, 1), 3), (2, 64, (1, 1, 1), 1)])
+                                                     (40, 576, (9, 3, 3), 24), (37, 1536, (3, 1, 1), 3), (2, 64, (1, 1, 1), 1)]
+                         + DRAWN_QKV)
 def test_fused_qkv_rotary_pack_against_separate_launches_and_oracle(runtime, m, k, heads, partial_count):
     rng = np.random.default_rng(1000 * m + k + partial_count)
     q_heads, k_heads, v_heads = heads
@@ -146,7 +168,7 @@ def test_fused_qkv_rotary_pack_against_separate_launches_and_oracle(runtime, m, 
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 1536, 576), (2, 1536, 576), (8, 1536, 576), (33, 1536, 576), (3, 2048, 1024),
-                                   (5, 128, 1408), (2, 64, 64), (4, 1024, 704)])
+                                   (5, 128, 1408), (2, 64, 64), (4, 1024, 704)] + DRAWN_FFN)
 def test_fused_ffn_partial_sums_against_separate_launches_and_oracle(runtime, m, n, k):
     rng = np.random.default_rng(7 * m + n + k)
     x = rng.standard_normal((m, k)).astype(np.float16)
@@ -190,7 +212,7 @@ def test_fused_ffn_partial_sums_against_separate_launches_and_oracle(runtime, m,
 
 
 @pytest.mark.parametrize("m,n,k,pending", [(1, 1536, 576, 9), (2, 1536, 576, 9), (8, 1536, 576, 9), (5, 128, 1024, 32),
-                                           (3, 256, 704, 1), (16, 1536, 576, 9), (4, 64, 576, 0)])
+                                           (3, 256, 704, 1), (16, 1536, 576, 9), (4, 64, 576, 0)] + DRAWN_SUMMING)
 def test_summing_ffn_forms_the_stream_and_leaves_the_partial_sums_of_the_plain_entry(runtime, m, n, k, pending):
     rng = np.random.default_rng(11 * m + n + k + pending)
     x, pending_sums, stream = pending_stream(rng, m, k, pending)
@@ -236,7 +258,7 @@ def paged_case(rng, batch, q_heads, kv_heads, lengths):
 @pytest.mark.parametrize("batch,q_heads,kv_heads,hidden,longest", [(1, 9, 3, 576, 2048), (1, 9, 3, 576, 64), (2, 9, 3, 576, 300),
                                                                    (8, 9, 3, 576, 2048), (5, 8, 2, 1024, 700),
                                                                    (16, 9, 3, 576, 500), (3, 4, 4, 64, 150),
-                                                                   (33, 2, 1, 704, 260)])
+                                                                   (33, 2, 1, 704, 260)] + DRAWN_PROJECTING)
 def test_projecting_attention_leaves_each_heads_share_of_the_output_projection(runtime, batch, q_heads, kv_heads, hidden,
                                                                                longest):
     rng = np.random.default_rng(batch * 1000 + hidden + longest)
