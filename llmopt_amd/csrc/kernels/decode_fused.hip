@@ -328,44 +328,53 @@ __global__ __launch_bounds__(kThreads) void fused_qkv_kernel(FusedQkvArgs a) {
 }
 
 // PER: pending partial sums a thread adds to the stream on the way in (0: none), as in fused_qkv_kernel.
-template <int M, int PER>
+// SLICE: columns of the intermediate a workgroup owns, 64 or 32.  Half the columns are half the bytes a CU has
+// to pull in before it can start (a CU fills its LDS at about 80 bytes a nanosecond: the 55 KB of a 64-wide
+// slice at hidden 576 were not all requested until 1.1 us into the kernel) and half the arithmetic on its four
+// SIMDs, for twice the partial sums the next reader adds.
+template <int M, int PER, int SLICE>
 __global__ __launch_bounds__(kThreads) void fused_ffn_kernel(FusedFfnArgs a) {
+  static_assert(SLICE == 32 || SLICE == 64, "whole 16-byte pieces of a down-projection row");
+  constexpr int kPieces = SLICE / 32;  // 16-byte pieces of a down-projection row inside the slice
   extern __shared__ __attribute__((aligned(16))) uint8_t fused_lds[];
   __shared__ float square_lds[M][kWaves];
-  __shared__ __attribute__((aligned(16))) uint16_t product_lds[M][kHead];
+  __shared__ __attribute__((aligned(16))) uint16_t product_lds[M][SLICE];
   Carve carve = {fused_lds};
-  const uint32_t row_bytes = a.k >> 1, scale_bytes = kHead * (a.k >> 6) * 2;
-  uint8_t *gate_lds = carve.take(kHead * row_bytes);
-  uint8_t *up_lds = carve.take(kHead * row_bytes);
+  const uint32_t row_bytes = a.k >> 1, scale_bytes = SLICE * (a.k >> 6) * 2;
+  uint8_t *gate_lds = carve.take(SLICE * row_bytes);
+  uint8_t *up_lds = carve.take(SLICE * row_bytes);
   uint16_t *gate_scales_lds = reinterpret_cast<uint16_t *>(carve.take(scale_bytes));
   uint16_t *up_scales_lds = reinterpret_cast<uint16_t *>(carve.take(scale_bytes));
-  uint8_t *down_lds = carve.take(a.k * 32);  // 32 bytes a row: the slice's 64 columns
+  uint8_t *down_lds = carve.take(a.k * (SLICE / 2));  // SLICE / 2 bytes a row: the slice's columns
   uint16_t *down_scales_lds = reinterpret_cast<uint16_t *>(carve.take(a.k * 2));
   uint16_t *x_lds = reinterpret_cast<uint16_t *>(carve.take(M * a.k * 2));
   f4_t *group_lds = reinterpret_cast<f4_t *>(carve.take(PER > 0 ? kThreads * 16 : 0));
   const uint32_t lane = threadIdx.x & 63;
   const uint32_t wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const uint32_t row0 = blockIdx.y * M;
-  const uint32_t slice = blockIdx.x;  // intermediate columns [64 slice, 64 slice + 64)
+  const uint32_t slice = blockIdx.x;  // intermediate columns [SLICE slice, SLICE slice + SLICE)
 
   FUSED_STAMP(0);
-  const uint8_t *gate_weights = a.gate.weight + (size_t)slice * kHead * row_bytes;
-  const uint8_t *up_weights = a.up.weight + (size_t)slice * kHead * row_bytes;
-  const uint8_t *gate_scales = reinterpret_cast<const uint8_t *>(a.gate.scale + (size_t)slice * kHead * (a.k >> 6));
-  const uint8_t *up_scales = reinterpret_cast<const uint8_t *>(a.up.scale + (size_t)slice * kHead * (a.k >> 6));
-  copy_to_lds(gate_lds, kHead * row_bytes, [&](uint32_t piece) { return gate_weights + (size_t)piece * 16; });
-  copy_to_lds(up_lds, kHead * row_bytes, [&](uint32_t piece) { return up_weights + (size_t)piece * 16; });
+  const uint8_t *gate_weights = a.gate.weight + (size_t)slice * SLICE * row_bytes;
+  const uint8_t *up_weights = a.up.weight + (size_t)slice * SLICE * row_bytes;
+  const uint8_t *gate_scales = reinterpret_cast<const uint8_t *>(a.gate.scale + (size_t)slice * SLICE * (a.k >> 6));
+  const uint8_t *up_scales = reinterpret_cast<const uint8_t *>(a.up.scale + (size_t)slice * SLICE * (a.k >> 6));
+  copy_to_lds(gate_lds, SLICE * row_bytes, [&](uint32_t piece) { return gate_weights + (size_t)piece * 16; });
+  copy_to_lds(up_lds, SLICE * row_bytes, [&](uint32_t piece) { return up_weights + (size_t)piece * 16; });
   copy_to_lds(reinterpret_cast<uint8_t *>(gate_scales_lds), scale_bytes, [&](uint32_t piece) { return gate_scales + (size_t)piece * 16; });
   copy_to_lds(reinterpret_cast<uint8_t *>(up_scales_lds), scale_bytes, [&](uint32_t piece) { return up_scales + (size_t)piece * 16; });
-  // down: row r of the slice is 32 bytes, pieces 2 r and 2 r + 1
-  const uint8_t *down_weights = a.down.weight + (size_t)slice * 32;
-  copy_to_lds(down_lds, a.k * 32, [&](uint32_t piece) { return down_weights + (size_t)(piece >> 1) * (a.n >> 1) + (piece & 1) * 16; });
+  // down: row r of the slice is SLICE / 2 bytes, kPieces pieces
+  const uint8_t *down_weights = a.down.weight + (size_t)slice * (SLICE / 2);
+  copy_to_lds(down_lds, a.k * (SLICE / 2), [&](uint32_t piece) {
+    return down_weights + (size_t)(piece / kPieces) * (a.n >> 1) + (piece % kPieces) * 16;
+  });
   // (the scales of the slice's down rows pass registers: two bytes a row, 2 n / 64 bytes apart)
   constexpr int kScalePasses = (int)kFusedMaxWidth / kThreads;
   uint16_t down_scales[kScalePasses];
+  const uint32_t down_group = (slice * SLICE) >> 6;  // the scale group of the down rows the slice lies in
 #pragma unroll
   for (int pass = 0; pass < kScalePasses; ++pass)
-    down_scales[pass] = a.down.scale[(size_t)min(threadIdx.x + pass * kThreads, a.k - 1) * (a.n >> 6) + slice];
+    down_scales[pass] = a.down.scale[(size_t)min(threadIdx.x + pass * kThreads, a.k - 1) * (a.n >> 6) + down_group];
   stage_normalised_rows<M, PER>(a.in, a.norm, a.m, a.k, row0, blockIdx.x == 0 && a.in.x_out != nullptr, x_lds, group_lds,
                                 square_lds);
 #pragma unroll
@@ -379,13 +388,13 @@ __global__ __launch_bounds__(kThreads) void fused_ffn_kernel(FusedFfnArgs a) {
     hold_rows<M>(held, x_lds, a.k, lanes.piece, lanes.present);
     FUSED_STAMP(4);
 #pragma unroll 1
-    for (uint32_t row = wave * lanes.rows_per_step; row < (uint32_t)kHead; row += kWaves * lanes.rows_per_step) {
+    for (uint32_t row = wave * lanes.rows_per_step; row < (uint32_t)SLICE; row += kWaves * lanes.rows_per_step) {
       float gate[M], up[M];
       rows_dot<M>(lanes, held, gate_lds + row * row_bytes, gate_scales_lds + row * (a.k >> 6), gate);
       rows_dot<M>(lanes, held, up_lds + row * row_bytes, up_scales_lds + row * (a.k >> 6), up);
 #pragma unroll
       for (int m = 0; m < M; ++m)
-        if (lane < lanes.rows_per_step && row + lane < (uint32_t)kHead)
+        if (lane < lanes.rows_per_step && row + lane < (uint32_t)SLICE)
           product_lds[m][row + lane] = float_to_half_bits(gate[m] / (1.0f + __expf(-gate[m])) * up[m]);
     }
     FUSED_STAMP(5);
@@ -393,20 +402,21 @@ __global__ __launch_bounds__(kThreads) void fused_ffn_kernel(FusedFfnArgs a) {
   __syncthreads();
   FUSED_STAMP(6);
 
-  // lane pair p owns output row p (+ kThreads / 2 per pass): each lane 32 of the slice's 64 columns
-  const uint32_t half_select = threadIdx.x & 1;
+  // kPieces neighbouring lanes own an output row (+ kThreads / kPieces per pass): each lane 32 of the slice's columns
+  const uint32_t piece_select = threadIdx.x % kPieces;
   Held<M> held;
-  hold_rows<M>(held, &product_lds[0][0], kHead, half_select, true);
+  hold_rows<M>(held, &product_lds[0][0], SLICE, piece_select, true);
 #pragma unroll 1
-  for (uint32_t column = threadIdx.x >> 1; column < a.k; column += kThreads / 2) {
-    const u32x4_t weights = *reinterpret_cast<const u32x4_t *>(down_lds + column * 32 + half_select * 16);
+  for (uint32_t column = threadIdx.x / kPieces; column < a.k; column += kThreads / kPieces) {
+    const u32x4_t weights = *reinterpret_cast<const u32x4_t *>(down_lds + column * (SLICE / 2) + piece_select * 16);
     float share[M];
     piece_dot<M>(weights, half_bits_to_float(down_scales_lds[column]), held, share);
 #pragma unroll
     for (int m = 0; m < M; ++m) {
-      const float total = share[m] + __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(
-                                         0, __builtin_bit_cast(int, share[m]), 0xB1, 0xF, 0xF, false));
-      if (half_select == 0 && row0 + m < a.m) a.partials[((size_t)slice * a.m + row0 + m) * a.k + column] = total;
+      float total = share[m];
+      if constexpr (kPieces == 2)
+        total += __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, share[m]), 0xB1, 0xF, 0xF, false));
+      if (piece_select == 0 && row0 + m < a.m) a.partials[((size_t)slice * a.m + row0 + m) * a.k + column] = total;
     }
   }
   FUSED_STAMP(8);
@@ -415,13 +425,13 @@ __global__ __launch_bounds__(kThreads) void fused_ffn_kernel(FusedFfnArgs a) {
 bool aligned16(const void *pointer) { return (reinterpret_cast<uintptr_t>(pointer) & 15) == 0; }
 
 constexpr size_t kLdsBudget = 150 * 1024;
-size_t ffn_lds_bytes(uint32_t rows, uint32_t k, bool partials);
+size_t ffn_lds_bytes(uint32_t rows, uint32_t k, bool partials, uint32_t slice = 64);
 
 // Sequences per workgroup: one, until the launch has more workgroups than the device holds at once
 // (two share a workgroup's decoded weights; their rows must fit one pass of the staging).
-uint32_t rows_per_workgroup(uint32_t m, uint32_t k, uint32_t column_blocks) {
+uint32_t rows_per_workgroup(uint32_t m, uint32_t k, uint32_t column_blocks, uint32_t slice = 64) {
   return (uint64_t)m * column_blocks > 2ull * (uint32_t)device_compute_units() && 2 * (k >> 2) <= (uint32_t)kThreads &&
-                 ffn_lds_bytes(2, k, true) <= kLdsBudget
+                 ffn_lds_bytes(2, k, true, slice) <= kLdsBudget
              ? 2
              : 1;
 }
@@ -432,8 +442,8 @@ size_t qkv_lds_bytes(uint32_t rows, uint32_t k, bool partials) {
   return padded(kHead * (k >> 1)) + padded(kHead * (k >> 6) * 2) + padded(rows * k * 2) + (partials ? kThreads * 16 : 0);
 }
 
-size_t ffn_lds_bytes(uint32_t rows, uint32_t k, bool partials) {
-  return 2 * padded(kHead * (k >> 1)) + 2 * padded(kHead * (k >> 6) * 2) + padded(k * 32) + padded(k * 2) +
+size_t ffn_lds_bytes(uint32_t rows, uint32_t k, bool partials, uint32_t slice) {
+  return 2 * padded(slice * (k >> 1)) + 2 * padded(slice * (k >> 6) * 2) + padded(k * (slice / 2)) + padded(k * 2) +
          padded(rows * k * 2) + (partials ? kThreads * 16 : 0);
 }
 
@@ -465,24 +475,25 @@ hipError_t launch_qkv_rows(const FusedQkvArgs &a, dim3 grid, hipStream_t stream)
   return launch_qkv_instance<M, 32>(a, grid, lds, stream);
 }
 
-template <int M, int PER>
+template <int M, int PER, int SLICE>
 hipError_t launch_ffn_instance(const FusedFfnArgs &a, dim3 grid, size_t lds, hipStream_t stream) {
   static bool configured[kMaxDevices] = {};
   if (lds > 64 * 1024)
-    if (hipError_t status = allow_dynamic_lds(reinterpret_cast<const void *>(fused_ffn_kernel<M, PER>), 158 * 1024, configured))
+    if (hipError_t status =
+            allow_dynamic_lds(reinterpret_cast<const void *>(fused_ffn_kernel<M, PER, SLICE>), 158 * 1024, configured))
       return status;
-  hipLaunchKernelGGL((fused_ffn_kernel<M, PER>), grid, dim3(kThreads), lds, stream, a);
+  hipLaunchKernelGGL((fused_ffn_kernel<M, PER, SLICE>), grid, dim3(kThreads), lds, stream, a);
   return hipGetLastError();
 }
 
-template <int M>
+template <int M, int SLICE>
 hipError_t launch_ffn_rows(const FusedFfnArgs &a, dim3 grid, hipStream_t stream) {
   const uint32_t per = partials_per_thread(M, a.k, a.in.partial_count);
-  const size_t lds = ffn_lds_bytes(M, a.k, per != 0);
-  if (per == 0) return launch_ffn_instance<M, 0>(a, grid, lds, stream);
-  if (per <= 8) return launch_ffn_instance<M, 8>(a, grid, lds, stream);
-  if (per <= 16) return launch_ffn_instance<M, 16>(a, grid, lds, stream);
-  return launch_ffn_instance<M, 32>(a, grid, lds, stream);
+  const size_t lds = ffn_lds_bytes(M, a.k, per != 0, SLICE);
+  if (per == 0) return launch_ffn_instance<M, 0, SLICE>(a, grid, lds, stream);
+  if (per <= 8) return launch_ffn_instance<M, 8, SLICE>(a, grid, lds, stream);
+  if (per <= 16) return launch_ffn_instance<M, 16, SLICE>(a, grid, lds, stream);
+  return launch_ffn_instance<M, 32, SLICE>(a, grid, lds, stream);
 }
 
 }  // namespace
@@ -492,6 +503,7 @@ bool fused_qkv_ok(const FusedQkvArgs &a) {
   for (int i = 0; i < 3; ++i)
     if (a.n[i] == 0 || a.n[i] % kHead != 0 || !aligned16(a.w[i].weight) || !aligned16(a.w[i].scale)) return false;
   if (a.in.partial_count > kFusedMaxPartials) return false;
+  if (partials_per_thread(1, a.k, a.in.partial_count) > 32) return false;
   if (a.in.partial_count != 0 && (a.in.partials == nullptr || !aligned16(a.in.partials))) return false;
   if (a.token_stride % 2 != 0 || a.token_elements % 2 != 0) return false;
   return aligned16(a.in.x) && aligned16(a.norm.weight) && (a.in.x_out == nullptr || aligned16(a.in.x_out));
@@ -500,28 +512,31 @@ bool fused_qkv_ok(const FusedQkvArgs &a) {
 hipError_t launch_fused_qkv(const FusedQkvArgs &a, hipStream_t stream) {
   if (!fused_qkv_ok(a)) return hipErrorInvalidValue;
   const uint32_t heads = (a.n[0] + a.n[1] + a.n[2]) / kHead;
-  const uint32_t per = rows_per_workgroup(a.m, a.k, heads);
+  uint32_t per = rows_per_workgroup(a.m, a.k, heads);
+  if (per == 2 && partials_per_thread(2, a.k, a.in.partial_count) > 32) per = 1;
   const dim3 grid(heads, (a.m + per - 1) / per);
   return per == 1 ? launch_qkv_rows<1>(a, grid, stream) : launch_qkv_rows<2>(a, grid, stream);
 }
 
-bool fused_ffn_ok(uint32_t m, uint32_t n, uint32_t k, bool pending) {
-  return m != 0 && k != 0 && k % 64 == 0 && k <= kFusedMaxWidth && ffn_lds_bytes(1, k, pending) <= kLdsBudget && n != 0 &&
-         n % kHead == 0 && n / kHead <= kFusedMaxPartials;
+bool fused_ffn_ok(uint32_t m, uint32_t n, uint32_t k, bool pending, uint32_t slice) {
+  return (slice == 32 || slice == 64) && m != 0 && k != 0 && k % 64 == 0 && k <= kFusedMaxWidth &&
+         ffn_lds_bytes(1, k, pending, slice) <= kLdsBudget && n != 0 && n % slice == 0 && n / slice <= kFusedMaxPartials;
 }
 
 hipError_t launch_fused_ffn(const FusedFfnArgs &a, hipStream_t stream) {
-  if (a.in.partial_count > kFusedMaxPartials) return hipErrorInvalidValue;
+  if (a.in.partial_count > kFusedMaxPartials || partials_per_thread(1, a.k, a.in.partial_count) > 32) return hipErrorInvalidValue;
   if (a.in.partial_count != 0 && (a.in.partials == nullptr || !aligned16(a.in.partials))) return hipErrorInvalidValue;
   if (a.in.x_out != nullptr && (!aligned16(a.in.x_out) || a.in.x_out == a.in.x)) return hipErrorInvalidValue;
-  if (!fused_ffn_ok(a.m, a.n, a.k, a.in.partial_count != 0) || !aligned16(a.in.x) || !aligned16(a.norm.weight) || !aligned16(a.gate.weight) ||
+  if (!fused_ffn_ok(a.m, a.n, a.k, a.in.partial_count != 0, a.slice) || !aligned16(a.in.x) || !aligned16(a.norm.weight) || !aligned16(a.gate.weight) ||
       !aligned16(a.up.weight) || !aligned16(a.down.weight) || !aligned16(a.partials) || !aligned16(a.gate.scale) ||
       !aligned16(a.up.scale))
     return hipErrorInvalidValue;
-  const uint32_t slices = a.n / kHead;
-  const uint32_t per = rows_per_workgroup(a.m, a.k, slices);
+  const uint32_t slices = a.n / a.slice;
+  uint32_t per = rows_per_workgroup(a.m, a.k, slices, a.slice);
+  if (per == 2 && partials_per_thread(2, a.k, a.in.partial_count) > 32) per = 1;
   const dim3 grid(slices, (a.m + per - 1) / per);
-  return per == 1 ? launch_ffn_rows<1>(a, grid, stream) : launch_ffn_rows<2>(a, grid, stream);
+  if (a.slice == 32) return per == 1 ? launch_ffn_rows<1, 32>(a, grid, stream) : launch_ffn_rows<2, 32>(a, grid, stream);
+  return per == 1 ? launch_ffn_rows<1, 64>(a, grid, stream) : launch_ffn_rows<2, 64>(a, grid, stream);
 }
 
 }  // namespace llmopt

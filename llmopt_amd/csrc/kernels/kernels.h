@@ -100,7 +100,8 @@ struct FusedResidual {
   uint32_t partial_count;
   uint16_t *x_out;        // f16 [m, k]
 };
-constexpr uint32_t kFusedMaxPartials = 32;
+// (and at most 32 per thread of the reader: a reader whose rows leave it one group of threads takes 32)
+constexpr uint32_t kFusedMaxPartials = 48;
 constexpr uint32_t kFusedMaxWidth = 2048;
 
 // llmopt_rms_norm_f16_simd + llmopt_w4a16_qkv_linear_f16_g64 + llmopt_rotary_qk_f16_simd_h64 +
@@ -133,11 +134,12 @@ struct FusedFfnArgs {
   W4Norm norm;         // weight_first = 1
   W4Matrix gate, up;   // [n, k/2]
   W4Matrix down;       // [k, n/2]
-  float *partials;     // f32 [n / 64, m, k]
+  float *partials;     // f32 [n / slice, m, k]
   uint32_t m, n, k;
+  uint32_t slice = 64;  // columns of the intermediate per workgroup and partial sum: 64 or 32
 };
 // pending: the input arrives with partial sums to add (their staging takes 8 KiB of the workgroup's memory)
-bool fused_ffn_ok(uint32_t m, uint32_t n, uint32_t k, bool pending = false);
+bool fused_ffn_ok(uint32_t m, uint32_t n, uint32_t k, bool pending = false, uint32_t slice = 64);
 hipError_t launch_fused_ffn(const FusedFfnArgs &args, hipStream_t stream);
 
 // The product kernels' own nibble decoders run over a whole matrix, as float32 [n, k]:

@@ -283,37 +283,42 @@ int rms_w4a16_qkv_rotary_pack(llmopt_hip_context *context, const DispatchRecord 
   args.pool = record.buffers[15].device;
   if (args.in.x == args.in.x_out)
     return fail(LLMOPT_ERR_INVALID, "%s writes the stream while other workgroups still read the input: two buffers", name);
-  if (!fused_qkv_ok(args)) return fail(LLMOPT_ERR_INVALID, "%s requires 16-byte aligned buffers", name);
+  if (!fused_qkv_ok(args))
+    return fail(LLMOPT_ERR_INVALID, "%s requires 16-byte aligned buffers, and rows of more than 1024 values take at most 32 "
+                "partial sums", name);
   return launched(launch_fused_qkv(args, context->stream), name);
 }
 
 // Extension (no reference kernel): llmopt_w4a16_swiglu_rms_f16_g64, llmopt_w4a16_dual_swiglu_f16_g64 and
-// the contraction of llmopt_w4a16_down_add_f16_g64 as ONE launch that leaves, per 64 columns of the
+// the contraction of llmopt_w4a16_down_add_f16_g64 as ONE launch that leaves, per `slice` columns of the
 // intermediate, a float32 partial sum of every output; the launch that reads the stream next adds them
-// and the residual (llmopt_rms_w4a16_qkv_rotary_pack_q8_f16_g64).  W4A16SwiGLUFFNParams {u32 m, n, k; f32 eps}.
-// buffers: input f16 [m,k], norm weight, gateW, gateS, upW, upS, downW, downS, partials f32 [n/64,m,k].
+// and the residual (llmopt_rms_w4a16_qkv_rotary_pack_q8_f16_g64).  W4A16SwiGLUFFNParams {u32 m, n, k; f32 eps},
+// then u32 slice: 64 or 32 (32: twice the workgroups with half the weights each, and twice the partial sums).
+// buffers: input f16 [m,k], norm weight, gateW, gateS, upW, upS, downW, downS, partials f32 [n/slice,m,k].
 // `summing` (llmopt_sum_rms_w4a16_swiglu_down_partial_f16_g64): the input itself arrives as rows plus
 // pending partial sums (of the projecting attention entry) and is written out whole: buffers input,
-// pending f32 [pending_count,m,k], stream f16 [m,k], then as above; u32 pending_count follows epsilon.
+// pending f32 [pending_count,m,k], stream f16 [m,k], then as above; u32 pending_count follows epsilon, slice follows it.
 int swiglu_down_partial(llmopt_hip_context *context, const DispatchRecord &record, bool summing) {
   const size_t b = summing ? 2 : 0;
   if (int status = require_buffer_count(record, 9 + b)) return status;
-  if (int status = require_parameter_bytes(record, summing ? 20 : 16)) return status;
+  if (int status = require_parameter_bytes(record, summing ? 24 : 20)) return status;
   const char *name = record.name.c_str();
   const uint32_t m = param_u32(record, 0), n = param_u32(record, 4), k = param_u32(record, 8);
   const float epsilon = param_f32(record, 12);
   if (int status = check_w4_shape(name, m, n, k)) return status;
-  if (!fused_ffn_ok(m, n, k, summing && param_u32(record, 16) != 0))
+  const uint32_t slice = param_u32(record, summing ? 20 : 16);
+  if (slice != 32 && slice != 64) return fail(LLMOPT_ERR_INVALID, "%s takes slices of 32 or 64 columns, got %u", name, slice);
+  if (!fused_ffn_ok(m, n, k, summing && param_u32(record, 16) != 0, slice))
     return fail(LLMOPT_ERR_INVALID, "%s takes a hidden width k whose slice of the three matrices fits a workgroup's "
-                "memory (k <= 1472, with pending sums k <= 1344) and n a multiple of 64 up to %u, got k = %u, n = %u", name,
-                64 * kFusedMaxPartials, k, n);
+                "memory (slices of 64: k <= 1472, with pending sums k <= 1344) and n a multiple of the slice up to %u "
+                "slices, got k = %u, n = %u, slice = %u", name, kFusedMaxPartials, k, n, slice);
   if (!std::isfinite(epsilon) || epsilon <= 0.0f) return fail(LLMOPT_ERR_INVALID, "%s requires a positive finite epsilon", name);
   if (int status = require_buffer_size(record.buffers[0], (uint64_t)m * k * 2, "input")) return status;
   if (int status = require_buffer_size(record.buffers[b + 1], (uint64_t)k * 2, "norm weight")) return status;
   if (int status = check_w4_matrix(record.buffers[b + 2], record.buffers[b + 3], n, k, "gate")) return status;
   if (int status = check_w4_matrix(record.buffers[b + 4], record.buffers[b + 5], n, k, "up")) return status;
   if (int status = check_w4_matrix(record.buffers[b + 6], record.buffers[b + 7], k, n, "down")) return status;
-  if (int status = require_buffer_size(record.buffers[b + 8], (uint64_t)(n / 64) * m * k * 4, "partial sums")) return status;
+  if (int status = require_buffer_size(record.buffers[b + 8], (uint64_t)(n / slice) * m * k * 4, "partial sums")) return status;
   FusedFfnArgs args = {};
   args.in.x = as_f16(record.buffers[0]);
   if (summing) {
@@ -337,6 +342,7 @@ int swiglu_down_partial(llmopt_hip_context *context, const DispatchRecord &recor
   args.m = m;
   args.n = n;
   args.k = k;
+  args.slice = slice;
   return launched(launch_fused_ffn(args, context->stream), name);
 }
 

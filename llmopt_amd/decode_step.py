@@ -38,6 +38,9 @@ FUSED_MAX_BATCH = 20
 # The attention launch multiplies its heads into the output projection where it can (three launches a
 # layer instead of four: batch 1 0.742 against 0.771 ms, 8 0.856 / 0.907, 16 1.052 / 1.096, 32 1.364 / 1.379).
 PROJECTING_ATTENTION = True
+# Columns of the intermediate per workgroup of the fused FFN launch (and per partial sum it leaves): 32 where that
+# stays within the 48 partial sums a reader takes, else 64.
+FFN_SLICE = 32
 
 
 def u32s(*values) -> bytes:
@@ -155,6 +158,10 @@ class DecodeStep:
         self.reference_entries = reference_entries
         if reference_entries and batch != 1:
             raise ValueError("the reference's paged attention entries share one slot table: batch 1")
+        # (slices of 32 while their workgroups fit the device's 256 CUs once; measured at the 30-layer model:
+        # batch 1 0.709 against 0.742 ms, 4 0.762 / 0.793, 8 0.873 / 0.856, 16 1.079 / 1.050)
+        self.ffn_slice = FFN_SLICE if config.mlp % FFN_SLICE == 0 and config.mlp // FFN_SLICE <= 48 and \
+            config.hidden <= 1024 and batch * (config.mlp // FFN_SLICE) <= 256 else 64
         can_fuse = (config.head_dim == 64 and config.hidden % 64 == 0 and config.hidden <= 1472 and
                     config.mlp % 64 == 0 and config.mlp // 64 <= 32)
         if fused and (reference_entries or not can_fuse):
@@ -202,7 +209,7 @@ class DecodeStep:
         }
         if self.fused:
             self.work["stream"] = create(batch * h * 2)
-            self.work["partials"] = create((c.mlp // 64) * batch * h * 4)
+            self.work["partials"] = create((c.mlp // self.ffn_slice) * batch * h * 4)
         if self.projecting:
             self.work["head_partials"] = create(c.q_heads * batch * h * 4)
         self.dispatches = self._build()
@@ -290,7 +297,7 @@ class DecodeStep:
         h, qd, kvd = c.hidden, c.q_heads * c.head_dim, c.kv_heads * c.head_dim
         group = (256, 1, 1)
         first, last = index == 0, index == c.layers - 1
-        slices = c.mlp // 64
+        slices = c.mlp // self.ffn_slice
         stream_in = w["x"][0] if first else w["x"][1]
         out = [("llmopt_rms_w4a16_qkv_rotary_pack_q8_f16_g64",
                 [stream_in, w["partials"], w["stream"], layer["attn_norm"], *layer["q"], *layer["k"], *layer["v"],
@@ -306,7 +313,7 @@ class DecodeStep:
             out.append(("llmopt_sum_rms_w4a16_swiglu_down_partial_f16_g64",
                         [w["stream"], w["head_partials"], w["x"][1], layer["ffn_norm"], *layer["gate"], *layer["up"],
                          *layer["down"], w["partials"]],
-                        ffn_params + u32s(c.q_heads), (slices * 256, m, 1), group))
+                        ffn_params + u32s(c.q_heads, self.ffn_slice), (slices * 256, m, 1), group))
             return out
         out.append(self._batched_attention(key_offset, value_offset))
         suffix, grid = self._linear_entry(h)
@@ -315,7 +322,7 @@ class DecodeStep:
         if not last:
             out.append(("llmopt_rms_w4a16_swiglu_down_partial_f16_g64",
                         [w["x"][1], layer["ffn_norm"], *layer["gate"], *layer["up"], *layer["down"], w["partials"]],
-                        ffn_params, (slices * 256, m, 1), group))
+                        ffn_params + u32s(self.ffn_slice), (slices * 256, m, 1), group))
             return out
         suffix, grid = self._linear_entry(c.mlp)
         out.append(("llmopt_rms_w4a16_dual_swiglu_f16_g64",

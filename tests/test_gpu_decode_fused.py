@@ -66,7 +66,9 @@ def pending_stream(rng, m, k, partial_count):
 
 @pytest.mark.parametrize("m,k,heads,partial_count", [(1, 576, (9, 3, 3), 0), (1, 576, (9, 3, 3), 24), (3, 576, (9, 3, 3), 24),
                                                      (8, 576, (9, 3, 3), 24), (5, 1024, (4, 2, 2), 7), (2, 2048, (2, 1, 1), 32),
-                                                     (40, 576, (9, 3, 3), 24), (37, 1536, (3, 1, 1), 3), (2, 64, (1, 1, 1), 1)]
+                                                     (40, 576, (9, 3, 3), 24), (37, 1536, (3, 1, 1), 3), (2, 64, (1, 1, 1), 1),
+                                                     (1, 576, (9, 3, 3), 48), (8, 576, (9, 3, 3), 48), (23, 576, (9, 3, 3), 48),
+                                                     (3, 1024, (4, 2, 2), 48)]
                          + DRAWN_QKV)
 def test_fused_qkv_rotary_pack_against_separate_launches_and_oracle(runtime, m, k, heads, partial_count):
     rng = np.random.default_rng(1000 * m + k + partial_count)
@@ -169,18 +171,21 @@ def test_fused_qkv_rotary_pack_against_separate_launches_and_oracle(runtime, m, 
 
 @pytest.mark.parametrize("m,n,k", [(1, 1536, 576), (2, 1536, 576), (8, 1536, 576), (33, 1536, 576), (3, 2048, 1024),
                                    (5, 128, 1408), (2, 64, 64), (4, 1024, 704)] + DRAWN_FFN)
-def test_fused_ffn_partial_sums_against_separate_launches_and_oracle(runtime, m, n, k):
+@pytest.mark.parametrize("width", [64, 32], ids=["slices_of_64", "slices_of_32"])
+def test_fused_ffn_partial_sums_against_separate_launches_and_oracle(runtime, m, n, k, width):
+    if n // width > 48:
+        pytest.skip("more slices than a reader takes partial sums")
     rng = np.random.default_rng(7 * m + n + k)
     x = rng.standard_normal((m, k)).astype(np.float16)
     gain = rng.uniform(0.5, 1.5, k).astype(np.float16)
     gate, up, down = random_w4(rng, n, k), random_w4(rng, n, k), random_w4(rng, k, n)
     b = runtime.buffer_of_bytes
     device = [b(a) for pair in (gate, up, down) for a in pair]
-    slices = n // 64
+    slices = n // width
     partials = b(np.full(slices * m * k, np.nan, dtype=np.float32))
     params = u32s(m, n, k) + struct.pack("<f", 1e-5)
-    runtime.dispatch("llmopt_rms_w4a16_swiglu_down_partial_f16_g64", [b(x), b(gain), *device, partials], params,
-                     grid=(256, 1, 1), group=GROUP)
+    runtime.dispatch("llmopt_rms_w4a16_swiglu_down_partial_f16_g64", [b(x), b(gain), *device, partials],
+                     params + u32s(width), grid=(256, 1, 1), group=GROUP)
     got_partials = partials.numpy(np.float32, (slices, m, k))
     assert np.all(np.isfinite(got_partials))
     total = np.zeros((m, k), dtype=np.float32)
@@ -202,29 +207,38 @@ def test_fused_ffn_partial_sums_against_separate_launches_and_oracle(runtime, m,
                                        oracle.w4a16_linear(normalised, *up, None)))
     want = oracle.add(oracle.w4a16_linear(want_product, *down, None), x.astype(np.float32))
     assert_close_to_oracle(got, want, "vs oracle")
-    # every partial sum is its own 64 columns of the contraction
+    # every partial sum is its own slice of the contraction (slices of 32: half a scale group, the group's scale)
     for p in sorted({0, slices // 2, slices - 1}):
-        columns = slice(64 * p, 64 * p + 64)
-        packed = np.ascontiguousarray(down[0][:, 32 * p:32 * p + 32])
-        want_partial = oracle.w4a16_linear(want_product[:, columns], packed, np.ascontiguousarray(down[1][:, p:p + 1]), None)
+        columns = slice(width * p, width * p + width)
+        packed = np.ascontiguousarray(down[0][:, width // 2 * p:width // 2 * p + width // 2])
+        scale = np.ascontiguousarray(down[1][:, width * p // 64:width * p // 64 + 1])
+        if width == 32:  # as a 64-wide group whose other half is zero
+            packed = np.concatenate([packed, np.zeros_like(packed)], axis=1)
+            padded_product = np.concatenate([want_product[:, columns], np.zeros((m, 32), dtype=np.float16)], axis=1)
+            want_partial = oracle.w4a16_linear(padded_product, packed, scale, None)
+        else:
+            want_partial = oracle.w4a16_linear(want_product[:, columns], packed, scale, None)
         error = np.linalg.norm(got_partials[p] - want_partial) / max(np.linalg.norm(want_partial), 1e-30)
         assert error <= 2e-3, f"partial sum {p}: {error:.3e}"  # the product's half rounding carries over
 
 
 @pytest.mark.parametrize("m,n,k,pending", [(1, 1536, 576, 9), (2, 1536, 576, 9), (8, 1536, 576, 9), (5, 128, 1024, 32),
                                            (3, 256, 704, 1), (16, 1536, 576, 9), (4, 64, 576, 0)] + DRAWN_SUMMING)
-def test_summing_ffn_forms_the_stream_and_leaves_the_partial_sums_of_the_plain_entry(runtime, m, n, k, pending):
+@pytest.mark.parametrize("width", [64, 32], ids=["slices_of_64", "slices_of_32"])
+def test_summing_ffn_forms_the_stream_and_leaves_the_partial_sums_of_the_plain_entry(runtime, m, n, k, pending, width):
+    if n // width > 48:
+        pytest.skip("more slices than a reader takes partial sums")
     rng = np.random.default_rng(11 * m + n + k + pending)
     x, pending_sums, stream = pending_stream(rng, m, k, pending)
     gain = rng.uniform(0.5, 1.5, k).astype(np.float16)
     b = runtime.buffer_of_bytes
     device = [b(a) for pair in (random_w4(rng, n, k), random_w4(rng, n, k), random_w4(rng, k, n)) for a in pair]
-    slices = n // 64
+    slices = n // width
     params = u32s(m, n, k) + struct.pack("<f", 1e-5)
     stream_out = b(np.full(m * k, np.nan, dtype=np.float16))
     partials = b(np.full(slices * m * k, np.nan, dtype=np.float32))
     runtime.dispatch("llmopt_sum_rms_w4a16_swiglu_down_partial_f16_g64",
-                     [b(x), b(pending_sums), stream_out, b(gain), *device, partials], params + u32s(pending),
+                     [b(x), b(pending_sums), stream_out, b(gain), *device, partials], params + u32s(pending, width),
                      grid=(256, 1, 1), group=GROUP)
     got_stream = stream_out.numpy(np.float16, (m, k))
     assert np.all(np.isfinite(got_stream))
@@ -234,8 +248,8 @@ def test_summing_ffn_forms_the_stream_and_leaves_the_partial_sums_of_the_plain_e
     assert np.mean(got_stream != stream) < 0.01
     # the plain entry on the stream this launch formed: the same kernel from there on, bit for bit
     plain = b(np.full(slices * m * k, np.nan, dtype=np.float32))
-    runtime.dispatch("llmopt_rms_w4a16_swiglu_down_partial_f16_g64", [b(got_stream), b(gain), *device, plain], params,
-                     grid=(256, 1, 1), group=GROUP)
+    runtime.dispatch("llmopt_rms_w4a16_swiglu_down_partial_f16_g64", [b(got_stream), b(gain), *device, plain],
+                     params + u32s(width), grid=(256, 1, 1), group=GROUP)
     np.testing.assert_array_equal(partials.numpy(np.uint32, (slices, m, k)), plain.numpy(np.uint32, (slices, m, k)))
 
 
@@ -310,7 +324,10 @@ def test_fused_entries_reject_what_they_cannot_take(runtime):
     any_buffer = b(np.zeros(4096, dtype=np.uint8))
     with pytest.raises(LlmoptError, match="k <= 1472,"):
         runtime.dispatch("llmopt_rms_w4a16_swiglu_down_partial_f16_g64", [any_buffer] * 9,
-                         u32s(1, 64, 4096) + struct.pack("<f", 1e-5), grid=(256, 1, 1), group=GROUP)
+                         u32s(1, 64, 4096) + struct.pack("<f", 1e-5) + u32s(64), grid=(256, 1, 1), group=GROUP)
+    with pytest.raises(LlmoptError, match="slices of 32 or 64"):
+        runtime.dispatch("llmopt_rms_w4a16_swiglu_down_partial_f16_g64", [any_buffer] * 9,
+                         u32s(1, 64, 64) + struct.pack("<f", 1e-5) + u32s(48), grid=(256, 1, 1), group=GROUP)
     with pytest.raises(LlmoptError, match="whole heads of 64"):
         runtime.dispatch("llmopt_rms_w4a16_qkv_rotary_pack_q8_f16_g64", [any_buffer] * 16,
                          u32s(1, 64, 64, 32, 32) + struct.pack("<f", 1e-5) + u32s(0, 0, 64, 128, 132),
@@ -320,9 +337,9 @@ def test_fused_entries_reject_what_they_cannot_take(runtime):
         runtime.dispatch("llmopt_attention_q8_paged_batched_w4a16_partial_g64", [big] * 11,
                          struct.pack("<12IfIII", 1, 1, 1, 0, 64, 0, 0, 128, 0, 64, 64, 132, 0.125, 1, 0, 0) + u32s(10, 64),
                          grid=(256, 1, 1), group=GROUP)
-    with pytest.raises(LlmoptError, match="at most 32 pending"):
+    with pytest.raises(LlmoptError, match="at most 48 pending"):
         runtime.dispatch("llmopt_sum_rms_w4a16_swiglu_down_partial_f16_g64", [any_buffer] * 11,
-                         u32s(1, 64, 64) + struct.pack("<f", 1e-5) + u32s(33), grid=(256, 1, 1), group=GROUP)
+                         u32s(1, 64, 64) + struct.pack("<f", 1e-5) + u32s(49, 64), grid=(256, 1, 1), group=GROUP)
     with pytest.raises(LlmoptError, match="two buffers"):
         big = b(np.zeros(1 << 16, dtype=np.uint8))
         runtime.dispatch("llmopt_rms_w4a16_qkv_rotary_pack_q8_f16_g64", [big] * 16,
