@@ -578,7 +578,8 @@ __global__ __launch_bounds__(kMergeSlices *D) void q8_attention_merge_kernel(Q8A
   // (chunk tid, tid + THREADS, ...), the first kAhead chunks of this thread's slice of the
   // weighted sum, the current token - so the kernel waits for memory once, not once per phase.
   constexpr int PER = kMaxSplitChunks / THREADS;  // chunks of phase 1 per thread
-  constexpr int kAhead = 8;
+  // (heads of 64: sixteen, so that the 64 chunks of a lone sequence of 2048 tokens are one trip to memory, not two)
+  constexpr int kAhead = D <= 64 ? 16 : 8;
   static_assert(PER * THREADS == kMaxSplitChunks, "phase 1 covers every chunk once");
   float chunk_max[PER], chunk_denominator[PER];
 #pragma unroll
