@@ -90,6 +90,52 @@ def test_decode_step_matches_oracle_chain(runtime, batch, lengths, launches):
     np.testing.assert_array_equal(got_pool[untouched], want_pool[untouched])
 
 
+@pytest.mark.parametrize("shape", [dict(hidden=256, q_heads=4, kv_heads=2, mlp=512), dict(hidden=1024, q_heads=16, kv_heads=4, mlp=2048),
+                                   dict(hidden=128, q_heads=2, kv_heads=2, mlp=1536), dict(hidden=704, q_heads=8, kv_heads=1, mlp=960)],
+                         ids=["256x512", "1024x2048", "128x1536", "704x960"])
+@pytest.mark.parametrize("launches", [6, 4, 3])
+def test_decode_step_of_other_models_matches_oracle_chain(runtime, shape, launches):
+    """The three launch forms on models other than the benchmark's: other widths, head counts and group
+    sizes (one KV head for eight query heads; as many KV heads as query heads), an FFN too wide for
+    slices of 32 columns (2048 / 32 = 64 partial sums) and one where they apply at every batch here."""
+    from llmopt_amd.decode_step import DecodeConfig, DecodeStep, random_weights
+    config = DecodeConfig(layers=2, vocabulary=512, **shape)
+    batch, lengths = 3, [90, 7, 140]
+    rng = np.random.default_rng(config.hidden + launches)
+    weights = random_weights(config, rng)
+    total = sum(lengths)
+    capacity = total + batch + 2
+    order = rng.permutation(capacity).astype(np.uint32)
+    slots, new_slots = order[:total], order[total:total + batch]
+    offsets = np.concatenate([[0], np.cumsum(lengths)[:-1]]).astype(np.uint32)
+    stride, elements = config.token_stride, config.token_elements
+    pool = np.zeros((capacity, stride), dtype=np.uint8)
+    pool[:, :elements] = np.clip(np.rint(rng.standard_normal((capacity, elements)) * 38), -127, 127) \
+        .astype(np.int8).view(np.uint8)
+    pool[:, elements:] = rng.uniform(0.02, 0.035, (capacity, elements // 64)).astype(np.float16) \
+        .view(np.uint8).reshape(capacity, -1)
+    pool = pool.reshape(-1)
+    tokens = rng.integers(0, config.vocabulary, batch)
+    device_pool = runtime.buffer_of_bytes(pool)
+    step = DecodeStep(runtime, config, weights, batch, device_pool, runtime.buffer_of_bytes(slots), offsets, lengths,
+                      new_slots, lengths, fused=launches < 6, projecting=launches == 3)
+    assert len(step.dispatches) == {6: 14, 4: 11, 3: 10}[launches]
+    got_tokens = step.run(tokens)
+    got_hidden = step.work["x"][0].numpy(np.float16, (batch, config.hidden))
+    hidden, logits, expected_pool = oracle_step(config, weights, pool, slots, offsets, lengths, new_slots, lengths, tokens)
+    assert_close_to_oracle(got_hidden, hidden, "hidden state after the last layer", rel_l2_tol=4e-3)
+    rms = float(np.sqrt(np.mean(logits.astype(np.float64) ** 2)))
+    for b in range(batch):
+        assert float(logits[b, got_tokens[b]]) >= float(logits[b].max()) - 2e-2 * rms
+    got_pool = device_pool.numpy(np.uint8, (capacity, stride))
+    want_pool = expected_pool.reshape(capacity, stride)
+    difference = got_pool[new_slots, :elements].view(np.int8).astype(np.int32) - \
+        want_pool[new_slots, :elements].view(np.int8).astype(np.int32)
+    assert np.abs(difference).max() <= 1
+    untouched = np.setdiff1d(np.arange(capacity), new_slots)
+    np.testing.assert_array_equal(got_pool[untouched], want_pool[untouched])
+
+
 @pytest.mark.parametrize("batch", [4, 8])
 def test_batched_decode_continues_from_prefilled_sequences(runtime, batch):
     """Every sequence of a batch is prefilled by its own PrefillStep into one shared pool; one
