@@ -451,7 +451,7 @@ def pool_block(rng, config, context):
     return block
 
 
-def verify_decode_chain(runtime, batch, context, rng, fused=None, projecting=None):
+def verify_decode_chain(runtime, batch, context, rng, fused=None, projecting=None, fused_qkv=None):
     """Checker: a two-layer copy of the timed decode step (same batch, same context, same kernels
     per layer; vocabulary 2048) against the oracle's chain on up to six of its sequences."""
     from llmopt_amd.decode_step import DecodeConfig, DecodeStep, random_weights
@@ -461,7 +461,8 @@ def verify_decode_chain(runtime, batch, context, rng, fused=None, projecting=Non
     block = pool_block(rng, small, context)
     pool, slots, offsets, new_slots = decode_inputs(runtime, small, batch, context, block)
     step = DecodeStep(runtime, small, weights, batch, pool, runtime.buffer_of_bytes(slots), offsets,
-                      [context] * batch, new_slots, [context] * batch, fused=fused, projecting=projecting)
+                      [context] * batch, new_slots, [context] * batch, fused=fused, projecting=projecting,
+                      fused_qkv=fused_qkv)
     tokens = rng.integers(0, small.vocabulary, batch)
     got_tokens = step.run(tokens)
     got_hidden = step.work["x"][0].numpy(np.float16, (batch, small.hidden)).astype(np.float64)
@@ -481,7 +482,8 @@ def verify_decode_chain(runtime, batch, context, rng, fused=None, projecting=Non
     return bool(np.all(np.isfinite(got_hidden)) and rel_l2 <= 4e-3 and tokens_ok), rel_l2, len(sample)
 
 
-def bench_decode_step(runtime, batches=(1, 8, 32, 128), context=2048, use_graph=True, fused=None, projecting=None):
+def bench_decode_step(runtime, batches=(1, 8, 32, 128), context=2048, use_graph=True, fused=None, projecting=None,
+                      fused_qkv=None):
     """C5: one decode step of the 30-layer model (hidden 576, 9/3 heads of 64, MLP 1536,
     vocabulary 49152), every sequence with `context` tokens in the Q8 pool, replayed as a
     HIP graph.  tokens/s = batch / step time.  Checked outside the timed region: what the replayed
@@ -498,7 +500,8 @@ def bench_decode_step(runtime, batches=(1, 8, 32, 128), context=2048, use_graph=
         # (a step that picks six launches a layer by itself has no projecting form to force)
         step_projecting = None if projecting and fused is None and batch > FUSED_MAX_BATCH else projecting
         step = DecodeStep(runtime, config, weights, batch, pool, runtime.buffer_of_bytes(slots), offsets,
-                          [context] * batch, new_slots, [context] * batch, fused=fused, projecting=step_projecting)
+                          [context] * batch, new_slots, [context] * batch, fused=fused, projecting=step_projecting,
+                          fused_qkv=None if fused_qkv and (fused or (fused is None and batch <= FUSED_MAX_BATCH)) else fused_qkv)
         tokens = rng.integers(0, config.vocabulary, batch)
         eager_tokens = step.run(tokens)  # first-use allocations; and the eager result the replay must repeat
         eager_hidden = step.work["x"][0].numpy(np.uint16, (batch, config.hidden))
@@ -531,11 +534,12 @@ def bench_decode_step(runtime, batches=(1, 8, 32, 128), context=2048, use_graph=
             single = plan.single_submission
             del plan
         launches, weight_bytes, kv_bytes = len(step.dispatches), step.weight_bytes(), step.kv_bytes()
-        fused_step, projecting_step = step.fused, step.projecting
+        fused_step, projecting_step, fused_qkv_step = step.fused, step.projecting, step.fused_qkv
         del step, pool
-        chain_ok, chain_rel_l2, chain_sequences = verify_decode_chain(runtime, batch, context, rng, fused_step, projecting_step)
+        chain_ok, chain_rel_l2, chain_sequences = verify_decode_chain(runtime, batch, context, rng, fused_step, projecting_step,
+                                                                      fused_qkv_step)
         results.append({"batch": batch, "context": context, "launches": launches,
-                        "launches_per_layer": 3 if projecting_step else 4 if fused_step else 6,
+                        "launches_per_layer": 3 if projecting_step else 4 if fused_step else 5 if fused_qkv_step else 6,
                         "ms_per_step": round(ms, 4), "tokens_per_s": round(batch / (ms * 1e-3), 1),
                         "prebaked_execute_wall_ms": None if execute_ms is None else round(execute_ms, 4),
                         "prebaked_execute_tokens_per_s": None if execute_ms is None
@@ -768,6 +772,9 @@ def main():
     parser.add_argument("--decode-batches", default="1,8,32,128", help="batch sizes of the decode-step extra")
     parser.add_argument("--decode-fused", choices=("auto", "on", "off"), default="auto",
                         help="the decode step as four launches a layer (on), six (off), or whichever the step picks")
+    parser.add_argument("--decode-fused-qkv", choices=("auto", "on", "off"), default="auto",
+                        help="a decode step that is not fused takes the fused QKV launch in front of the reference's "
+                             "entries (five launches a layer), or not (six)")
     parser.add_argument("--decode-projecting", choices=("auto", "on", "off"), default="auto",
                         help="a fused decode step's attention launch multiplies its heads into the output projection "
                              "(three launches a layer), or not (four)")
@@ -834,7 +841,8 @@ def main():
         extras["decode_step"] = bench_decode_step(
             runtime, batches=tuple(int(b) for b in args.decode_batches.split(",")), use_graph=not args.decode_eager,
             fused={"auto": None, "on": True, "off": False}[args.decode_fused],
-            projecting={"auto": None, "on": True, "off": False}[args.decode_projecting])
+            projecting={"auto": None, "on": True, "off": False}[args.decode_projecting],
+            fused_qkv={"auto": None, "on": True, "off": False}[args.decode_fused_qkv])
     if "prefill" in wanted:
         extras["prefill_step"] = bench_prefill(runtime)
     # refuse to print numbers whose outputs did not match the oracle

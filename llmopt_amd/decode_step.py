@@ -29,12 +29,14 @@ import numpy as np
 from .native import Buffer, Runtime
 
 
-# Above this many sequences the fused launches (one or two sequences per workgroup, every workgroup
-# reading and decoding its weights again) cost more than the launches they save: measured at 2048
-# tokens of context, ms per step as three launches a layer / as six: batch 1 0.742 / 0.794, 2 0.785 / 0.977,
-# 8 0.856 / 1.048, 12 1.011 / 1.072, 16 1.050 / 1.136, 20 1.161 / 1.260, 24 1.292 / 1.279, 28 1.313 / 1.299,
-# 32 1.361 / 1.321.
-FUSED_MAX_BATCH = 20
+# Up to this many sequences a step takes the fused layer of three launches; above it every workgroup
+# re-reading and re-decoding its weights per sequence costs more than the launches saved, and the step takes
+# five launches a layer (the fused QKV launch in front of the reference's entries).  Measured at 2048 tokens
+# of context, ms per step as three / five / six launches a layer: batch 1 0.703 / - / 0.794, 6 0.814 / 0.914 /
+# -, 8 0.828 / 0.926 / 1.048, 10 0.908 / 0.966 / -, 12 1.014 / 0.988 / 1.077, 14 1.040 / 1.023 / -,
+# 16 1.050 / 1.048 / 1.141, 20 1.161 / 1.168 / 1.263, 24 1.292 / 1.187 / 1.280, 32 1.361 / 1.232 / 1.324,
+# 64 - / 1.705 / 1.890, 128 - / 2.722 / 2.759.
+FUSED_MAX_BATCH = 10
 # The attention launch multiplies its heads into the output projection where it can (three launches a
 # layer instead of four: batch 1 0.742 against 0.771 ms, 8 0.856 / 0.907, 16 1.052 / 1.096, 32 1.364 / 1.379).
 PROJECTING_ATTENTION = True
@@ -142,7 +144,7 @@ class DecodeStep:
     def __init__(self, runtime: Runtime, config: DecodeConfig, weights: dict, batch: int, pool: Buffer,
                  slots: Buffer, slot_offsets, past_lengths, new_slots, positions, max_context=None,
                  slots_host=None, reference_entries: bool = False, fused: bool | None = None,
-                 projecting: bool | None = None):
+                 projecting: bool | None = None, fused_qkv: bool | None = None):
         """max_context: the longest context any later step will have (sizes the attention launch;
         default: the longest now).  slots_host: the host copy of the slot table, with room behind
         every sequence's slots for the tokens `advance` will add.  reference_entries (batch 1):
@@ -153,7 +155,11 @@ class DecodeStep:
         + cache pack as one launch, attention, output projection, and the SwiGLU FFN as one that leaves
         partial sums for the next layer's first launch - four launches a layer instead of six; three
         where the attention launch can multiply its heads into the output projection itself
-        (`self.projecting`: contexts of 64 tokens and more, hidden <= 1024, at most 32 query heads)."""
+        (`self.projecting`: contexts of 64 tokens and more, hidden <= 1024, at most 32 query heads).
+        fused_qkv (a step that is not `fused`; default: whenever the shapes allow): the first of those launches
+        in front of the reference's entries for the rest of the layer - five launches a layer, which is what
+        larger batches take (measured against six: 1.188 / 1.280 ms at batch 24, 1.232 / 1.324 at 32,
+        1.705 / 1.890 at 64, 2.722 / 2.759 at 128)."""
         self.runtime, self.config, self.batch = runtime, config, batch
         self.reference_entries = reference_entries
         if reference_entries and batch != 1:
@@ -167,6 +173,11 @@ class DecodeStep:
         if fused and (reference_entries or not can_fuse):
             raise ValueError("the fused launches take heads of 64, hidden <= 1472 and mlp <= 2048")
         self.fused = can_fuse and not reference_entries and batch <= FUSED_MAX_BATCH if fused is None else fused
+        can_fuse_qkv = (not self.fused and not reference_entries and config.head_dim == 64 and config.hidden % 64 == 0 and
+                        config.hidden <= 2048)
+        if fused_qkv and not can_fuse_qkv:
+            raise ValueError("the fused QKV launch takes a step that is not fused, heads of 64 and hidden <= 2048")
+        self.fused_qkv = can_fuse_qkv if fused_qkv is None else fused_qkv
         self.max_past = int(max(past_lengths)) if max_context is None else int(max_context)
         can_project = bool(self.fused and self.max_past >= 64 and config.hidden <= 1024 and config.q_heads <= 32)
         if projecting and not can_project:
@@ -207,8 +218,9 @@ class DecodeStep:
             "attention": create(q_bytes),
             "product": create(batch * c.mlp * 2),
         }
-        if self.fused:
+        if self.fused or self.fused_qkv:
             self.work["stream"] = create(batch * h * 2)
+        if self.fused:
             self.work["partials"] = create((c.mlp // self.ffn_slice) * batch * h * 4)
         if self.projecting:
             self.work["head_partials"] = create(c.q_heads * batch * h * 4)
@@ -236,6 +248,28 @@ class DecodeStep:
             value_offset = key_offset + kvd
             if self.fused:
                 out += self._fused_layer(index, layer, key_offset, value_offset)
+                continue
+            if self.fused_qkv:
+                # norm + QKV + rotation + cache pack as one launch (no pending sums: the stream is whole; the
+                # copy of it that the launch writes is not read), the rest as the reference's entries
+                out.append(("llmopt_rms_w4a16_qkv_rotary_pack_q8_f16_g64",
+                            [x_in, x_in, w["stream"], layer["attn_norm"], *layer["q"], *layer["k"], *layer["v"],
+                             self.trig, w["q_rot"], w["k_rot"], w["v"], self.new_slots, self.pool],
+                            u32s(m, h, qd, kvd, kvd) + struct.pack("<f", c.epsilon) +
+                            u32s(0, key_offset, value_offset, c.token_elements, c.token_stride),
+                            (((qd + 2 * kvd) // 64) * 256, m, 1), group))
+                out.append(self._batched_attention(key_offset, value_offset))
+                suffix, grid = self._linear_entry(h)
+                out.append(("llmopt_w4a16_linear_f16_g64" + suffix,
+                            [w["attention"], *layer["o"], x_in, x_mid], u32s(m, h, qd, 1, h), grid, group))
+                ffn_params = u32s(m, c.mlp, h) + struct.pack("<f", c.epsilon)
+                suffix, grid = self._linear_entry(c.mlp)
+                out.append(("llmopt_rms_w4a16_dual_swiglu_f16_g64",
+                            [x_mid, layer["ffn_norm"], *layer["gate"], *layer["up"], w["product"]], ffn_params, grid,
+                            group))
+                suffix, grid = self._linear_entry(h)
+                out.append(("llmopt_w4a16_down_add_f16_g64" + suffix,
+                            [w["product"], *layer["down"], x_mid, x_in], ffn_params, grid, group))
                 continue
             # each RMSNorm rides in the projection launch that reads it
             suffix, grid = self._linear_entry(qd + 2 * kvd)

@@ -372,17 +372,19 @@ def test_fused_step_leaves_what_the_unfused_step_leaves(runtime, batch):
     tokens = rng.integers(0, config.vocabulary, batch)
     results = {}
     # six launches a layer, four, and three (the last layer of a fused step: five)
-    launches = {"unfused": 2 + 6 * config.layers, "fused": 2 + 4 * config.layers + 1, "projecting": 2 + 3 * (config.layers - 1) + 5}
+    launches = {"unfused": 2 + 6 * config.layers, "fused_qkv": 2 + 5 * config.layers, "fused": 2 + 4 * config.layers + 1,
+                "projecting": 2 + 3 * (config.layers - 1) + 5}
     for mode in launches:
         device_pool = runtime.buffer_of_bytes(pool)
         step = DecodeStep(runtime, config, weights, batch, device_pool, runtime.buffer_of_bytes(slots), offsets,
-                          lengths, new_slots, lengths, fused=mode != "unfused", projecting=mode == "projecting")
-        assert step.fused == (mode != "unfused") and step.projecting == (mode == "projecting")
+                          lengths, new_slots, lengths, fused=mode in ("fused", "projecting"), projecting=mode == "projecting",
+                          fused_qkv=mode == "fused_qkv")
+        assert step.fused == (mode in ("fused", "projecting")) and step.projecting == (mode == "projecting")
         assert len(step.dispatches) == launches[mode]
         got_tokens = step.run(tokens)
         results[mode] = (got_tokens, step.work["x"][0].numpy(np.float16, (batch, config.hidden)),
                          device_pool.numpy(np.uint8, (capacity, stride)))
-    for mode in ("fused", "projecting"):
+    for mode in ("fused_qkv", "fused", "projecting"):
         assert_close_to_oracle(results[mode][1], results["unfused"][1].astype(np.float32), f"{mode} vs unfused hidden state",
                                rel_l2_tol=2e-3)
         difference = results[mode][2][:, :elements].view(np.int8).astype(np.int32) - \

@@ -30,7 +30,8 @@ def ragged_lengths(batch, seed):
 # itself), 9-32 its row-grouped form: batch 8 and 32 are the sizes the decode-step benchmark times.
 @pytest.mark.parametrize("batch,lengths", [(1, [37]), (1, [77]), (2, [130, 9]), (3, [64, 5, 300]), (8, ragged_lengths(8, 5)),
                                            (32, ragged_lengths(32, 6))])
-@pytest.mark.parametrize("launches", [6, 4, 3], ids=["six_launches_a_layer", "four_launches_a_layer", "three_launches_a_layer"])
+@pytest.mark.parametrize("launches", [6, 5, 4, 3], ids=["six_launches_a_layer", "five_launches_a_layer", "four_launches_a_layer",
+                                                        "three_launches_a_layer"])
 def test_decode_step_matches_oracle_chain(runtime, batch, lengths, launches):
     from llmopt_amd.decode_step import DecodeConfig, DecodeStep, random_weights
     if launches == 3 and max(lengths) < 64:
@@ -55,8 +56,8 @@ def test_decode_step_matches_oracle_chain(runtime, batch, lengths, launches):
 
     device_pool = runtime.buffer_of_bytes(pool)
     step = DecodeStep(runtime, config, weights, batch, device_pool, runtime.buffer_of_bytes(slots), offsets,
-                      lengths, new_slots, positions, fused=launches < 6, projecting=launches == 3)
-    assert len(step.dispatches) == {6: 14, 4: 11, 3: 10}[launches]  # (the last layer of a fused step: five)
+                      lengths, new_slots, positions, fused=launches < 5, projecting=launches == 3, fused_qkv=launches == 5)
+    assert len(step.dispatches) == {6: 14, 5: 12, 4: 11, 3: 10}[launches]  # (the last layer of a fused step: five)
     got_tokens = step.run(tokens)
     got_hidden = step.work["x"][0].numpy(np.float16, (batch, config.hidden))
 
@@ -93,7 +94,7 @@ def test_decode_step_matches_oracle_chain(runtime, batch, lengths, launches):
 @pytest.mark.parametrize("shape", [dict(hidden=256, q_heads=4, kv_heads=2, mlp=512), dict(hidden=1024, q_heads=16, kv_heads=4, mlp=2048),
                                    dict(hidden=128, q_heads=2, kv_heads=2, mlp=1536), dict(hidden=704, q_heads=8, kv_heads=1, mlp=960)],
                          ids=["256x512", "1024x2048", "128x1536", "704x960"])
-@pytest.mark.parametrize("launches", [6, 4, 3])
+@pytest.mark.parametrize("launches", [6, 5, 4, 3])
 def test_decode_step_of_other_models_matches_oracle_chain(runtime, shape, launches):
     """The three launch forms on models other than the benchmark's: other widths, head counts and group
     sizes (one KV head for eight query heads; as many KV heads as query heads), an FFN too wide for
@@ -118,8 +119,8 @@ def test_decode_step_of_other_models_matches_oracle_chain(runtime, shape, launch
     tokens = rng.integers(0, config.vocabulary, batch)
     device_pool = runtime.buffer_of_bytes(pool)
     step = DecodeStep(runtime, config, weights, batch, device_pool, runtime.buffer_of_bytes(slots), offsets, lengths,
-                      new_slots, lengths, fused=launches < 6, projecting=launches == 3)
-    assert len(step.dispatches) == {6: 14, 4: 11, 3: 10}[launches]
+                      new_slots, lengths, fused=launches < 5, projecting=launches == 3, fused_qkv=launches == 5)
+    assert len(step.dispatches) == {6: 14, 5: 12, 4: 11, 3: 10}[launches]
     got_tokens = step.run(tokens)
     got_hidden = step.work["x"][0].numpy(np.float16, (batch, config.hidden))
     hidden, logits, expected_pool = oracle_step(config, weights, pool, slots, offsets, lengths, new_slots, lengths, tokens)
