@@ -8,6 +8,7 @@
 #include <cstring>
 
 #include "kernels/kernels.h"
+#include "kernels/kernels_internal.h"
 #include "runtime.h"
 
 namespace llmopt {
@@ -242,9 +243,12 @@ int lm_head(llmopt_hip_context *context, const DispatchRecord &record, LmHeadVar
   norm.epsilon = epsilon;
   if (int status = launched(launch_rms_norm_split(norm, context->stream), name)) return status;
 
-  // the decode GEMV keeps float32 results; more rows go through it in groups
-  for (uint32_t first = 0; first < gemv_rows; first += kGemvMaxRows) {
-    const uint32_t rows = std::min(kGemvMaxRows, gemv_rows - first);
+  // the decode GEMV keeps float32 results; more rows go through it in groups: of eight a launch, or - when one
+  // workgroup covers K, so that nothing is handed over between workgroups - up to 128 rows a launch as row groups
+  // of one grid (the 64 rows of 32 sequences at 49152 x 576: one launch instead of eight)
+  const uint32_t rows_per_launch = w4a16_gemv_mfma_needs_split(k) ? kGemvMaxRows : 128;
+  for (uint32_t first = 0; first < gemv_rows; first += rows_per_launch) {
+    const uint32_t rows = std::min(rows_per_launch, gemv_rows - first);
     W4LinearArgs linear = {};
     linear.x = normalized + (size_t)first * k;
     linear.w = {record.buffers[2].device, as_f16(record.buffers[3])};
@@ -259,7 +263,10 @@ int lm_head(llmopt_hip_context *context, const DispatchRecord &record, LmHeadVar
       linear.counters = context_counters(context, &linear.counter_count);
       if (linear.counters == nullptr) return LLMOPT_ERR_FAILURE;
     }
-    if (int status = launched(launch_w4a16_linear(linear, context->stream), name)) return status;
+    if (int status = launched(rows > kGemvMaxRows ? launch_w4a16_gemv_mfma_linear(linear, context->stream)
+                                                  : launch_w4a16_linear(linear, context->stream),
+                              name))
+      return status;
   }
   uint16_t *half_logits = variant.extra ? as_f16_out(record.buffers[5]) : nullptr;
   if (int status = launched(launch_argmax_candidates(logits, candidates, m, n, true, half_logits, context->stream),

@@ -375,7 +375,10 @@ def check_tokens(tokens, expected_logits):
     (2, 16400, 576, np.float16, True, False),   # a wide head with its logits
     (3, 2048, 640, np.float32, True, True),
     (8, 520, 2048, np.float16, False, False),
-    (11, 300, 128, np.float16, True, False),    # more rows than one GEMV launch takes
+    (11, 300, 128, np.float16, True, False),    # more rows than one GEMV launch of eight takes: three row groups
+    (32, 49152, 576, np.float16, False, False),  # the decode LM head at batch 32: 64 rows, eight row groups, one launch
+    (70, 1024, 576, np.float16, True, False),   # 140 rows: two launches of row groups
+    (9, 1040, 5120, np.float16, True, False),   # K split over workgroups: groups of eight rows, a launch each
 ])
 def test_lm_head_argmax(runtime, m, n, k, dtype, extra, staged):
     rng = np.random.default_rng(m * 7 + n)
