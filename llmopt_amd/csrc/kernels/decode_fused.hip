@@ -12,11 +12,13 @@
 //    group are its own, nothing is handed over between workgroups.
 //  * fused_ffn_kernel: llmopt_w4a16_swiglu_rms_f16_g64, llmopt_w4a16_dual_swiglu_f16_g64 and the
 //    contraction of llmopt_w4a16_down_add_f16_g64 (lib/metal_w4a16_source.ml:496-611).  Workgroup j
-//    owns 64 columns of the intermediate: gate and up for them, product = half(silu(gate) * up), and
-//    that product times its 64 columns of the down matrix - a partial sum of every output, float32.
-//    The sums over j and the residual are taken by whoever reads the stream next (the next layer's
-//    fused_qkv_kernel): every workgroup there adds the partial sums in the same fixed order, so the
-//    result does not depend on scheduling and no workgroup waits for another.
+//    owns a slice of 64 or 32 columns of the intermediate: gate and up for them, product =
+//    half(silu(gate) * up), and that product times its columns of the down matrix - a partial sum of
+//    every output, float32.  The sums over j and the residual are taken by whoever reads the stream
+//    next (the next layer's fused_qkv_kernel): every workgroup there adds the partial sums in the
+//    same fixed order, so the result does not depend on scheduling and no workgroup waits for
+//    another.  Its own input may arrive the same way (rows plus the partial sums the projecting
+//    attention merge left, one per head).
 //
 // What bounds a launch like these, measured with time stamps inside the kernels: the first trip to
 // memory (about 2 us: argument block, then weights / activations / partial sums, all requested
