@@ -28,7 +28,7 @@ def ragged_lengths(batch, seed):
 
 # Batch 1-2 run the register-activation GEMV, 3-8 the matrix-core GEMV (normalising its rows
 # itself), 9-32 its row-grouped form: batch 8 and 32 are the sizes the decode-step benchmark times.
-@pytest.mark.parametrize("batch,lengths", [(1, [37]), (1, [77]), (2, [130, 9]), (3, [64, 5, 300]), (8, ragged_lengths(8, 5)),
+@pytest.mark.parametrize("batch,lengths", [(1, [37]), (1, [77]), (2, [130, 9]), (3, [0, 70, 12]), (3, [64, 5, 300]), (8, ragged_lengths(8, 5)),
                                            (32, ragged_lengths(32, 6))])
 @pytest.mark.parametrize("launches", [6, 5, 4, 3], ids=["six_launches_a_layer", "five_launches_a_layer", "four_launches_a_layer",
                                                         "three_launches_a_layer"])
